@@ -1,0 +1,229 @@
+// C-ABI layer of libfdma_hip.so: argument validation, kernel-parameter set-up and dispatch.
+//
+// Host-side counterpart of mha_fwd / mha_bwd with set_params_fprop / set_params_dgrad
+// (csrc/flash_sparse_attn/flash_api.cpp:24-249, 351-554, 792-1050 of the reference).  The checks and
+// their messages follow the reference's TORCH_CHECKs so callers see the same errors; everything
+// torch-specific (allocation, device guard, current stream) stays with the caller.
+#include "../../include/fdma.h"
+
+#include <hip/hip_runtime.h>
+
+#include <cmath>
+#include <cstdarg>
+#include <cstdio>
+#include <cstring>
+
+#include "fdma_params.h"
+
+namespace {
+
+thread_local char g_err[512] = "";
+
+int fail(int code, const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_err, sizeof(g_err), fmt, ap);
+    va_end(ap);
+    return code;
+}
+
+inline int64_t round_up(int64_t x, int64_t m) { return (x + m - 1) / m * m; }
+
+inline bool aligned16(const void *p) { return (reinterpret_cast<uintptr_t>(p) & 15) == 0; }
+
+bool strides_ok(const int64_t s[3], int mult) {
+    for (int i = 0; i < 3; i++)
+        if (s[i] % mult != 0) return false;
+    return true;
+}
+
+// Shape / dtype / stride rules of flash_api.cpp:371-438 (forward) -- shared by backward (:824-898).
+int validate_common(const fdma_fwd_args *a, bool backward) {
+    if (!a) return fail(FDMA_ERR_INVALID, "args must not be NULL");
+    if (a->dtype != FDMA_DTYPE_BF16 && a->dtype != FDMA_DTYPE_FP16)
+        return fail(FDMA_ERR_INVALID, "FlashSparseAttention only support fp16 and bf16 data type");
+    if (a->batch <= 0) return fail(FDMA_ERR_INVALID, "batch size must be positive");
+    if (a->seqlen_q < 0 || a->seqlen_k < 0) return fail(FDMA_ERR_INVALID, "sequence lengths must be non-negative");
+    if (a->num_heads <= 0 || a->num_heads_k <= 0) return fail(FDMA_ERR_INVALID, "number of heads must be positive");
+    if (a->head_dim > 256)
+        return fail(FDMA_ERR_INVALID, "FlashSparseAttention %s only supports head dimension at most 256", backward ? "backward" : "forward");
+    if (a->head_dim <= 0 || a->head_dim % 8 != 0)
+        return fail(FDMA_ERR_INVALID, backward ? "head_size should be a multiple of 8"
+                                               : "query, key, value, and out_ must have a head_size that is a multiple of 8");
+    if (a->num_heads % a->num_heads_k != 0)
+        return fail(FDMA_ERR_INVALID, "Number of heads in key/value must divide number of heads in query");
+    if (!a->q || !a->k || !a->v) return fail(FDMA_ERR_INVALID, "q, k, v must be device pointers");
+    if (!a->out) return fail(FDMA_ERR_INVALID, "out must be a device pointer");
+    if (!a->lse) return fail(FDMA_ERR_INVALID, "softmax_lse must be a device pointer");
+    if (a->mask) {
+        const int hm = a->num_heads_mask;
+        if (!(hm == 1 || hm == a->num_heads_k || hm == a->num_heads))
+            return fail(FDMA_ERR_INVALID, "Number of heads in mask must be 1, h_k or h");
+        if (!aligned16(a->mask) || !strides_ok(a->mask_strides, 16))
+            return fail(FDMA_ERR_INVALID, "mask must be 16-byte aligned with strides that are multiples of 16 (pad the key dimension)");
+    }
+    if (a->bias) {
+        const int hb = a->num_heads_bias;
+        if (!(hb == 1 || hb == a->num_heads_k || hb == a->num_heads))
+            return fail(FDMA_ERR_INVALID, "Number of heads in bias must be 1, h_k or h");
+        if (!aligned16(a->bias) || !strides_ok(a->bias_strides, 8))
+            return fail(FDMA_ERR_INVALID, "bias must be 16-byte aligned with strides that are multiples of 8 (pad the key dimension)");
+    }
+    if (!aligned16(a->q) || !aligned16(a->k) || !aligned16(a->v) || !aligned16(a->out) || !strides_ok(a->q_strides, 8) ||
+        !strides_ok(a->k_strides, 8) || !strides_ok(a->v_strides, 8) || !strides_ok(a->o_strides, 8))
+        return fail(FDMA_ERR_INVALID, "q, k, v, out must be 16-byte aligned with strides that are multiples of 8 elements");
+    if (a->softcap != 0.f) return fail(FDMA_ERR_UNSUPPORTED, "softcap is not supported by this build");
+    if (a->head_dim > 128) return fail(FDMA_ERR_UNSUPPORTED, "head dimensions above 128 are not built yet (got %d)", a->head_dim);
+    if (!std::isfinite(a->softmax_scale)) return fail(FDMA_ERR_INVALID, "softmax_scale must be finite");
+    return FDMA_OK;
+}
+
+void fill_fwd_params(const fdma_fwd_args *a, fdma::FwdParams &p) {
+    std::memset(&p, 0, sizeof(p));
+    p.q = a->q; p.k = a->k; p.v = a->v;
+    p.mask = static_cast<const uint8_t *>(a->mask);
+    p.bias = a->bias;
+    p.o = a->out;
+    p.lse = a->lse;
+    p.q_b = a->q_strides[0]; p.q_r = a->q_strides[1]; p.q_h = a->q_strides[2];
+    p.k_b = a->k_strides[0]; p.k_r = a->k_strides[1]; p.k_h = a->k_strides[2];
+    p.v_b = a->v_strides[0]; p.v_r = a->v_strides[1]; p.v_h = a->v_strides[2];
+    p.o_b = a->o_strides[0]; p.o_r = a->o_strides[1]; p.o_h = a->o_strides[2];
+    if (a->mask) { p.m_b = a->mask_strides[0]; p.m_h = a->mask_strides[1]; p.m_r = a->mask_strides[2]; }
+    if (a->bias) { p.bi_b = a->bias_strides[0]; p.bi_h = a->bias_strides[1]; p.bi_r = a->bias_strides[2]; }
+    p.B = a->batch; p.Lq = a->seqlen_q; p.Lk = a->seqlen_k;
+    p.H = a->num_heads; p.Hk = a->num_heads_k;
+    p.Hm = a->mask ? a->num_heads_mask : 1;
+    p.Hb = a->bias ? a->num_heads_bias : 1;
+    p.d = a->head_dim;
+    // seqlen_q == 1 makes causal a no-op (flash_api.cpp:441)
+    p.causal = (a->is_causal && a->seqlen_q != 1) ? 1 : 0;
+    p.scale = a->softmax_scale;
+    p.scale_log2 = a->softmax_scale * 1.4426950408889634f;
+    p.splits = 1;
+}
+
+}  // namespace
+
+extern "C" {
+
+const char *fdma_last_error(void) { return g_err; }
+int fdma_abi_version(void) { return FDMA_ABI_VERSION; }
+size_t fdma_sizeof_fwd_args(void) { return sizeof(fdma_fwd_args); }
+size_t fdma_sizeof_bwd_args(void) { return sizeof(fdma_bwd_args); }
+
+int fdma_fwd_validate(const fdma_fwd_args *a) {
+    g_err[0] = 0;
+    return validate_common(a, false);
+}
+
+size_t fdma_fwd_workspace_bytes(const fdma_fwd_args *a) {
+    if (!a) return 0;
+    if (!fdma::use_decode_path(a->seqlen_q, a->num_heads, a->num_heads_k)) return 0;
+    const int splits = fdma::decode_num_splits(a->batch, a->num_heads_k, a->seqlen_k);
+    if (splits <= 1) return 0;
+    const size_t rows = (size_t)splits * a->batch * a->num_heads * a->seqlen_q;
+    return rows * (size_t)(a->head_dim + 1) * sizeof(float);
+}
+
+int fdma_fwd(const fdma_fwd_args *a, void *hip_stream) {
+    g_err[0] = 0;
+    int rc = validate_common(a, false);
+    if (rc != FDMA_OK) return rc;
+    fdma::FwdParams p;
+    fill_fwd_params(a, p);
+    hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    hipError_t e;
+    if (a->seqlen_q == 0) return FDMA_OK;
+    if (fdma::use_decode_path(a->seqlen_q, a->num_heads, a->num_heads_k) && a->seqlen_k > 0) {
+        p.splits = fdma::decode_num_splits(a->batch, a->num_heads_k, a->seqlen_k);
+        if (p.splits > 1) {
+            const size_t need = fdma_fwd_workspace_bytes(a);
+            if (!a->workspace || a->workspace_bytes < need)
+                return fail(FDMA_ERR_WORKSPACE, "forward workspace too small: need %zu bytes, got %zu", need, a->workspace_bytes);
+            const size_t rows = (size_t)p.splits * a->batch * a->num_heads * a->seqlen_q;
+            p.o_part = static_cast<float *>(a->workspace);
+            p.lse_part = p.o_part + rows * a->head_dim;
+        }
+        e = fdma::launch_fwd_decode(p, a->dtype, stream);
+    } else {
+        // seqlen_k == 0 falls out of the kernel as O = 0, LSE = +inf (flash_api.cpp:535-539)
+        e = fdma::launch_fwd(p, a->dtype, stream);
+    }
+    if (e != hipSuccess) return fail(FDMA_ERR_LAUNCH, "forward launch failed: %s", hipGetErrorString(e));
+    return FDMA_OK;
+}
+
+int fdma_bwd_validate(const fdma_bwd_args *a) {
+    g_err[0] = 0;
+    if (!a) return fail(FDMA_ERR_INVALID, "args must not be NULL");
+    int rc = validate_common(&a->f, true);
+    if (rc != FDMA_OK) return rc;
+    if (!a->dout || !a->dq || !a->dk || !a->dv) return fail(FDMA_ERR_INVALID, "dout, dq, dk, dv must be device pointers");
+    if (!a->softmax_d) return fail(FDMA_ERR_INVALID, "softmax_d must be a device pointer");
+    if ((a->f.bias != nullptr) != (a->dbias != nullptr))
+        return fail(FDMA_ERR_INVALID, "dbias must be given exactly when bias is given");
+    if (!aligned16(a->dout) || !aligned16(a->dq) || !aligned16(a->dk) || !aligned16(a->dv) || !strides_ok(a->do_strides, 8) ||
+        !strides_ok(a->dq_strides, 8) || !strides_ok(a->dk_strides, 8) || !strides_ok(a->dv_strides, 8))
+        return fail(FDMA_ERR_INVALID, "dout, dq, dk, dv must be 16-byte aligned with strides that are multiples of 8 elements");
+    if (a->dbias) {
+        if (!aligned16(a->dbias) || !strides_ok(a->dbias_strides, 8))
+            return fail(FDMA_ERR_INVALID, "dbias must be 16-byte aligned with strides that are multiples of 8");
+        for (int i = 0; i < 3; i++)
+            if ((a->dbias_strides[i] == 0) != (a->f.bias_strides[i] == 0))
+                return fail(FDMA_ERR_INVALID, "dbias must have the broadcast pattern of bias");
+    }
+    return FDMA_OK;
+}
+
+// fp32 accumulation scratch for dbias when several workgroups add into one dbias element:
+// bias broadcast over batch (with batch > 1) or over kv-head groups (bias heads == 1 < Hk).
+static bool dbias_shared(const fdma_bwd_args *a) {
+    if (!a->dbias) return false;
+    const bool batch_bcast = a->f.batch > 1 && a->f.bias_strides[0] == 0;
+    const bool head_bcast = a->f.num_heads_bias == 1 && a->f.num_heads_k > 1;
+    return batch_bcast || head_bcast;
+}
+
+static size_t dbias_accum_elems(const fdma_bwd_args *a) {
+    const size_t nb = a->f.bias_strides[0] == 0 ? 1 : a->f.batch;
+    const size_t nr = a->f.bias_strides[2] == 0 ? 1 : a->f.seqlen_q;
+    return nb * a->f.num_heads_bias * nr * (size_t)round_up(a->f.seqlen_k, 8);
+}
+
+size_t fdma_bwd_workspace_bytes(const fdma_bwd_args *a) {
+    if (!a) return 0;
+    return dbias_shared(a) ? dbias_accum_elems(a) * sizeof(float) : 0;
+}
+
+int fdma_bwd(const fdma_bwd_args *a, void *hip_stream) {
+    int rc = fdma_bwd_validate(a);
+    if (rc != FDMA_OK) return rc;
+    fdma::BwdParams p;
+    std::memset(&p, 0, sizeof(p));
+    fill_fwd_params(&a->f, p.f);
+    p.dout = a->dout; p.dq = a->dq; p.dk = a->dk; p.dv = a->dv; p.dbias = a->dbias;
+    p.do_b = a->do_strides[0]; p.do_r = a->do_strides[1]; p.do_h = a->do_strides[2];
+    p.dq_b = a->dq_strides[0]; p.dq_r = a->dq_strides[1]; p.dq_h = a->dq_strides[2];
+    p.dk_b = a->dk_strides[0]; p.dk_r = a->dk_strides[1]; p.dk_h = a->dk_strides[2];
+    p.dv_b = a->dv_strides[0]; p.dv_r = a->dv_strides[1]; p.dv_h = a->dv_strides[2];
+    if (a->dbias) { p.db_b = a->dbias_strides[0]; p.db_h = a->dbias_strides[1]; p.db_r = a->dbias_strides[2]; }
+    p.softmax_d = a->softmax_d;
+    p.Lq_rounded = (int32_t)round_up(a->f.seqlen_q, 128);
+    if (dbias_shared(a)) {
+        const size_t need = fdma_bwd_workspace_bytes(a);
+        if (!a->workspace || a->workspace_bytes < need)
+            return fail(FDMA_ERR_WORKSPACE, "backward workspace too small: need %zu bytes, got %zu", need, a->workspace_bytes);
+        p.dbias_accum = static_cast<float *>(a->workspace);
+        const int64_t lkr = round_up(a->f.seqlen_k, 8);
+        const int64_t nr = a->f.bias_strides[2] == 0 ? 1 : a->f.seqlen_q;
+        p.dba_r = a->f.bias_strides[2] == 0 ? 0 : lkr;
+        p.dba_h = nr * lkr;
+        p.dba_b = a->f.bias_strides[0] == 0 ? 0 : p.dba_h * a->f.num_heads_bias;
+    }
+    hipError_t e = fdma::launch_bwd(p, a->f.dtype, static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(FDMA_ERR_LAUNCH, "backward launch failed: %s", hipGetErrorString(e));
+    return FDMA_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,154 @@
+"""ctypes binding of libfdma_hip.so (declared in include/fdma.h).
+
+This is the only place the Python operator touches native code.  It plays the part of the
+reference's ``import flash_sparse_attn_cuda`` (flash_sparse_attn/flash_sparse_attn_interface.py:7):
+importing this module raises ImportError when the HIP library has not been built, and there is no
+CPU or eager fallback behind it.
+"""
+import ctypes
+import os
+from typing import Optional, Sequence
+
+import torch
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_DEFAULT_LIB = os.path.normpath(os.path.join(_HERE, "..", "lib", "libfdma_hip.so"))
+
+
+class FwdArgs(ctypes.Structure):
+    _fields_ = [
+        ("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p),
+        ("mask", ctypes.c_void_p), ("bias", ctypes.c_void_p),
+        ("out", ctypes.c_void_p), ("lse", ctypes.c_void_p),
+        ("q_strides", ctypes.c_int64 * 3), ("k_strides", ctypes.c_int64 * 3),
+        ("v_strides", ctypes.c_int64 * 3), ("o_strides", ctypes.c_int64 * 3),
+        ("mask_strides", ctypes.c_int64 * 3), ("bias_strides", ctypes.c_int64 * 3),
+        ("batch", ctypes.c_int32), ("seqlen_q", ctypes.c_int32), ("seqlen_k", ctypes.c_int32),
+        ("num_heads", ctypes.c_int32), ("num_heads_k", ctypes.c_int32),
+        ("num_heads_mask", ctypes.c_int32), ("num_heads_bias", ctypes.c_int32),
+        ("head_dim", ctypes.c_int32), ("dtype", ctypes.c_int32), ("is_causal", ctypes.c_int32),
+        ("softmax_scale", ctypes.c_float), ("softcap", ctypes.c_float),
+        ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
+    ]
+
+
+class BwdArgs(ctypes.Structure):
+    _fields_ = [
+        ("f", FwdArgs),
+        ("dout", ctypes.c_void_p),
+        ("dq", ctypes.c_void_p), ("dk", ctypes.c_void_p), ("dv", ctypes.c_void_p),
+        ("dbias", ctypes.c_void_p),
+        ("do_strides", ctypes.c_int64 * 3), ("dq_strides", ctypes.c_int64 * 3),
+        ("dk_strides", ctypes.c_int64 * 3), ("dv_strides", ctypes.c_int64 * 3),
+        ("dbias_strides", ctypes.c_int64 * 3),
+        ("softmax_d", ctypes.c_void_p),
+        ("deterministic", ctypes.c_int32),
+        ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
+    ]
+
+
+EXPORTS = (
+    "fdma_fwd", "fdma_bwd", "fdma_fwd_workspace_bytes", "fdma_bwd_workspace_bytes",
+    "fdma_fwd_validate", "fdma_bwd_validate", "fdma_last_error", "fdma_abi_version",
+    "fdma_sizeof_fwd_args", "fdma_sizeof_bwd_args",
+)
+
+
+def lib_path() -> str:
+    return os.environ.get("FDMA_LIB", _DEFAULT_LIB)
+
+
+def _load() -> ctypes.CDLL:
+    path = lib_path()
+    if not os.path.exists(path):
+        raise ImportError(
+            f"libfdma_hip.so not found at {path}: build it with `make -C flash-dmattn_amd/csrc` "
+            "(or __graft_entry__.build()); there is no fallback implementation"
+        )
+    try:
+        lib = ctypes.CDLL(path)
+    except OSError as e:  # missing HIP runtime etc.
+        raise ImportError(f"cannot load {path}: {e}") from e
+    lib.fdma_fwd.argtypes = [ctypes.POINTER(FwdArgs), ctypes.c_void_p]
+    lib.fdma_fwd.restype = ctypes.c_int
+    lib.fdma_bwd.argtypes = [ctypes.POINTER(BwdArgs), ctypes.c_void_p]
+    lib.fdma_bwd.restype = ctypes.c_int
+    lib.fdma_fwd_validate.argtypes = [ctypes.POINTER(FwdArgs)]
+    lib.fdma_fwd_validate.restype = ctypes.c_int
+    lib.fdma_bwd_validate.argtypes = [ctypes.POINTER(BwdArgs)]
+    lib.fdma_bwd_validate.restype = ctypes.c_int
+    lib.fdma_fwd_workspace_bytes.argtypes = [ctypes.POINTER(FwdArgs)]
+    lib.fdma_fwd_workspace_bytes.restype = ctypes.c_size_t
+    lib.fdma_bwd_workspace_bytes.argtypes = [ctypes.POINTER(BwdArgs)]
+    lib.fdma_bwd_workspace_bytes.restype = ctypes.c_size_t
+    lib.fdma_last_error.argtypes = []
+    lib.fdma_last_error.restype = ctypes.c_char_p
+    lib.fdma_abi_version.restype = ctypes.c_int
+    lib.fdma_sizeof_fwd_args.restype = ctypes.c_size_t
+    lib.fdma_sizeof_bwd_args.restype = ctypes.c_size_t
+    if lib.fdma_abi_version() != 1:
+        raise ImportError(f"{path}: ABI version {lib.fdma_abi_version()} != 1")
+    if lib.fdma_sizeof_fwd_args() != ctypes.sizeof(FwdArgs) or lib.fdma_sizeof_bwd_args() != ctypes.sizeof(BwdArgs):
+        raise ImportError(f"{path}: argument block size differs from the Python mirror")
+    return lib
+
+
+lib = _load()
+
+
+def last_error() -> str:
+    return lib.fdma_last_error().decode()
+
+
+def check(rc: int) -> None:
+    """Every failure of the native layer surfaces as RuntimeError, as TORCH_CHECK does."""
+    if rc != 0:
+        raise RuntimeError(last_error() or f"libfdma_hip error {rc}")
+
+
+_DTYPES = {torch.bfloat16: 0, torch.float16: 1}
+
+
+def dtype_code(t: torch.Tensor) -> int:
+    if t.dtype not in _DTYPES:
+        raise RuntimeError("FlashSparseAttention only support fp16 and bf16 data type")
+    return _DTYPES[t.dtype]
+
+
+def _ptr(t: Optional[torch.Tensor]) -> Optional[int]:
+    return None if t is None else t.data_ptr()
+
+
+def _s3(t: torch.Tensor) -> Sequence[int]:
+    """(batch, row, head) strides of a (B, L, H, D) tensor."""
+    return (t.stride(0), t.stride(1), t.stride(2))
+
+
+def _bcast3(t: torch.Tensor) -> Sequence[int]:
+    """(batch, head, row) strides of a 4-D mask / bias, 0 for size-1 (broadcast) dims."""
+    return tuple(0 if t.size(i) == 1 else t.stride(i) for i in range(3))
+
+
+def fill_fwd(a: FwdArgs, q, k, v, mask, bias, out, lse, softmax_scale, is_causal, softcap) -> None:
+    a.q, a.k, a.v = _ptr(q), _ptr(k), _ptr(v)
+    a.mask, a.bias = _ptr(mask), _ptr(bias)
+    a.out, a.lse = _ptr(out), _ptr(lse)
+    a.q_strides[:] = _s3(q)
+    a.k_strides[:] = _s3(k)
+    a.v_strides[:] = _s3(v)
+    a.o_strides[:] = _s3(out)
+    a.mask_strides[:] = _bcast3(mask) if mask is not None else (0, 0, 0)
+    a.bias_strides[:] = _bcast3(bias) if bias is not None else (0, 0, 0)
+    a.batch, a.seqlen_q, a.num_heads, a.head_dim = q.shape
+    a.seqlen_k, a.num_heads_k = k.shape[1], k.shape[2]
+    a.num_heads_mask = mask.shape[1] if mask is not None else 1
+    a.num_heads_bias = bias.shape[1] if bias is not None else 1
+    a.dtype = dtype_code(q)
+    a.is_causal = int(bool(is_causal))
+    a.softmax_scale = float(softmax_scale)
+    a.softcap = float(softcap)
+    a.workspace, a.workspace_bytes = None, 0
+
+
+def current_stream(device: torch.device) -> int:
+    return torch.cuda.current_stream(device).cuda_stream

@@ -1,0 +1,452 @@
+"""Python operator of Flash Dynamic Mask Attention on MI355X.
+
+Host-side mirror of the reference's flash_sparse_attn/flash_sparse_attn_interface.py: the same public
+functions, argument meaning, defaults, return conventions and error behaviour
+(`flash_sparse_attn_func` :610-684, `FlashDMAttnFunc` :382-498, the custom ops
+`flash_sparse_attn::_flash_sparse_attn_forward/_backward` :73-123, 206-285), but the compiled
+extension behind it is libfdma_hip.so (hand-written gfx950 kernels behind a C ABI) instead of
+`flash_sparse_attn_cuda`.  PyTorch is used for device memory, streams and autograd only.
+
+Differences that are visible only in cost, not in results:
+  * gradients are allocated with ``empty_like`` (the kernels write every element exactly once)
+    instead of ``zeros_like`` (:463-464);
+  * mask / bias are padded along the key dimension only when the kernels' 16-byte row alignment
+    needs it, not always to a multiple of 128 (:420-430);
+  * dK / dV / dBias come out of the kernels at their final shapes; there are no expanded
+    temporaries or host-side reductions (flash_api.cpp:970-983, 1027-1047).
+"""
+from typing import Any, Optional, Tuple
+
+import torch
+
+from . import _cabi
+
+
+def maybe_contiguous(x: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
+    return x.contiguous() if x is not None and x.stride(-1) != 1 else x
+
+
+def round_multiple(x, m):
+    return (x + m - 1) // m * m
+
+
+def _aligned(x: Optional[torch.Tensor], elems: int) -> Optional[torch.Tensor]:
+    """Make x usable by the kernels' 16-byte vector accesses: last dim contiguous, base pointer
+    16-byte aligned, every other stride a multiple of `elems` elements."""
+    if x is None:
+        return None
+    x = maybe_contiguous(x)
+    ok = x.data_ptr() % 16 == 0 and all(x.size(i) == 1 or x.stride(i) % elems == 0 for i in range(x.dim() - 1))
+    return x if ok else x.contiguous().clone(memory_format=torch.contiguous_format)
+
+
+def _check_inputs(q, k, v, mask, bias) -> None:
+    """Device / dtype / rank / shape checks of mha_fwd (flash_api.cpp:371-438, 477-479)."""
+    if q.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("FlashSparseAttention only support fp16 and bf16 data type")
+    if k.dtype != q.dtype:
+        raise RuntimeError("query and key must have the same dtype")
+    if v.dtype != q.dtype:
+        raise RuntimeError("query and value must have the same dtype")
+    for name, t in (("q", q), ("k", k), ("v", v), ("mask", mask), ("bias", bias)):
+        if t is not None and not t.is_cuda:
+            raise RuntimeError(f"{name} must be on CUDA")
+    if q.dim() != 4 or k.dim() != 4 or v.dim() != 4:
+        raise RuntimeError("q, k, v must have shape (batch_size, seqlen, nheads, headdim)")
+    batch, seqlen_q, num_heads, head_size = q.shape
+    seqlen_k, num_heads_k = k.shape[1], k.shape[2]
+    if batch <= 0:
+        raise RuntimeError("batch size must be positive")
+    if head_size > 256:
+        raise RuntimeError("FlashSparseAttention forward only supports head dimension at most 256")
+    if head_size % 8 != 0:
+        raise RuntimeError("query, key, value, and out_ must have a head_size that is a multiple of 8")
+    if num_heads_k <= 0 or num_heads % num_heads_k != 0:
+        raise RuntimeError("Number of heads in key/value must divide number of heads in query")
+    if tuple(k.shape) != (batch, seqlen_k, num_heads_k, head_size):
+        raise RuntimeError(f"k must have shape ({batch}, {seqlen_k}, {num_heads_k}, {head_size})")
+    if tuple(v.shape) != (batch, seqlen_k, num_heads_k, head_size):
+        raise RuntimeError(f"v must have shape ({batch}, {seqlen_k}, {num_heads_k}, {head_size})")
+    for name, t in (("mask", mask), ("bias", bias)):
+        if t is None:
+            continue
+        if name == "mask" and t.dtype != torch.bool:
+            raise RuntimeError("mask must have dtype bool")
+        if name == "bias" and t.dtype != q.dtype:
+            raise RuntimeError("bias must have the same dtype as inputs")
+        if t.dim() != 4:
+            raise RuntimeError(f"{name} must have 4 dimensions with shape (batch_size, nheads, seqlen_q, seqlen_k_rounded)")
+        if t.size(0) not in (batch, 1):
+            raise RuntimeError(f"Batch dimension in {name} must be 1 or equal to batch size")
+        if t.size(1) not in (1, num_heads_k, num_heads):
+            raise RuntimeError(f"Number of heads in {name} must be 1, h_k or h")
+        if t.size(2) not in (1, seqlen_q):
+            raise RuntimeError(f"Query length dimension in {name} must be 1 or equal to seqlen_q")
+        if t.size(3) < seqlen_k:
+            raise RuntimeError(f"Key length dimension in {name} must be seqlen_k_rounded")
+
+
+@torch.library.custom_op("flash_sparse_attn::_flash_sparse_attn_forward", mutates_args=(), device_types="cuda")
+def _flash_sparse_attn_forward(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    mask: Optional[torch.Tensor],
+    bias: Optional[torch.Tensor],
+    softmax_scale: float,
+    is_causal: bool,
+    softcap: float,
+    return_softmax: bool,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    _check_inputs(q, k, v, mask, bias)
+    q, k, v = [_aligned(x, 8) for x in (q, k, v)]
+    mask = _aligned(mask, 16)
+    bias = _aligned(bias, 8)
+    batch, seqlen_q, num_heads, _ = q.shape
+    out = torch.empty_like(q, memory_format=torch.contiguous_format)
+    softmax_lse = torch.empty((batch, num_heads, seqlen_q), dtype=torch.float32, device=q.device)
+    # The attention-probability dump is a debugging aid of the reference ("for testing only",
+    # interface.py:661-663); it is not produced here.
+    p = torch.empty((0,), dtype=q.dtype, device=q.device)
+    if seqlen_q == 0:
+        return out, softmax_lse, p
+    args = _cabi.FwdArgs()
+    _cabi.fill_fwd(args, q, k, v, mask, bias, out, softmax_lse, softmax_scale, is_causal, softcap)
+    with torch.cuda.device(q.device):
+        nbytes = _cabi.lib.fdma_fwd_workspace_bytes(args)
+        workspace = None
+        if nbytes:
+            workspace = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+            args.workspace, args.workspace_bytes = workspace.data_ptr(), nbytes
+        _cabi.check(_cabi.lib.fdma_fwd(args, _cabi.current_stream(q.device)))
+    return out, softmax_lse, p
+
+
+@torch.library.register_fake("flash_sparse_attn::_flash_sparse_attn_forward")
+def _flash_sparse_attn_forward_fake(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    mask: Optional[torch.Tensor],
+    bias: Optional[torch.Tensor],
+    softmax_scale: float,
+    is_causal: bool,
+    softcap: float,
+    return_softmax: bool,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    batch_size, seqlen_q, num_heads, _ = q.shape
+    out = torch.empty_like(q, memory_format=torch.contiguous_format)
+    softmax_lse = torch.empty((batch_size, num_heads, seqlen_q), dtype=torch.float32, device=q.device)
+    p = torch.empty((0,), dtype=q.dtype, device=q.device)
+    return out, softmax_lse, p
+
+
+_wrapped_flash_sparse_attn_forward = _flash_sparse_attn_forward
+
+
+@torch.library.custom_op(
+    "flash_sparse_attn::_flash_sparse_attn_backward", mutates_args=("dq", "dk", "dv", "dbias"), device_types="cuda"
+)
+def _flash_sparse_attn_backward(
+    dout: torch.Tensor,
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    mask: Optional[torch.Tensor],
+    bias: Optional[torch.Tensor],
+    out: torch.Tensor,
+    softmax_lse: torch.Tensor,
+    dq: Optional[torch.Tensor],
+    dk: Optional[torch.Tensor],
+    dv: Optional[torch.Tensor],
+    dbias: Optional[torch.Tensor],
+    softmax_scale: float,
+    is_causal: bool,
+    softcap: float,
+    deterministic: bool,
+) -> torch.Tensor:
+    _check_inputs(q, k, v, mask, bias)
+    if out.dtype != q.dtype:
+        raise RuntimeError("query and out must have the same dtype")
+    if dout.dtype != q.dtype:
+        raise RuntimeError("query and dout must have the same dtype")
+    if tuple(out.shape) != tuple(q.shape) or tuple(dout.shape) != tuple(q.shape):
+        raise RuntimeError("out and dout must have the shape of q")
+    dout, q, k, v, out = [_aligned(x, 8) for x in (dout, q, k, v, out)]
+    mask = _aligned(mask, 16)
+    bias = _aligned(bias, 8)
+    softmax_lse = softmax_lse.contiguous()
+    batch, seqlen_q, num_heads, _ = q.shape
+    softmax_d = torch.empty((batch, num_heads, round_multiple(seqlen_q, 128)), device=q.device, dtype=torch.float32)
+
+    # Outputs handed in by the caller are written in place when their layout allows the kernels'
+    # vector stores; otherwise a staging tensor is filled and copied back.
+    def staging(t, like, name):
+        if t is None:
+            raise RuntimeError(f"{name} must be provided")
+        if t.dtype != q.dtype:
+            raise RuntimeError(f"{name} must have the same dtype as q")
+        if tuple(t.shape) != tuple(like.shape):
+            raise RuntimeError(f"{name} must have the shape of its input")
+        ok = t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(
+            t.size(i) == 1 or t.stride(i) % 8 == 0 for i in range(t.dim() - 1))
+        return t if ok else torch.empty_like(t, memory_format=torch.contiguous_format)
+
+    dq_w, dk_w, dv_w = staging(dq, q, "dq"), staging(dk, k, "dk"), staging(dv, v, "dv")
+    dbias_w = staging(dbias, bias, "dbias") if bias is not None else None
+
+    args = _cabi.BwdArgs()
+    _cabi.fill_fwd(args.f, q, k, v, mask, bias, out, softmax_lse, softmax_scale, is_causal, softcap)
+    args.dout = dout.data_ptr()
+    args.dq, args.dk, args.dv = dq_w.data_ptr(), dk_w.data_ptr(), dv_w.data_ptr()
+    args.dbias = dbias_w.data_ptr() if dbias_w is not None else None
+    args.do_strides[:] = _cabi._s3(dout)
+    args.dq_strides[:] = _cabi._s3(dq_w)
+    args.dk_strides[:] = _cabi._s3(dk_w)
+    args.dv_strides[:] = _cabi._s3(dv_w)
+    args.dbias_strides[:] = _cabi._bcast3(dbias_w) if dbias_w is not None else (0, 0, 0)
+    args.softmax_d = softmax_d.data_ptr()
+    args.deterministic = int(bool(deterministic))
+    with torch.cuda.device(q.device):
+        nbytes = _cabi.lib.fdma_bwd_workspace_bytes(args)
+        workspace = None
+        if nbytes:
+            workspace = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+            args.workspace, args.workspace_bytes = workspace.data_ptr(), nbytes
+        else:
+            args.workspace, args.workspace_bytes = None, 0
+        if seqlen_q > 0:
+            _cabi.check(_cabi.lib.fdma_bwd(args, _cabi.current_stream(q.device)))
+        else:  # empty query: gradients are zero (flash_api.cpp:1019-1025)
+            for t in (dk_w, dv_w, dbias_w, softmax_d):
+                if t is not None:
+                    t.zero_()
+    for given, work in ((dq, dq_w), (dk, dk_w), (dv, dv_w), (dbias, dbias_w)):
+        if given is not None and work is not given:
+            given.copy_(work)
+    return softmax_d
+
+
+@torch.library.register_fake("flash_sparse_attn::_flash_sparse_attn_backward")
+def _flash_sparse_attn_backward_fake(
+    dout: torch.Tensor,
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    mask: Optional[torch.Tensor],
+    bias: Optional[torch.Tensor],
+    out: torch.Tensor,
+    softmax_lse: torch.Tensor,
+    dq: Optional[torch.Tensor],
+    dk: Optional[torch.Tensor],
+    dv: Optional[torch.Tensor],
+    dbias: Optional[torch.Tensor],
+    softmax_scale: float,
+    is_causal: bool,
+    softcap: float,
+    deterministic: bool,
+) -> torch.Tensor:
+    batch_size, seqlen_q, num_heads, _ = q.shape
+    return torch.empty((batch_size, num_heads, round_multiple(seqlen_q, 128)), device=q.device, dtype=torch.float32)
+
+
+_wrapped_flash_sparse_attn_backward = _flash_sparse_attn_backward
+
+
+def _pad_key_dim(t: Optional[torch.Tensor], seqlen_k: int, elems: int) -> Optional[torch.Tensor]:
+    """Key-dimension rule of FlashDMAttnFunc.forward (interface.py:420-430): a size-1 key dim is
+    expanded, any other length is padded.  The reference pads to a multiple of 128 always; the
+    kernels here only need rows of a whole number of 16-byte vectors."""
+    if t is None:
+        return None
+    if t.shape[-1] == 1 and seqlen_k != 1:
+        return t.expand(*t.shape[:-1], round_multiple(seqlen_k, 128))
+    if t.shape[-1] % elems != 0:
+        return torch.nn.functional.pad(t, [0, round_multiple(max(seqlen_k, t.shape[-1]), 128) - t.shape[-1]])
+    return t
+
+
+class FlashDMAttnFunc(torch.autograd.Function):
+
+    @staticmethod
+    def forward(
+        ctx: torch.autograd.function.FunctionCtx,
+        q: torch.Tensor,
+        k: torch.Tensor,
+        v: torch.Tensor,
+        mask: Optional[torch.Tensor],
+        bias: Optional[torch.Tensor],
+        softmax_scale: Optional[float],
+        is_causal: Optional[bool],
+        softcap: Optional[float],
+        deterministic: Optional[bool],
+        return_softmax: Optional[bool],
+        is_grad_enabled: bool = True,
+    ):
+        is_grad = is_grad_enabled and any(x.requires_grad for x in [q, k, v])
+        if softmax_scale is None:
+            softmax_scale = q.shape[-1] ** (-0.5)
+        if is_causal is None:
+            is_causal = False
+        if softcap is None:
+            softcap = 0.0
+        if deterministic is None:
+            deterministic = False
+        if return_softmax is None:
+            return_softmax = False
+        seqlen_k_bias_og = bias.shape[-1] if bias is not None else 0
+
+        # Padding to multiple of 8 for 16-bit memory allocations
+        head_size_og = q.size(3)
+        if head_size_og % 8 != 0:
+            q = torch.nn.functional.pad(q, [0, 8 - head_size_og % 8])
+            k = torch.nn.functional.pad(k, [0, 8 - head_size_og % 8])
+            v = torch.nn.functional.pad(v, [0, 8 - head_size_og % 8])
+        mask = _pad_key_dim(mask, k.shape[1], 16)
+        bias = _pad_key_dim(bias, k.shape[1], 8)
+
+        out_padded, softmax_lse, S_dmask = _wrapped_flash_sparse_attn_forward(
+            q,
+            k,
+            v,
+            mask,
+            bias,
+            softmax_scale,
+            is_causal=is_causal,
+            softcap=softcap,
+            return_softmax=return_softmax,
+        )
+
+        if is_grad:
+            ctx.save_for_backward(q, k, v, mask, bias, out_padded, softmax_lse)
+            ctx.softmax_scale = softmax_scale
+            ctx.is_causal = is_causal
+            ctx.softcap = softcap
+            ctx.deterministic = deterministic
+            ctx.seqlen_k_bias_og = seqlen_k_bias_og
+
+        out = out_padded[..., :head_size_og]
+
+        return out if not return_softmax else (out, softmax_lse, S_dmask)
+
+    @staticmethod
+    def backward(
+        ctx: torch.autograd.function.FunctionCtx,
+        dout: torch.Tensor,
+        *args: Any,
+    ):
+        q, k, v, mask, bias, out, softmax_lse = ctx.saved_tensors
+        # every element of the gradients is written by the kernels: no zero fill
+        dq = torch.empty_like(q, memory_format=torch.contiguous_format)
+        dk = torch.empty_like(k, memory_format=torch.contiguous_format)
+        dv = torch.empty_like(v, memory_format=torch.contiguous_format)
+        dbias = torch.empty(bias.shape, dtype=bias.dtype, device=bias.device) if bias is not None else None
+
+        head_size_og = dout.size(3)
+        dout_padded = dout
+        if head_size_og % 8 != 0:
+            dout_padded = torch.nn.functional.pad(dout, [0, 8 - head_size_og % 8])
+
+        _wrapped_flash_sparse_attn_backward(
+            dout_padded,
+            q,
+            k,
+            v,
+            mask,
+            bias,
+            out,
+            softmax_lse,
+            dq,
+            dk,
+            dv,
+            dbias,
+            ctx.softmax_scale,
+            ctx.is_causal,
+            ctx.softcap,
+            ctx.deterministic,
+        )
+
+        # We could have padded the head dimension
+        dq = dq[..., : dout.shape[-1]]
+        dk = dk[..., : dout.shape[-1]]
+        dv = dv[..., : dout.shape[-1]]
+
+        if dbias is not None:
+            dbias = (
+                dbias[..., : k.shape[1]].sum(dim=-1, keepdim=True)
+                if ctx.seqlen_k_bias_og == 1
+                else dbias[..., : k.shape[1]]
+            )
+
+        return dq, dk, dv, None, dbias, None, None, None, None, None, None
+
+
+def flash_sparse_attn_func(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    attn_mask: Optional[torch.Tensor] = None,
+    attn_bias: Optional[torch.Tensor] = None,
+    softmax_scale: Optional[float] = None,
+    is_causal: Optional[bool] = None,
+    softcap: Optional[float] = None,
+    deterministic: Optional[bool] = None,
+    return_attn_probs: Optional[bool] = None,
+):
+    """Dynamic-mask attention with MQA/GQA: K, V may have fewer heads than Q (the number of Q heads
+    must be divisible by the number of KV heads; Q head h attends to KV head h // (H // Hkv)).
+
+    attn_mask and attn_bias may have a head dimension of 1, nheads_k or nheads, a batch dimension
+    of 1 or batch_size, and a query dimension of 1 or seqlen_q; size-1 dimensions broadcast.
+
+    If is_causal=True, the causal mask is aligned to the bottom right corner of the attention
+    matrix.  For seqlen_q = 2 and seqlen_k = 5 the causal mask (1 = keep, 0 = masked out) is:
+        1 1 1 1 0
+        1 1 1 1 1
+    and for seqlen_q = 5 and seqlen_k = 2:
+        0 0
+        0 0
+        0 0
+        1 0
+        1 1
+    If a row of the mask is all zero, the output row is zero.
+
+    Arguments:
+        query: (batch_size, seqlen, nheads, headdim)
+        key: (batch_size, seqlen_k, nheads_k, headdim)
+        value: (batch_size, seqlen_k, nheads_k, headdim)
+        attn_mask: optional bool tensor ({batch_size|1}, {nheads|nheads_k|1}, {seqlen_q|1}, {seqlen_k|1});
+            True keeps a score, False masks it out.
+        attn_bias: optional tensor of query's dtype, same shape rules, added to the scaled scores.
+        softmax_scale: scaling of QK^T before the bias is added. Default 1 / sqrt(headdim).
+        is_causal: apply the (bottom-right aligned) causal mask.
+        softcap: must be None or 0 (soft-capping is not built).
+        deterministic: accepted; the backward pass never uses atomics on dQ/dK/dV and is
+            deterministic regardless.
+        return_attn_probs: also return (softmax_lse, S_dmask); S_dmask is an empty tensor.
+    Return:
+        out: (batch_size, seqlen, nheads, headdim).
+        softmax_lse [optional]: (batch_size, nheads, seqlen), fp32 logsumexp of each score row
+            (+inf for rows with no visible key).
+    """
+    return FlashDMAttnFunc.apply(
+        query,
+        key,
+        value,
+        attn_mask,
+        attn_bias,
+        softmax_scale,
+        is_causal,
+        softcap,
+        deterministic,
+        return_attn_probs,
+        torch.is_grad_enabled(),
+    )
+
+
+def flash_sparse_attn_varlen_func(*args, **kwargs):
+    """Ragged-batch entry point of the reference (interface.py:687-760).  It takes no mask or bias
+    and is not part of the dynamic-mask hot path; it is not built here."""
+    raise NotImplementedError(
+        "flash_sparse_attn_varlen_func (cu_seqlens path without mask/bias) is not provided by the MI355X build"
+    )

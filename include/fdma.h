@@ -1,0 +1,116 @@
+/*
+ * fdma.h -- C ABI of libfdma_hip.so, the gfx950 (MI355X) implementation of Flash Dynamic Mask
+ * Attention (dense path: Q,K,V + boolean keep-mask + additive bias, causal, MQA/GQA,
+ * dQ/dK/dV/dBias).
+ *
+ * The library is a drop-in for the compiled extension of SmallDoges/flash-dmattn: each entry point
+ * below replaces one function the reference's Python operator binds from `flash_sparse_attn_cuda`
+ * (reference paths are relative to its checkout):
+ *
+ *   fdma_fwd   <-  mha_fwd            csrc/flash_sparse_attn/flash_api.cpp:351-554  (pybind "fwd",  :1272)
+ *   fdma_bwd   <-  mha_bwd            csrc/flash_sparse_attn/flash_api.cpp:792-1050 (pybind "bwd",  :1274)
+ *   fdma_fwd_args / fdma_bwd_args
+ *              <-  Flash_fwd_params / Flash_bwd_params   csrc/flash_sparse_attn/src/flash.h:20-198
+ *
+ * Differences from the reference boundary, all on purpose:
+ *   - plain C: device pointers, sizes and element strides; no torch / pybind types;
+ *   - the caller owns every buffer (outputs, LSE, softmax_d, workspace); the library never
+ *     allocates, frees or synchronises and launches on the HIP stream it is handed;
+ *   - dK/dV are written at their true (Hkv) shape and dBias at the bias's own broadcast shape,
+ *     so there are no "expanded" temporaries and no host-side reductions
+ *     (flash_api.cpp:970-983, 1027-1047 are fused into the kernels);
+ *   - errors are returned as negative codes with a thread-local message (fdma_last_error)
+ *     carrying the same text the reference's TORCH_CHECKs raise.
+ *
+ * Layouts (all strides in ELEMENTS, innermost dimension contiguous):
+ *   q, out, dout, dq : (batch, seqlen_q, num_heads,   head_dim)   strides {batch, row, head}
+ *   k, v, dk, dv     : (batch, seqlen_k, num_heads_k, head_dim)   strides {batch, row, head}
+ *   mask  (uint8 / bool, 1 = keep) : ({batch|1}, {1|Hk|H}, {seqlen_q|1}, >= seqlen_k)
+ *   bias, dbias (same dtype as q)  : ({batch|1}, {1|Hk|H}, {seqlen_q|1}, >= seqlen_k)
+ *                                     strides {batch, head, row}; 0 marks a broadcast dim
+ *   lse       : (batch, num_heads, seqlen_q) fp32, contiguous; +inf for rows with no visible key
+ *   softmax_d : (batch, num_heads, round_up(seqlen_q,128)) fp32, contiguous
+ */
+#ifndef FDMA_H_
+#define FDMA_H_
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define FDMA_ABI_VERSION 1
+
+enum { FDMA_DTYPE_BF16 = 0, FDMA_DTYPE_FP16 = 1 };
+
+enum {
+    FDMA_OK = 0,
+    FDMA_ERR_INVALID = -1,     /* argument validation failed (the reference raises RuntimeError) */
+    FDMA_ERR_UNSUPPORTED = -2, /* valid for the reference, not built here (e.g. head_dim > 128)   */
+    FDMA_ERR_WORKSPACE = -3,   /* workspace missing or too small                                  */
+    FDMA_ERR_LAUNCH = -4       /* the HIP runtime refused a launch                                */
+};
+
+typedef struct fdma_fwd_args {
+    const void *q, *k, *v;
+    const void *mask; /* NULL = no mask */
+    const void *bias; /* NULL = no bias */
+    void *out;
+    float *lse;
+    int64_t q_strides[3], k_strides[3], v_strides[3], o_strides[3];
+    int64_t mask_strides[3], bias_strides[3];
+    int32_t batch, seqlen_q, seqlen_k;
+    int32_t num_heads, num_heads_k, num_heads_mask, num_heads_bias;
+    int32_t head_dim;
+    int32_t dtype;
+    int32_t is_causal;
+    float softmax_scale;
+    float softcap; /* must be 0: softcapping is not built */
+    void *workspace;        /* split-KV partials for the decode path; may be NULL if bytes == 0 */
+    size_t workspace_bytes; /* >= fdma_fwd_workspace_bytes(args) */
+} fdma_fwd_args;
+
+typedef struct fdma_bwd_args {
+    fdma_fwd_args f; /* q,k,v,mask,bias as in forward; f.out and f.lse are the forward RESULTS (read) */
+    const void *dout;
+    void *dq, *dk, *dv;
+    void *dbias; /* NULL iff f.bias == NULL; shape and broadcast pattern of the bias */
+    int64_t do_strides[3], dq_strides[3], dk_strides[3], dv_strides[3];
+    int64_t dbias_strides[3];
+    float *softmax_d; /* out: rowsum(dO * O) */
+    int32_t deterministic;
+    void *workspace;
+    size_t workspace_bytes; /* >= fdma_bwd_workspace_bytes(args) */
+} fdma_bwd_args;
+
+/* Forward attention.  Asynchronous on `hip_stream` (a hipStream_t).  Returns FDMA_OK or < 0. */
+int fdma_fwd(const fdma_fwd_args *args, void *hip_stream);
+
+/* Backward attention: dq, dk, dv, dbias, softmax_d.  Every output element is written exactly once
+ * (no zero-fill needed by the caller), including masked / skipped regions of dbias. */
+int fdma_bwd(const fdma_bwd_args *args, void *hip_stream);
+
+/* Scratch the caller must provide.  0 when none is needed.  Validate nothing but shapes. */
+size_t fdma_fwd_workspace_bytes(const fdma_fwd_args *args);
+size_t fdma_bwd_workspace_bytes(const fdma_bwd_args *args);
+
+/* Argument validation only (no GPU work, callable on a host without a device). */
+int fdma_fwd_validate(const fdma_fwd_args *args);
+int fdma_bwd_validate(const fdma_bwd_args *args);
+
+/* Message of the last error raised on the calling thread ("" if none). */
+const char *fdma_last_error(void);
+
+int fdma_abi_version(void);
+
+/* sizeof() of the two argument blocks as compiled, so a foreign-language binding can check its
+ * struct packing before the first call. */
+size_t fdma_sizeof_fwd_args(void);
+size_t fdma_sizeof_bwd_args(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FDMA_H_ */
