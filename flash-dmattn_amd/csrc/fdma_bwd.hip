@@ -1,5 +1,663 @@
+// Backward dynamic-mask attention for gfx950.
+//
+// Replaces the reference's backward pipeline (csrc/flash_sparse_attn/src/flash_bwd_launch_template.h:71-117):
+//   flash_bwd_dot_do_o_kernel                       src/flash_bwd_preprocess_kernel.h:24-162
+//   flash_bwd_dq_dk_dv_loop_seqk_parallel_kernel    src/flash_bwd_kernel.h:79-1142
+//   flash_bwd_convert_dq_kernel                     src/flash_bwd_preprocess_kernel.h:212-304
+// and the host-side GQA / broadcast reductions of mha_bwd (csrc/flash_sparse_attn/flash_api.cpp:970-983, 1027-1047).
+//
+// Same math, recomputing P from the saved LSE:
+//     P = exp(S - LSE) ; dP = dO V^T ; D = rowsum(dO * O) ; dS = P * (dP - D)
+//     dQ = scale * dS K ; dK = scale * dS^T Q ; dV = P^T dO ; dBias = dS (summed over broadcast dims)
+//
+// Different structure: no fp32 dQ accumulator, no atomics on dQ/dK/dV, no expanded GQA buffers.
+//   1. bwd_dot_kernel   : D = rowsum(dO * O)
+//   2. bwd_dkdv_kernel  : one workgroup per (key block, batch, KV head); K/V stationary, loops over the
+//                         query heads of the group and over query blocks; dK, dV and dBias complete in
+//                         registers (S is computed un-transposed so a lane owns one key column);
+//   3. bwd_dq_kernel    : one workgroup per (query block, batch, head); loops over key blocks exactly like
+//                         the forward kernel (transposed scores, a lane owns one query row).
+// Work is therefore 7 tile GEMMs instead of 5, in exchange for a deterministic result and no
+// read-modify-write traffic.
 #include "fdma_common.h"
 #include "fdma_params.h"
+
 namespace fdma {
-hipError_t launch_bwd(const BwdParams &, int, hipStream_t) { return hipErrorNotSupported; }
+
+namespace {
+
+constexpr int NTHREADS = 256;
+
+// nonzero bytes of x -> bit k of the result is set iff byte k of x != 0
+__device__ __forceinline__ uint32_t nz_bytes_to_bits(uint32_t x) {
+    uint32_t y = (((x & 0x7f7f7f7fu) + 0x7f7f7f7fu) | x) & 0x80808080u;
+    return ((y >> 7) * 0x10204080u) >> 28;
 }
+
+// ------------------------------------------------------------------------------------------------
+// 1. D = rowsum(dO * O)   (softmax_d, padded rows are zero)
+// ------------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256) bwd_dot_kernel(const BwdParams p) {
+    using E = Elem<T>;
+    const int CH = (p.f.d + 7) / 8;               // 16-byte chunks per row
+    const int lanes = CH <= 8 ? 8 : 16;           // lanes cooperating on one row (power of two)
+    const int rows_per_block = 256 / lanes;
+    const int sub = threadIdx.x % lanes;
+    const int row = blockIdx.x * rows_per_block + threadIdx.x / lanes;
+    const int h = blockIdx.y, b = blockIdx.z;
+    float acc = 0.f;
+    if (row < p.f.Lq) {
+        const uint16_t *op = (const uint16_t *)p.f.o + b * p.f.o_b + (int64_t)row * p.f.o_r + h * p.f.o_h;
+        const uint16_t *dp = (const uint16_t *)p.dout + b * p.do_b + (int64_t)row * p.do_r + h * p.do_h;
+        for (int c = sub; c < CH; c += lanes) {
+            u32x4_t ov = *(const u32x4_t *)(op + c * 8);
+            u32x4_t dv = *(const u32x4_t *)(dp + c * 8);
+#pragma unroll
+            for (int e = 0; e < 4; e++) acc += E::lo(ov[e]) * E::lo(dv[e]) + E::hi(ov[e]) * E::hi(dv[e]);
+        }
+    }
+    for (int off = lanes / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
+    if (sub == 0 && row < p.Lq_rounded) p.softmax_d[((int64_t)b * p.f.H + h) * p.Lq_rounded + row] = acc;
+}
+
+// ------------------------------------------------------------------------------------------------
+// 2. dK / dV / dBias
+// ------------------------------------------------------------------------------------------------
+constexpr int KV_BM = 64;   // query rows per step
+constexpr int KV_BN = 128;  // key columns per workgroup (32 per wave)
+
+template <int D> struct KvSmem {
+    static constexpr int S = D + 8;  // row stride (elements) of every tile
+    static constexpr int K_BYTES = KV_BN * S * 2;
+    static constexpr int Q_BYTES = KV_BM * S * 2;
+    static constexpr int STAT_BYTES = KV_BM * 4;
+    static constexpr int OFF_K = 0;
+    static constexpr int OFF_V = OFF_K + K_BYTES;
+    static constexpr int OFF_Q = OFF_V + K_BYTES;
+    static constexpr int OFF_DO = OFF_Q + Q_BYTES;
+    static constexpr int OFF_LSE = OFF_DO + Q_BYTES;
+    static constexpr int OFF_DD = OFF_LSE + STAT_BYTES;
+    static constexpr int TOTAL = OFF_DD + STAT_BYTES;
+};
+
+template <typename T, int D, bool CAUSAL>
+__global__ void __launch_bounds__(NTHREADS) bwd_dkdv_kernel(const BwdParams p) {
+    using E = Elem<T>;
+    using SM = KvSmem<D>;
+    constexpr int KS = D / 16;
+    constexpr int DB = D / 32;
+    constexpr int MB = KV_BM / 32;
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    char *sK = smem + SM::OFF_K, *sV = smem + SM::OFF_V, *sQ = smem + SM::OFF_Q, *sDO = smem + SM::OFF_DO;
+    float *sLSE = (float *)(smem + SM::OFF_LSE), *sDD = (float *)(smem + SM::OFF_DD);
+
+    const FwdParams &f = p.f;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 31, g = lane >> 5;
+    const int n_block = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
+    const int G = f.H / f.Hk;
+    const int n0 = n_block * KV_BN;
+    const int key = n0 + wave * 32 + r;  // the key column this lane owns
+    const int shift = f.Lk - f.Lq;
+
+    // ---- stage K and V (rows beyond Lk zero-filled)
+    {
+        constexpr int CH = D / 8, RPP = NTHREADS / CH;
+        const int c = tid % CH, r0 = tid / CH;
+        const uint16_t *kbase = (const uint16_t *)f.k + b * f.k_b + hk * f.k_h;
+        const uint16_t *vbase = (const uint16_t *)f.v + b * f.v_b + hk * f.v_h;
+#pragma unroll
+        for (int it = 0; it < KV_BN / RPP; it++) {
+            int row = r0 + it * RPP, kk = n0 + row;
+            u32x4_t kv = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
+            if (kk < f.Lk && c * 8 < f.d) {
+                kv = *(const u32x4_t *)(kbase + (int64_t)kk * f.k_r + c * 8);
+                vv = *(const u32x4_t *)(vbase + (int64_t)kk * f.v_r + c * 8);
+            }
+            *(u32x4_t *)(sK + (row * SM::S + c * 8) * 2) = kv;
+            *(u32x4_t *)(sV + (row * SM::S + c * 8) * 2) = vv;
+        }
+    }
+
+    f32x16_t dk[DB], dv[DB];
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) { dk[db][i] = 0.f; dv[db][i] = 0.f; }
+
+    const int M_blocks = (f.Lq + KV_BM - 1) / KV_BM;
+    int m_start = 0;
+    if (CAUSAL) {
+        int first_q = n0 - shift;  // first query row that sees key n0
+        if (first_q > 0) m_start = first_q / KV_BM;
+        if (m_start > M_blocks) m_start = M_blocks;
+    }
+
+    const bool has_bias = f.bias != nullptr;
+    const bool bias_rows = has_bias && f.bi_r != 0;   // per-query bias (and dbias) rows
+    const bool mask_rows = f.mask != nullptr && f.m_r != 0;
+    const bool use_accum = p.dbias_accum != nullptr;   // several workgroups share a dbias element
+    // loop order: per-query dbias wants (m outer, g inner) to sum dS over the group in registers;
+    // row-broadcast dbias wants (g outer, m inner) to keep one column sum per bias head.
+    const bool m_outer = bias_rows;
+    const int n_m = M_blocks - m_start;
+    const int n_steps = n_m * G;
+
+    // zero the part of a per-query dbias this workgroup owns but never visits (above the causal
+    // diagonal); visited tiles are written below.
+    if (bias_rows && !use_accum && m_start > 0) {
+        const int ngh = (f.Hb == f.H) ? G : 1;
+        for (int gh = 0; gh < ngh; gh++) {
+            const int hb = f.Hb == f.H ? hk * G + gh : (f.Hb == 1 ? 0 : hk);
+            uint16_t *dbp = (uint16_t *)p.dbias + b * p.db_b + hb * p.db_h;
+            const int rows = m_start * KV_BM < f.Lq ? m_start * KV_BM : f.Lq;
+            // 16 chunks of 8 keys per row
+            for (int idx = tid; idx < rows * 16; idx += NTHREADS) {
+                int row = idx >> 4, c = idx & 15;
+                int kk = n0 + c * 8;
+                if (kk < f.Lk) *(u32x4_t *)(dbp + (int64_t)row * p.db_r + kk) = u32x4_t{0, 0, 0, 0};
+            }
+        }
+    }
+
+    // per-lane constants for row-broadcast mask / bias
+    const int a_row = pi_row(r);
+    const int tj = lane & 15, te = tj >> 2, tc = tj & 3;
+    const int tcp = (tc == 1) ? 2 : (tc == 2 ? 1 : tc);
+    const int tdh = (lane >> 4) & 1;
+    const uint32_t tr_off = (uint32_t)(((8 * g + te) * SM::S + 16 * tdh + 4 * tcp) * 2);
+
+    float colsum = 0.f;       // row-broadcast dbias: sum over queries of dS for this lane's key
+    f32x16_t dsum[MB];        // per-query dbias with bias heads < H: sum over the group
+#pragma unroll
+    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) dsum[mb][i] = 0.f;
+
+    for (int step = 0; step < n_steps; step++) {
+        const int gi = m_outer ? step % G : step / n_m;
+        const int mi = m_start + (m_outer ? step / G : step % n_m);
+        const int h = hk * G + gi;
+        const int m0 = mi * KV_BM;
+        const int hm = f.mask ? (f.Hm == f.H ? h : (f.Hm == 1 ? 0 : hk)) : 0;
+        const int hb = has_bias ? (f.Hb == f.H ? h : (f.Hb == 1 ? 0 : hk)) : 0;
+        const bool first_of_group = gi == 0;
+        const bool last_of_group = gi == G - 1;
+
+        __syncthreads();  // previous step finished reading sQ / sDO / stats (also covers the K/V staging)
+        // ---- stage Q, dO, LSE, D for (h, m-block)
+        {
+            constexpr int CH = D / 8, RPP = NTHREADS / CH;
+            const int c = tid % CH, r0 = tid / CH;
+            const uint16_t *qbase = (const uint16_t *)f.q + b * f.q_b + h * f.q_h;
+            const uint16_t *dobase = (const uint16_t *)p.dout + b * p.do_b + h * p.do_h;
+#pragma unroll
+            for (int it = 0; it < KV_BM / RPP; it++) {
+                int row = r0 + it * RPP, qq = m0 + row;
+                u32x4_t qv = {0, 0, 0, 0}, dov = {0, 0, 0, 0};
+                if (qq < f.Lq && c * 8 < f.d) {
+                    qv = *(const u32x4_t *)(qbase + (int64_t)qq * f.q_r + c * 8);
+                    dov = *(const u32x4_t *)(dobase + (int64_t)qq * p.do_r + c * 8);
+                }
+                *(u32x4_t *)(sQ + (row * SM::S + c * 8) * 2) = qv;
+                *(u32x4_t *)(sDO + (row * SM::S + c * 8) * 2) = dov;
+            }
+            if (tid < KV_BM) {
+                int qq = m0 + tid;
+                float l = INFINITY, dd = 0.f;
+                if (qq < f.Lq) {
+                    l = f.lse[((int64_t)b * f.H + h) * f.Lq + qq] * kLog2e;
+                    dd = p.softmax_d[((int64_t)b * f.H + h) * p.Lq_rounded + qq];
+                }
+                sLSE[tid] = l;
+                sDD[tid] = dd;
+            }
+        }
+
+        // ---- keep bits: bit 16*mb + i  <->  query m0 + 32mb + 16(i/8) + 8g + i%8, this lane's key
+        uint32_t keep = 0;
+        {
+            const uint8_t *mp = f.mask ? f.mask + b * f.m_b + hm * f.m_h + key : nullptr;
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    int qq = m0 + 32 * mb + 16 * (i >> 3) + 8 * g + (i & 7);
+                    bool vis = key < f.Lk && qq < f.Lq;
+                    if (CAUSAL) vis = vis && key <= qq + shift;
+                    if (vis && mp) vis = mp[(int64_t)(mask_rows ? qq : 0) * f.m_r] != 0;
+                    keep |= (vis ? 1u : 0u) << (16 * mb + i);
+                }
+        }
+        __syncthreads();
+
+        f32x16_t ds[MB];
+        if (keep != 0 || true) {
+            // ---- S = Q K^T and dP = dO V^T  (M = query, N = key)
+            f32x16_t s[MB], dp[MB];
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++) {
+#pragma unroll
+                for (int i = 0; i < 16; i++) { s[mb][i] = 0.f; dp[mb][i] = 0.f; }
+            }
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                u32x4_t kb = *(const u32x4_t *)(sK + ((32 * wave + r) * SM::S + ks * 16 + g * 8) * 2);
+                u32x4_t vb = *(const u32x4_t *)(sV + ((32 * wave + r) * SM::S + ks * 16 + g * 8) * 2);
+#pragma unroll
+                for (int mb = 0; mb < MB; mb++) {
+                    u32x4_t qa = *(const u32x4_t *)(sQ + ((32 * mb + a_row) * SM::S + ks * 16 + g * 8) * 2);
+                    u32x4_t da = *(const u32x4_t *)(sDO + ((32 * mb + a_row) * SM::S + ks * 16 + g * 8) * 2);
+                    s[mb] = E::mfma(qa, kb, s[mb]);
+                    dp[mb] = E::mfma(da, vb, dp[mb]);
+                }
+            }
+            // ---- P and dS
+            uint32_t ppk[MB * 8], dpk[MB * 8];
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++) {
+#pragma unroll
+                for (int i = 0; i < 16; i += 2) {
+                    float pv[2], dsv[2];
+#pragma unroll
+                    for (int e = 0; e < 2; e++) {
+                        const int ii = i + e;
+                        const int ql = 32 * mb + 16 * (ii >> 3) + 8 * g + (ii & 7);
+                        float bl2 = 0.f;
+                        if (has_bias) {
+                            const uint16_t *bp = (const uint16_t *)f.bias + b * f.bi_b + hb * f.bi_h;
+                            int qq = m0 + ql;
+                            qq = qq < f.Lq ? qq : f.Lq - 1;
+                            int kk = key < f.Lk ? key : f.Lk - 1;
+                            uint32_t raw = bp[(int64_t)(bias_rows ? qq : 0) * f.bi_r + kk];
+                            bl2 = E::lo(raw) * kLog2e;
+                        }
+                        float x = fmaf(s[mb][ii], f.scale_log2, bl2) - sLSE[ql];
+                        float pe = ((keep >> (16 * mb + ii)) & 1u) ? fast_exp2(x) : 0.f;
+                        float de = pe * (dp[mb][ii] - sDD[ql]);
+                        pv[e] = pe;
+                        dsv[e] = de;
+                        ds[mb][ii] = de;
+                    }
+                    ppk[mb * 8 + i / 2] = E::pack2(pv[0], pv[1]);
+                    dpk[mb * 8 + i / 2] = E::pack2(dsv[0], dsv[1]);
+                }
+            }
+            // ---- dV^T += dO^T P ; dK^T += Q^T dS   (M = d, N = key, contraction = query)
+#pragma unroll
+            for (int qb = 0; qb < KV_BM / 16; qb++) {
+                u32x4_t pb = {ppk[4 * qb], ppk[4 * qb + 1], ppk[4 * qb + 2], ppk[4 * qb + 3]};
+                u32x4_t sb = {dpk[4 * qb], dpk[4 * qb + 1], dpk[4 * qb + 2], dpk[4 * qb + 3]};
+#pragma unroll
+                for (int db = 0; db < DB; db++) {
+                    uint32_t off = tr_off + (uint32_t)((16 * qb * SM::S + 32 * db) * 2);
+                    u32x2_t lo = lds_read_tr16(sDO, off), hi = lds_read_tr16(sDO, off + 4 * SM::S * 2);
+                    u32x4_t a = {lo[0], lo[1], hi[0], hi[1]};
+                    dv[db] = E::mfma(a, pb, dv[db]);
+                    lo = lds_read_tr16(sQ, off);
+                    hi = lds_read_tr16(sQ, off + 4 * SM::S * 2);
+                    u32x4_t a2 = {lo[0], lo[1], hi[0], hi[1]};
+                    dk[db] = E::mfma(a2, sb, dk[db]);
+                }
+            }
+        }
+
+        // ---- dBias
+        if (has_bias) {
+            if (!bias_rows) {
+                float part = 0.f;
+#pragma unroll
+                for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) part += ds[mb][i];
+                colsum += part;
+                // flush when the bias head changes (g outer, m inner)
+                const bool last_m = (step % n_m) == n_m - 1;
+                const bool flush = last_m && (f.Hb == f.H || last_of_group);
+                if (flush) {
+                    float tot = xhalf_sum(colsum);
+                    if (g == 0 && key < f.Lk) {
+                        if (use_accum)
+                            atomicAdd(p.dbias_accum + b * p.dba_b + hb * p.dba_h + key, tot);
+                        else
+                            ((uint16_t *)p.dbias)[b * p.db_b + hb * p.db_h + key] = (uint16_t)(E::pack2(tot, 0.f) & 0xffffu);
+                    }
+                    colsum = 0.f;
+                }
+            } else {
+                const bool per_head = f.Hb == f.H;
+#pragma unroll
+                for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) dsum[mb][i] = (per_head || first_of_group) ? ds[mb][i] : dsum[mb][i] + ds[mb][i];
+                if (per_head || last_of_group) {
+#pragma unroll
+                    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+                        for (int i = 0; i < 16; i++) {
+                            int qq = m0 + 32 * mb + 16 * (i >> 3) + 8 * g + (i & 7);
+                            if (qq < f.Lq && key < f.Lk) {
+                                if (use_accum)
+                                    atomicAdd(p.dbias_accum + b * p.dba_b + hb * p.dba_h + (int64_t)qq * p.dba_r + key, dsum[mb][i]);
+                                else
+                                    ((uint16_t *)p.dbias)[b * p.db_b + hb * p.db_h + (int64_t)qq * p.db_r + key] =
+                                        (uint16_t)(E::pack2(dsum[mb][i], 0.f) & 0xffffu);
+                            }
+                        }
+                }
+            }
+        }
+    }
+
+    // a key block that no query can see still owns its dbias column (row-broadcast case)
+    if (has_bias && !bias_rows && n_steps == 0 && !use_accum && g == 0 && key < f.Lk) {
+        const int ngh = (f.Hb == f.H) ? G : 1;
+        for (int gh = 0; gh < ngh; gh++) {
+            const int hb = f.Hb == f.H ? hk * G + gh : (f.Hb == 1 ? 0 : hk);
+            ((uint16_t *)p.dbias)[b * p.db_b + hb * p.db_h + key] = 0;
+        }
+    }
+
+    // ---- store dK (scaled) and dV: lane owns one key row, 8 consecutive head-dim elements per store
+    if (key < f.Lk) {
+        uint16_t *dkp = (uint16_t *)p.dk + b * p.dk_b + (int64_t)key * p.dk_r + hk * p.dk_h;
+        uint16_t *dvp = (uint16_t *)p.dv + b * p.dv_b + (int64_t)key * p.dv_r + hk * p.dv_h;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int blk = 0; blk < 2; blk++) {
+                int c = 32 * db + 16 * blk + 8 * g;
+                if (c < f.d) {
+                    u32x4_t wk, wv;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        wk[e] = E::pack2(dk[db][8 * blk + 2 * e] * f.scale, dk[db][8 * blk + 2 * e + 1] * f.scale);
+                        wv[e] = E::pack2(dv[db][8 * blk + 2 * e], dv[db][8 * blk + 2 * e + 1]);
+                    }
+                    *(u32x4_t *)(dkp + c) = wk;
+                    *(u32x4_t *)(dvp + c) = wv;
+                }
+            }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// 3. dQ
+// ------------------------------------------------------------------------------------------------
+constexpr int Q_BM = 128;
+constexpr int Q_BN = 64;
+
+template <int D> struct DqSmem {
+    static constexpr int S = D + 8;
+    static constexpr int K_BYTES = Q_BN * S * 2;
+    static constexpr int TOTAL = 2 * K_BYTES;
+};
+
+template <typename T, int D, bool CAUSAL>
+__global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_kernel(const BwdParams p) {
+    using E = Elem<T>;
+    using SM = DqSmem<D>;
+    constexpr int KS = D / 16;
+    constexpr int DB = D / 32;
+
+    __shared__ __attribute__((aligned(16))) char smem[SM::TOTAL];
+    char *sK = smem, *sV = smem + SM::K_BYTES;
+
+    const FwdParams &f = p.f;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 31, g = lane >> 5;
+    const int m_block = gridDim.x - 1 - blockIdx.x;
+    const int h = blockIdx.y, b = blockIdx.z;
+    const int hk = h / (f.H / f.Hk);
+    const int m0 = m_block * Q_BM;
+    const int qrow = m0 + wave * 32 + r;
+    const int qrow_c = qrow < f.Lq ? qrow : f.Lq - 1;
+    const int shift = f.Lk - f.Lq;
+
+    u32x4_t qf[KS], dof[KS];
+    {
+        const uint16_t *qp = (const uint16_t *)f.q + b * f.q_b + (int64_t)qrow_c * f.q_r + h * f.q_h;
+        const uint16_t *dp = (const uint16_t *)p.dout + b * p.do_b + (int64_t)qrow_c * p.do_r + h * p.do_h;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            int c = ks * 16 + g * 8;
+            u32x4_t qv = {0, 0, 0, 0}, dv = {0, 0, 0, 0};
+            if (qrow < f.Lq && c < f.d) { qv = *(const u32x4_t *)(qp + c); dv = *(const u32x4_t *)(dp + c); }
+            qf[ks] = qv;
+            dof[ks] = dv;
+        }
+    }
+    float lse2 = INFINITY, dd = 0.f;
+    if (qrow < f.Lq) {
+        lse2 = f.lse[((int64_t)b * f.H + h) * f.Lq + qrow] * kLog2e;
+        dd = p.softmax_d[((int64_t)b * f.H + h) * p.Lq_rounded + qrow];
+    }
+
+    int n_end = (f.Lk + Q_BN - 1) / Q_BN;
+    if (CAUSAL) {
+        int lim = m0 + Q_BM + shift;
+        if (lim < 0) lim = 0;
+        int ne = (lim + Q_BN - 1) / Q_BN;
+        if (ne < n_end) n_end = ne;
+    }
+
+    f32x16_t dq[DB];
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) dq[db][i] = 0.f;
+
+    const int hm = f.mask ? (f.Hm == f.H ? h : (f.Hm == 1 ? 0 : h / (f.H / f.Hm))) : 0;
+    const int hb = f.bias ? (f.Hb == f.H ? h : (f.Hb == 1 ? 0 : h / (f.H / f.Hb))) : 0;
+    const uint8_t *mrow = f.mask ? f.mask + b * f.m_b + hm * f.m_h + (int64_t)qrow_c * f.m_r : nullptr;
+    const uint16_t *brow = f.bias ? (const uint16_t *)f.bias + b * f.bi_b + hb * f.bi_h + (int64_t)qrow_c * f.bi_r : nullptr;
+    const uint16_t *kbase = (const uint16_t *)f.k + b * f.k_b + hk * f.k_h;
+    const uint16_t *vbase = (const uint16_t *)f.v + b * f.v_b + hk * f.v_h;
+
+    const int a_row = pi_row(r);
+    const int tj = lane & 15, te = tj >> 2, tc = tj & 3;
+    const int tcp = (tc == 1) ? 2 : (tc == 2 ? 1 : tc);
+    const int tdh = (lane >> 4) & 1;
+    const uint32_t tr_off = (uint32_t)(((8 * g + te) * SM::S + 16 * tdh + 4 * tcp) * 2);
+
+    for (int j = 0; j < n_end; j++) {
+        const int n0 = j * Q_BN;
+        uint32_t keep = 0;
+#pragma unroll
+        for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+            for (int blk = 0; blk < 2; blk++) {
+                int c0 = n0 + 32 * mb + 16 * blk + 8 * g;
+                uint32_t bits = 0xffu;
+                if (mrow) {
+                    bits = 0;
+                    if (c0 < f.Lk) {
+                        u32x2_t mv = *(const u32x2_t *)(mrow + c0);
+                        bits = nz_bytes_to_bits(mv[0]) | (nz_bytes_to_bits(mv[1]) << 4);
+                    }
+                }
+                int lim = f.Lk;
+                if (CAUSAL) { int cl = qrow + 1 + shift; lim = cl < lim ? cl : lim; }
+                int nvis = lim - c0;
+                uint32_t vis = nvis >= 8 ? 0xffu : (nvis <= 0 ? 0u : ((1u << nvis) - 1u));
+                bits &= vis;
+                if (qrow >= f.Lq) bits = 0;
+                keep |= bits << (16 * mb + 8 * blk);
+            }
+        const int active = __syncthreads_or(keep != 0);
+        if (!active) continue;
+
+        {
+            constexpr int CH = D / 8, RPP = NTHREADS / CH;
+            const int c = tid % CH, r0 = tid / CH;
+#pragma unroll
+            for (int it = 0; it < Q_BN / RPP; it++) {
+                int row = r0 + it * RPP, kk = n0 + row;
+                u32x4_t kv = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
+                if (kk < f.Lk && c * 8 < f.d) {
+                    kv = *(const u32x4_t *)(kbase + (int64_t)kk * f.k_r + c * 8);
+                    vv = *(const u32x4_t *)(vbase + (int64_t)kk * f.v_r + c * 8);
+                }
+                *(u32x4_t *)(sK + (row * SM::S + c * 8) * 2) = kv;
+                *(u32x4_t *)(sV + (row * SM::S + c * 8) * 2) = vv;
+            }
+        }
+        float bl2[32];
+#pragma unroll
+        for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+            for (int blk = 0; blk < 2; blk++) {
+                int c0 = n0 + 32 * mb + 16 * blk + 8 * g;
+                u32x4_t bv = {0, 0, 0, 0};
+                if (brow && c0 < f.Lk) bv = *(const u32x4_t *)(brow + c0);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    bl2[16 * mb + 8 * blk + 2 * e] = E::lo(bv[e]) * kLog2e;
+                    bl2[16 * mb + 8 * blk + 2 * e + 1] = E::hi(bv[e]) * kLog2e;
+                }
+            }
+        __syncthreads();
+
+        // ---- S^T = K Q^T, dP^T = V dO^T
+        f32x16_t s[2], dp[2];
+#pragma unroll
+        for (int mb = 0; mb < 2; mb++) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) { s[mb][i] = 0.f; dp[mb][i] = 0.f; }
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                u32x4_t ka = *(const u32x4_t *)(sK + ((32 * mb + a_row) * SM::S + ks * 16 + g * 8) * 2);
+                u32x4_t va = *(const u32x4_t *)(sV + ((32 * mb + a_row) * SM::S + ks * 16 + g * 8) * 2);
+                s[mb] = E::mfma(ka, qf[ks], s[mb]);
+                dp[mb] = E::mfma(va, dof[ks], dp[mb]);
+            }
+        }
+        uint32_t dpk[16];
+#pragma unroll
+        for (int mb = 0; mb < 2; mb++)
+#pragma unroll
+            for (int i = 0; i < 16; i += 2) {
+                float d2[2];
+#pragma unroll
+                for (int e = 0; e < 2; e++) {
+                    const int ii = i + e;
+                    float x = fmaf(s[mb][ii], f.scale_log2, bl2[16 * mb + ii]) - lse2;
+                    float pe = ((keep >> (16 * mb + ii)) & 1u) ? fast_exp2(x) : 0.f;
+                    d2[e] = pe * (dp[mb][ii] - dd);
+                }
+                dpk[8 * mb + i / 2] = E::pack2(d2[0], d2[1]);
+            }
+        // ---- dQ^T += K^T dS^T
+#pragma unroll
+        for (int kb = 0; kb < 4; kb++) {
+            u32x4_t bop = {dpk[4 * kb], dpk[4 * kb + 1], dpk[4 * kb + 2], dpk[4 * kb + 3]};
+#pragma unroll
+            for (int db = 0; db < DB; db++) {
+                uint32_t off = tr_off + (uint32_t)((16 * kb * SM::S + 32 * db) * 2);
+                u32x2_t lo = lds_read_tr16(sK, off), hi = lds_read_tr16(sK, off + 4 * SM::S * 2);
+                u32x4_t a = {lo[0], lo[1], hi[0], hi[1]};
+                dq[db] = E::mfma(a, bop, dq[db]);
+            }
+        }
+    }
+
+    if (qrow < f.Lq) {
+        uint16_t *dqp = (uint16_t *)p.dq + b * p.dq_b + (int64_t)qrow * p.dq_r + h * p.dq_h;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int blk = 0; blk < 2; blk++) {
+                int c = 32 * db + 16 * blk + 8 * g;
+                if (c < f.d) {
+                    u32x4_t w;
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        w[e] = E::pack2(dq[db][8 * blk + 2 * e] * f.scale, dq[db][8 * blk + 2 * e + 1] * f.scale);
+                    *(u32x4_t *)(dqp + c) = w;
+                }
+            }
+    }
+}
+
+// ------------------------------------------------------------------------------------------------
+// fp32 dbias accumulator helpers (only when several workgroups share a dbias element)
+// ------------------------------------------------------------------------------------------------
+__global__ void fill_zero_kernel(float *ptr, size_t n) {
+    size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x, stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < n; i += stride) ptr[i] = 0.f;
+}
+
+template <typename T>
+__global__ void dbias_convert_kernel(const BwdParams p, int nb, int nh, int nr, int lk) {
+    using E = Elem<T>;
+    size_t total = (size_t)nb * nh * nr * lk;
+    size_t i = blockIdx.x * (size_t)blockDim.x + threadIdx.x, stride = (size_t)gridDim.x * blockDim.x;
+    for (; i < total; i += stride) {
+        int k = (int)(i % lk);
+        size_t t = i / lk;
+        int rr = (int)(t % nr); t /= nr;
+        int hh = (int)(t % nh);
+        int bb = (int)(t / nh);
+        float v = p.dbias_accum[bb * p.dba_b + hh * p.dba_h + (int64_t)rr * p.dba_r + k];
+        ((uint16_t *)p.dbias)[bb * p.db_b + hh * p.db_h + (int64_t)rr * p.db_r + k] = (uint16_t)(E::pack2(v, 0.f) & 0xffffu);
+    }
+}
+
+template <typename T, int D>
+hipError_t launch_bwd_t(const BwdParams &p, hipStream_t stream) {
+    const FwdParams &f = p.f;
+    hipError_t e;
+    // 1. D = rowsum(dO * O)
+    {
+        const int CH = (f.d + 7) / 8, lanes = CH <= 8 ? 8 : 16, rpb = 256 / lanes;
+        dim3 grid((p.Lq_rounded + rpb - 1) / rpb, f.H, f.B);
+        hipLaunchKernelGGL((bwd_dot_kernel<T>), grid, dim3(256), 0, stream, p);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+    }
+    const int nb = f.bi_b == 0 ? 1 : f.B, nr = f.bi_r == 0 ? 1 : f.Lq;
+    if (p.dbias_accum) {
+        size_t n = (size_t)nb * f.Hb * nr * ((f.Lk + 7) / 8 * 8);
+        hipLaunchKernelGGL(fill_zero_kernel, dim3(1024), dim3(256), 0, stream, p.dbias_accum, n);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+    }
+    // 2. dK, dV, dBias
+    if (f.Lk > 0) {
+        dim3 grid((f.Lk + KV_BN - 1) / KV_BN, f.Hk, f.B);
+        const size_t smem = KvSmem<D>::TOTAL;
+        if (f.causal) {
+            auto kern = bwd_dkdv_kernel<T, D, true>;
+            if ((e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem)) != hipSuccess) return e;
+            hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, stream, p);
+        } else {
+            auto kern = bwd_dkdv_kernel<T, D, false>;
+            if ((e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem)) != hipSuccess) return e;
+            hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, stream, p);
+        }
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+    }
+    if (p.dbias_accum) {
+        hipLaunchKernelGGL((dbias_convert_kernel<T>), dim3(1024), dim3(256), 0, stream, p, nb, f.Hb, nr, f.Lk);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+    }
+    // 3. dQ
+    {
+        dim3 grid((f.Lq + Q_BM - 1) / Q_BM, f.H, f.B);
+        if (f.causal)
+            hipLaunchKernelGGL((bwd_dq_kernel<T, D, true>), grid, dim3(NTHREADS), 0, stream, p);
+        else
+            hipLaunchKernelGGL((bwd_dq_kernel<T, D, false>), grid, dim3(NTHREADS), 0, stream, p);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+    }
+    return hipSuccess;
+}
+
+}  // namespace
+
+hipError_t launch_bwd(const BwdParams &p, int dtype, hipStream_t stream) {
+    if (p.f.B <= 0 || p.f.Lq <= 0) return hipSuccess;
+    const bool d64 = p.f.d <= 64;
+    if (dtype == 0) return d64 ? launch_bwd_t<bf16_tag, 64>(p, stream) : launch_bwd_t<bf16_tag, 128>(p, stream);
+    return d64 ? launch_bwd_t<fp16_tag, 64>(p, stream) : launch_bwd_t<fp16_tag, 128>(p, stream);
+}
+
+}  // namespace fdma
