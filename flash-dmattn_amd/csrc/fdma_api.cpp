@@ -52,7 +52,7 @@ int validate_common(const fdma_fwd_args *a, bool backward) {
                                                : "query, key, value, and out_ must have a head_size that is a multiple of 8");
     if (a->num_heads % a->num_heads_k != 0)
         return fail(FDMA_ERR_INVALID, "Number of heads in key/value must divide number of heads in query");
-    if (!a->q || !a->k || !a->v) return fail(FDMA_ERR_INVALID, "q, k, v must be device pointers");
+    if (!a->q || ((!a->k || !a->v) && a->seqlen_k > 0)) return fail(FDMA_ERR_INVALID, "q, k, v must be device pointers");
     if (!a->out) return fail(FDMA_ERR_INVALID, "out must be a device pointer");
     if (!a->lse) return fail(FDMA_ERR_INVALID, "softmax_lse must be a device pointer");
     if (a->mask) {

@@ -1,0 +1,165 @@
+"""CPU-only checks of the drop-in boundary: the C-ABI library loads and exports every symbol that
+include/fdma.h declares, the ctypes mirrors match the compiled structs, argument validation
+reproduces the reference's error rules (csrc/flash_sparse_attn/flash_api.cpp:371-438, 824-898 of the
+reference) without touching a GPU, and the Python surface has the reference's names and signatures
+(flash_sparse_attn/__init__.py:87-97, flash_sparse_attn_interface.py:610-621)."""
+import ctypes
+import inspect
+import os
+import re
+
+import pytest
+import torch
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    from flash_sparse_attn import _cabi
+
+    header = open(os.path.join(ROOT, "include", "fdma.h")).read()
+    header = re.sub(r"/\*.*?\*/", "", header, flags=re.S)
+    declared = set(re.findall(r"\b(fdma_[a-z_0-9]+)\s*\(", header))
+    assert declared == set(_cabi.EXPORTS), declared ^ set(_cabi.EXPORTS)
+    lib = ctypes.CDLL(_cabi.lib_path())
+    for name in declared:
+        assert hasattr(lib, name), f"{name} not exported"
+    assert lib.fdma_abi_version() == 1
+
+
+def test_struct_mirrors_match_compiled_sizes():
+    from flash_sparse_attn import _cabi
+
+    assert _cabi.lib.fdma_sizeof_fwd_args() == ctypes.sizeof(_cabi.FwdArgs)
+    assert _cabi.lib.fdma_sizeof_bwd_args() == ctypes.sizeof(_cabi.BwdArgs)
+
+
+def _valid_fwd():
+    from flash_sparse_attn import _cabi
+
+    a = _cabi.FwdArgs()
+    for name in ("q", "k", "v", "out", "lse"):
+        setattr(a, name, 0x1000)
+    a.batch, a.seqlen_q, a.seqlen_k = 2, 128, 256
+    a.num_heads, a.num_heads_k, a.num_heads_mask, a.num_heads_bias = 8, 2, 1, 1
+    a.head_dim, a.dtype, a.is_causal, a.softmax_scale, a.softcap = 64, 0, 1, 0.125, 0.0
+    for s, v in (("q_strides", (128 * 8 * 64, 8 * 64, 64)), ("k_strides", (256 * 2 * 64, 2 * 64, 64)),
+                 ("v_strides", (256 * 2 * 64, 2 * 64, 64)), ("o_strides", (128 * 8 * 64, 8 * 64, 64))):
+        getattr(a, s)[:] = v
+    return a
+
+
+def test_validation_accepts_a_good_call_and_needs_no_gpu():
+    from flash_sparse_attn import _cabi
+
+    a = _valid_fwd()
+    assert _cabi.lib.fdma_fwd_validate(a) == 0, _cabi.last_error()
+    assert _cabi.lib.fdma_fwd_workspace_bytes(a) == 0
+
+
+@pytest.mark.parametrize(
+    "mutate,needle",
+    [
+        (lambda a: setattr(a, "dtype", 7), "only support fp16 and bf16"),
+        (lambda a: setattr(a, "batch", 0), "batch size must be positive"),
+        (lambda a: setattr(a, "head_dim", 264), "at most 256"),
+        (lambda a: setattr(a, "head_dim", 60), "multiple of 8"),
+        (lambda a: setattr(a, "num_heads_k", 3), "must divide number of heads in query"),
+        (lambda a: (setattr(a, "mask", 0x2000), setattr(a, "num_heads_mask", 3)), "Number of heads in mask must be 1, h_k or h"),
+        (lambda a: (setattr(a, "bias", 0x2000), setattr(a, "num_heads_bias", 5)), "Number of heads in bias must be 1, h_k or h"),
+        (lambda a: setattr(a, "q", 0x1004), "16-byte aligned"),
+        (lambda a: setattr(a, "softcap", 30.0), "softcap"),
+    ],
+)
+def test_validation_errors(mutate, needle):
+    from flash_sparse_attn import _cabi
+
+    a = _valid_fwd()
+    mutate(a)
+    rc = _cabi.lib.fdma_fwd_validate(a)
+    assert rc < 0
+    assert needle in _cabi.last_error(), _cabi.last_error()
+    with pytest.raises(RuntimeError, match=re.escape(needle)):
+        _cabi.check(rc)
+
+
+def test_backward_validation():
+    from flash_sparse_attn import _cabi
+
+    b = _cabi.BwdArgs()
+    ctypes.memmove(ctypes.byref(b.f), ctypes.byref(_valid_fwd()), ctypes.sizeof(_cabi.FwdArgs))
+    for name in ("dout", "dq", "dk", "dv", "softmax_d"):
+        setattr(b, name, 0x3000)
+    for s, src in (("do_strides", b.f.q_strides), ("dq_strides", b.f.q_strides), ("dk_strides", b.f.k_strides), ("dv_strides", b.f.k_strides)):
+        getattr(b, s)[:] = list(src)
+    assert _cabi.lib.fdma_bwd_validate(b) == 0, _cabi.last_error()
+    b.f.bias = 0x4000  # bias without dbias
+    assert _cabi.lib.fdma_bwd_validate(b) < 0 and "dbias" in _cabi.last_error()
+    b.dbias = 0x5000
+    b.f.bias_strides[:] = (512, 256, 0)
+    b.dbias_strides[:] = (512, 256, 256)  # broadcast pattern differs from the bias
+    assert _cabi.lib.fdma_bwd_validate(b) < 0 and "broadcast pattern" in _cabi.last_error()
+    b.dbias_strides[:] = (512, 256, 0)
+    assert _cabi.lib.fdma_bwd_validate(b) == 0, _cabi.last_error()
+    # bias broadcast over kv groups (1 head, Hk = 2): shared dbias elements need fp32 scratch
+    assert _cabi.lib.fdma_bwd_workspace_bytes(b) == 2 * 1 * 1 * 256 * 4
+    b.f.num_heads_bias = 2
+    assert _cabi.lib.fdma_bwd_workspace_bytes(b) == 0
+    b.f.bias_strides[0] = b.dbias_strides[0] = 0  # batch-broadcast bias with batch 2: shared again
+    assert _cabi.lib.fdma_bwd_workspace_bytes(b) == 1 * 2 * 1 * 256 * 4
+
+
+def test_decode_workspace_size():
+    from flash_sparse_attn import _cabi
+
+    a = _valid_fwd()
+    a.batch, a.seqlen_q, a.seqlen_k, a.num_heads, a.num_heads_k, a.head_dim = 8, 1, 65536, 32, 8, 128
+    n = _cabi.lib.fdma_fwd_workspace_bytes(a)
+    assert n > 0 and n % ((128 + 1) * 4 * 8 * 32) == 0  # splits * B * H rows of (d + 1) floats
+
+
+def test_python_surface_matches_reference_names():
+    import flash_sparse_attn as fsa
+    from flash_sparse_attn import flash_sparse_attn_interface as itf
+
+    assert fsa.__version__ == "1.2.3"
+    assert set(fsa.__all__) == {
+        "CUDA_AVAILABLE", "TRITON_AVAILABLE", "FLEX_AVAILABLE", "flash_sparse_attn_func", "flash_sparse_attn_varlen_func",
+        "triton_sparse_attn_func", "flex_sparse_attn_func", "get_available_backends", "flash_sparse_attn_func_auto"}
+    assert fsa.CUDA_AVAILABLE and fsa.get_available_backends() == ["cuda"]
+    assert fsa.flash_sparse_attn_func_auto() is fsa.flash_sparse_attn_func
+    assert fsa.flash_sparse_attn_func_auto(backend="cuda") is itf.flash_sparse_attn_func
+    with pytest.raises(RuntimeError, match="Triton backend is not available"):
+        fsa.flash_sparse_attn_func_auto(backend="triton")
+    with pytest.raises(RuntimeError, match="Flex backend is not available"):
+        fsa.flash_sparse_attn_func_auto(backend="flex")
+    with pytest.raises(ValueError, match="Unknown backend"):
+        fsa.flash_sparse_attn_func_auto(backend="nope")
+    sig = inspect.signature(itf.flash_sparse_attn_func)
+    assert list(sig.parameters) == ["query", "key", "value", "attn_mask", "attn_bias", "softmax_scale", "is_causal",
+                                    "softcap", "deterministic", "return_attn_probs"]
+    assert all(p.default is None for n, p in sig.parameters.items() if n not in ("query", "key", "value"))
+    for name in ("FlashDMAttnFunc", "_flash_sparse_attn_forward", "_flash_sparse_attn_backward", "maybe_contiguous",
+                 "round_multiple", "flash_sparse_attn_varlen_func"):
+        assert hasattr(itf, name)
+    # the custom ops are registered under the reference's names
+    assert hasattr(torch.ops.flash_sparse_attn, "_flash_sparse_attn_forward")
+    assert hasattr(torch.ops.flash_sparse_attn, "_flash_sparse_attn_backward")
+
+
+def test_cpu_tensors_are_rejected_loudly():
+    """No CPU fallback: the operator only exists for device tensors (device_types="cuda")."""
+    from flash_sparse_attn import flash_sparse_attn_func
+
+    q = torch.randn(1, 8, 2, 64, dtype=torch.bfloat16)
+    with pytest.raises((RuntimeError, NotImplementedError)):
+        flash_sparse_attn_func(q, q, q)
+
+
+def test_product_package_never_imports_the_oracle():
+    pkg = os.path.join(ROOT, "flash-dmattn_amd")
+    for dirpath, _, files in os.walk(pkg):
+        for fn in files:
+            if fn.endswith((".py", ".cpp", ".hip", ".h")):
+                text = open(os.path.join(dirpath, fn)).read()
+                assert "oracle" not in text.lower(), f"{fn} mentions the oracle"

@@ -1,0 +1,279 @@
+"""GPU parity tests of the hot path (run with `-m gpu` on an MI355X).
+
+Every case goes through the Python operator, i.e. through the C ABI of libfdma_hip.so, and is
+compared with the oracle on identical seeded inputs:
+  * small shapes against the C oracle (oracle/fdma_oracle.c, IEEE double on the same bf16 bits);
+  * larger shapes against the fp32 safe-eager restatement evaluated on the GPU (the C oracle would
+    take minutes), which test_oracle.py ties to the C oracle.
+Tolerances (bf16 compute): max-abs error of the output <= 2e-2; gradients within rtol 5e-2 as
+defined in _util.assert_grad_close.
+"""
+import pytest
+import torch
+
+from oracle import c_oracle, eager
+from _util import assert_grad_close, assert_out_close, make_inputs, topk_keep_mask
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _op():
+    from flash_sparse_attn import flash_sparse_attn_func
+    return flash_sparse_attn_func
+
+
+def _to_dev(*ts):
+    return [t.to(DEV) if t is not None else None for t in ts]
+
+
+def _run_fwd_bwd(q, k, v, mask, bias, causal, scale=None, dout=None, need_grad=True):
+    qd, kd, vd, md, bd = _to_dev(q, k, v, mask, bias)
+    if need_grad:
+        qd, kd, vd = [t.requires_grad_(True) for t in (qd, kd, vd)]
+        if bd is not None:
+            bd.requires_grad_(True)
+    out, lse, _ = _op()(qd, kd, vd, md, bd, scale, causal, None, None, True)
+    grads = None
+    if need_grad:
+        do = torch.ones_like(out) if dout is None else dout.to(DEV)
+        out.backward(do)
+        grads = (qd.grad, kd.grad, vd.grad, bd.grad if bd is not None else None)
+    torch.cuda.synchronize()
+    return out.detach(), lse.detach(), grads
+
+
+def _check_lse(lse, ref):
+    ref = ref.to(lse.device)
+    assert torch.equal(torch.isinf(lse), torch.isinf(ref)), "empty-row pattern of the LSE differs"
+    fin = torch.isfinite(ref)
+    if fin.any():
+        assert (lse[fin] - ref[fin]).abs().max().item() <= 1e-2
+    assert (lse[~fin] > 0).all()
+
+
+SMALL_CASES = {
+    # name: (B, Lq, Lk, H, Hk, D, bias_shape, mask_shape, window, causal)
+    "cfg1_mqa_rowbias_topk128": (1, 256, 256, 2, 1, 64, (1, 1, 1, 256), (1, 1, 1, 256), 128, True),
+    "plain_noncausal_d128": (1, 256, 256, 2, 2, 128, None, None, None, False),
+    "plain_causal_ragged": (2, 300, 300, 4, 2, 128, None, None, None, True),
+    "bias_only_per_head": (1, 256, 320, 4, 2, 64, (1, 4, 1, 320), None, None, True),
+    "full_mask_full_bias": (2, 200, 264, 4, 2, 64, (2, 4, 200, 264), (2, 4, 200, 264), 64, True),
+    "full_bias_kv_heads": (2, 200, 264, 4, 2, 64, (2, 2, 200, 264), (2, 1, 200, 264), 64, True),
+    "full_bias_batch_broadcast": (2, 200, 264, 4, 2, 64, (1, 2, 200, 264), (2, 1, 200, 264), 64, True),
+    "row_bias_single_head": (2, 200, 264, 4, 2, 64, (2, 1, 1, 264), (2, 1, 1, 264), 64, False),
+    "lq_lt_lk_bottom_right": (1, 100, 333, 2, 2, 128, (1, 2, 1, 333), (1, 1, 100, 333), 100, True),
+    "lq_gt_lk_empty_rows": (1, 333, 100, 2, 2, 128, (1, 2, 1, 100), (1, 1, 333, 100), 50, True),
+    "head_dim_96": (1, 256, 256, 2, 1, 96, (1, 1, 1, 256), (1, 1, 1, 256), 128, True),
+    "head_dim_32": (1, 192, 256, 2, 1, 32, (1, 1, 1, 256), (1, 1, 1, 256), 128, False),
+    "tiny": (1, 3, 5, 2, 1, 8, (1, 1, 3, 5), (1, 1, 3, 5), 2, True),
+}
+
+
+@pytest.mark.parametrize("name", list(SMALL_CASES))
+def test_forward_backward_vs_c_oracle(name):
+    B, Lq, Lk, H, Hk, D, bshape, mshape, W, causal = SMALL_CASES[name]
+    q, k, v, mask, bias = make_inputs(B, Lq, Lk, H, Hk, D, bshape, mshape, W, seed=0)
+    dout = torch.randn(B, Lq, H, D, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16)
+    out, lse, (dq, dk, dv, db) = _run_fwd_bwd(q, k, v, mask, bias, causal, dout=dout)
+    ro, rl = c_oracle.forward(q, k, v, mask, bias, None, causal)
+    assert out.dtype == torch.bfloat16 and out.shape == q.shape and lse.shape == (B, H, Lq)
+    assert_out_close(out.cpu(), ro)
+    _check_lse(lse.cpu(), rl)
+    rdq, rdk, rdv, rdb = c_oracle.backward(q, k, v, dout, mask, bias, None, causal)
+    assert_grad_close(dq.cpu(), rdq, "dq")
+    assert_grad_close(dk.cpu(), rdk, "dk")
+    assert_grad_close(dv.cpu(), rdv, "dv")
+    if bias is not None:
+        assert db.shape == bias.shape and db.dtype == bias.dtype
+        assert_grad_close(db.cpu(), rdb, "dbias")
+
+
+def test_fp16_inputs():
+    q, k, v, mask, bias = make_inputs(1, 256, 256, 2, 1, 64, (1, 1, 1, 256), (1, 1, 1, 256), 128, seed=0, dtype=torch.float16)
+    out, lse, (dq, dk, dv, db) = _run_fwd_bwd(q, k, v, mask, bias, True)
+    ro, rl = c_oracle.forward(q, k, v, mask, bias, None, True)
+    assert out.dtype == torch.float16
+    assert_out_close(out.cpu(), ro)
+    rdq, rdk, rdv, rdb = c_oracle.backward(q, k, v, torch.ones_like(ro), mask, bias, None, True)
+    for g, r, n in ((dq, rdq, "dq"), (dk, rdk, "dk"), (dv, rdv, "dv"), (db, rdb, "dbias")):
+        assert_grad_close(g.cpu(), r, n)
+
+
+def test_cfg1_reference_plumbing_config():
+    """Config 1 of the benchmark: B=1, L=256, H=2, Hkv=1 (MQA), d=64, bias [B,Hkv,1,Lk], mask = top-128
+    keys by bias intersected with causal (given both as a full-shape mask and as column mask +
+    is_causal), scale 1/8, loss = out.sum()."""
+    q, k, v, colmask, bias = make_inputs(1, 256, 256, 2, 1, 64, (1, 1, 1, 256), (1, 1, 1, 256), 128, seed=0)
+    full = colmask.expand(1, 1, 256, 256) & torch.tril(torch.ones(256, 256, dtype=torch.bool))
+    ro, rl = c_oracle.forward(q, k, v, full, bias, 0.125, True)
+    rdq, rdk, rdv, rdb = c_oracle.backward(q, k, v, torch.ones_like(ro), full, bias, 0.125, True)
+    for m in (full, colmask):
+        out, lse, (dq, dk, dv, db) = _run_fwd_bwd(q, k, v, m, bias, True, scale=0.125)
+        assert_out_close(out.cpu(), ro)
+        _check_lse(lse.cpu(), rl)
+        for g, r, n in ((dq, rdq, "dq"), (dk, rdk, "dk"), (dv, rdv, "dv"), (db, rdb, "dbias")):
+            assert_grad_close(g.cpu(), r, n)
+    assert int(torch.isinf(rl).sum()) > 0, "this config is expected to contain rows without a visible key"
+
+
+def test_non_contiguous_views_and_mask_bias_key_dim_one():
+    # q/k/v given as transposed views of (B,H,L,D) tensors (forward_equivalence.py:175-177 pattern),
+    # bias with key dim 1 (expanded by the operator; dbias summed back over keys, interface.py:495-496)
+    B, L, H, Hk, D = 2, 192, 4, 2, 64
+    g = torch.Generator().manual_seed(3)
+    q = torch.randn(B, H, L, D, generator=g).to(torch.bfloat16).transpose(1, 2)
+    k = torch.randn(B, Hk, L, D, generator=g).to(torch.bfloat16).transpose(1, 2)
+    v = torch.randn(B, Hk, L, D, generator=g).to(torch.bfloat16).transpose(1, 2)
+    bias = torch.randn(B, Hk, L, 1, generator=g).to(torch.bfloat16)
+    mask = torch.rand(B, 1, L, L, generator=g) > 0.3
+    out, lse, (dq, dk, dv, db) = _run_fwd_bwd(q, k, v, mask, bias, True)
+    ro, _ = c_oracle.forward(q, k, v, mask, bias.expand(B, Hk, L, L), None, True)
+    assert_out_close(out.cpu(), ro)
+    rdq, rdk, rdv, rdb = c_oracle.backward(q, k, v, torch.ones_like(ro), mask, bias.expand(B, Hk, L, L), None, True)
+    assert db.shape == bias.shape
+    assert_grad_close(dq.cpu(), rdq, "dq")
+    assert_grad_close(dk.cpu(), rdk, "dk")
+    assert_grad_close(dv.cpu(), rdv, "dv")
+    # rows of dS sum to zero, so the exact dbias of a key-broadcast bias is 0; what the operator returns
+    # is the sum over keys of bf16-rounded dS elements: rounding noise of about sqrt(L) half-ulps
+    assert rdb.sum(-1, keepdim=True).abs().max() < 1e-4
+    noise = 3.0 * (L ** 0.5) * 2.0 ** -9 * rdb.abs().max().item()
+    worst = db.float().abs().max().item()
+    assert worst <= noise, f"key-broadcast dbias {worst:.3e} exceeds rounding noise bound {noise:.3e}"
+
+
+def test_fully_masked_tiles_are_skipped_and_rows_without_keys_give_zero():
+    # block-structured mask: whole 64-key tiles masked out, plus a band of query rows with nothing kept
+    B, L, H, Hk, D = 1, 512, 2, 2, 128
+    q, k, v, _, bias = make_inputs(B, L, L, H, Hk, D, (B, Hk, 1, L), None, seed=5)
+    mask = torch.zeros(B, 1, L, L, dtype=torch.bool)
+    mask[..., 64:128] = True
+    mask[..., 320:384] = True
+    mask[:, :, 200:260, :] = False
+    out, lse, (dq, dk, dv, db) = _run_fwd_bwd(q, k, v, mask, bias, False)
+    ro, rl = c_oracle.forward(q, k, v, mask, bias, None, False)
+    assert_out_close(out.cpu(), ro)
+    _check_lse(lse.cpu(), rl)
+    assert torch.equal(out[:, 200:260].cpu(), torch.zeros(B, 60, H, D, dtype=torch.bfloat16))
+    rdq, rdk, rdv, rdb = c_oracle.backward(q, k, v, torch.ones_like(ro), mask, bias, None, False)
+    for g, r, n in ((dq, rdq, "dq"), (dk, rdk, "dk"), (dv, rdv, "dv"), (db, rdb, "dbias")):
+        assert_grad_close(g.cpu(), r, n)
+    assert torch.equal(dk[:, :64].cpu(), torch.zeros(B, 64, Hk, D, dtype=torch.bfloat16))  # keys nobody keeps
+
+
+def test_seqlen_k_zero_and_no_grad_path():
+    q = torch.randn(1, 16, 2, 64, dtype=torch.bfloat16, device=DEV)
+    k = torch.empty(1, 0, 2, 64, dtype=torch.bfloat16, device=DEV)
+    out, lse, _ = _op()(q, k, k, None, None, None, False, None, None, True)
+    assert torch.equal(out, torch.zeros_like(out)) and torch.isinf(lse).all() and (lse > 0).all()
+    with torch.no_grad():
+        q2 = torch.randn(1, 64, 2, 64, dtype=torch.bfloat16, device=DEV)
+        o = _op()(q2, q2, q2, is_causal=True)
+    assert o.shape == q2.shape and not o.requires_grad
+
+
+def test_deterministic_rerun_is_bit_identical():
+    q, k, v, mask, bias = make_inputs(2, 384, 384, 4, 2, 64, (2, 2, 384, 384), (2, 2, 384, 384), 96, seed=7)
+    a = _run_fwd_bwd(q, k, v, mask, bias, True)
+    b = _run_fwd_bwd(q, k, v, mask, bias, True)
+    assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
+    for x, y in zip(a[2], b[2]):
+        assert torch.equal(x, y)
+
+
+MID_CASES = {
+    # scaled-down versions of benchmark configs 2-4 (same head structure, shorter sequences),
+    # checked against the fp32 eager restatement on the GPU
+    "cfg2_like_gqa4_d128": (1, 2048, 2048, 8, 2, 128, (1, 2, 1, 2048), (1, 2, 1, 2048), 512, True),
+    "cfg3_like_full_dbias_d64": (2, 1024, 1024, 4, 4, 64, (2, 4, 1024, 1024), (2, 4, 1024, 1024), 256, True),
+    "cfg4_like_sparse_d128": (1, 4096, 4096, 4, 1, 128, (1, 1, 1, 4096), (1, 1, 1, 4096), 128, True),
+}
+
+
+@pytest.mark.parametrize("name", list(MID_CASES))
+def test_mid_size_vs_eager_fp32(name):
+    B, Lq, Lk, H, Hk, D, bshape, mshape, W, causal = MID_CASES[name]
+    q, k, v, mask, bias = make_inputs(B, Lq, Lk, H, Hk, D, bshape, mshape, W, seed=11)
+    out, lse, (dq, dk, dv, db) = _run_fwd_bwd(q, k, v, mask, bias, causal)
+    qd, kd, vd, md, bd = _to_dev(q, k, v, mask, bias)
+    ro, rdq, rdk, rdv, rdb = eager.attention_forward_backward(qd, kd, vd, md, bd, None, causal)
+    assert_out_close(out, ro)
+    for g, r, n in ((dq, rdq, "dq"), (dk, rdk, "dk"), (dv, rdv, "dv"), (db, rdb, "dbias")):
+        assert_grad_close(g, r, n)
+
+
+def test_cfg2_full_size_forward_properties():
+    """Config 2 at full size (B=1, L=8192, H=32, Hkv=8, d=128, bias [1,8,1,8192], top-2048 ∩ causal).
+    Checked through size-independent properties plus an eager check of one KV group:
+      * V = 1  =>  O = 1 on rows with a visible key, 0 elsewhere (rows of P sum to one);
+      * a per-head constant added to the bias leaves O unchanged and shifts the LSE by it;
+      * the 4 query heads of KV group 0 against fp32 eager."""
+    B, L, H, Hk, D, W = 1, 8192, 32, 8, 128, 2048
+    q, k, v, mask, bias = make_inputs(B, L, L, H, Hk, D, (B, Hk, 1, L), (B, Hk, 1, L), W, seed=0)
+    qd, kd, vd, md, bd = _to_dev(q, k, v, mask, bias)
+    f = _op()
+    out, lse, _ = f(qd, kd, vd, md, bd, None, True, None, None, True)
+    ones, _, _ = f(qd, kd, torch.ones_like(vd), md, bd, None, True, None, None, True)
+    nonempty = torch.isfinite(lse).transpose(1, 2)[..., None].expand_as(ones)  # (B, L, H, 1)
+    assert torch.equal(ones[nonempty], torch.ones_like(ones[nonempty]))
+    assert torch.equal(ones[~nonempty], torch.zeros_like(ones[~nonempty]))
+    shifted, lse_s, _ = f(qd, kd, vd, md, bd + 2.0, None, True, None, None, True)
+    assert (shifted.float() - out.float()).abs().max().item() <= 2e-2
+    fin = torch.isfinite(lse)
+    assert (lse_s[fin] - lse[fin] - 2.0).abs().max().item() <= 2e-2
+    ro, rl = eager.attention_forward(qd[:, :, :4], kd[:, :, :1], vd[:, :, :1], md[:, :1], bd[:, :1], None, True)
+    assert_out_close(out[:, :, :4], ro)
+    _check_lse(lse[:, :4], rl)
+
+
+DECODE_CASES = {
+    # name: (B, Lk, H, Hk, D, mask heads, bias heads, window)
+    "gqa4_topk": (2, 4096, 8, 2, 128, 2, 2, 256),
+    "mqa_per_head_mask": (1, 1000, 4, 1, 64, 4, 4, 100),
+    "mha_no_mask": (2, 777, 4, 4, 128, None, 1, None),
+    "gqa8_shared_mask": (1, 3000, 16, 2, 128, 1, 16, 64),
+    "short": (3, 40, 8, 2, 64, 2, 2, 7),
+}
+
+
+@pytest.mark.parametrize("name", list(DECODE_CASES))
+def test_decode_vs_c_oracle(name):
+    B, Lk, H, Hk, D, hm, hb, W = DECODE_CASES[name]
+    q, k, v, mask, bias = make_inputs(B, 1, Lk, H, Hk, D, (B, hb, 1, Lk), (B, hm, 1, Lk) if hm else None, W, seed=13)
+    qd, kd, vd, md, bd = _to_dev(q, k, v, mask, bias)
+    out, lse, _ = _op()(qd, kd, vd, md, bd, None, False, None, None, True)
+    ro, rl = c_oracle.forward(q, k, v, mask, bias, None, False)
+    assert_out_close(out.cpu(), ro)
+    _check_lse(lse.cpu(), rl)
+    # is_causal is a no-op for a single query token (flash_api.cpp:441)
+    out_c = _op()(qd, kd, vd, md, bd, None, True)
+    assert torch.equal(out_c, out)
+
+
+def test_cfg5_full_size_decode():
+    """Config 5: B=8, Lq=1, Lk=65536, H=32, Hkv=8, d=128, bias [8,8,1,65536], top-2048, no causal."""
+    B, Lk, H, Hk, D, W = 8, 65536, 32, 8, 128, 2048
+    q, k, v, mask, bias = make_inputs(B, 1, Lk, H, Hk, D, (B, Hk, 1, Lk), (B, Hk, 1, Lk), W, seed=0)
+    qd, kd, vd, md, bd = _to_dev(q, k, v, mask, bias)
+    out, lse, _ = _op()(qd, kd, vd, md, bd, None, False, None, None, True)
+    ro, rl = eager.attention_forward(qd, kd, vd, md, bd, None, False)
+    assert_out_close(out, ro)
+    _check_lse(lse, rl)
+
+
+def test_direct_c_abi_call_without_the_python_operator():
+    """Calls fdma_fwd through ctypes exactly as a foreign-language binding would."""
+    from flash_sparse_attn import _cabi
+
+    q, k, v, mask, bias = make_inputs(1, 128, 128, 2, 1, 64, (1, 1, 1, 128), (1, 1, 1, 128), 64, seed=17)
+    qd, kd, vd, md, bd = _to_dev(q, k, v, mask, bias)
+    out = torch.empty_like(qd)
+    lse = torch.empty(1, 2, 128, dtype=torch.float32, device=DEV)
+    a = _cabi.FwdArgs()
+    _cabi.fill_fwd(a, qd, kd, vd, md, bd, out, lse, 0.125, True, 0.0)
+    assert _cabi.lib.fdma_fwd(a, _cabi.current_stream(qd.device)) == 0, _cabi.last_error()
+    torch.cuda.synchronize()
+    ro, rl = c_oracle.forward(q, k, v, mask, bias, 0.125, True)
+    assert_out_close(out.cpu(), ro)
+    _check_lse(lse.cpu(), rl)
