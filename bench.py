@@ -1,0 +1,251 @@
+#!/usr/bin/env python3
+"""Benchmark of the dynamic-mask attention hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all] [--no-cpu]
+
+A "step" is one forward pass of `flash_sparse_attn_func` over one synthetic batch of the headline
+configuration: B=1, Lq=Lk=8192, H=32, Hkv=8 (GQA 4:1), d=128, bf16, bias [B,Hkv,1,Lk] ~ N(0,1),
+keep-mask = per-row top-2048 keys by bias intersected with causal, scale 1/sqrt(128).
+Prints ONE JSON line.  `value` is the forward's effective TFLOP/s counting only executed tiles on
+the canonical 64x64 tile grid (a tile is executed iff it holds at least one mask-and-causal-visible
+element); forward+backward, the other configurations, the roofline of the dominant kernel and a CPU
+baseline on the host cores ride along in the same line.
+
+Inputs are resident in HBM before the timed region starts; timing uses HIP events on the stream the
+kernels are launched on (torch's current stream).
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for _p in (ROOT, os.path.join(ROOT, "flash-dmattn_amd")):
+    if _p not in sys.path:
+        sys.path.insert(0, _p)
+
+import torch  # noqa: E402
+
+PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
+PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+
+CONFIGS = {
+    # name: B, Lq, Lk, H, Hk, D, bias shape, window, causal, passes
+    "cfg1": dict(B=1, Lq=256, Lk=256, H=2, Hk=1, D=64, bias=(1, 1, 1, 256), W=128, causal=True, bwd=True, scale=0.125),
+    "cfg2": dict(B=1, Lq=8192, Lk=8192, H=32, Hk=8, D=128, bias=(1, 8, 1, 8192), W=2048, causal=True, bwd=True, scale=None),
+    "cfg3": dict(B=2, Lq=4096, Lk=4096, H=16, Hk=16, D=64, bias=(2, 16, 4096, 4096), W=1024, causal=True, bwd=True, scale=None),
+    "cfg4": dict(B=1, Lq=32768, Lk=32768, H=16, Hk=4, D=128, bias=(1, 4, 1, 32768), W=1024, causal=True, bwd=True, scale=None),
+    "cfg5": dict(B=8, Lq=1, Lk=65536, H=32, Hk=8, D=128, bias=(8, 8, 1, 65536), W=2048, causal=False, bwd=False, scale=None),
+}
+
+
+def make_case(c, device, seed=0):
+    """Synthetic inputs.  The mask has the bias's shape (top-W per row); the causal intersection is
+    applied by is_causal=True, which is the identical keep-set."""
+    g = torch.Generator(device="cpu").manual_seed(seed)
+    dt = torch.bfloat16
+    q = torch.randn(c["B"], c["Lq"], c["H"], c["D"], generator=g).to(dt).to(device)
+    k = torch.randn(c["B"], c["Lk"], c["Hk"], c["D"], generator=g).to(dt).to(device)
+    v = torch.randn(c["B"], c["Lk"], c["Hk"], c["D"], generator=g).to(dt).to(device)
+    if c["bias"][2] == 1:
+        bias = torch.randn(*c["bias"], generator=g).to(dt).to(device)
+    else:  # the per-query bias of cfg3 is 1 GiB: draw it on the device
+        gd = torch.Generator(device=device).manual_seed(seed)
+        bias = torch.randn(*c["bias"], generator=gd, device=device, dtype=torch.float32).to(dt)
+    idx = bias.float().topk(min(c["W"], c["Lk"]), dim=-1).indices
+    mask = torch.zeros(bias.shape, dtype=torch.bool, device=device).scatter_(-1, idx, True)
+    return q, k, v, mask, bias
+
+
+def count_tiles(mask, Lq, Lk, causal, H, tile=64):
+    """Canonical 64x64 tile statistics from the actual mask: (executed tiles, causal tiles, nnz)
+    summed over batch and query heads."""
+    Bm, Hm, Rm, _ = mask.shape
+    shift = Lk - Lq
+    nq, nk = (Lq + tile - 1) // tile, (Lk + tile - 1) // tile
+    dev = mask.device
+    last_row = torch.clamp(torch.arange(nq, device=dev) * tile + tile - 1, max=Lq - 1)  # most permissive row
+    kblock_lo = torch.arange(nk, device=dev) * tile
+    causal_tile = (kblock_lo[None, :] <= last_row[:, None] + shift) if causal else torch.ones(nq, nk, dtype=torch.bool, device=dev)
+    rep = H // Hm
+    if Rm == 1:
+        m = mask[:, :, 0, :Lk]
+        pad = nk * tile - Lk
+        mp = torch.nn.functional.pad(m, (0, pad)).view(Bm, Hm, nk, tile)
+        cols = torch.arange(nk * tile, device=dev).view(nk, tile)
+        big = torch.iinfo(torch.int64).max
+        first_kept = torch.where(mp, cols, torch.full_like(cols, big)).min(-1).values  # (Bm,Hm,nk)
+        if causal:
+            ex = first_kept[:, :, None, :] <= last_row[None, None, :, None] + shift
+            executed = int(ex.sum().item()) * rep
+        else:
+            executed = int((first_kept < big).sum().item()) * nq * rep
+        if causal:
+            rows = torch.arange(Lq, device=dev)
+            csum = torch.cumsum(m.to(torch.int64), -1)
+            lim = torch.clamp(rows + shift, max=Lk - 1)
+            nnz = int(torch.where(lim >= 0, csum[..., torch.clamp(lim, min=0)], torch.zeros((), dtype=torch.int64, device=dev)).sum().item()) * rep
+        else:
+            nnz = int(m.sum().item()) * Lq * rep
+    else:
+        executed, nnz = 0, 0
+        cm = None
+        if causal:
+            i = torch.arange(Lq, device=dev)[:, None]
+            j = torch.arange(Lk, device=dev)[None, :]
+            cm = j <= i + shift
+        for b in range(Bm):
+            for h in range(Hm):
+                m = mask[b, h, :, :Lk]
+                if cm is not None:
+                    m = m & cm
+                nnz += int(m.sum().item())
+                mp = torch.nn.functional.pad(m, (0, nk * tile - Lk, 0, nq * tile - Lq))
+                executed += int(mp.view(nq, tile, nk, tile).any(3).any(1).sum().item())
+        executed *= rep
+        nnz *= rep
+    Bfull = mask.shape[0]
+    return executed, int(causal_tile.sum().item()) * H * Bfull, nnz
+
+
+def time_gpu(fn, steps, warmup):
+    for _ in range(warmup):
+        fn()
+    torch.cuda.synchronize()
+    e0 = torch.cuda.Event(enable_timing=True)
+    e1 = torch.cuda.Event(enable_timing=True)
+    e0.record()
+    for _ in range(steps):
+        fn()
+    e1.record()
+    torch.cuda.synchronize()
+    return e0.elapsed_time(e1) / steps
+
+
+def run_config(name, steps, warmup, device):
+    from flash_sparse_attn import flash_sparse_attn_func
+
+    c = CONFIGS[name]
+    q, k, v, mask, bias = make_case(c, device)
+    scale = c["scale"]
+    res = {"name": name, "mask_form": "[B,Hm,%s,Lk] bool + is_causal" % ("1" if mask.shape[2] == 1 else "Lq")}
+    with torch.no_grad():
+        ms_fwd = time_gpu(lambda: flash_sparse_attn_func(q, k, v, mask, bias, scale, c["causal"]), steps, warmup)
+    res["ms_fwd"] = ms_fwd
+    if c["Lq"] > 1:
+        n_exec, n_causal, nnz = count_tiles(mask, c["Lq"], c["Lk"], c["causal"], c["H"])
+        res.update(n_exec=n_exec, tile_occupancy=n_exec / max(1, n_causal), nnz=nnz)
+        fl_fwd = 4.0 * 64 * 64 * c["D"] * n_exec
+        res["tflops_fwd"] = fl_fwd / ms_fwd / 1e9
+        res["tflops_fwd_elementwise"] = 4.0 * c["D"] * nnz / ms_fwd / 1e9
+    else:
+        kept = int(mask.sum().item())  # per (b, mask head); all heads of a group share the rows
+        rows = kept * (c["Hk"] // mask.shape[1] if mask.shape[1] <= c["Hk"] else 1)
+        kv_bytes = 2.0 * rows * c["D"] * 2
+        side = mask.numel() + bias.numel() * 2 + q.numel() * 2 * 2
+        res.update(kept_rows=rows, touched_bytes=kv_bytes + side, hbm_gbs=(kv_bytes + side) / ms_fwd / 1e6,
+                   hbm_gbs_tile64=None)
+        m = mask[:, :, 0, :]
+        blocks = int(m.view(m.shape[0], m.shape[1], -1, 64).any(-1).sum().item())
+        res["tile64_bytes"] = 2.0 * blocks * 64 * c["D"] * 2 + side
+        res["hbm_gbs_tile64"] = res["tile64_bytes"] / ms_fwd / 1e6
+    if c["bwd"]:
+        qg, kg, vg = [t.clone().requires_grad_(True) for t in (q, k, v)]
+        bg = bias.clone().requires_grad_(True)
+
+        def step():
+            out = flash_sparse_attn_func(qg, kg, vg, mask, bg, scale, c["causal"])
+            out.backward(torch.ones_like(out))
+            qg.grad = kg.grad = vg.grad = bg.grad = None
+
+        ms_fb = time_gpu(step, max(2, steps // 2), max(1, warmup // 2))
+        res["ms_fwd_bwd"] = ms_fb
+        res["tflops_fwd_bwd"] = 14.0 * 64 * 64 * c["D"] * res["n_exec"] / ms_fb / 1e9
+    return res
+
+
+def cpu_baseline(device_cfg="cfg2", groups=1):
+    """The fp32 safe-eager restatement (oracle/eager.py, a port of the reference's eager formula) timed
+    on the host cores for a bounded sample of the headline workload: `groups` KV groups (each with its
+    4 query heads) of the 8, full sequence length."""
+    from oracle import eager
+
+    c = dict(CONFIGS[device_cfg])
+    q, k, v, mask, bias = make_case(c, "cpu")
+    G = c["H"] // c["Hk"]
+    qs, ks, vs = q[:, :, : G * groups].float(), k[:, :, :groups].float(), v[:, :, :groups].float()
+    ms_, bs = mask[:, :groups], bias[:, :groups].float()
+    cores = os.cpu_count() or 1
+    torch.set_num_threads(cores)
+    with torch.no_grad():
+        t0 = time.perf_counter()
+        eager.attention_forward(qs, ks, vs, ms_, bs, c["scale"], c["causal"])
+        dt = time.perf_counter() - t0
+    n_exec, _, _ = count_tiles(ms_, c["Lq"], c["Lk"], c["causal"], G * groups)
+    tfl = 4.0 * 64 * 64 * c["D"] * n_exec / dt / 1e12
+    return {"value": tfl, "unit": "TFLOP/s", "cores": cores, "kind": "port",
+            "sample": f"{groups} of {c['Hk']} KV groups ({G * groups} query heads) of {device_cfg} forward, fp32 eager on host, "
+                      f"{dt:.2f} s; same executed-tile FLOP count as the GPU figure",
+            "ms_scaled_to_full": dt * 1e3 * c["Hk"] / groups}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--all", action="store_true", help="also time configurations 1, 3, 4, 5")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the hot path has no multi-GPU part in this build; run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+    if not torch.cuda.is_available():
+        print("bench.py needs an MI355X", file=sys.stderr)
+        sys.exit(1)
+    device = torch.device("cuda:0")
+    torch.cuda.set_device(device)
+
+    main_res = run_config("cfg2", args.steps, args.warmup, device)
+    c = CONFIGS["cfg2"]
+    out = {
+        "metric": "fwd effective TFLOP/s on executed 64x64 tiles (L=8192, W=2048, d=128, bf16, GQA 4:1, mask+bias+causal)",
+        "value": main_res["tflops_fwd"],
+        "unit": "TFLOP/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": main_res["ms_fwd"],
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "bf16",
+        "data": "synthetic",
+        "config": {"workload": "cfg2: B=1 Lq=Lk=8192 H=32 Hkv=8 d=128 bias[1,8,1,8192] top-2048 ∩ causal, forward",
+                   "mask_form": main_res["mask_form"], "n_exec_tiles": main_res["n_exec"],
+                   "tile_occupancy": main_res["tile_occupancy"]},
+        "ms_fwd": main_res["ms_fwd"],
+        "ms_fwd_bwd": main_res.get("ms_fwd_bwd"),
+        "tflops_fwd_bwd": main_res.get("tflops_fwd_bwd"),
+        "roofline": {
+            "bound": "mfma",
+            "achieved": main_res["tflops_fwd"],
+            "peak": PEAK_BF16_TFLOPS,
+            "unit": "TFLOP/s",
+            "frac": main_res["tflops_fwd"] / PEAK_BF16_TFLOPS,
+            "traffic": None,
+            "kernel": "fdma::fwd_kernel<bf16, 128, causal>",
+            "flops_per_launch": 4.0 * 64 * 64 * c["D"] * main_res["n_exec"],
+        },
+    }
+    if args.all:
+        out["other_configs"] = [run_config(n, max(3, args.steps // 4), max(1, args.warmup // 2), device)
+                                for n in ("cfg1", "cfg3", "cfg4", "cfg5")]
+    if not args.no_cpu:
+        out["cpu_baseline"] = cpu_baseline("cfg2", groups=1)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
