@@ -1,0 +1,479 @@
+// Forward dynamic-mask attention for gfx950, column-mask specialisation.
+//
+// Same math and same reference counterparts as fdma_fwd.hip (compute_attn_1rowblock,
+// csrc/flash_sparse_attn/src/flash_fwd_kernel.h:53-804 of the reference), for the case that dominates
+// dynamic-mask attention in practice: mask and bias are absent or broadcast over the query
+// dimension (shape [B, {1,Hk,H}, 1, Lk]), so "keep" is a property of the key column and the
+// per-query part of the mask is only the causal triangle.
+//
+// What that buys:
+//   * the set of KV tiles with at least one kept key is known before the main loop: the workgroup
+//     scans its mask row once into an LDS bitmap and then visits active tiles only -- no per-tile
+//     workgroup-wide OR, no loads and no MFMA work for skipped tiles;
+//   * bias and mask fuse into one fp32 vector per tile (bias*log2e, or -inf where masked or beyond
+//     Lk) staged in LDS, so the score epilogue is a single FMA per element;
+//   * causal masking costs instructions on diagonal tiles only.
+//
+// Pipeline (one barrier per tile): K tiles are double-buffered in LDS, V tiles are transposed in
+// registers while being staged and double-buffered as V^T, the fused bias vector is triple-buffered.
+// Global loads for tile i+2 (K, bias) and i+1 (V) are in flight while tile i is computed, and the
+// score MFMAs of tile i+1 are issued before the softmax of tile i so the matrix pipe has work
+// during the vector-ALU phase.  Each wave owns 32*NQ query rows; with NQ = 2 every K / V^T
+// fragment read from LDS feeds two MFMAs, halving LDS traffic per flop.
+#include "fdma_common.h"
+#include "fdma_params.h"
+
+namespace fdma {
+
+namespace {
+
+constexpr int NTHREADS = 256;
+constexpr int MAX_TILES = 16384;  // bitmap capacity: Lk <= 1 Mi keys
+
+template <int D, int BN> struct CmSmem {
+    static constexpr int SK = D + 8;        // K tile row stride (elements)
+    static constexpr int SVT = BN + 8;      // V^T tile row stride (elements)
+    static constexpr int K_BYTES = BN * SK * 2;
+    static constexpr int VT_BYTES = D * SVT * 2;
+    static constexpr int OFF_K = 0;
+    static constexpr int OFF_VT = OFF_K + 2 * K_BYTES;
+    static constexpr int OFF_BIAS = OFF_VT + 2 * VT_BYTES;
+    static constexpr int OFF_BITS = OFF_BIAS + 3 * BN * 4;
+    static constexpr int TOTAL = OFF_BITS + MAX_TILES / 8;
+};
+
+template <typename T, int D, int NQ, int BN, bool PIPE, bool CAUSAL>
+__global__ void __launch_bounds__(NTHREADS, NQ == 1 ? 2 : 1) fwd_colmask_kernel(const FwdParams p) {
+    using E = Elem<T>;
+    using SM = CmSmem<D, BN>;
+    constexpr int MB = BN / 32;               // 32-key blocks per tile
+    constexpr int KB = BN / 16;               // 16-key contraction blocks per tile
+    constexpr int KQ = BN / 4;                // key quads per tile
+    constexpr int KS = D / 16;
+    constexpr int DB = D / 32;
+    constexpr int BM = 128 * NQ;
+    constexpr int CH = D / 8;                 // 16-byte chunks per K row
+    constexpr int K_RPP = NTHREADS / CH;      // K rows staged per pass
+    constexpr int K_IT = BN / K_RPP;          // passes (registers) per K tile
+    constexpr int V_ITEMS = KQ * CH;          // (key quad, d chunk) items of a V tile
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    float *sBias = (float *)(smem + SM::OFF_BIAS);
+    uint32_t *sBits = (uint32_t *)(smem + SM::OFF_BITS);
+
+    const int tid = threadIdx.x;
+    const int wave = tid >> 6;
+    const int lane = tid & 63;
+    const int r = lane & 31;
+    const int g = lane >> 5;
+
+    const int m_block = gridDim.x - 1 - blockIdx.x;
+    const int h = blockIdx.y;
+    const int b = blockIdx.z;
+    const int hk = h / (p.H / p.Hk);
+    const int m0 = m_block * BM;
+    const int shift = p.Lk - p.Lq;
+    const int wrow0 = m0 + wave * 32 * NQ;  // first query row of this wave
+
+    const int hm = p.mask ? (p.Hm == p.H ? h : (p.Hm == 1 ? 0 : h / (p.H / p.Hm))) : 0;
+    const int hb = p.bias ? (p.Hb == p.H ? h : (p.Hb == 1 ? 0 : h / (p.H / p.Hb))) : 0;
+    const uint8_t *mrow = p.mask ? p.mask + b * p.m_b + hm * p.m_h : nullptr;
+    const uint16_t *brow = p.bias ? (const uint16_t *)p.bias + b * p.bi_b + hb * p.bi_h : nullptr;
+    const uint16_t *kbase = (const uint16_t *)p.k + b * p.k_b + hk * p.k_h;
+    const uint16_t *vbase = (const uint16_t *)p.v + b * p.v_b + hk * p.v_h;
+
+    int n_end = (p.Lk + BN - 1) / BN;
+    if (CAUSAL) {
+        int lim = m0 + BM + shift;
+        if (lim > p.Lq + shift) lim = p.Lq + shift;  // rows beyond Lq do not exist
+        if (lim < 0) lim = 0;
+        int ne = (lim + BN - 1) / BN;
+        if (ne < n_end) n_end = ne;
+    }
+
+    // ---- active-tile bitmap
+    for (int base = 0; base < n_end; base += NTHREADS) {
+        const int j = base + tid;
+        bool act = false;
+        if (j < n_end) {
+            if (mrow) {
+                uint32_t any = 0;
+#pragma unroll
+                for (int c = 0; c < BN / 16; c++) {
+                    const int col = j * BN + c * 16;
+                    if (col < p.Lk) {
+                        u32x4_t mv = *(const u32x4_t *)(mrow + col);
+                        any |= mv[0] | mv[1] | mv[2] | mv[3];
+                    }
+                }
+                act = any != 0;
+            } else {
+                act = true;
+            }
+        }
+        const uint64_t ball = __ballot(act);
+        if (lane == 0) {
+            const int w0 = (base + wave * 64) >> 5;
+            sBits[w0] = (uint32_t)ball;
+            sBits[w0 + 1] = (uint32_t)(ball >> 32);
+        }
+    }
+    __syncthreads();
+
+    auto next_active = [&](int j) -> int {  // smallest active tile >= j, or n_end
+        while (j < n_end) {
+            uint32_t w = sBits[j >> 5] >> (j & 31);
+            if (w) {
+                j += __builtin_ctz(w);
+                return j < n_end ? j : n_end;
+            }
+            j = (j | 31) + 1;
+        }
+        return n_end;
+    };
+
+    // ---- Q fragments
+    u32x4_t qf[NQ][KS];
+#pragma unroll
+    for (int nb = 0; nb < NQ; nb++) {
+        const int qrow = wrow0 + nb * 32 + r;
+        const int qc = qrow < p.Lq ? qrow : p.Lq - 1;
+        const uint16_t *qp = (const uint16_t *)p.q + b * p.q_b + (int64_t)qc * p.q_r + h * p.q_h;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            const int c = ks * 16 + g * 8;
+            u32x4_t v = {0, 0, 0, 0};
+            if (qrow < p.Lq && c < p.d) v = *(const u32x4_t *)(qp + c);
+            qf[nb][ks] = v;
+        }
+    }
+
+    f32x16_t o[NQ][DB];
+    float row_max[NQ], row_sum[NQ];
+#pragma unroll
+    for (int nb = 0; nb < NQ; nb++) {
+        row_max[nb] = -INFINITY;
+        row_sum[nb] = 0.f;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) o[nb][db][i] = 0.f;
+    }
+
+    // ---- staging helpers (global -> registers -> LDS)
+    // Per-thread byte offsets inside a tile are 32-bit and computed once; the per-tile base is
+    // wave-uniform, so a full tile costs no vector address arithmetic and no predication.
+    const int kc = tid % CH, kr0 = tid / CH;
+    const int vkg = tid % KQ, vc = tid / KQ;  // V: key quad and d chunk of this thread
+    const bool k_dvalid = kc * 8 < p.d, v_dvalid = vc * 8 < p.d;
+    uint32_t koff[K_IT], voff[4];
+#pragma unroll
+    for (int it = 0; it < K_IT; it++) koff[it] = (uint32_t)(((int64_t)(kr0 + it * K_RPP) * p.k_r + (k_dvalid ? kc * 8 : 0)) * 2);
+#pragma unroll
+    for (int i = 0; i < 4; i++) voff[i] = (uint32_t)(((int64_t)(4 * vkg + i) * p.v_r + (v_dvalid ? vc * 8 : 0)) * 2);
+    const bool d_full = p.d == D;
+    u32x4_t kreg[K_IT], vreg[4];
+    float breg = 0.f;
+
+    auto load_k = [&](int j) {
+        const int n0 = j * BN;
+        const char *tb = (const char *)kbase + (int64_t)n0 * p.k_r * 2;
+        if (n0 + BN <= p.Lk) {
+#pragma unroll
+            for (int it = 0; it < K_IT; it++) kreg[it] = *(const u32x4_t *)(tb + koff[it]);
+            if (!d_full) {
+#pragma unroll
+                for (int it = 0; it < K_IT; it++)
+                    if (!k_dvalid) kreg[it] = u32x4_t{0, 0, 0, 0};
+            }
+        } else {
+#pragma unroll
+            for (int it = 0; it < K_IT; it++) {
+                const int key = n0 + kr0 + it * K_RPP;
+                u32x4_t kv = {0, 0, 0, 0};
+                if (key < p.Lk && k_dvalid) kv = *(const u32x4_t *)(tb + koff[it]);
+                kreg[it] = kv;
+            }
+        }
+        if (tid < BN) {
+            const int col = n0 + tid;
+            float v = -INFINITY;
+            if (col < p.Lk && (!mrow || mrow[col])) {
+                v = 0.f;
+                if (brow) v = E::lo((uint32_t)brow[col]) * kLog2e;
+            }
+            breg = v;
+        }
+    };
+    auto store_k = [&](int buf, int slot) {
+        char *sK = smem + SM::OFF_K + buf * SM::K_BYTES;
+#pragma unroll
+        for (int it = 0; it < K_IT; it++)
+            *(u32x4_t *)(sK + ((kr0 + it * K_RPP) * SM::SK + kc * 8) * 2) = kreg[it];
+        if (tid < BN) sBias[slot * BN + tid] = breg;
+    };
+    auto load_v = [&](int j) {
+        const int n0 = j * BN;
+        const char *tb = (const char *)vbase + (int64_t)n0 * p.v_r * 2;
+        if (tid < V_ITEMS) {
+            if (n0 + BN <= p.Lk) {
+#pragma unroll
+                for (int i = 0; i < 4; i++) vreg[i] = *(const u32x4_t *)(tb + voff[i]);
+                if (!d_full) {
+#pragma unroll
+                    for (int i = 0; i < 4; i++)
+                        if (!v_dvalid) vreg[i] = u32x4_t{0, 0, 0, 0};
+                }
+            } else {
+#pragma unroll
+                for (int i = 0; i < 4; i++) {
+                    const int key = n0 + 4 * vkg + i;
+                    u32x4_t vv = {0, 0, 0, 0};
+                    if (key < p.Lk && v_dvalid) vv = *(const u32x4_t *)(tb + voff[i]);
+                    vreg[i] = vv;
+                }
+            }
+        }
+    };
+    auto store_v = [&](int buf) {  // transpose 4 keys x 8 d in registers, write V^T[d][key quad]
+        char *sVt = smem + SM::OFF_VT + buf * SM::VT_BYTES;
+        if (tid < V_ITEMS) {
+#pragma unroll
+            for (int dd = 0; dd < 8; dd++) {
+                const int w = dd >> 1;
+                const uint32_t sel = (dd & 1) ? 0x07060302u : 0x05040100u;
+                u32x2_t out;
+                out[0] = __builtin_amdgcn_perm(vreg[1][w], vreg[0][w], sel);
+                out[1] = __builtin_amdgcn_perm(vreg[3][w], vreg[2][w], sel);
+                *(u32x2_t *)(sVt + ((vc * 8 + dd) * SM::SVT + 4 * vkg) * 2) = out;
+            }
+        }
+    };
+
+    const int a_row = pi_row(r);
+
+    auto qk = [&](f32x16_t (&s)[NQ][MB], int buf) {
+        const char *sK = smem + SM::OFF_K + buf * SM::K_BYTES;
+#pragma unroll
+        for (int nb = 0; nb < NQ; nb++)
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) s[nb][mb][i] = 0.f;
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                u32x4_t a = *(const u32x4_t *)(sK + ((32 * mb + a_row) * SM::SK + ks * 16 + g * 8) * 2);
+#pragma unroll
+                for (int nb = 0; nb < NQ; nb++) s[nb][mb] = E::mfma(a, qf[nb][ks], s[nb][mb]);
+            }
+    };
+
+    auto softmax_pv = [&](f32x16_t (&s)[NQ][MB], int j, int slot, int vbuf) {
+        const int n0 = j * BN;
+        const float *bs = sBias + slot * BN;
+        float bl2[16 * MB];
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+            for (int blk = 0; blk < 2; blk++) {
+                const f32x4_t b0 = *(const f32x4_t *)(bs + 32 * mb + 16 * blk + 8 * g);
+                const f32x4_t b1 = *(const f32x4_t *)(bs + 32 * mb + 16 * blk + 8 * g + 4);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    bl2[16 * mb + 8 * blk + e] = b0[e];
+                    bl2[16 * mb + 8 * blk + 4 + e] = b1[e];
+                }
+            }
+        uint32_t pk[NQ][8 * MB];
+#pragma unroll
+        for (int nb = 0; nb < NQ; nb++) {
+            const int qrow = wrow0 + nb * 32 + r;
+            // diagonal tile for this 32-row block? (wave-uniform)
+            const bool diag = CAUSAL && (n0 + BN - 1 > wrow0 + nb * 32 + shift);
+            float tmax = -INFINITY;
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) s[nb][mb][i] = fmaf(s[nb][mb][i], p.scale_log2, bl2[16 * mb + i]);
+            if (diag) {
+                asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch: only diagonal tiles pay
+                const int lim = qrow + shift - n0 - 8 * g;  // local column limit for this lane
+#pragma unroll
+                for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) {
+                        const int lc = 32 * mb + 16 * (i >> 3) + (i & 7);
+                        s[nb][mb][i] = lc <= lim ? s[nb][mb][i] : -INFINITY;
+                    }
+            }
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) tmax = fmaxf(tmax, s[nb][mb][i]);
+            tmax = xhalf_max(tmax);
+            if (__any(tmax > row_max[nb])) {
+                const float new_max = fmaxf(row_max[nb], tmax);
+                const float safe = new_max == -INFINITY ? 0.f : new_max;
+                const float alpha = fast_exp2(row_max[nb] - safe);
+                row_max[nb] = new_max;
+                row_sum[nb] *= alpha;
+#pragma unroll
+                for (int db = 0; db < DB; db++)
+#pragma unroll
+                    for (int i = 0; i < 16; i++) o[nb][db][i] *= alpha;
+            }
+            const float m_use = row_max[nb] == -INFINITY ? 0.f : row_max[nb];
+            float psum = 0.f;
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+                for (int i = 0; i < 16; i += 2) {
+                    const float p0 = fast_exp2(s[nb][mb][i] - m_use);
+                    const float p1 = fast_exp2(s[nb][mb][i + 1] - m_use);
+                    psum += p0 + p1;
+                    pk[nb][8 * mb + i / 2] = E::pack2(p0, p1);
+                }
+            row_sum[nb] += psum;
+        }
+        const char *sVt = smem + SM::OFF_VT + vbuf * SM::VT_BYTES;
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++)
+#pragma unroll
+            for (int db = 0; db < DB; db++) {
+                u32x4_t a = *(const u32x4_t *)(sVt + ((32 * db + a_row) * SM::SVT + 16 * kb + 8 * g) * 2);
+#pragma unroll
+                for (int nb = 0; nb < NQ; nb++) {
+                    u32x4_t bop = {pk[nb][4 * kb], pk[nb][4 * kb + 1], pk[nb][4 * kb + 2], pk[nb][4 * kb + 3]};
+                    o[nb][db] = E::mfma(a, bop, o[nb][db]);
+                }
+            }
+    };
+
+    // ---- prologue: tiles t0 (K, bias, V) and t1 (K, bias)
+    int j0 = next_active(0);
+    if (j0 < n_end) {
+        int j1 = next_active(j0 + 1);
+        load_k(j0);
+        load_v(j0);
+        store_k(0, 0);
+        store_v(0);
+        if (j1 < n_end) {
+            load_k(j1);
+            store_k(1, 1);
+        }
+        __syncthreads();
+
+        if constexpr (PIPE) {
+            f32x16_t sa[NQ][MB], sb[NQ][MB];
+            qk(sa, 0);
+            __syncthreads();  // nobody may overwrite K buffer 0 (end of step 0) before every wave has read it
+
+            // one pipeline step: tile jc is current (scores in s_cur), jn1 next, jn2 the one after
+            auto step = [&](f32x16_t (&s_cur)[NQ][MB], f32x16_t (&s_next)[NQ][MB], int i, int jc, int jn1, int jn2) {
+                if (jn2 < n_end) load_k(jn2);
+                if (jn1 < n_end) {
+                    load_v(jn1);
+                    qk(s_next, (i + 1) & 1);
+                }
+                softmax_pv(s_cur, jc, i % 3, i & 1);
+                if (jn2 < n_end) store_k(i & 1, (i + 2) % 3);
+                if (jn1 < n_end) store_v((i + 1) & 1);
+                __syncthreads();
+            };
+
+            int i = 0, jc = j0, jn1 = j1;
+            while (jc < n_end) {
+                int jn2 = jn1 < n_end ? next_active(jn1 + 1) : n_end;
+                step(sa, sb, i, jc, jn1, jn2);
+                i++; jc = jn1; jn1 = jn2;
+                if (jc >= n_end) break;
+                jn2 = jn1 < n_end ? next_active(jn1 + 1) : n_end;
+                step(sb, sa, i, jc, jn1, jn2);
+                i++; jc = jn1; jn1 = jn2;
+            }
+        } else {
+            // same buffer rotation without the cross-tile score prefetch (one score buffer)
+            f32x16_t sa[NQ][MB];
+            int i = 0, jc = j0, jn1 = j1;
+            while (jc < n_end) {
+                const int jn2 = jn1 < n_end ? next_active(jn1 + 1) : n_end;
+                if (jn2 < n_end) load_k(jn2);
+                if (jn1 < n_end) load_v(jn1);
+                qk(sa, i & 1);
+                softmax_pv(sa, jc, i % 3, i & 1);
+                __syncthreads();  // every wave is done with K buffer i&1 before it is refilled
+                if (jn2 < n_end) store_k(i & 1, (i + 2) % 3);
+                if (jn1 < n_end) store_v((i + 1) & 1);
+                __syncthreads();
+                i++; jc = jn1; jn1 = jn2;
+            }
+        }
+    }
+
+    // ---- epilogue
+#pragma unroll
+    for (int nb = 0; nb < NQ; nb++) {
+        const int qrow = wrow0 + nb * 32 + r;
+        const float total = xhalf_sum(row_sum[nb]);
+        const float inv = total > 0.f ? 1.f / total : 0.f;
+        if (qrow < p.Lq) {
+            uint16_t *op = (uint16_t *)p.o + b * p.o_b + (int64_t)qrow * p.o_r + h * p.o_h;
+#pragma unroll
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int blk = 0; blk < 2; blk++) {
+                    const int c = 32 * db + 16 * blk + 8 * g;
+                    if (c < p.d) {
+                        u32x4_t w;
+#pragma unroll
+                        for (int e = 0; e < 4; e++)
+                            w[e] = E::pack2(o[nb][db][8 * blk + 2 * e] * inv, o[nb][db][8 * blk + 2 * e + 1] * inv);
+                        *(u32x4_t *)(op + c) = w;
+                    }
+                }
+            if (g == 0) {
+                const float lse = total > 0.f ? (row_max[nb] + __builtin_amdgcn_logf(total)) * kLn2 : INFINITY;
+                p.lse[((int64_t)b * p.H + h) * p.Lq + qrow] = lse;
+            }
+        }
+    }
+}
+
+template <typename T, int D, int NQ, int BN, bool PIPE, bool CAUSAL>
+hipError_t launch_one(const FwdParams &p, hipStream_t stream) {
+    constexpr int BM = 128 * NQ;
+    auto kern = fwd_colmask_kernel<T, D, NQ, BN, PIPE, CAUSAL>;
+    const int smem = CmSmem<D, BN>::TOTAL;
+    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return e;
+    dim3 grid((p.Lq + BM - 1) / BM, p.H, p.B);
+    hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, stream, p);
+    return hipGetLastError();
+}
+
+template <typename T, int D>
+hipError_t launch_d(const FwdParams &p, int variant, hipStream_t stream) {
+    switch (variant) {
+        case 2: return p.causal ? launch_one<T, D, 2, 32, true, true>(p, stream) : launch_one<T, D, 2, 32, true, false>(p, stream);
+        case 3: return p.causal ? launch_one<T, D, 1, 32, true, true>(p, stream) : launch_one<T, D, 1, 32, true, false>(p, stream);
+        default: return p.causal ? launch_one<T, D, 1, 64, false, true>(p, stream) : launch_one<T, D, 1, 64, false, false>(p, stream);
+    }
+}
+
+}  // namespace
+
+bool fwd_colmask_applicable(const FwdParams &p) {
+    const bool mask_ok = !p.mask || p.m_r == 0;
+    const bool bias_ok = !p.bias || p.bi_r == 0;
+    return mask_ok && bias_ok && (p.Lk + 31) / 32 <= MAX_TILES;
+}
+
+hipError_t launch_fwd_colmask(const FwdParams &p, int dtype, int nq, hipStream_t stream) {
+    const bool d64 = p.d <= 64;
+    if (dtype == 0) return d64 ? launch_d<bf16_tag, 64>(p, nq, stream) : launch_d<bf16_tag, 128>(p, nq, stream);
+    return d64 ? launch_d<fp16_tag, 64>(p, nq, stream) : launch_d<fp16_tag, 128>(p, nq, stream);
+}
+
+}  // namespace fdma

@@ -47,6 +47,9 @@ struct BwdParams {
 
 // dtype: 0 = bf16, 1 = fp16.  All launches are asynchronous on `stream`; return hipError_t.
 hipError_t launch_fwd(const FwdParams &p, int dtype, hipStream_t stream);
+// column-mask specialisation (mask / bias absent or broadcast over queries); nq = 32-row blocks per wave
+bool fwd_colmask_applicable(const FwdParams &p);
+hipError_t launch_fwd_colmask(const FwdParams &p, int dtype, int nq, hipStream_t stream);
 hipError_t launch_fwd_decode(const FwdParams &p, int dtype, hipStream_t stream);
 hipError_t launch_bwd(const BwdParams &p, int dtype, hipStream_t stream);
 
