@@ -14,12 +14,11 @@
 //     Lk) staged in LDS, so the score epilogue is a single FMA per element;
 //   * causal masking costs instructions on diagonal tiles only.
 //
-// Pipeline (one barrier per tile): K tiles are double-buffered in LDS, V tiles are transposed in
-// registers while being staged and double-buffered as V^T, the fused bias vector is triple-buffered.
-// Global loads for tile i+2 (K, bias) and i+1 (V) are in flight while tile i is computed, and the
-// score MFMAs of tile i+1 are issued before the softmax of tile i so the matrix pipe has work
-// during the vector-ALU phase.  Each wave owns 32*NQ query rows; with NQ = 2 every K / V^T
-// fragment read from LDS feeds two MFMAs, halving LDS traffic per flop.
+// Pipeline: K tiles are double-buffered in LDS, V tiles are transposed in registers while being
+// staged and double-buffered as V^T, the fused bias vector is triple-buffered.  Global loads for
+// tile i+2 (K, bias) and i+1 (V) are in flight while tile i is computed; LDS fragment reads run a
+// batch ahead of the MFMAs that consume them.  Workgroup ids are remapped so that the workgroups
+// sharing one XCD's L2 also share K / V.
 #include "fdma_common.h"
 #include "fdma_params.h"
 
@@ -27,7 +26,6 @@ namespace fdma {
 
 namespace {
 
-constexpr int NTHREADS = 256;
 constexpr int MAX_TILES = 16384;  // bitmap capacity: Lk <= 1 Mi keys
 
 template <int D, int BN> struct CmSmem {
@@ -42,8 +40,12 @@ template <int D, int BN> struct CmSmem {
     static constexpr int TOTAL = OFF_BITS + MAX_TILES / 8;
 };
 
-template <typename T, int D, int NQ, int BN, bool PIPE, bool CAUSAL>
-__global__ void __launch_bounds__(NTHREADS, NQ == 1 ? 2 : 1) fwd_colmask_kernel(const FwdParams p) {
+template <typename T, int D, int NQ, int BN, bool CAUSAL, int NW>
+__global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(const FwdParams p) {
+    constexpr int NTHREADS = 64 * NW;
+    // with 8 waves the staging work is split by role: waves 0-3 stage V, waves 4-7 stage K and bias
+    constexpr bool SPLIT_ROLES = NW == 8;
+    constexpr int STHREADS = SPLIT_ROLES ? NTHREADS / 2 : NTHREADS;  // threads staging one operand
     using E = Elem<T>;
     using SM = CmSmem<D, BN>;
     constexpr int MB = BN / 32;               // 32-key blocks per tile
@@ -51,9 +53,9 @@ __global__ void __launch_bounds__(NTHREADS, NQ == 1 ? 2 : 1) fwd_colmask_kernel(
     constexpr int KQ = BN / 4;                // key quads per tile
     constexpr int KS = D / 16;
     constexpr int DB = D / 32;
-    constexpr int BM = 128 * NQ;
+    constexpr int BM = 32 * NQ * NW;
     constexpr int CH = D / 8;                 // 16-byte chunks per K row
-    constexpr int K_RPP = NTHREADS / CH;      // K rows staged per pass
+    constexpr int K_RPP = STHREADS / CH;      // K rows staged per pass
     constexpr int K_IT = BN / K_RPP;          // passes (registers) per K tile
     constexpr int V_ITEMS = KQ * CH;          // (key quad, d chunk) items of a V tile
 
@@ -67,9 +69,28 @@ __global__ void __launch_bounds__(NTHREADS, NQ == 1 ? 2 : 1) fwd_colmask_kernel(
     const int r = lane & 31;
     const int g = lane >> 5;
 
-    const int m_block = gridDim.x - 1 - blockIdx.x;
-    const int h = blockIdx.y;
-    const int b = blockIdx.z;
+    // Workgroup -> (batch, kv head, query head, query block), XCD-aware.  Workgroups are dealt to the 8
+    // XCDs round-robin by linear id and every XCD has its own L2.  The id is remapped so that the
+    // workgroups running at the same time on one XCD share K / V: the (batch, kv head) pairs are
+    // split into k = 8 / gcd(pairs, 8) interleaved lists of query blocks each, the resulting
+    // multiple-of-8 lists are dealt to the XCDs, and an XCD walks its lists one after the other,
+    // heaviest query block first, the G query heads of a block side by side.  Re-reads of K / V
+    // tiles then hit in that XCD's L2, and every XCD gets the same amount of work.
+    const int n_mb = (p.Lq + BM - 1) / BM;
+    const int G = p.H / p.Hk;
+    const int pairs = p.B * p.Hk;
+    const int gcd8 = (pairs % 8 == 0) ? 8 : ((pairs % 4 == 0) ? 4 : ((pairs % 2 == 0) ? 2 : 1));
+    const int k_split = 8 / gcd8;
+    const int list_len = ((n_mb + k_split - 1) / k_split) * G;  // workgroups per list
+    const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
+    const int vlist = xcd + 8 * (slot / list_len);
+    const int pos = slot % list_len;
+    const int pair = vlist / k_split;
+    const int mslot = (pos / G) * k_split + vlist % k_split;
+    if (mslot >= n_mb) return;
+    const int m_block = n_mb - 1 - mslot;
+    const int b = pair / p.Hk;
+    const int h = (pair % p.Hk) * G + pos % G;
     const int hk = h / (p.H / p.Hk);
     const int m0 = m_block * BM;
     const int shift = p.Lk - p.Lq;
@@ -163,8 +184,11 @@ __global__ void __launch_bounds__(NTHREADS, NQ == 1 ? 2 : 1) fwd_colmask_kernel(
     // ---- staging helpers (global -> registers -> LDS)
     // Per-thread byte offsets inside a tile are 32-bit and computed once; the per-tile base is
     // wave-uniform, so a full tile costs no vector address arithmetic and no predication.
-    const int kc = tid % CH, kr0 = tid / CH;
-    const int vkg = tid % KQ, vc = tid / KQ;  // V: key quad and d chunk of this thread
+    const bool k_role = !SPLIT_ROLES || tid >= STHREADS;
+    const bool v_role = !SPLIT_ROLES || tid < STHREADS;
+    const int ktid = SPLIT_ROLES ? (tid - STHREADS) & (STHREADS - 1) : tid;
+    const int kc = ktid % CH, kr0 = ktid / CH;
+    const int vkg = tid % KQ, vc = (tid / KQ) % CH;  // V: key quad and d chunk of this thread
     const bool k_dvalid = kc * 8 < p.d, v_dvalid = vc * 8 < p.d;
     uint32_t koff[K_IT], voff[4];
 #pragma unroll
@@ -172,10 +196,14 @@ __global__ void __launch_bounds__(NTHREADS, NQ == 1 ? 2 : 1) fwd_colmask_kernel(
 #pragma unroll
     for (int i = 0; i < 4; i++) voff[i] = (uint32_t)(((int64_t)(4 * vkg + i) * p.v_r + (v_dvalid ? vc * 8 : 0)) * 2);
     const bool d_full = p.d == D;
-    u32x4_t kreg[K_IT], vreg[4];
+    // staging registers; with split roles a thread stages either K or V, so the two share storage
+    u32x4_t stage_regs[SPLIT_ROLES ? 4 : K_IT + 4];
+    u32x4_t *kreg = stage_regs;
+    u32x4_t *vreg = stage_regs + (SPLIT_ROLES ? 0 : K_IT);
     float breg = 0.f;
 
     auto load_k = [&](int j) {
+        if (!k_role) return;
         const int n0 = j * BN;
         const char *tb = (const char *)kbase + (int64_t)n0 * p.k_r * 2;
         if (n0 + BN <= p.Lk) {
@@ -195,8 +223,8 @@ __global__ void __launch_bounds__(NTHREADS, NQ == 1 ? 2 : 1) fwd_colmask_kernel(
                 kreg[it] = kv;
             }
         }
-        if (tid < BN) {
-            const int col = n0 + tid;
+        if (ktid < BN) {
+            const int col = n0 + ktid;
             float v = -INFINITY;
             if (col < p.Lk && (!mrow || mrow[col])) {
                 v = 0.f;
@@ -206,16 +234,17 @@ __global__ void __launch_bounds__(NTHREADS, NQ == 1 ? 2 : 1) fwd_colmask_kernel(
         }
     };
     auto store_k = [&](int buf, int slot) {
+        if (!k_role) return;
         char *sK = smem + SM::OFF_K + buf * SM::K_BYTES;
 #pragma unroll
         for (int it = 0; it < K_IT; it++)
             *(u32x4_t *)(sK + ((kr0 + it * K_RPP) * SM::SK + kc * 8) * 2) = kreg[it];
-        if (tid < BN) sBias[slot * BN + tid] = breg;
+        if (ktid < BN) sBias[slot * BN + ktid] = breg;
     };
     auto load_v = [&](int j) {
         const int n0 = j * BN;
         const char *tb = (const char *)vbase + (int64_t)n0 * p.v_r * 2;
-        if (tid < V_ITEMS) {
+        if (v_role && tid < V_ITEMS) {
             if (n0 + BN <= p.Lk) {
 #pragma unroll
                 for (int i = 0; i < 4; i++) vreg[i] = *(const u32x4_t *)(tb + voff[i]);
@@ -237,7 +266,7 @@ __global__ void __launch_bounds__(NTHREADS, NQ == 1 ? 2 : 1) fwd_colmask_kernel(
     };
     auto store_v = [&](int buf) {  // transpose 4 keys x 8 d in registers, write V^T[d][key quad]
         char *sVt = smem + SM::OFF_VT + buf * SM::VT_BYTES;
-        if (tid < V_ITEMS) {
+        if (v_role && tid < V_ITEMS) {
 #pragma unroll
             for (int dd = 0; dd < 8; dd++) {
                 const int w = dd >> 1;
@@ -260,14 +289,30 @@ __global__ void __launch_bounds__(NTHREADS, NQ == 1 ? 2 : 1) fwd_colmask_kernel(
             for (int mb = 0; mb < MB; mb++)
 #pragma unroll
                 for (int i = 0; i < 16; i++) s[nb][mb][i] = 0.f;
+        // fragment reads run FR ahead of the MFMAs that consume them, so the LDS latency is paid once
+        // per batch instead of once per MFMA; (ks, mb) order alternates accumulators
+        constexpr int NF = MB * KS, FR = NF < 8 ? NF : 8;
+        u32x4_t a[NF];
+        auto frag = [&](int f) {
+            const int ks = f / MB, mb = f % MB;
+            return *(const u32x4_t *)(sK + ((32 * mb + a_row) * SM::SK + ks * 16 + g * 8) * 2);
+        };
 #pragma unroll
-        for (int mb = 0; mb < MB; mb++)
+        for (int f = 0; f < FR; f++) a[f] = frag(f);
 #pragma unroll
-            for (int ks = 0; ks < KS; ks++) {
-                u32x4_t a = *(const u32x4_t *)(sK + ((32 * mb + a_row) * SM::SK + ks * 16 + g * 8) * 2);
+        for (int f = 0; f < NF; f++) {
+            if (f + FR < NF) a[f + FR] = frag(f + FR);
+            const int ks = f / MB, mb = f % MB;
 #pragma unroll
-                for (int nb = 0; nb < NQ; nb++) s[nb][mb] = E::mfma(a, qf[nb][ks], s[nb][mb]);
-            }
+            for (int nb = 0; nb < NQ; nb++) s[nb][mb] = E::mfma(a[f], qf[nb][ks], s[nb][mb]);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x100, FR, 0);
+#pragma unroll
+        for (int f = 0; f < NF - FR; f++) {
+            __builtin_amdgcn_sched_group_barrier(0x008, NQ, 0);
+            __builtin_amdgcn_sched_group_barrier(0x100, 1, 0);
+        }
+        __builtin_amdgcn_sched_group_barrier(0x008, FR * NQ, 0);
     };
 
     auto softmax_pv = [&](f32x16_t (&s)[NQ][MB], int j, int slot, int vbuf) {
@@ -338,17 +383,26 @@ __global__ void __launch_bounds__(NTHREADS, NQ == 1 ? 2 : 1) fwd_colmask_kernel(
             row_sum[nb] += psum;
         }
         const char *sVt = smem + SM::OFF_VT + vbuf * SM::VT_BYTES;
+        {
+            constexpr int NF = KB * DB, FR = NF < 8 ? NF : 8;
+            u32x4_t a[NF];
+            auto frag = [&](int f) {
+                const int kb = f / DB, db = f % DB;
+                return *(const u32x4_t *)(sVt + ((32 * db + a_row) * SM::SVT + 16 * kb + 8 * g) * 2);
+            };
 #pragma unroll
-        for (int kb = 0; kb < KB; kb++)
+            for (int f = 0; f < FR; f++) a[f] = frag(f);
 #pragma unroll
-            for (int db = 0; db < DB; db++) {
-                u32x4_t a = *(const u32x4_t *)(sVt + ((32 * db + a_row) * SM::SVT + 16 * kb + 8 * g) * 2);
+            for (int f = 0; f < NF; f++) {
+                if (f + FR < NF) a[f + FR] = frag(f + FR);
+                const int kb = f / DB, db = f % DB;
 #pragma unroll
                 for (int nb = 0; nb < NQ; nb++) {
                     u32x4_t bop = {pk[nb][4 * kb], pk[nb][4 * kb + 1], pk[nb][4 * kb + 2], pk[nb][4 * kb + 3]};
-                    o[nb][db] = E::mfma(a, bop, o[nb][db]);
+                    o[nb][db] = E::mfma(a[f], bop, o[nb][db]);
                 }
             }
+        }
     };
 
     // ---- prologue: tiles t0 (K, bias, V) and t1 (K, bias)
@@ -365,50 +419,19 @@ __global__ void __launch_bounds__(NTHREADS, NQ == 1 ? 2 : 1) fwd_colmask_kernel(
         }
         __syncthreads();
 
-        if constexpr (PIPE) {
-            f32x16_t sa[NQ][MB], sb[NQ][MB];
-            qk(sa, 0);
-            __syncthreads();  // nobody may overwrite K buffer 0 (end of step 0) before every wave has read it
-
-            // one pipeline step: tile jc is current (scores in s_cur), jn1 next, jn2 the one after
-            auto step = [&](f32x16_t (&s_cur)[NQ][MB], f32x16_t (&s_next)[NQ][MB], int i, int jc, int jn1, int jn2) {
-                if (jn2 < n_end) load_k(jn2);
-                if (jn1 < n_end) {
-                    load_v(jn1);
-                    qk(s_next, (i + 1) & 1);
-                }
-                softmax_pv(s_cur, jc, i % 3, i & 1);
-                if (jn2 < n_end) store_k(i & 1, (i + 2) % 3);
-                if (jn1 < n_end) store_v((i + 1) & 1);
-                __syncthreads();
-            };
-
-            int i = 0, jc = j0, jn1 = j1;
-            while (jc < n_end) {
-                int jn2 = jn1 < n_end ? next_active(jn1 + 1) : n_end;
-                step(sa, sb, i, jc, jn1, jn2);
-                i++; jc = jn1; jn1 = jn2;
-                if (jc >= n_end) break;
-                jn2 = jn1 < n_end ? next_active(jn1 + 1) : n_end;
-                step(sb, sa, i, jc, jn1, jn2);
-                i++; jc = jn1; jn1 = jn2;
-            }
-        } else {
-            // same buffer rotation without the cross-tile score prefetch (one score buffer)
-            f32x16_t sa[NQ][MB];
-            int i = 0, jc = j0, jn1 = j1;
-            while (jc < n_end) {
-                const int jn2 = jn1 < n_end ? next_active(jn1 + 1) : n_end;
-                if (jn2 < n_end) load_k(jn2);
-                if (jn1 < n_end) load_v(jn1);
-                qk(sa, i & 1);
-                softmax_pv(sa, jc, i % 3, i & 1);
-                __syncthreads();  // every wave is done with K buffer i&1 before it is refilled
-                if (jn2 < n_end) store_k(i & 1, (i + 2) % 3);
-                if (jn1 < n_end) store_v((i + 1) & 1);
-                __syncthreads();
-                i++; jc = jn1; jn1 = jn2;
-            }
+        f32x16_t sa[NQ][MB];
+        int i = 0, jc = j0, jn1 = j1;
+        while (jc < n_end) {
+            const int jn2 = jn1 < n_end ? next_active(jn1 + 1) : n_end;
+            if (jn2 < n_end) load_k(jn2);
+            if (jn1 < n_end) load_v(jn1);
+            qk(sa, i & 1);
+            softmax_pv(sa, jc, i % 3, i & 1);
+            __syncthreads();  // every wave is done with K buffer i&1 before it is refilled
+            if (jn2 < n_end) store_k(i & 1, (i + 2) % 3);
+            if (jn1 < n_end) store_v((i + 1) & 1);
+            __syncthreads();
+            i++; jc = jn1; jn1 = jn2;
         }
     }
 
@@ -441,25 +464,25 @@ __global__ void __launch_bounds__(NTHREADS, NQ == 1 ? 2 : 1) fwd_colmask_kernel(
     }
 }
 
-template <typename T, int D, int NQ, int BN, bool PIPE, bool CAUSAL>
+template <typename T, int D, int NQ, int BN, bool CAUSAL, int NW = 4>
 hipError_t launch_one(const FwdParams &p, hipStream_t stream) {
-    constexpr int BM = 128 * NQ;
-    auto kern = fwd_colmask_kernel<T, D, NQ, BN, PIPE, CAUSAL>;
+    constexpr int BM = 32 * NQ * NW;
+    auto kern = fwd_colmask_kernel<T, D, NQ, BN, CAUSAL, NW>;
     const int smem = CmSmem<D, BN>::TOTAL;
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    dim3 grid((p.Lq + BM - 1) / BM, p.H, p.B);
-    hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, stream, p);
+    const int n_mb = (p.Lq + BM - 1) / BM, G = p.H / p.Hk, pairs = p.B * p.Hk;
+    const int gcd8 = (pairs % 8 == 0) ? 8 : ((pairs % 4 == 0) ? 4 : ((pairs % 2 == 0) ? 2 : 1));
+    const int k_split = 8 / gcd8;
+    dim3 grid(pairs * k_split * ((n_mb + k_split - 1) / k_split) * G);
+    hipLaunchKernelGGL(kern, grid, dim3(64 * NW), smem, stream, p);
     return hipGetLastError();
 }
 
 template <typename T, int D>
 hipError_t launch_d(const FwdParams &p, int variant, hipStream_t stream) {
-    switch (variant) {
-        case 2: return p.causal ? launch_one<T, D, 2, 32, true, true>(p, stream) : launch_one<T, D, 2, 32, true, false>(p, stream);
-        case 3: return p.causal ? launch_one<T, D, 1, 32, true, true>(p, stream) : launch_one<T, D, 1, 32, true, false>(p, stream);
-        default: return p.causal ? launch_one<T, D, 1, 64, false, true>(p, stream) : launch_one<T, D, 1, 64, false, false>(p, stream);
-    }
+    (void)variant;
+    return p.causal ? launch_one<T, D, 1, 64, true>(p, stream) : launch_one<T, D, 1, 64, false>(p, stream);
 }
 
 }  // namespace
