@@ -22,6 +22,8 @@
 #include "fdma_common.h"
 #include "fdma_params.h"
 
+#include <type_traits>
+
 namespace fdma {
 
 namespace {
@@ -621,7 +623,11 @@ hipError_t launch_bwd_t(const BwdParams &p, hipStream_t stream) {
         if ((e = hipGetLastError()) != hipSuccess) return e;
     }
     // 2. dK, dV, dBias
-    if (f.Lk > 0) {
+    const int dtype_code = std::is_same<T, bf16_tag>::value ? 0 : 1;
+    const bool colmask = bwd_colmask_applicable(p);
+    if (f.Lk > 0 && colmask) {
+        if ((e = launch_bwd_dkdv_colmask(p, dtype_code, stream)) != hipSuccess) return e;
+    } else if (f.Lk > 0) {
         dim3 grid((f.Lk + KV_BN - 1) / KV_BN, f.Hk, f.B);
         const size_t smem = KvSmem<D>::TOTAL;
         if (f.causal) {
@@ -640,7 +646,9 @@ hipError_t launch_bwd_t(const BwdParams &p, hipStream_t stream) {
         if ((e = hipGetLastError()) != hipSuccess) return e;
     }
     // 3. dQ
-    {
+    if (colmask) {
+        if ((e = launch_bwd_dq_colmask(p, dtype_code, stream)) != hipSuccess) return e;
+    } else {
         dim3 grid((f.Lq + Q_BM - 1) / Q_BM, f.H, f.B);
         if (f.causal)
             hipLaunchKernelGGL((bwd_dq_kernel<T, D, true>), grid, dim3(NTHREADS), 0, stream, p);

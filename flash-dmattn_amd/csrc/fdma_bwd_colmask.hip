@@ -1,0 +1,667 @@
+// Backward dynamic-mask attention for gfx950, column-mask specialisation of the two main kernels.
+//
+// Same math and same reference counterparts as fdma_bwd.hip
+// (compute_dq_dk_dv_1colblock, csrc/flash_sparse_attn/src/flash_bwd_kernel.h:79-1142 of the reference), for
+// mask and bias that are absent or broadcast over the query dimension ([B, {1,Hk,H}, 1, Lk]).
+// "Keep" and the bias are then properties of the key column:
+//   * in the dK/dV kernel a lane owns one key column for the whole kernel, so mask and bias
+//     collapse to one fused per-lane constant (bias*log2e, or -inf when masked / beyond Lk): no
+//     mask or bias loads in the loop, no selects -- exp2(-inf) = 0 does the masking;
+//   * dBias is the column sum of dS, accumulated in a register and written once;
+//   * in the dQ kernel the fused vector is staged per tile exactly as in the forward kernel and
+//     fully masked 64-key tiles are skipped through the same LDS bitmap.
+// K and V are stationary in registers in the dK/dV kernel (B operands), Q / dO tiles and the row
+// statistics stream through double-buffered LDS with the next step's global loads in flight during
+// the current step.  Workgroup ids are remapped so that workgroups sharing an XCD's L2 share the
+// streamed operands.
+#include "fdma_common.h"
+#include "fdma_params.h"
+
+namespace fdma {
+
+namespace {
+
+constexpr int NTHREADS = 256;
+
+// XCD-aware work distribution shared by both kernels: `pairs` independent (batch, kv head) pairs with
+// `n_units` units of work each (heaviest first); see the forward column-mask kernel for the rationale.
+struct XcdMap {
+    int pair, unit;
+    bool valid;
+};
+__device__ __forceinline__ XcdMap xcd_map(int lid, int pairs, int n_units, int per_unit) {
+    const int gcd8 = (pairs % 8 == 0) ? 8 : ((pairs % 4 == 0) ? 4 : ((pairs % 2 == 0) ? 2 : 1));
+    const int k_split = 8 / gcd8;
+    const int list_len = ((n_units + k_split - 1) / k_split) * per_unit;
+    const int xcd = lid % 8, slot = lid / 8;
+    const int vlist = xcd + 8 * (slot / list_len);
+    const int pos = slot % list_len;
+    XcdMap m;
+    m.pair = vlist / k_split;
+    m.unit = (pos / per_unit) * k_split + vlist % k_split;
+    m.valid = m.unit < n_units;
+    return m;
+}
+inline int xcd_grid(int pairs, int n_units, int per_unit) {
+    const int gcd8 = (pairs % 8 == 0) ? 8 : ((pairs % 4 == 0) ? 4 : ((pairs % 2 == 0) ? 2 : 1));
+    const int k_split = 8 / gcd8;
+    return pairs * k_split * ((n_units + k_split - 1) / k_split) * per_unit;
+}
+
+// ------------------------------------------------------------------------------------------------
+// dK / dV / dBias
+// ------------------------------------------------------------------------------------------------
+constexpr int KV_BM = 64;   // query rows per step
+constexpr int KV_BN = 128;  // key columns per workgroup (32 per wave)
+
+template <int D> struct KvcSmem {
+    static constexpr int S = D + 8;
+    static constexpr int Q_BYTES = KV_BM * S * 2;
+    static constexpr int STAGE = 2 * Q_BYTES + 2 * KV_BM * 4;  // Q, dO, LSE, D
+    static constexpr int TOTAL = 2 * STAGE;
+};
+
+template <typename T, int D, bool CAUSAL>
+__global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_kernel(const BwdParams p) {
+    using E = Elem<T>;
+    using SM = KvcSmem<D>;
+    constexpr int KS = D / 16;
+    constexpr int DB = D / 32;
+    constexpr int MB = KV_BM / 32;
+    constexpr int CH = D / 8, RPP = NTHREADS / CH, Q_IT = KV_BM / RPP;
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+
+    const FwdParams &f = p.f;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 31, g = lane >> 5;
+    const int G = f.H / f.Hk;
+    const int n_nb = (f.Lk + KV_BN - 1) / KV_BN;
+    const XcdMap wm = xcd_map(blockIdx.x, f.B * f.Hk, n_nb, 1);
+    if (!wm.valid) return;
+    const int n_block = wm.unit;  // low key blocks are seen by the most queries under causal: heaviest first
+    const int b = wm.pair / f.Hk, hk = wm.pair % f.Hk;
+    const int n0 = n_block * KV_BN;
+    const int key = n0 + wave * 32 + r;  // the key column this lane owns
+    const int key_c = key < f.Lk ? key : f.Lk - 1;
+    const int shift = f.Lk - f.Lq;
+
+    // ---- stationary K / V fragments (B operands): lane holds K[key][16ks + 8g .. +8]
+    u32x4_t kf[KS], vf[KS];
+    {
+        const uint16_t *kp = (const uint16_t *)f.k + b * f.k_b + (int64_t)key_c * f.k_r + hk * f.k_h;
+        const uint16_t *vp = (const uint16_t *)f.v + b * f.v_b + (int64_t)key_c * f.v_r + hk * f.v_h;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            const int c = ks * 16 + g * 8;
+            u32x4_t kv = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
+            if (c < f.d) { kv = *(const u32x4_t *)(kp + c); vv = *(const u32x4_t *)(vp + c); }
+            kf[ks] = kv;
+            vf[ks] = vv;
+        }
+    }
+
+    f32x16_t dk[DB], dv[DB];
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) { dk[db][i] = 0.f; dv[db][i] = 0.f; }
+
+    const int M_blocks = (f.Lq + KV_BM - 1) / KV_BM;
+    int m_start = 0;
+    if (CAUSAL) {
+        const int first_q = n0 - shift;  // first query row that sees key n0
+        if (first_q > 0) m_start = first_q / KV_BM;
+        if (m_start > M_blocks) m_start = M_blocks;
+    }
+    const int n_m = M_blocks - m_start;
+    const int n_steps = n_m * G;  // (g outer, m inner)
+
+    const bool has_bias = f.bias != nullptr;
+    const bool use_accum = p.dbias_accum != nullptr;
+
+    // fused per-lane column constant for query head h: bias*log2e, or -inf when the column is dropped
+    auto column_const = [&](int h) -> float {
+        if (key >= f.Lk) return -INFINITY;
+        if (f.mask) {
+            const int hm = f.Hm == f.H ? h : (f.Hm == 1 ? 0 : hk);
+            if (!f.mask[b * f.m_b + hm * f.m_h + key]) return -INFINITY;
+        }
+        if (has_bias) {
+            const int hb = f.Hb == f.H ? h : (f.Hb == 1 ? 0 : hk);
+            return E::lo((uint32_t)((const uint16_t *)f.bias)[b * f.bi_b + hb * f.bi_h + key]) * kLog2e;
+        }
+        return 0.f;
+    };
+
+    // ---- staging of Q / dO / LSE / D for one step (global -> registers -> LDS)
+    const int qc = tid % CH, qr0 = tid / CH;
+    const int qcol = (qc * 8 < f.d) ? qc * 8 : 0;  // head-dim chunks beyond d: re-read chunk 0 (K/V fragments there are zero)
+    u32x4_t qreg[Q_IT], doreg[Q_IT];
+    float lreg = INFINITY, dreg = 0.f;
+    auto load_step = [&](int step) {
+        const int gi = step / n_m, mi = m_start + step % n_m;
+        const int h = hk * G + gi, m0 = mi * KV_BM;
+        const uint16_t *qbase = (const uint16_t *)f.q + b * f.q_b + h * f.q_h + qcol;
+        const uint16_t *dobase = (const uint16_t *)p.dout + b * p.do_b + h * p.do_h + qcol;
+#pragma unroll
+        for (int it = 0; it < Q_IT; it++) {
+            int qq = m0 + qr0 + it * RPP;
+            qq = qq < f.Lq ? qq : f.Lq - 1;  // rows beyond Lq: finite duplicates, cancelled by LSE = +inf
+            qreg[it] = *(const u32x4_t *)(qbase + (int64_t)qq * f.q_r);
+            doreg[it] = *(const u32x4_t *)(dobase + (int64_t)qq * p.do_r);
+        }
+        if (tid < KV_BM) {
+            const int qq = m0 + tid;
+            lreg = INFINITY;
+            dreg = 0.f;
+            if (qq < f.Lq) {
+                lreg = f.lse[((int64_t)b * f.H + h) * f.Lq + qq] * kLog2e;
+                dreg = p.softmax_d[((int64_t)b * f.H + h) * p.Lq_rounded + qq];
+            }
+        }
+    };
+    auto store_step = [&](int buf) {
+        char *base = smem + buf * SM::STAGE;
+#pragma unroll
+        for (int it = 0; it < Q_IT; it++) {
+            const int off = ((qr0 + it * RPP) * SM::S + qc * 8) * 2;
+            *(u32x4_t *)(base + off) = qreg[it];
+            *(u32x4_t *)(base + SM::Q_BYTES + off) = doreg[it];
+        }
+        if (tid < KV_BM) {
+            ((float *)(base + 2 * SM::Q_BYTES))[tid] = lreg;
+            ((float *)(base + 2 * SM::Q_BYTES + KV_BM * 4))[tid] = dreg;
+        }
+    };
+
+    const int a_row = pi_row(r);
+    const int tj = lane & 15, te = tj >> 2, tc = tj & 3;
+    const int tcp = (tc == 1) ? 2 : (tc == 2 ? 1 : tc);
+    const int tdh = (lane >> 4) & 1;
+    const uint32_t tr_off = (uint32_t)(((8 * g + te) * SM::S + 16 * tdh + 4 * tcp) * 2);
+    const uint32_t a_off = (uint32_t)((a_row * SM::S + g * 8) * 2);
+
+    float colsum = 0.f;
+    float cconst = 0.f;
+
+    if (n_steps > 0) {
+        load_step(0);
+        store_step(0);
+        __syncthreads();
+    }
+
+    for (int step = 0; step < n_steps; step++) {
+        const int gi = step / n_m, mi = m_start + step % n_m;
+        const int h = hk * G + gi;
+        const int m0 = mi * KV_BM;
+        const int buf = step & 1;
+        if (step % n_m == 0) cconst = column_const(h);
+        if (step + 1 < n_steps) load_step(step + 1);
+
+        const char *sQ = smem + buf * SM::STAGE;
+        const char *sDO = sQ + SM::Q_BYTES;
+        const float *sLSE = (const float *)(sQ + 2 * SM::Q_BYTES);
+        const float *sDD = sLSE + KV_BM;
+
+        // ---- S = Q K^T and dP = dO V^T (M = query, N = key); fragment reads run a batch ahead
+        f32x16_t s[MB], dp[MB];
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) { s[mb][i] = 0.f; dp[mb][i] = 0.f; }
+        {
+            constexpr int NF = 2 * MB * KS, FR = 8;  // fragment f: (ks, mb, which) with which = 0: Q, 1: dO
+            u32x4_t a[NF];
+            auto frag = [&](int fi) {
+                const int which = fi & 1, mb = (fi >> 1) % MB, ks = (fi >> 1) / MB;
+                return *(const u32x4_t *)((which ? sDO : sQ) + a_off + (32 * mb * SM::S + ks * 16) * 2);
+            };
+#pragma unroll
+            for (int fi = 0; fi < FR; fi++) a[fi] = frag(fi);
+#pragma unroll
+            for (int fi = 0; fi < NF; fi++) {
+                if (fi + FR < NF) a[fi + FR] = frag(fi + FR);
+                const int which = fi & 1, mb = (fi >> 1) % MB, ks = (fi >> 1) / MB;
+                if (which) dp[mb] = E::mfma(a[fi], vf[ks], dp[mb]);
+                else s[mb] = E::mfma(a[fi], kf[ks], s[mb]);
+            }
+        }
+
+        // ---- P = exp2(S*scale*log2e + c - LSE*log2e) ; dS = P * (dP - D)
+        // diagonal step: some (query, key) pairs of this wave are above the causal diagonal
+        const bool diag = CAUSAL && (n0 + wave * 32 + 31 > m0 + shift);
+        uint32_t ppk[MB * 8], dpk[MB * 8];
+        float part = 0.f;
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+            for (int blk = 0; blk < 2; blk++) {
+                const float *lp = sLSE + 32 * mb + 16 * blk + 8 * g;
+                const float *dpn = sDD + 32 * mb + 16 * blk + 8 * g;
+                const f32x4_t l0 = *(const f32x4_t *)lp, l1 = *(const f32x4_t *)(lp + 4);
+                const f32x4_t d0 = *(const f32x4_t *)dpn, d1 = *(const f32x4_t *)(dpn + 4);
+                float pv[8], dsv[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const int ii = 8 * blk + e;
+                    const float lse2 = e < 4 ? l0[e] : l1[e - 4];
+                    const float dd = e < 4 ? d0[e] : d1[e - 4];
+                    const float x = fmaf(s[mb][ii], f.scale_log2, cconst) - lse2;
+                    pv[e] = fast_exp2(x);
+                    dsv[e] = dp[mb][ii] - dd;
+                }
+                if (diag) {
+                    asm volatile("" ::: "memory");  // keep a real branch: only diagonal steps pay
+                    const int lim = key - shift - m0 - 32 * mb - 16 * blk - 8 * g;  // rows e >= lim see this key
+#pragma unroll
+                    for (int e = 0; e < 8; e++) pv[e] = e >= lim ? pv[e] : 0.f;
+                }
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    dsv[e] *= pv[e];
+                    part += dsv[e];
+                }
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    ppk[mb * 8 + blk * 4 + e] = E::pack2(pv[2 * e], pv[2 * e + 1]);
+                    dpk[mb * 8 + blk * 4 + e] = E::pack2(dsv[2 * e], dsv[2 * e + 1]);
+                }
+            }
+        colsum += part;
+
+        // ---- dV^T += dO^T P ; dK^T += Q^T dS   (M = d, N = key, contraction = query)
+#pragma unroll
+        for (int qb = 0; qb < KV_BM / 16; qb++) {
+            const u32x4_t pb = {ppk[4 * qb], ppk[4 * qb + 1], ppk[4 * qb + 2], ppk[4 * qb + 3]};
+            const u32x4_t sb = {dpk[4 * qb], dpk[4 * qb + 1], dpk[4 * qb + 2], dpk[4 * qb + 3]};
+#pragma unroll
+            for (int db = 0; db < DB; db++) {
+                const uint32_t off = tr_off + (uint32_t)((16 * qb * SM::S + 32 * db) * 2);
+                const u32x2_t lo = lds_read_tr16(sDO, off), hi = lds_read_tr16(sDO, off + 4 * SM::S * 2);
+                const u32x2_t lo2 = lds_read_tr16(sQ, off), hi2 = lds_read_tr16(sQ, off + 4 * SM::S * 2);
+                const u32x4_t a1 = {lo[0], lo[1], hi[0], hi[1]};
+                const u32x4_t a2 = {lo2[0], lo2[1], hi2[0], hi2[1]};
+                dv[db] = E::mfma(a1, pb, dv[db]);
+                dk[db] = E::mfma(a2, sb, dk[db]);
+            }
+        }
+
+        // ---- dBias column sum: flush when the bias head changes
+        if (has_bias) {
+            const bool last_m = (step % n_m) == n_m - 1;
+            if (last_m && (f.Hb == f.H || gi == G - 1)) {
+                const float tot = xhalf_sum(colsum);
+                const int hb = f.Hb == f.H ? h : (f.Hb == 1 ? 0 : hk);
+                if (g == 0 && key < f.Lk) {
+                    if (use_accum) atomicAdd(p.dbias_accum + b * p.dba_b + hb * p.dba_h + key, tot);
+                    else ((uint16_t *)p.dbias)[b * p.db_b + hb * p.db_h + key] = (uint16_t)(E::pack2(tot, 0.f) & 0xffffu);
+                }
+                colsum = 0.f;
+            }
+        }
+
+        if (step + 1 < n_steps) store_step(buf ^ 1);
+        __syncthreads();
+    }
+
+    // a key block that no query can see still owns its dbias column
+    if (has_bias && n_steps == 0 && !use_accum && g == 0 && key < f.Lk) {
+        const int ngh = (f.Hb == f.H) ? G : 1;
+        for (int gh = 0; gh < ngh; gh++) {
+            const int hb = f.Hb == f.H ? hk * G + gh : (f.Hb == 1 ? 0 : hk);
+            ((uint16_t *)p.dbias)[b * p.db_b + hb * p.db_h + key] = 0;
+        }
+    }
+
+    // ---- store dK (scaled) and dV
+    if (key < f.Lk) {
+        uint16_t *dkp = (uint16_t *)p.dk + b * p.dk_b + (int64_t)key * p.dk_r + hk * p.dk_h;
+        uint16_t *dvp = (uint16_t *)p.dv + b * p.dv_b + (int64_t)key * p.dv_r + hk * p.dv_h;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int blk = 0; blk < 2; blk++) {
+                const int c = 32 * db + 16 * blk + 8 * g;
+                if (c < f.d) {
+                    u32x4_t wk, wv;
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        wk[e] = E::pack2(dk[db][8 * blk + 2 * e] * f.scale, dk[db][8 * blk + 2 * e + 1] * f.scale);
+                        wv[e] = E::pack2(dv[db][8 * blk + 2 * e], dv[db][8 * blk + 2 * e + 1]);
+                    }
+                    *(u32x4_t *)(dkp + c) = wk;
+                    *(u32x4_t *)(dvp + c) = wv;
+                }
+            }
+    }
+}
+
+template <typename T, int D, bool CAUSAL>
+hipError_t launch_dkdv(const BwdParams &p, hipStream_t stream) {
+    const FwdParams &f = p.f;
+    auto kern = bwd_dkdv_colmask_kernel<T, D, CAUSAL>;
+    const int smem = KvcSmem<D>::TOTAL;
+    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return e;
+    dim3 grid(xcd_grid(f.B * f.Hk, (f.Lk + KV_BN - 1) / KV_BN, 1));
+    hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, stream, p);
+    return hipGetLastError();
+}
+
+
+// ------------------------------------------------------------------------------------------------
+// dQ
+// ------------------------------------------------------------------------------------------------
+constexpr int Q_BM = 128;
+constexpr int MAX_TILES = 16384;
+
+
+template <int D, int BN> struct DqcSmem {
+    static constexpr int S = D + 8;
+    static constexpr int K_BYTES = BN * S * 2;
+    static constexpr int OFF_K = 0;
+    static constexpr int OFF_V = OFF_K + 2 * K_BYTES;
+    static constexpr int OFF_BIAS = OFF_V + 2 * K_BYTES;
+    static constexpr int OFF_BITS = OFF_BIAS + 3 * BN * 4;
+    static constexpr int TOTAL = OFF_BITS + MAX_TILES / 8;
+};
+
+template <typename T, int D, int BN, bool CAUSAL>
+__global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdParams p) {
+    using E = Elem<T>;
+    using SM = DqcSmem<D, BN>;
+    constexpr int KS = D / 16;
+    constexpr int DB = D / 32;
+    constexpr int MB = BN / 32;
+    constexpr int KB = BN / 16;
+    constexpr int CH = D / 8, RPP = NTHREADS / CH, K_IT = BN / RPP;
+
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    float *sBias = (float *)(smem + SM::OFF_BIAS);
+    uint32_t *sBits = (uint32_t *)(smem + SM::OFF_BITS);
+
+    const FwdParams &f = p.f;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 31, g = lane >> 5;
+    const int G = f.H / f.Hk;
+    const int n_mb = (f.Lq + Q_BM - 1) / Q_BM;
+    const XcdMap wm = xcd_map(blockIdx.x, f.B * f.Hk, n_mb, G);
+    if (!wm.valid) return;
+    const int m_block = n_mb - 1 - wm.unit;  // heaviest first under causal
+    const int b = wm.pair / f.Hk, hk = wm.pair % f.Hk;
+    const int h = hk * G + (blockIdx.x / 8) % G;
+    const int m0 = m_block * Q_BM;
+    const int qrow = m0 + wave * 32 + r;
+    const int qrow_c = qrow < f.Lq ? qrow : f.Lq - 1;
+    const int shift = f.Lk - f.Lq;
+
+    const int hm = f.mask ? (f.Hm == f.H ? h : (f.Hm == 1 ? 0 : hk)) : 0;
+    const int hb = f.bias ? (f.Hb == f.H ? h : (f.Hb == 1 ? 0 : hk)) : 0;
+    const uint8_t *mrow = f.mask ? f.mask + b * f.m_b + hm * f.m_h : nullptr;
+    const uint16_t *brow = f.bias ? (const uint16_t *)f.bias + b * f.bi_b + hb * f.bi_h : nullptr;
+    const uint16_t *kbase = (const uint16_t *)f.k + b * f.k_b + hk * f.k_h;
+    const uint16_t *vbase = (const uint16_t *)f.v + b * f.v_b + hk * f.v_h;
+
+    int n_end = (f.Lk + BN - 1) / BN;
+    if (CAUSAL) {
+        int lim = m0 + Q_BM + shift;
+        if (lim > f.Lq + shift) lim = f.Lq + shift;
+        if (lim < 0) lim = 0;
+        const int ne = (lim + BN - 1) / BN;
+        if (ne < n_end) n_end = ne;
+    }
+
+    // ---- active-tile bitmap (tiles with at least one kept key)
+    for (int base = 0; base < n_end; base += NTHREADS) {
+        const int j = base + tid;
+        bool act = false;
+        if (j < n_end) {
+            if (mrow) {
+                uint32_t any = 0;
+#pragma unroll
+                for (int c = 0; c < BN / 16; c++) {
+                    const int col = j * BN + c * 16;
+                    if (col < f.Lk) {
+                        const u32x4_t mv = *(const u32x4_t *)(mrow + col);
+                        any |= mv[0] | mv[1] | mv[2] | mv[3];
+                    }
+                }
+                act = any != 0;
+            } else {
+                act = true;
+            }
+        }
+        const uint64_t ball = __ballot(act);
+        if (lane == 0) {
+            const int w0 = (base + wave * 64) >> 5;
+            sBits[w0] = (uint32_t)ball;
+            sBits[w0 + 1] = (uint32_t)(ball >> 32);
+        }
+    }
+    __syncthreads();
+    auto next_active = [&](int j) -> int {
+        while (j < n_end) {
+            const uint32_t w = sBits[j >> 5] >> (j & 31);
+            if (w) {
+                j += __builtin_ctz(w);
+                return j < n_end ? j : n_end;
+            }
+            j = (j | 31) + 1;
+        }
+        return n_end;
+    };
+
+    // ---- Q and dO fragments (B operands), row statistics
+    u32x4_t qf[KS], dof[KS];
+    {
+        const uint16_t *qp = (const uint16_t *)f.q + b * f.q_b + (int64_t)qrow_c * f.q_r + h * f.q_h;
+        const uint16_t *dp = (const uint16_t *)p.dout + b * p.do_b + (int64_t)qrow_c * p.do_r + h * p.do_h;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            const int c = ks * 16 + g * 8;
+            u32x4_t qv = {0, 0, 0, 0}, dv = {0, 0, 0, 0};
+            if (qrow < f.Lq && c < f.d) { qv = *(const u32x4_t *)(qp + c); dv = *(const u32x4_t *)(dp + c); }
+            qf[ks] = qv;
+            dof[ks] = dv;
+        }
+    }
+    float lse2 = INFINITY, dd = 0.f;
+    if (qrow < f.Lq) {
+        lse2 = f.lse[((int64_t)b * f.H + h) * f.Lq + qrow] * kLog2e;
+        dd = p.softmax_d[((int64_t)b * f.H + h) * p.Lq_rounded + qrow];
+    }
+
+    f32x16_t dq[DB];
+#pragma unroll
+    for (int db = 0; db < DB; db++)
+#pragma unroll
+        for (int i = 0; i < 16; i++) dq[db][i] = 0.f;
+
+    // ---- staging: rows beyond Lk are clamped (their fused bias is -inf), head-dim chunks beyond d re-read chunk 0
+    const int kc = tid % CH, kr0 = tid / CH;
+    const int kcol = (kc * 8 < f.d) ? kc * 8 : 0;
+    u32x4_t kreg[K_IT], vreg[K_IT];
+    float breg = 0.f;
+    auto load_tile = [&](int j) {
+        const int n0 = j * BN;
+#pragma unroll
+        for (int it = 0; it < K_IT; it++) {
+            int key = n0 + kr0 + it * RPP;
+            key = key < f.Lk ? key : f.Lk - 1;
+            kreg[it] = *(const u32x4_t *)(kbase + (int64_t)key * f.k_r + kcol);
+            vreg[it] = *(const u32x4_t *)(vbase + (int64_t)key * f.v_r + kcol);
+        }
+        if (tid < BN) {
+            const int col = n0 + tid;
+            float v = -INFINITY;
+            if (col < f.Lk && (!mrow || mrow[col])) {
+                v = 0.f;
+                if (brow) v = E::lo((uint32_t)brow[col]) * kLog2e;
+            }
+            breg = v;
+        }
+    };
+    auto store_tile = [&](int buf, int slot) {
+        char *sK = smem + SM::OFF_K + buf * SM::K_BYTES;
+        char *sV = smem + SM::OFF_V + buf * SM::K_BYTES;
+#pragma unroll
+        for (int it = 0; it < K_IT; it++) {
+            const int off = ((kr0 + it * RPP) * SM::S + kc * 8) * 2;
+            *(u32x4_t *)(sK + off) = kreg[it];
+            *(u32x4_t *)(sV + off) = vreg[it];
+        }
+        if (tid < BN) sBias[slot * BN + tid] = breg;
+    };
+
+    const int a_row = pi_row(r);
+    const uint32_t a_off = (uint32_t)((a_row * SM::S + g * 8) * 2);
+    const int tj = lane & 15, te = tj >> 2, tc = tj & 3;
+    const int tcp = (tc == 1) ? 2 : (tc == 2 ? 1 : tc);
+    const int tdh = (lane >> 4) & 1;
+    const uint32_t tr_off = (uint32_t)(((8 * g + te) * SM::S + 16 * tdh + 4 * tcp) * 2);
+
+    int jc = next_active(0);
+    if (jc < n_end) {
+        load_tile(jc);
+        store_tile(0, 0);
+        __syncthreads();
+    }
+    int i = 0;
+    while (jc < n_end) {
+        const int jn = next_active(jc + 1);
+        if (jn < n_end) load_tile(jn);
+        const int n0 = jc * BN;
+        const char *sK = smem + SM::OFF_K + (i & 1) * SM::K_BYTES;
+        const char *sV = smem + SM::OFF_V + (i & 1) * SM::K_BYTES;
+        const float *bs = sBias + (i % 3) * BN + 8 * g;
+
+        // ---- S^T = K Q^T, dP^T = V dO^T
+        f32x16_t s[MB], dp[MB];
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+            for (int ii = 0; ii < 16; ii++) { s[mb][ii] = 0.f; dp[mb][ii] = 0.f; }
+        {
+            constexpr int NF = 2 * MB * KS, FR = 8;
+            u32x4_t a[NF];
+            auto frag = [&](int fi) {
+                const int which = fi & 1, mb = (fi >> 1) % MB, ks = (fi >> 1) / MB;
+                return *(const u32x4_t *)((which ? sV : sK) + a_off + (32 * mb * SM::S + ks * 16) * 2);
+            };
+#pragma unroll
+            for (int fi = 0; fi < FR; fi++) a[fi] = frag(fi);
+#pragma unroll
+            for (int fi = 0; fi < NF; fi++) {
+                if (fi + FR < NF) a[fi + FR] = frag(fi + FR);
+                const int which = fi & 1, mb = (fi >> 1) % MB, ks = (fi >> 1) / MB;
+                if (which) dp[mb] = E::mfma(a[fi], dof[ks], dp[mb]);
+                else s[mb] = E::mfma(a[fi], qf[ks], s[mb]);
+            }
+        }
+        // ---- dS^T = P^T * (dP^T - D)
+        const bool diag = CAUSAL && (n0 + BN - 1 > m0 + wave * 32 + shift);
+        uint32_t dpk[8 * MB];
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+            for (int blk = 0; blk < 2; blk++) {
+                const f32x4_t b0 = *(const f32x4_t *)(bs + 32 * mb + 16 * blk);
+                const f32x4_t b1 = *(const f32x4_t *)(bs + 32 * mb + 16 * blk + 4);
+                float pv[8];
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    const float bl = e < 4 ? b0[e] : b1[e - 4];
+                    pv[e] = fast_exp2(fmaf(s[mb][8 * blk + e], f.scale_log2, bl) - lse2);
+                }
+                if (diag) {
+                    asm volatile("" ::: "memory");
+                    const int lim = qrow + shift - n0 - 32 * mb - 16 * blk - 8 * g;  // local columns e <= lim are visible
+#pragma unroll
+                    for (int e = 0; e < 8; e++) pv[e] = e <= lim ? pv[e] : 0.f;
+                }
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const float d0 = pv[2 * e] * (dp[mb][8 * blk + 2 * e] - dd);
+                    const float d1 = pv[2 * e + 1] * (dp[mb][8 * blk + 2 * e + 1] - dd);
+                    dpk[8 * mb + 4 * blk + e] = E::pack2(d0, d1);
+                }
+            }
+        // ---- dQ^T += K^T dS^T  (K^T through transposing LDS reads of the row-major K tile)
+#pragma unroll
+        for (int kb = 0; kb < KB; kb++) {
+            const u32x4_t bop = {dpk[4 * kb], dpk[4 * kb + 1], dpk[4 * kb + 2], dpk[4 * kb + 3]};
+#pragma unroll
+            for (int db = 0; db < DB; db++) {
+                const uint32_t off = tr_off + (uint32_t)((16 * kb * SM::S + 32 * db) * 2);
+                const u32x2_t lo = lds_read_tr16(sK, off), hi = lds_read_tr16(sK, off + 4 * SM::S * 2);
+                const u32x4_t a = {lo[0], lo[1], hi[0], hi[1]};
+                dq[db] = E::mfma(a, bop, dq[db]);
+            }
+        }
+        if (jn < n_end) store_tile((i + 1) & 1, (i + 1) % 3);
+        __syncthreads();
+        i++;
+        jc = jn;
+    }
+
+    if (qrow < f.Lq) {
+        uint16_t *dqp = (uint16_t *)p.dq + b * p.dq_b + (int64_t)qrow * p.dq_r + h * p.dq_h;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int blk = 0; blk < 2; blk++) {
+                const int c = 32 * db + 16 * blk + 8 * g;
+                if (c < f.d) {
+                    u32x4_t w;
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        w[e] = E::pack2(dq[db][8 * blk + 2 * e] * f.scale, dq[db][8 * blk + 2 * e + 1] * f.scale);
+                    *(u32x4_t *)(dqp + c) = w;
+                }
+            }
+    }
+}
+
+template <typename T, int D, bool CAUSAL>
+hipError_t launch_dq(const BwdParams &p, hipStream_t stream) {
+    const FwdParams &f = p.f;
+    constexpr int BN = D > 64 ? 32 : 64;  // at d = 128 a 64-key tile would spill registers
+    auto kern = bwd_dq_colmask_kernel<T, D, BN, CAUSAL>;
+    const int smem = DqcSmem<D, BN>::TOTAL;
+    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return e;
+    dim3 grid(xcd_grid(f.B * f.Hk, (f.Lq + Q_BM - 1) / Q_BM, f.H / f.Hk));
+    hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, stream, p);
+    return hipGetLastError();
+}
+
+}  // namespace
+
+bool bwd_colmask_applicable(const BwdParams &p) {
+    const bool mask_ok = !p.f.mask || p.f.m_r == 0;
+    const bool bias_ok = !p.f.bias || p.f.bi_r == 0;
+    return mask_ok && bias_ok && (p.f.Lk + 63) / 64 <= MAX_TILES;
+}
+
+hipError_t launch_bwd_dkdv_colmask(const BwdParams &p, int dtype, hipStream_t stream) {
+    const bool d64 = p.f.d <= 64, c = p.f.causal != 0;
+    if (dtype == 0) {
+        if (d64) return c ? launch_dkdv<bf16_tag, 64, true>(p, stream) : launch_dkdv<bf16_tag, 64, false>(p, stream);
+        return c ? launch_dkdv<bf16_tag, 128, true>(p, stream) : launch_dkdv<bf16_tag, 128, false>(p, stream);
+    }
+    if (d64) return c ? launch_dkdv<fp16_tag, 64, true>(p, stream) : launch_dkdv<fp16_tag, 64, false>(p, stream);
+    return c ? launch_dkdv<fp16_tag, 128, true>(p, stream) : launch_dkdv<fp16_tag, 128, false>(p, stream);
+}
+
+}  // namespace fdma
+
+namespace fdma {
+hipError_t launch_bwd_dq_colmask(const BwdParams &p, int dtype, hipStream_t stream) {
+    const bool d64 = p.f.d <= 64, c = p.f.causal != 0;
+    if (dtype == 0) {
+        if (d64) return c ? launch_dq<bf16_tag, 64, true>(p, stream) : launch_dq<bf16_tag, 64, false>(p, stream);
+        return c ? launch_dq<bf16_tag, 128, true>(p, stream) : launch_dq<bf16_tag, 128, false>(p, stream);
+    }
+    if (d64) return c ? launch_dq<fp16_tag, 64, true>(p, stream) : launch_dq<fp16_tag, 64, false>(p, stream);
+    return c ? launch_dq<fp16_tag, 128, true>(p, stream) : launch_dq<fp16_tag, 128, false>(p, stream);
+}
+}  // namespace fdma

@@ -52,6 +52,10 @@ bool fwd_colmask_applicable(const FwdParams &p);
 hipError_t launch_fwd_colmask(const FwdParams &p, int dtype, int nq, hipStream_t stream);
 hipError_t launch_fwd_decode(const FwdParams &p, int dtype, hipStream_t stream);
 hipError_t launch_bwd(const BwdParams &p, int dtype, hipStream_t stream);
+// column-mask specialisations of the two main backward kernels
+bool bwd_colmask_applicable(const BwdParams &p);
+hipError_t launch_bwd_dkdv_colmask(const BwdParams &p, int dtype, hipStream_t stream);
+hipError_t launch_bwd_dq_colmask(const BwdParams &p, int dtype, hipStream_t stream);
 
 // number of KV splits the decode path uses for this shape (1 = no workspace needed)
 int decode_num_splits(int B, int Hk, int Lk);
