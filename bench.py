@@ -29,6 +29,10 @@ import torch  # noqa: E402
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
+# HBM bytes per launch of the forward kernel on the headline workload, from two rocprofv3 --pmc runs of
+# this script (FETCH_SIZE, WRITE_SIZE; each scaled by what the counter reads for a 256 MiB device copy,
+# see --calib-copy): 143 MiB read + 65 MiB written.  Override with --traffic-bytes after re-measuring.
+MEASURED_FWD_TRAFFIC_BYTES = 208.0 * 1024 * 1024
 
 CONFIGS = {
     # name: B, Lq, Lk, H, Hk, D, bias shape, window, causal, passes
@@ -197,6 +201,10 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--all", action="store_true", help="also time configurations 1, 3, 4, 5")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--calib-copy", action="store_true",
+                    help="also run one plain 256 MiB device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
+    ap.add_argument("--traffic-bytes", type=float, default=None,
+                    help="HBM bytes per launch of the dominant kernel from rocprofv3 --pmc runs (reported as roofline.traffic)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the hot path has no multi-GPU part in this build; run with --gpus 1", file=sys.stderr)
@@ -234,11 +242,18 @@ def main():
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": main_res["tflops_fwd"] / PEAK_BF16_TFLOPS,
-            "traffic": None,
+            "traffic": MEASURED_FWD_TRAFFIC_BYTES,
             "kernel": "fdma::fwd_kernel<bf16, 128, causal>",
             "flops_per_launch": 4.0 * 64 * 64 * c["D"] * main_res["n_exec"],
         },
     }
+    if args.traffic_bytes is not None:
+        out["roofline"]["traffic"] = args.traffic_bytes
+    if args.calib_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=device).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
     if args.all:
         out["other_configs"] = [run_config(n, max(3, args.steps // 4), max(1, args.warmup // 2), device)
                                 for n in ("cfg1", "cfg3", "cfg4", "cfg5")]

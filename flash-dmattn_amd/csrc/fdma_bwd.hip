@@ -179,7 +179,7 @@ __global__ void __launch_bounds__(NTHREADS) bwd_dkdv_kernel(const BwdParams p) {
 
     for (int step = 0; step < n_steps; step++) {
         const int gi = m_outer ? step % G : step / n_m;
-        const int mi = m_start + (m_outer ? step / G : step % n_m);
+        const int mi = M_blocks - 1 - (m_outer ? step / G : step % n_m);  // last query block first (shared L2 streaming)
         const int h = hk * G + gi;
         const int m0 = mi * KV_BM;
         const int hm = f.mask ? (f.Hm == f.H ? h : (f.Hm == 1 ? 0 : hk)) : 0;

@@ -114,7 +114,10 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
         if (m_start > M_blocks) m_start = M_blocks;
     }
     const int n_m = M_blocks - m_start;
-    const int n_steps = n_m * G;  // (g outer, m inner)
+    // (g outer, m inner); the query blocks are walked from the LAST one down to m_start, so that the
+    // workgroups of one (batch, kv head) pair, which run side by side on an XCD, all begin at the same
+    // Q / dO tile and stream the same tiles at the same time (L2 hits instead of re-fetches)
+    const int n_steps = n_m * G;
 
     const bool has_bias = f.bias != nullptr;
     const bool use_accum = p.dbias_accum != nullptr;
@@ -139,7 +142,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
     u32x4_t qreg[Q_IT], doreg[Q_IT];
     float lreg = INFINITY, dreg = 0.f;
     auto load_step = [&](int step) {
-        const int gi = step / n_m, mi = m_start + step % n_m;
+        const int gi = step / n_m, mi = M_blocks - 1 - step % n_m;  // last query block first: see below
         const int h = hk * G + gi, m0 = mi * KV_BM;
         const uint16_t *qbase = (const uint16_t *)f.q + b * f.q_b + h * f.q_h + qcol;
         const uint16_t *dobase = (const uint16_t *)p.dout + b * p.do_b + h * p.do_h + qcol;
@@ -191,7 +194,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
     }
 
     for (int step = 0; step < n_steps; step++) {
-        const int gi = step / n_m, mi = m_start + step % n_m;
+        const int gi = step / n_m, mi = M_blocks - 1 - step % n_m;  // last query block first: see below
         const int h = hk * G + gi;
         const int m0 = mi * KV_BM;
         const int buf = step & 1;
