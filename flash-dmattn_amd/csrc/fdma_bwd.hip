@@ -64,36 +64,41 @@ __global__ void __launch_bounds__(256) bwd_dot_kernel(const BwdParams p) {
 }
 
 // ------------------------------------------------------------------------------------------------
-// 2. dK / dV / dBias
+// 2. dK / dV / dBias with a per-query mask and / or bias
 // ------------------------------------------------------------------------------------------------
+// One workgroup = 128 keys (32 per wave) of one (batch, kv head); K and V stay in registers as MFMA B
+// operands.  Per step (64 query rows of one query head) the workgroup stages Q, dO, LSE, D and a FUSED
+// bias tile through LDS: fused[q][k] = bias[q][k] where (mask[q][k] and k < Lk), else -inf, built from
+// coalesced 16-byte bias / 8-byte mask loads (broadcast dims simply have stride 0).  exp2(-inf) = 0 does
+// the masking.  dS goes back through an LDS tile so that dBias is written with coalesced 16-byte stores
+// at the bias's own shape; over the query heads of a group it is summed in registers first.
 constexpr int KV_BM = 64;   // query rows per step
 constexpr int KV_BN = 128;  // key columns per workgroup (32 per wave)
 
 template <int D> struct KvSmem {
-    static constexpr int S = D + 8;  // row stride (elements) of every tile
-    static constexpr int K_BYTES = KV_BN * S * 2;
+    static constexpr int S = D + 8;          // Q / dO row stride (elements)
+    static constexpr int SB = KV_BN + 8;     // fused-bias / dS tile row stride (elements)
     static constexpr int Q_BYTES = KV_BM * S * 2;
-    static constexpr int STAT_BYTES = KV_BM * 4;
-    static constexpr int OFF_K = 0;
-    static constexpr int OFF_V = OFF_K + K_BYTES;
-    static constexpr int OFF_Q = OFF_V + K_BYTES;
-    static constexpr int OFF_DO = OFF_Q + Q_BYTES;
-    static constexpr int OFF_LSE = OFF_DO + Q_BYTES;
-    static constexpr int OFF_DD = OFF_LSE + STAT_BYTES;
-    static constexpr int TOTAL = OFF_DD + STAT_BYTES;
+    static constexpr int FB_BYTES = KV_BM * SB * 2;
+    static constexpr int STAGE = 2 * Q_BYTES + 2 * KV_BM * 4 + FB_BYTES;  // Q, dO, LSE, D, fused bias
+    static constexpr int OFF_DS = 2 * STAGE;
+    static constexpr int TOTAL = OFF_DS + FB_BYTES;
 };
 
+template <typename T> struct NegInfPair;
+template <> struct NegInfPair<bf16_tag> { static constexpr uint32_t value = 0xFF80FF80u; };
+template <> struct NegInfPair<fp16_tag> { static constexpr uint32_t value = 0xFC00FC00u; };
+
 template <typename T, int D, bool CAUSAL>
-__global__ void __launch_bounds__(NTHREADS) bwd_dkdv_kernel(const BwdParams p) {
+__global__ void __launch_bounds__(NTHREADS, 1) bwd_dkdv_kernel(const BwdParams p) {
     using E = Elem<T>;
     using SM = KvSmem<D>;
     constexpr int KS = D / 16;
     constexpr int DB = D / 32;
     constexpr int MB = KV_BM / 32;
+    constexpr int CH = D / 8, RPP = NTHREADS / CH, Q_IT = KV_BM / RPP;
 
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    char *sK = smem + SM::OFF_K, *sV = smem + SM::OFF_V, *sQ = smem + SM::OFF_Q, *sDO = smem + SM::OFF_DO;
-    float *sLSE = (float *)(smem + SM::OFF_LSE), *sDD = (float *)(smem + SM::OFF_DD);
 
     const FwdParams &f = p.f;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 31, g = lane >> 5;
@@ -101,24 +106,21 @@ __global__ void __launch_bounds__(NTHREADS) bwd_dkdv_kernel(const BwdParams p) {
     const int G = f.H / f.Hk;
     const int n0 = n_block * KV_BN;
     const int key = n0 + wave * 32 + r;  // the key column this lane owns
+    const int key_c = key < f.Lk ? key : f.Lk - 1;
     const int shift = f.Lk - f.Lq;
 
-    // ---- stage K and V (rows beyond Lk zero-filled)
+    // ---- stationary K / V fragments (B operands)
+    u32x4_t kf[KS], vf[KS];
     {
-        constexpr int CH = D / 8, RPP = NTHREADS / CH;
-        const int c = tid % CH, r0 = tid / CH;
-        const uint16_t *kbase = (const uint16_t *)f.k + b * f.k_b + hk * f.k_h;
-        const uint16_t *vbase = (const uint16_t *)f.v + b * f.v_b + hk * f.v_h;
+        const uint16_t *kp = (const uint16_t *)f.k + b * f.k_b + (int64_t)key_c * f.k_r + hk * f.k_h;
+        const uint16_t *vp = (const uint16_t *)f.v + b * f.v_b + (int64_t)key_c * f.v_r + hk * f.v_h;
 #pragma unroll
-        for (int it = 0; it < KV_BN / RPP; it++) {
-            int row = r0 + it * RPP, kk = n0 + row;
+        for (int ks = 0; ks < KS; ks++) {
+            const int c = ks * 16 + g * 8;
             u32x4_t kv = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
-            if (kk < f.Lk && c * 8 < f.d) {
-                kv = *(const u32x4_t *)(kbase + (int64_t)kk * f.k_r + c * 8);
-                vv = *(const u32x4_t *)(vbase + (int64_t)kk * f.v_r + c * 8);
-            }
-            *(u32x4_t *)(sK + (row * SM::S + c * 8) * 2) = kv;
-            *(u32x4_t *)(sV + (row * SM::S + c * 8) * 2) = vv;
+            if (c < f.d) { kv = *(const u32x4_t *)(kp + c); vv = *(const u32x4_t *)(vp + c); }
+            kf[ks] = kv;
+            vf[ks] = vv;
         }
     }
 
@@ -131,44 +133,127 @@ __global__ void __launch_bounds__(NTHREADS) bwd_dkdv_kernel(const BwdParams p) {
     const int M_blocks = (f.Lq + KV_BM - 1) / KV_BM;
     int m_start = 0;
     if (CAUSAL) {
-        int first_q = n0 - shift;  // first query row that sees key n0
+        const int first_q = n0 - shift;  // first query row that sees key n0
         if (first_q > 0) m_start = first_q / KV_BM;
         if (m_start > M_blocks) m_start = M_blocks;
     }
 
     const bool has_bias = f.bias != nullptr;
     const bool bias_rows = has_bias && f.bi_r != 0;   // per-query bias (and dbias) rows
-    const bool mask_rows = f.mask != nullptr && f.m_r != 0;
     const bool use_accum = p.dbias_accum != nullptr;   // several workgroups share a dbias element
     // loop order: per-query dbias wants (m outer, g inner) to sum dS over the group in registers;
-    // row-broadcast dbias wants (g outer, m inner) to keep one column sum per bias head.
+    // row-broadcast dbias wants (g outer, m inner) to keep one column sum per bias head.  Query blocks
+    // are walked from the last one down so that neighbouring workgroups stream the same tiles together.
     const bool m_outer = bias_rows;
     const int n_m = M_blocks - m_start;
     const int n_steps = n_m * G;
 
-    // zero the part of a per-query dbias this workgroup owns but never visits (above the causal
-    // diagonal); visited tiles are written below.
+    // zero the part of a per-query dbias this workgroup owns but never visits (above the causal diagonal)
     if (bias_rows && !use_accum && m_start > 0) {
         const int ngh = (f.Hb == f.H) ? G : 1;
         for (int gh = 0; gh < ngh; gh++) {
             const int hb = f.Hb == f.H ? hk * G + gh : (f.Hb == 1 ? 0 : hk);
             uint16_t *dbp = (uint16_t *)p.dbias + b * p.db_b + hb * p.db_h;
             const int rows = m_start * KV_BM < f.Lq ? m_start * KV_BM : f.Lq;
-            // 16 chunks of 8 keys per row
             for (int idx = tid; idx < rows * 16; idx += NTHREADS) {
-                int row = idx >> 4, c = idx & 15;
-                int kk = n0 + c * 8;
+                const int row = idx >> 4, c = idx & 15;
+                const int kk = n0 + c * 8;
                 if (kk < f.Lk) *(u32x4_t *)(dbp + (int64_t)row * p.db_r + kk) = u32x4_t{0, 0, 0, 0};
             }
         }
     }
 
-    // per-lane constants for row-broadcast mask / bias
+    // ---- staging for one step (global -> registers -> LDS)
+    const int qc = tid % CH, qr0 = tid / CH;
+    const int qcol = (qc * 8 < f.d) ? qc * 8 : 0;
+    const int bc = tid & 15, br0 = tid >> 4;  // fused-bias tile: 8-key chunk and first row of this thread
+    u32x4_t qreg[Q_IT], doreg[Q_IT], fbreg[4];
+    float lreg = INFINITY, dreg = 0.f;
+    auto step_head = [&](int step, int &gi, int &mi) {
+        gi = m_outer ? step % G : step / n_m;
+        mi = M_blocks - 1 - (m_outer ? step / G : step % n_m);
+    };
+    auto load_step = [&](int step) {
+        int gi, mi;
+        step_head(step, gi, mi);
+        const int h = hk * G + gi, m0 = mi * KV_BM;
+        const uint16_t *qbase = (const uint16_t *)f.q + b * f.q_b + h * f.q_h + qcol;
+        const uint16_t *dobase = (const uint16_t *)p.dout + b * p.do_b + h * p.do_h + qcol;
+#pragma unroll
+        for (int it = 0; it < Q_IT; it++) {
+            int qq = m0 + qr0 + it * RPP;
+            qq = qq < f.Lq ? qq : f.Lq - 1;
+            qreg[it] = *(const u32x4_t *)(qbase + (int64_t)qq * f.q_r);
+            doreg[it] = *(const u32x4_t *)(dobase + (int64_t)qq * p.do_r);
+        }
+        if (tid < KV_BM) {
+            const int qq = m0 + tid;
+            lreg = INFINITY;
+            dreg = 0.f;
+            if (qq < f.Lq) {
+                lreg = f.lse[((int64_t)b * f.H + h) * f.Lq + qq] * kLog2e;
+                dreg = p.softmax_d[((int64_t)b * f.H + h) * p.Lq_rounded + qq];
+            }
+        }
+        // fused bias chunks: rows br0 + 16*it, keys n0 + 8*bc .. +8
+        const int hm = f.mask ? (f.Hm == f.H ? h : (f.Hm == 1 ? 0 : hk)) : 0;
+        const int hb = has_bias ? (f.Hb == f.H ? h : (f.Hb == 1 ? 0 : hk)) : 0;
+        const int kk = n0 + 8 * bc;
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+            int qq = m0 + br0 + 16 * it;
+            qq = qq < f.Lq ? qq : f.Lq - 1;
+            u32x4_t bv = {0, 0, 0, 0};
+            u32x2_t mv = {0x01010101u, 0x01010101u};
+            if (kk < f.Lk) {
+                if (has_bias) bv = *(const u32x4_t *)((const uint16_t *)f.bias + b * f.bi_b + hb * f.bi_h + (int64_t)qq * f.bi_r + kk);
+                if (f.mask) mv = *(const u32x2_t *)(f.mask + b * f.m_b + hm * f.m_h + (int64_t)qq * f.m_r + kk);
+            } else {
+                mv = u32x2_t{0, 0};
+            }
+            if (kk + 8 > f.Lk && kk < f.Lk) {  // chunk straddles the end of the keys
+                const int nv = f.Lk - kk;       // 1..7 valid keys
+                const uint64_t keepm = (1ull << (8 * nv)) - 1ull;
+                mv[0] &= (uint32_t)keepm;
+                mv[1] &= (uint32_t)(keepm >> 32);
+            }
+#pragma unroll
+            for (int hlf = 0; hlf < 2; hlf++) {
+                uint32_t x = mv[hlf];
+                x = ((((x & 0x7f7f7f7fu) + 0x7f7f7f7fu) | x) >> 7) & 0x01010101u;  // nonzero byte -> 0x01
+                const uint32_t z = (x << 8) - x;                                      // 0x01 -> 0xFF per byte
+                const uint32_t m0w = __builtin_amdgcn_perm(0, z, 0x01010000u);        // [b0 b0 b1 b1]
+                const uint32_t m1w = __builtin_amdgcn_perm(0, z, 0x03030202u);        // [b2 b2 b3 b3]
+                bv[2 * hlf] = (bv[2 * hlf] & m0w) | (NegInfPair<T>::value & ~m0w);
+                bv[2 * hlf + 1] = (bv[2 * hlf + 1] & m1w) | (NegInfPair<T>::value & ~m1w);
+            }
+            fbreg[it] = bv;
+        }
+    };
+    auto store_step = [&](int buf) {
+        char *base = smem + buf * SM::STAGE;
+#pragma unroll
+        for (int it = 0; it < Q_IT; it++) {
+            const int off = ((qr0 + it * RPP) * SM::S + qc * 8) * 2;
+            *(u32x4_t *)(base + off) = qreg[it];
+            *(u32x4_t *)(base + SM::Q_BYTES + off) = doreg[it];
+        }
+        if (tid < KV_BM) {
+            ((float *)(base + 2 * SM::Q_BYTES))[tid] = lreg;
+            ((float *)(base + 2 * SM::Q_BYTES + KV_BM * 4))[tid] = dreg;
+        }
+        char *fb = base + 2 * SM::Q_BYTES + 2 * KV_BM * 4;
+#pragma unroll
+        for (int it = 0; it < 4; it++) *(u32x4_t *)(fb + ((br0 + 16 * it) * SM::SB + 8 * bc) * 2) = fbreg[it];
+    };
+
     const int a_row = pi_row(r);
     const int tj = lane & 15, te = tj >> 2, tc = tj & 3;
     const int tcp = (tc == 1) ? 2 : (tc == 2 ? 1 : tc);
     const int tdh = (lane >> 4) & 1;
     const uint32_t tr_off = (uint32_t)(((8 * g + te) * SM::S + 16 * tdh + 4 * tcp) * 2);
+    const uint32_t a_off = (uint32_t)((a_row * SM::S + g * 8) * 2);
+    uint16_t *sDS = (uint16_t *)(smem + SM::OFF_DS);
 
     float colsum = 0.f;       // row-broadcast dbias: sum over queries of dS for this lane's key
     f32x16_t dsum[MB];        // per-query dbias with bias heads < H: sum over the group
@@ -177,135 +262,110 @@ __global__ void __launch_bounds__(NTHREADS) bwd_dkdv_kernel(const BwdParams p) {
 #pragma unroll
         for (int i = 0; i < 16; i++) dsum[mb][i] = 0.f;
 
+    if (n_steps > 0) {
+        load_step(0);
+        store_step(0);
+        __syncthreads();
+    }
+
     for (int step = 0; step < n_steps; step++) {
-        const int gi = m_outer ? step % G : step / n_m;
-        const int mi = M_blocks - 1 - (m_outer ? step / G : step % n_m);  // last query block first (shared L2 streaming)
+        int gi, mi;
+        step_head(step, gi, mi);
         const int h = hk * G + gi;
         const int m0 = mi * KV_BM;
-        const int hm = f.mask ? (f.Hm == f.H ? h : (f.Hm == 1 ? 0 : hk)) : 0;
+        const int buf = step & 1;
         const int hb = has_bias ? (f.Hb == f.H ? h : (f.Hb == 1 ? 0 : hk)) : 0;
-        const bool first_of_group = gi == 0;
-        const bool last_of_group = gi == G - 1;
+        if (step + 1 < n_steps) load_step(step + 1);
 
-        __syncthreads();  // previous step finished reading sQ / sDO / stats (also covers the K/V staging)
-        // ---- stage Q, dO, LSE, D for (h, m-block)
-        {
-            constexpr int CH = D / 8, RPP = NTHREADS / CH;
-            const int c = tid % CH, r0 = tid / CH;
-            const uint16_t *qbase = (const uint16_t *)f.q + b * f.q_b + h * f.q_h;
-            const uint16_t *dobase = (const uint16_t *)p.dout + b * p.do_b + h * p.do_h;
+        const char *sQ = smem + buf * SM::STAGE;
+        const char *sDO = sQ + SM::Q_BYTES;
+        const float *sLSE = (const float *)(sQ + 2 * SM::Q_BYTES);
+        const float *sDD = sLSE + KV_BM;
+        const uint16_t *sFB = (const uint16_t *)(sDD + KV_BM) + wave * 32 + r;  // this lane's column
+
+        // ---- S = Q K^T and dP = dO V^T
+        f32x16_t s[MB], dp[MB];
 #pragma unroll
-            for (int it = 0; it < KV_BM / RPP; it++) {
-                int row = r0 + it * RPP, qq = m0 + row;
-                u32x4_t qv = {0, 0, 0, 0}, dov = {0, 0, 0, 0};
-                if (qq < f.Lq && c * 8 < f.d) {
-                    qv = *(const u32x4_t *)(qbase + (int64_t)qq * f.q_r + c * 8);
-                    dov = *(const u32x4_t *)(dobase + (int64_t)qq * p.do_r + c * 8);
-                }
-                *(u32x4_t *)(sQ + (row * SM::S + c * 8) * 2) = qv;
-                *(u32x4_t *)(sDO + (row * SM::S + c * 8) * 2) = dov;
-            }
-            if (tid < KV_BM) {
-                int qq = m0 + tid;
-                float l = INFINITY, dd = 0.f;
-                if (qq < f.Lq) {
-                    l = f.lse[((int64_t)b * f.H + h) * f.Lq + qq] * kLog2e;
-                    dd = p.softmax_d[((int64_t)b * f.H + h) * p.Lq_rounded + qq];
-                }
-                sLSE[tid] = l;
-                sDD[tid] = dd;
+        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) { s[mb][i] = 0.f; dp[mb][i] = 0.f; }
+        {
+            constexpr int NF = 2 * MB * KS, FR = 8;
+            u32x4_t a[NF];
+            auto frag = [&](int fi) {
+                const int which = fi & 1, mb = (fi >> 1) % MB, ks = (fi >> 1) / MB;
+                return *(const u32x4_t *)((which ? sDO : sQ) + a_off + (32 * mb * SM::S + ks * 16) * 2);
+            };
+#pragma unroll
+            for (int fi = 0; fi < FR; fi++) a[fi] = frag(fi);
+#pragma unroll
+            for (int fi = 0; fi < NF; fi++) {
+                if (fi + FR < NF) a[fi + FR] = frag(fi + FR);
+                const int which = fi & 1, mb = (fi >> 1) % MB, ks = (fi >> 1) / MB;
+                if (which) dp[mb] = E::mfma(a[fi], vf[ks], dp[mb]);
+                else s[mb] = E::mfma(a[fi], kf[ks], s[mb]);
             }
         }
 
-        // ---- keep bits: bit 16*mb + i  <->  query m0 + 32mb + 16(i/8) + 8g + i%8, this lane's key
-        uint32_t keep = 0;
-        {
-            const uint8_t *mp = f.mask ? f.mask + b * f.m_b + hm * f.m_h + key : nullptr;
-#pragma unroll
-            for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) {
-                    int qq = m0 + 32 * mb + 16 * (i >> 3) + 8 * g + (i & 7);
-                    bool vis = key < f.Lk && qq < f.Lq;
-                    if (CAUSAL) vis = vis && key <= qq + shift;
-                    if (vis && mp) vis = mp[(int64_t)(mask_rows ? qq : 0) * f.m_r] != 0;
-                    keep |= (vis ? 1u : 0u) << (16 * mb + i);
-                }
-        }
-        __syncthreads();
-
+        // ---- P = exp2((S*scale + fused)*log2e - LSE*log2e) ; dS = P * (dP - D)
+        const bool diag = CAUSAL && (n0 + wave * 32 + 31 > m0 + shift);
+        uint32_t ppk[MB * 8], dpk[MB * 8];
         f32x16_t ds[MB];
-        if (keep != 0 || true) {
-            // ---- S = Q K^T and dP = dO V^T  (M = query, N = key)
-            f32x16_t s[MB], dp[MB];
 #pragma unroll
-            for (int mb = 0; mb < MB; mb++) {
+        for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-                for (int i = 0; i < 16; i++) { s[mb][i] = 0.f; dp[mb][i] = 0.f; }
-            }
+            for (int blk = 0; blk < 2; blk++) {
+                const int q0l = 32 * mb + 16 * blk + 8 * g;  // first local query row of these 8 registers
+                const f32x4_t l0 = *(const f32x4_t *)(sLSE + q0l), l1 = *(const f32x4_t *)(sLSE + q0l + 4);
+                const f32x4_t d0 = *(const f32x4_t *)(sDD + q0l), d1 = *(const f32x4_t *)(sDD + q0l + 4);
+                float pv[8], dsv[8];
 #pragma unroll
-            for (int ks = 0; ks < KS; ks++) {
-                u32x4_t kb = *(const u32x4_t *)(sK + ((32 * wave + r) * SM::S + ks * 16 + g * 8) * 2);
-                u32x4_t vb = *(const u32x4_t *)(sV + ((32 * wave + r) * SM::S + ks * 16 + g * 8) * 2);
+                for (int e = 0; e < 8; e++) {
+                    const int ii = 8 * blk + e;
+                    const float lse2 = e < 4 ? l0[e] : l1[e - 4];
+                    const float dd = e < 4 ? d0[e] : d1[e - 4];
+                    const float fb = E::lo((uint32_t)sFB[(q0l + e) * SM::SB]);
+                    const float x = fmaf(fmaf(s[mb][ii], f.scale, fb), kLog2e, -lse2);
+                    pv[e] = fast_exp2(x);
+                    dsv[e] = dp[mb][ii] - dd;
+                }
+                if (diag) {
+                    asm volatile("" ::: "memory");
+                    const int lim = key - shift - m0 - q0l;  // rows e >= lim see this key
 #pragma unroll
-                for (int mb = 0; mb < MB; mb++) {
-                    u32x4_t qa = *(const u32x4_t *)(sQ + ((32 * mb + a_row) * SM::S + ks * 16 + g * 8) * 2);
-                    u32x4_t da = *(const u32x4_t *)(sDO + ((32 * mb + a_row) * SM::S + ks * 16 + g * 8) * 2);
-                    s[mb] = E::mfma(qa, kb, s[mb]);
-                    dp[mb] = E::mfma(da, vb, dp[mb]);
+                    for (int e = 0; e < 8; e++) pv[e] = e >= lim ? pv[e] : 0.f;
+                }
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    dsv[e] *= pv[e];
+                    ds[mb][8 * blk + e] = dsv[e];
+                }
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    ppk[mb * 8 + blk * 4 + e] = E::pack2(pv[2 * e], pv[2 * e + 1]);
+                    dpk[mb * 8 + blk * 4 + e] = E::pack2(dsv[2 * e], dsv[2 * e + 1]);
                 }
             }
-            // ---- P and dS
-            uint32_t ppk[MB * 8], dpk[MB * 8];
+
+        // ---- dV^T += dO^T P ; dK^T += Q^T dS
 #pragma unroll
-            for (int mb = 0; mb < MB; mb++) {
+        for (int qb = 0; qb < KV_BM / 16; qb++) {
+            const u32x4_t pb = {ppk[4 * qb], ppk[4 * qb + 1], ppk[4 * qb + 2], ppk[4 * qb + 3]};
+            const u32x4_t sb = {dpk[4 * qb], dpk[4 * qb + 1], dpk[4 * qb + 2], dpk[4 * qb + 3]};
 #pragma unroll
-                for (int i = 0; i < 16; i += 2) {
-                    float pv[2], dsv[2];
-#pragma unroll
-                    for (int e = 0; e < 2; e++) {
-                        const int ii = i + e;
-                        const int ql = 32 * mb + 16 * (ii >> 3) + 8 * g + (ii & 7);
-                        float bl2 = 0.f;
-                        if (has_bias) {
-                            const uint16_t *bp = (const uint16_t *)f.bias + b * f.bi_b + hb * f.bi_h;
-                            int qq = m0 + ql;
-                            qq = qq < f.Lq ? qq : f.Lq - 1;
-                            int kk = key < f.Lk ? key : f.Lk - 1;
-                            uint32_t raw = bp[(int64_t)(bias_rows ? qq : 0) * f.bi_r + kk];
-                            bl2 = E::lo(raw) * kLog2e;
-                        }
-                        float x = fmaf(s[mb][ii], f.scale_log2, bl2) - sLSE[ql];
-                        float pe = ((keep >> (16 * mb + ii)) & 1u) ? fast_exp2(x) : 0.f;
-                        float de = pe * (dp[mb][ii] - sDD[ql]);
-                        pv[e] = pe;
-                        dsv[e] = de;
-                        ds[mb][ii] = de;
-                    }
-                    ppk[mb * 8 + i / 2] = E::pack2(pv[0], pv[1]);
-                    dpk[mb * 8 + i / 2] = E::pack2(dsv[0], dsv[1]);
-                }
-            }
-            // ---- dV^T += dO^T P ; dK^T += Q^T dS   (M = d, N = key, contraction = query)
-#pragma unroll
-            for (int qb = 0; qb < KV_BM / 16; qb++) {
-                u32x4_t pb = {ppk[4 * qb], ppk[4 * qb + 1], ppk[4 * qb + 2], ppk[4 * qb + 3]};
-                u32x4_t sb = {dpk[4 * qb], dpk[4 * qb + 1], dpk[4 * qb + 2], dpk[4 * qb + 3]};
-#pragma unroll
-                for (int db = 0; db < DB; db++) {
-                    uint32_t off = tr_off + (uint32_t)((16 * qb * SM::S + 32 * db) * 2);
-                    u32x2_t lo = lds_read_tr16(sDO, off), hi = lds_read_tr16(sDO, off + 4 * SM::S * 2);
-                    u32x4_t a = {lo[0], lo[1], hi[0], hi[1]};
-                    dv[db] = E::mfma(a, pb, dv[db]);
-                    lo = lds_read_tr16(sQ, off);
-                    hi = lds_read_tr16(sQ, off + 4 * SM::S * 2);
-                    u32x4_t a2 = {lo[0], lo[1], hi[0], hi[1]};
-                    dk[db] = E::mfma(a2, sb, dk[db]);
-                }
+            for (int db = 0; db < DB; db++) {
+                const uint32_t off = tr_off + (uint32_t)((16 * qb * SM::S + 32 * db) * 2);
+                const u32x2_t lo = lds_read_tr16(sDO, off), hi = lds_read_tr16(sDO, off + 4 * SM::S * 2);
+                const u32x2_t lo2 = lds_read_tr16(sQ, off), hi2 = lds_read_tr16(sQ, off + 4 * SM::S * 2);
+                const u32x4_t a1 = {lo[0], lo[1], hi[0], hi[1]};
+                const u32x4_t a2 = {lo2[0], lo2[1], hi2[0], hi2[1]};
+                dv[db] = E::mfma(a1, pb, dv[db]);
+                dk[db] = E::mfma(a2, sb, dk[db]);
             }
         }
 
         // ---- dBias
+        bool tile_out = false;  // this step leaves a dS tile in LDS to be stored (uniform)
         if (has_bias) {
             if (!bias_rows) {
                 float part = 0.f;
@@ -314,16 +374,12 @@ __global__ void __launch_bounds__(NTHREADS) bwd_dkdv_kernel(const BwdParams p) {
 #pragma unroll
                     for (int i = 0; i < 16; i++) part += ds[mb][i];
                 colsum += part;
-                // flush when the bias head changes (g outer, m inner)
                 const bool last_m = (step % n_m) == n_m - 1;
-                const bool flush = last_m && (f.Hb == f.H || last_of_group);
-                if (flush) {
-                    float tot = xhalf_sum(colsum);
+                if (last_m && (f.Hb == f.H || gi == G - 1)) {
+                    const float tot = xhalf_sum(colsum);
                     if (g == 0 && key < f.Lk) {
-                        if (use_accum)
-                            atomicAdd(p.dbias_accum + b * p.dba_b + hb * p.dba_h + key, tot);
-                        else
-                            ((uint16_t *)p.dbias)[b * p.db_b + hb * p.db_h + key] = (uint16_t)(E::pack2(tot, 0.f) & 0xffffu);
+                        if (use_accum) atomicAdd(p.dbias_accum + b * p.dba_b + hb * p.dba_h + key, tot);
+                        else ((uint16_t *)p.dbias)[b * p.db_b + hb * p.db_h + key] = (uint16_t)(E::pack2(tot, 0.f) & 0xffffu);
                     }
                     colsum = 0.f;
                 }
@@ -332,24 +388,43 @@ __global__ void __launch_bounds__(NTHREADS) bwd_dkdv_kernel(const BwdParams p) {
 #pragma unroll
                 for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-                    for (int i = 0; i < 16; i++) dsum[mb][i] = (per_head || first_of_group) ? ds[mb][i] : dsum[mb][i] + ds[mb][i];
-                if (per_head || last_of_group) {
+                    for (int i = 0; i < 16; i++) dsum[mb][i] = (per_head || gi == 0) ? ds[mb][i] : dsum[mb][i] + ds[mb][i];
+                if (per_head || gi == G - 1) {
+                    if (use_accum) {
 #pragma unroll
-                    for (int mb = 0; mb < MB; mb++)
+                        for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-                        for (int i = 0; i < 16; i++) {
-                            int qq = m0 + 32 * mb + 16 * (i >> 3) + 8 * g + (i & 7);
-                            if (qq < f.Lq && key < f.Lk) {
-                                if (use_accum)
+                            for (int i = 0; i < 16; i++) {
+                                const int qq = m0 + 32 * mb + 16 * (i >> 3) + 8 * g + (i & 7);
+                                if (qq < f.Lq && key < f.Lk)
                                     atomicAdd(p.dbias_accum + b * p.dba_b + hb * p.dba_h + (int64_t)qq * p.dba_r + key, dsum[mb][i]);
-                                else
-                                    ((uint16_t *)p.dbias)[b * p.db_b + hb * p.db_h + (int64_t)qq * p.db_r + key] =
-                                        (uint16_t)(E::pack2(dsum[mb][i], 0.f) & 0xffffu);
                             }
-                        }
+                    } else {
+                        tile_out = true;
+#pragma unroll
+                        for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+                            for (int i = 0; i < 16; i++) {
+                                const int ql = 32 * mb + 16 * (i >> 3) + 8 * g + (i & 7);
+                                sDS[ql * SM::SB + wave * 32 + r] = (uint16_t)(E::pack2(dsum[mb][i], 0.f) & 0xffffu);
+                            }
+                    }
                 }
             }
         }
+        if (tile_out) __syncthreads();  // the dS tile is complete
+        if (step + 1 < n_steps) store_step(buf ^ 1);
+        if (tile_out) {
+            uint16_t *dbp = (uint16_t *)p.dbias + b * p.db_b + hb * p.db_h;
+            const int kk = n0 + 8 * bc;
+#pragma unroll
+            for (int it = 0; it < 4; it++) {
+                const int ql = br0 + 16 * it, qq = m0 + ql;
+                if (qq < f.Lq && kk < f.Lk)
+                    *(u32x4_t *)(dbp + (int64_t)qq * p.db_r + kk) = *(const u32x4_t *)(sDS + ql * SM::SB + 8 * bc);
+            }
+        }
+        __syncthreads();
     }
 
     // a key block that no query can see still owns its dbias column (row-broadcast case)
@@ -361,7 +436,7 @@ __global__ void __launch_bounds__(NTHREADS) bwd_dkdv_kernel(const BwdParams p) {
         }
     }
 
-    // ---- store dK (scaled) and dV: lane owns one key row, 8 consecutive head-dim elements per store
+    // ---- store dK (scaled) and dV
     if (key < f.Lk) {
         uint16_t *dkp = (uint16_t *)p.dk + b * p.dk_b + (int64_t)key * p.dk_r + hk * p.dk_h;
         uint16_t *dvp = (uint16_t *)p.dv + b * p.dv_b + (int64_t)key * p.dv_r + hk * p.dv_h;
@@ -369,7 +444,7 @@ __global__ void __launch_bounds__(NTHREADS) bwd_dkdv_kernel(const BwdParams p) {
         for (int db = 0; db < DB; db++)
 #pragma unroll
             for (int blk = 0; blk < 2; blk++) {
-                int c = 32 * db + 16 * blk + 8 * g;
+                const int c = 32 * db + 16 * blk + 8 * g;
                 if (c < f.d) {
                     u32x4_t wk, wv;
 #pragma unroll
