@@ -7,6 +7,7 @@ CPU or eager fallback behind it.
 """
 import ctypes
 import os
+import struct
 from typing import Optional, Sequence
 
 import torch
@@ -129,25 +130,32 @@ def _bcast3(t: torch.Tensor) -> Sequence[int]:
     return tuple(0 if t.size(i) == 1 else t.stride(i) for i in range(3))
 
 
+_FWD_STRUCT = struct.Struct("@7P18q10i2fPN")
+assert _FWD_STRUCT.size == ctypes.sizeof(FwdArgs)
+
+
 def fill_fwd(a: FwdArgs, q, k, v, mask, bias, out, lse, softmax_scale, is_causal, softcap) -> None:
-    a.q, a.k, a.v = _ptr(q), _ptr(k), _ptr(v)
-    a.mask, a.bias = _ptr(mask), _ptr(bias)
-    a.out, a.lse = _ptr(out), _ptr(lse)
-    a.q_strides[:] = _s3(q)
-    a.k_strides[:] = _s3(k)
-    a.v_strides[:] = _s3(v)
-    a.o_strides[:] = _s3(out)
-    a.mask_strides[:] = _bcast3(mask) if mask is not None else (0, 0, 0)
-    a.bias_strides[:] = _bcast3(bias) if bias is not None else (0, 0, 0)
-    a.batch, a.seqlen_q, a.num_heads, a.head_dim = q.shape
-    a.seqlen_k, a.num_heads_k = k.shape[1], k.shape[2]
-    a.num_heads_mask = mask.shape[1] if mask is not None else 1
-    a.num_heads_bias = bias.shape[1] if bias is not None else 1
-    a.dtype = dtype_code(q)
-    a.is_causal = int(bool(is_causal))
-    a.softmax_scale = float(softmax_scale)
-    a.softcap = float(softcap)
-    a.workspace, a.workspace_bytes = None, 0
+    """Fill the argument block in one struct.pack (ctypes field-by-field assignment costs ~10 us a call)."""
+    ms = _bcast3(mask) if mask is not None else (0, 0, 0)
+    bs = _bcast3(bias) if bias is not None else (0, 0, 0)
+    batch, seqlen_q, num_heads, head_dim = q.shape
+    _FWD_STRUCT.pack_into(
+        _as_buffer(a), 0,
+        q.data_ptr(), k.data_ptr(), v.data_ptr(),
+        mask.data_ptr() if mask is not None else 0, bias.data_ptr() if bias is not None else 0,
+        out.data_ptr(), lse.data_ptr(),
+        q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
+        v.stride(0), v.stride(1), v.stride(2), out.stride(0), out.stride(1), out.stride(2),
+        ms[0], ms[1], ms[2], bs[0], bs[1], bs[2],
+        batch, seqlen_q, k.shape[1], num_heads, k.shape[2],
+        mask.shape[1] if mask is not None else 1, bias.shape[1] if bias is not None else 1,
+        head_dim, dtype_code(q), int(bool(is_causal)),
+        float(softmax_scale), float(softcap), 0, 0,
+    )
+
+
+def _as_buffer(a):
+    return (ctypes.c_char * ctypes.sizeof(a)).from_address(ctypes.addressof(a))
 
 
 def current_stream(device: torch.device) -> int:

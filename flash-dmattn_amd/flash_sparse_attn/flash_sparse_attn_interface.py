@@ -35,6 +35,8 @@ def _aligned(x: Optional[torch.Tensor], elems: int) -> Optional[torch.Tensor]:
     16-byte aligned, every other stride a multiple of `elems` elements."""
     if x is None:
         return None
+    if x.is_contiguous() and x.shape[-1] % elems == 0 and x.data_ptr() % 16 == 0:
+        return x  # fast path: every stride of a contiguous tensor is a multiple of its last dim
     x = maybe_contiguous(x)
     ok = x.data_ptr() % 16 == 0 and all(x.size(i) == 1 or x.stride(i) % elems == 0 for i in range(x.dim() - 1))
     return x if ok else x.contiguous().clone(memory_format=torch.contiguous_format)
