@@ -113,6 +113,31 @@ def count_tiles(mask, Lq, Lk, causal, H, tile=64):
     return executed, int(causal_tile.sum().item()) * H * Bfull, nnz
 
 
+def compaction_applies(mask, c):
+    """Mirror of the library's rule for taking the column-compaction path (query-broadcast keep-mask with
+    1 or Hkv heads, at least 128 queries and keys, not switched off)."""
+    return (mask.shape[2] == 1 and mask.shape[1] in (1, c["Hk"]) and c["Lq"] >= 128 and c["Lk"] >= 128
+            and os.environ.get("FDMA_COMPACT", "1")[:1] != "0")
+
+
+def count_compacted_tiles(mask, Lq, Lk, causal, H, tile=64):
+    """64x64 tiles the compacted kernels execute: per (batch, mask head) the kept columns are packed to the
+    front, and a 64-row query block runs over ceil(visible / 64) tiles, visible = kept columns at or below
+    the causal limit of the block's last row.  Summed over batch and query heads."""
+    Bm, Hm, _, _ = mask.shape
+    dev = mask.device
+    m = mask[:, :, 0, :Lk]
+    csum = torch.cumsum(m.to(torch.int64), -1)
+    nq = (Lq + tile - 1) // tile
+    if causal:
+        last_row = torch.clamp(torch.arange(nq, device=dev) * tile + tile - 1, max=Lq - 1)
+        lim = last_row + (Lk - Lq)
+        vis = torch.where(lim >= 0, csum[..., torch.clamp(lim, 0, Lk - 1)], torch.zeros((), dtype=torch.int64, device=dev))
+    else:
+        vis = csum[..., -1:].expand(Bm, Hm, nq)
+    return int(((vis + tile - 1) // tile).sum().item()) * (H // Hm)
+
+
 def time_gpu(fn, steps, warmup):
     for _ in range(warmup):
         fn()
@@ -140,6 +165,14 @@ def run_config(name, steps, warmup, device):
     if c["Lq"] > 1:
         n_exec, n_causal, nnz = count_tiles(mask, c["Lq"], c["Lk"], c["causal"], c["H"])
         res.update(n_exec=n_exec, tile_occupancy=n_exec / max(1, n_causal), nnz=nnz)
+        res["compacted"] = compaction_applies(mask, c)
+        if res["compacted"]:
+            # the kernels run on the compacted key axis: their executed tiles are counted there; the tile
+            # count of the original layout (what a tile-skipping kernel would execute) is kept beside it
+            res["n_exec_original_layout"] = n_exec
+            res["tflops_fwd_original_layout_tiles"] = 4.0 * 64 * 64 * c["D"] * n_exec / ms_fwd / 1e9
+            n_exec = count_compacted_tiles(mask, c["Lq"], c["Lk"], c["causal"], c["H"])
+            res["n_exec"] = n_exec
         fl_fwd = 4.0 * 64 * 64 * c["D"] * n_exec
         res["tflops_fwd"] = fl_fwd / ms_fwd / 1e9
         res["tflops_fwd_elementwise"] = 4.0 * c["D"] * nnz / ms_fwd / 1e9
@@ -201,6 +234,8 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--all", action="store_true", help="also time configurations 1, 3, 4, 5")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-compact", action="store_true",
+                    help="switch the column-compaction path off (FDMA_COMPACT=0): time the tile-skipping kernels")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--traffic-bytes", type=float, default=None,
@@ -214,6 +249,8 @@ def main():
         sys.exit(1)
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
+    if args.no_compact:
+        os.environ["FDMA_COMPACT"] = "0"  # read once by the library, which is loaded on first use below
 
     main_res = run_config("cfg2", args.steps, args.warmup, device)
     c = CONFIGS["cfg2"]

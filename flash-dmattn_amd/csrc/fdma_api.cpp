@@ -119,7 +119,11 @@ int fdma_fwd_validate(const fdma_fwd_args *a) {
 
 size_t fdma_fwd_workspace_bytes(const fdma_fwd_args *a) {
     if (!a) return 0;
-    if (!fdma::use_decode_path(a->seqlen_q, a->num_heads, a->num_heads_k)) return 0;
+    if (!fdma::use_decode_path(a->seqlen_q, a->num_heads, a->num_heads_k)) {
+        fdma::FwdParams p;
+        fill_fwd_params(a, p);
+        return fdma::use_compact(p) ? fdma::compact_bytes(p) : 0;
+    }
     const int splits = fdma::decode_num_splits(a->batch, a->num_heads_k, a->seqlen_k);
     if (splits <= 1) return 0;
     const size_t rows = (size_t)splits * a->batch * a->num_heads * a->seqlen_q;
@@ -148,6 +152,13 @@ int fdma_fwd(const fdma_fwd_args *a, void *hip_stream) {
         e = fdma::launch_fwd_decode(p, a->dtype, stream);
     } else {
         // seqlen_k == 0 falls out of the kernel as O = 0, LSE = +inf (flash_api.cpp:535-539)
+        if (fdma::use_compact(p)) {
+            const size_t need = fdma::compact_bytes(p);
+            if (!a->workspace || a->workspace_bytes < need)
+                return fail(FDMA_ERR_WORKSPACE, "forward workspace too small: need %zu bytes, got %zu", need, a->workspace_bytes);
+            if ((e = fdma::compact_setup(p, a->workspace, a->dtype, stream)) != hipSuccess)
+                return fail(FDMA_ERR_LAUNCH, "forward launch failed: %s", hipGetErrorString(e));
+        }
         e = fdma::launch_fwd(p, a->dtype, stream);
     }
     if (e != hipSuccess) return fail(FDMA_ERR_LAUNCH, "forward launch failed: %s", hipGetErrorString(e));
@@ -191,9 +202,15 @@ static size_t dbias_accum_elems(const fdma_bwd_args *a) {
     return nb * a->f.num_heads_bias * nr * (size_t)round_up(a->f.seqlen_k, 8);
 }
 
+static size_t dbias_accum_bytes(const fdma_bwd_args *a) {
+    return dbias_shared(a) ? (size_t)round_up(dbias_accum_elems(a) * sizeof(float), 256) : 0;
+}
+
 size_t fdma_bwd_workspace_bytes(const fdma_bwd_args *a) {
     if (!a) return 0;
-    return dbias_shared(a) ? dbias_accum_elems(a) * sizeof(float) : 0;
+    fdma::FwdParams p;
+    fill_fwd_params(&a->f, p);
+    return dbias_accum_bytes(a) + (fdma::use_compact(p) ? fdma::compact_bytes(p) : 0);
 }
 
 int fdma_bwd(const fdma_bwd_args *a, void *hip_stream) {
@@ -210,10 +227,10 @@ int fdma_bwd(const fdma_bwd_args *a, void *hip_stream) {
     if (a->dbias) { p.db_b = a->dbias_strides[0]; p.db_h = a->dbias_strides[1]; p.db_r = a->dbias_strides[2]; }
     p.softmax_d = a->softmax_d;
     p.Lq_rounded = (int32_t)round_up(a->f.seqlen_q, 128);
+    const size_t need = fdma_bwd_workspace_bytes(a);
+    if (need && (!a->workspace || a->workspace_bytes < need))
+        return fail(FDMA_ERR_WORKSPACE, "backward workspace too small: need %zu bytes, got %zu", need, a->workspace_bytes);
     if (dbias_shared(a)) {
-        const size_t need = fdma_bwd_workspace_bytes(a);
-        if (!a->workspace || a->workspace_bytes < need)
-            return fail(FDMA_ERR_WORKSPACE, "backward workspace too small: need %zu bytes, got %zu", need, a->workspace_bytes);
         p.dbias_accum = static_cast<float *>(a->workspace);
         const int64_t lkr = round_up(a->f.seqlen_k, 8);
         const int64_t nr = a->f.bias_strides[2] == 0 ? 1 : a->f.seqlen_q;
@@ -221,7 +238,15 @@ int fdma_bwd(const fdma_bwd_args *a, void *hip_stream) {
         p.dba_h = nr * lkr;
         p.dba_b = a->f.bias_strides[0] == 0 ? 0 : p.dba_h * a->f.num_heads_bias;
     }
-    hipError_t e = fdma::launch_bwd(p, a->f.dtype, static_cast<hipStream_t>(hip_stream));
+    hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    hipError_t e;
+    if (a->f.seqlen_q > 0 && fdma::use_compact(p.f)) {
+        const fdma::FwdParams orig = p.f;
+        e = fdma::compact_setup(p.f, static_cast<char *>(a->workspace) + dbias_accum_bytes(a), a->f.dtype, stream);
+        if (e == hipSuccess) e = fdma::compact_zero_dropped(p, orig, stream);
+        if (e != hipSuccess) return fail(FDMA_ERR_LAUNCH, "backward launch failed: %s", hipGetErrorString(e));
+    }
+    e = fdma::launch_bwd(p, a->f.dtype, stream);
     if (e != hipSuccess) return fail(FDMA_ERR_LAUNCH, "backward launch failed: %s", hipGetErrorString(e));
     return FDMA_OK;
 }

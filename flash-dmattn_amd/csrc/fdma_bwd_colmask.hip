@@ -61,7 +61,9 @@ template <int D> struct KvcSmem {
     static constexpr int TOTAL = 2 * STAGE;
 };
 
-template <typename T, int D, bool CAUSAL>
+// CMP: the key axis is the compacted list of kept columns (fdma_compact.hip); a lane still owns one key,
+// reads it from the dense copies, and writes its gradients to the key's original row / column.
+template <typename T, int D, bool CAUSAL, bool CMP>
 __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_kernel(const BwdParams p) {
     using E = Elem<T>;
     using SM = KvcSmem<D>;
@@ -81,9 +83,16 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
     const int n_block = wm.unit;  // low key blocks are seen by the most queries under causal: heaviest first
     const int b = wm.pair / f.Hk, hk = wm.pair % f.Hk;
     const int n0 = n_block * KV_BN;
+    const int Lk = CMP ? f.cmp.count[wm.pair] : f.Lk;  // key columns on this pair's (possibly compacted) key axis
+    if (CMP && n0 >= Lk) return;
     const int key = n0 + wave * 32 + r;  // the key column this lane owns
-    const int key_c = key < f.Lk ? key : f.Lk - 1;
+    const int key_c = key < Lk ? key : Lk - 1;
     const int shift = f.Lk - f.Lq;
+    // original column indices: of this lane's key, of the workgroup's first key and of the wave's last key
+    const int32_t *cidx = CMP ? f.cmp.idx + (int64_t)wm.pair * f.cmp.ld : nullptr;
+    const int okey = CMP ? cidx[key_c] : key;
+    const int okey_first = CMP ? cidx[n0] : n0;
+    const int okey_wlast = CMP ? cidx[n0 + wave * 32 + 31 < Lk ? n0 + wave * 32 + 31 : Lk - 1] : n0 + wave * 32 + 31;
 
     // ---- stationary K / V fragments (B operands): lane holds K[key][16ks + 8g .. +8]
     u32x4_t kf[KS], vf[KS];
@@ -109,7 +118,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
     const int M_blocks = (f.Lq + KV_BM - 1) / KV_BM;
     int m_start = 0;
     if (CAUSAL) {
-        const int first_q = n0 - shift;  // first query row that sees key n0
+        const int first_q = okey_first - shift;  // first query row that sees the workgroup's first key
         if (first_q > 0) m_start = first_q / KV_BM;
         if (m_start > M_blocks) m_start = M_blocks;
     }
@@ -124,7 +133,8 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
 
     // fused per-lane column constant for query head h: bias*log2e, or -inf when the column is dropped
     auto column_const = [&](int h) -> float {
-        if (key >= f.Lk) return -INFINITY;
+        if (key >= Lk) return -INFINITY;
+        if (CMP) return f.cmp.fb[(int64_t)(b * f.cmp.Hfb + (f.cmp.Hfb == f.H ? h : hk)) * f.cmp.ld + key];
         if (f.mask) {
             const int hm = f.Hm == f.H ? h : (f.Hm == 1 ? 0 : hk);
             if (!f.mask[b * f.m_b + hm * f.m_h + key]) return -INFINITY;
@@ -232,7 +242,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
 
         // ---- P = exp2(S*scale*log2e + c - LSE*log2e) ; dS = P * (dP - D)
         // diagonal step: some (query, key) pairs of this wave are above the causal diagonal
-        const bool diag = CAUSAL && (n0 + wave * 32 + 31 > m0 + shift);
+        const bool diag = CAUSAL && (okey_wlast > m0 + shift);
         uint32_t ppk[MB * 8], dpk[MB * 8];
         float part = 0.f;
 #pragma unroll
@@ -255,7 +265,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
                 }
                 if (diag) {
                     asm volatile("" ::: "memory");  // keep a real branch: only diagonal steps pay
-                    const int lim = key - shift - m0 - 32 * mb - 16 * blk - 8 * g;  // rows e >= lim see this key
+                    const int lim = okey - shift - m0 - 32 * mb - 16 * blk - 8 * g;  // rows e >= lim see this key
 #pragma unroll
                     for (int e = 0; e < 8; e++) pv[e] = e >= lim ? pv[e] : 0.f;
                 }
@@ -295,9 +305,9 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
             if (last_m && (f.Hb == f.H || gi == G - 1)) {
                 const float tot = xhalf_sum(colsum);
                 const int hb = f.Hb == f.H ? h : (f.Hb == 1 ? 0 : hk);
-                if (g == 0 && key < f.Lk) {
-                    if (use_accum) atomicAdd(p.dbias_accum + b * p.dba_b + hb * p.dba_h + key, tot);
-                    else ((uint16_t *)p.dbias)[b * p.db_b + hb * p.db_h + key] = (uint16_t)(E::pack2(tot, 0.f) & 0xffffu);
+                if (g == 0 && key < Lk) {
+                    if (use_accum) atomicAdd(p.dbias_accum + b * p.dba_b + hb * p.dba_h + okey, tot);
+                    else ((uint16_t *)p.dbias)[b * p.db_b + hb * p.db_h + okey] = (uint16_t)(E::pack2(tot, 0.f) & 0xffffu);
                 }
                 colsum = 0.f;
             }
@@ -308,18 +318,18 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
     }
 
     // a key block that no query can see still owns its dbias column
-    if (has_bias && n_steps == 0 && !use_accum && g == 0 && key < f.Lk) {
+    if (has_bias && n_steps == 0 && !use_accum && g == 0 && key < Lk) {
         const int ngh = (f.Hb == f.H) ? G : 1;
         for (int gh = 0; gh < ngh; gh++) {
             const int hb = f.Hb == f.H ? hk * G + gh : (f.Hb == 1 ? 0 : hk);
-            ((uint16_t *)p.dbias)[b * p.db_b + hb * p.db_h + key] = 0;
+            ((uint16_t *)p.dbias)[b * p.db_b + hb * p.db_h + okey] = 0;
         }
     }
 
     // ---- store dK (scaled) and dV
-    if (key < f.Lk) {
-        uint16_t *dkp = (uint16_t *)p.dk + b * p.dk_b + (int64_t)key * p.dk_r + hk * p.dk_h;
-        uint16_t *dvp = (uint16_t *)p.dv + b * p.dv_b + (int64_t)key * p.dv_r + hk * p.dv_h;
+    if (key < Lk) {
+        uint16_t *dkp = (uint16_t *)p.dk + b * p.dk_b + (int64_t)okey * p.dk_r + hk * p.dk_h;
+        uint16_t *dvp = (uint16_t *)p.dv + b * p.dv_b + (int64_t)okey * p.dv_r + hk * p.dv_h;
 #pragma unroll
         for (int db = 0; db < DB; db++)
 #pragma unroll
@@ -339,16 +349,20 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
     }
 }
 
-template <typename T, int D, bool CAUSAL>
-hipError_t launch_dkdv(const BwdParams &p, hipStream_t stream) {
+template <typename T, int D, bool CAUSAL, bool CMP>
+hipError_t launch_dkdv_c(const BwdParams &p, hipStream_t stream) {
     const FwdParams &f = p.f;
-    auto kern = bwd_dkdv_colmask_kernel<T, D, CAUSAL>;
+    auto kern = bwd_dkdv_colmask_kernel<T, D, CAUSAL, CMP>;
     const int smem = KvcSmem<D>::TOTAL;
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
     dim3 grid(xcd_grid(f.B * f.Hk, (f.Lk + KV_BN - 1) / KV_BN, 1));
     hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, stream, p);
     return hipGetLastError();
+}
+template <typename T, int D, bool CAUSAL>
+hipError_t launch_dkdv(const BwdParams &p, hipStream_t stream) {
+    return p.f.cmp.on ? launch_dkdv_c<T, D, CAUSAL, true>(p, stream) : launch_dkdv_c<T, D, CAUSAL, false>(p, stream);
 }
 
 
@@ -369,7 +383,7 @@ template <int D, int BN> struct DqcSmem {
     static constexpr int TOTAL = OFF_BITS + MAX_TILES / 8;
 };
 
-template <typename T, int D, int BN, bool CAUSAL>
+template <typename T, int D, int BN, bool CAUSAL, bool CMP>
 __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdParams p) {
     using E = Elem<T>;
     using SM = DqcSmem<D, BN>;
@@ -404,17 +418,30 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
     const uint16_t *kbase = (const uint16_t *)f.k + b * f.k_b + hk * f.k_h;
     const uint16_t *vbase = (const uint16_t *)f.v + b * f.v_b + hk * f.v_h;
 
-    int n_end = (f.Lk + BN - 1) / BN;
+    // key columns this workgroup iterates over (the compacted list with CMP), and how many a row may see
+    const int Lk = CMP ? f.cmp.count[wm.pair] : f.Lk;
+    const int32_t *ccnt = CMP ? f.cmp.cnt + (int64_t)wm.pair * f.cmp.ld : nullptr;
+    const float *fbrow = CMP ? f.cmp.fb + (int64_t)(b * f.cmp.Hfb + (f.cmp.Hfb == f.H ? h : hk)) * f.cmp.ld : nullptr;
+    auto visible = [&](int row) -> int {  // columns [0, visible(row)) pass the causal test for `row`
+        if (row >= f.Lq) row = f.Lq - 1;
+        const int c = row + shift;
+        if (!CMP) return c + 1;
+        if (c < 0) return 0;
+        return ccnt[c < f.Lk ? c : f.Lk - 1];
+    };
+    const int vis_lane = CAUSAL ? visible(qrow) : 0;
+    const int vis_wave = CAUSAL ? visible(m0 + wave * 32) : 0;
+
+    int n_end = (Lk + BN - 1) / BN;
     if (CAUSAL) {
-        int lim = m0 + Q_BM + shift;
-        if (lim > f.Lq + shift) lim = f.Lq + shift;
+        int lim = visible(m0 + Q_BM - 1);
         if (lim < 0) lim = 0;
         const int ne = (lim + BN - 1) / BN;
         if (ne < n_end) n_end = ne;
     }
 
     // ---- active-tile bitmap (tiles with at least one kept key)
-    for (int base = 0; base < n_end; base += NTHREADS) {
+    for (int base = 0; !CMP && base < n_end; base += NTHREADS) {
         const int j = base + tid;
         bool act = false;
         if (j < n_end) {
@@ -442,6 +469,7 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
     }
     __syncthreads();
     auto next_active = [&](int j) -> int {
+        if (CMP) return j < n_end ? j : n_end;
         while (j < n_end) {
             const uint32_t w = sBits[j >> 5] >> (j & 31);
             if (w) {
@@ -489,14 +517,16 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
 #pragma unroll
         for (int it = 0; it < K_IT; it++) {
             int key = n0 + kr0 + it * RPP;
-            key = key < f.Lk ? key : f.Lk - 1;
+            key = key < Lk ? key : Lk - 1;
             kreg[it] = *(const u32x4_t *)(kbase + (int64_t)key * f.k_r + kcol);
             vreg[it] = *(const u32x4_t *)(vbase + (int64_t)key * f.v_r + kcol);
         }
         if (tid < BN) {
             const int col = n0 + tid;
             float v = -INFINITY;
-            if (col < f.Lk && (!mrow || mrow[col])) {
+            if (CMP) {
+                if (col < Lk) v = fbrow[col];
+            } else if (col < Lk && (!mrow || mrow[col])) {
                 v = 0.f;
                 if (brow) v = E::lo((uint32_t)brow[col]) * kLog2e;
             }
@@ -561,7 +591,7 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
             }
         }
         // ---- dS^T = P^T * (dP^T - D)
-        const bool diag = CAUSAL && (n0 + BN - 1 > m0 + wave * 32 + shift);
+        const bool diag = CAUSAL && (n0 + BN > vis_wave);
         uint32_t dpk[8 * MB];
 #pragma unroll
         for (int mb = 0; mb < MB; mb++)
@@ -577,7 +607,7 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
                 }
                 if (diag) {
                     asm volatile("" ::: "memory");
-                    const int lim = qrow + shift - n0 - 32 * mb - 16 * blk - 8 * g;  // local columns e <= lim are visible
+                    const int lim = vis_lane - 1 - n0 - 32 * mb - 16 * blk - 8 * g;  // local columns e <= lim are visible
 #pragma unroll
                     for (int e = 0; e < 8; e++) pv[e] = e <= lim ? pv[e] : 0.f;
                 }
@@ -628,7 +658,7 @@ template <typename T, int D, bool CAUSAL>
 hipError_t launch_dq(const BwdParams &p, hipStream_t stream) {
     const FwdParams &f = p.f;
     constexpr int BN = D > 64 ? 32 : 64;  // at d = 128 a 64-key tile would spill registers
-    auto kern = bwd_dq_colmask_kernel<T, D, BN, CAUSAL>;
+    auto kern = p.f.cmp.on ? bwd_dq_colmask_kernel<T, D, BN, CAUSAL, true> : bwd_dq_colmask_kernel<T, D, BN, CAUSAL, false>;
     const int smem = DqcSmem<D, BN>::TOTAL;
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;

@@ -1,0 +1,248 @@
+// Column compaction pre-pass for keep-masks that are broadcast over the query dimension.
+//
+// With a mask of shape [B, {1,Hk}, 1, Lk] a key column is kept or dropped for every query of a
+// (batch, kv head) pair at once, so attention over the kept columns only is the same function as
+// masked attention over all of them (the reference shows the equivalence on the CPU in
+// benchmarks/grad_equivalence.py:55-140, and its Triton variant gathers K / V the same way,
+// flash_sparse_attn/flash_dmattn_triton.py:50-211).  Tile skipping cannot exploit such a mask when the
+// kept columns are scattered -- nearly every 64-key tile holds a kept key -- but gathering them makes
+// the work proportional to the number of kept keys:
+//   scan    one workgroup per (batch, kv head): ordered list `idx` of kept columns, inclusive prefix
+//           counts `cnt` (what a causal query row needs: how many kept columns are <= its limit), total;
+//   gather  wide grid: K / V rows of the kept columns copied into dense [B, Hk, count, d] buffers, bias
+//           gathered and pre-scaled into an fp32 vector;
+//   (backward) zero   rows of dK / dV and columns of dBias that belong to dropped keys.
+// All of this is O(Lk * d) traffic in front of O(Lq * count * d) MFMA work.
+#include <cstdlib>
+
+#include "fdma_common.h"
+#include "fdma_params.h"
+
+namespace fdma {
+
+namespace {
+
+constexpr int SCAN_THREADS = 1024;
+constexpr int SCAN_KEYS = 16;                          // mask bytes per thread per pass
+constexpr int SCAN_RANGE = SCAN_THREADS * SCAN_KEYS;   // keys per pass
+constexpr int GATHER_KEYS = 64;                        // compacted keys per gather workgroup
+
+inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
+
+struct Layout {
+    size_t off_idx, off_cnt, off_count, off_fb, off_k, off_v, total;
+    int ld, Hfb;
+};
+
+Layout layout_of(const FwdParams &p) {
+    Layout l;
+    l.ld = (p.Lk + 15) / 16 * 16;
+    l.Hfb = (p.bias && p.Hb == p.H) ? p.H : p.Hk;
+    const size_t pairs = (size_t)p.B * p.Hk;
+    size_t o = 0;
+    l.off_idx = o;   o += align256(pairs * l.ld * 4);
+    l.off_cnt = o;   o += align256(pairs * l.ld * 4);
+    l.off_count = o; o += align256(pairs * 4);
+    l.off_fb = o;    o += align256((size_t)p.B * l.Hfb * l.ld * 4);
+    l.off_k = o;     o += align256(pairs * p.Lk * p.d * 2);
+    l.off_v = o;     o += align256(pairs * p.Lk * p.d * 2);
+    l.total = o;
+    return l;
+}
+
+__global__ void __launch_bounds__(SCAN_THREADS) compact_scan_kernel(const FwdParams p, int32_t *idx, int32_t *cnt,
+                                                                     int32_t *count, int ld) {
+    __shared__ int s_wave[SCAN_THREADS / 64];
+    const int pair = blockIdx.x, b = pair / p.Hk, hk = pair % p.Hk;
+    const int hm = p.Hm == 1 ? 0 : hk;
+    const uint8_t *mrow = p.mask + b * p.m_b + hm * p.m_h;
+    int32_t *irow = idx + (size_t)pair * ld;
+    int32_t *crow = cnt + (size_t)pair * ld;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int base = 0;
+    for (int c0 = 0; c0 < p.Lk; c0 += SCAN_RANGE) {
+        const int col = c0 + tid * SCAN_KEYS;
+        uint32_t bits = 0;
+        if (col < p.Lk) {
+            const u32x4_t mv = *(const u32x4_t *)(mrow + col);
+#pragma unroll
+            for (int e = 0; e < SCAN_KEYS; e++) {
+                const uint32_t byte = (mv[e >> 2] >> (8 * (e & 3))) & 0xffu;
+                if (byte && col + e < p.Lk) bits |= 1u << e;
+            }
+        }
+        const int n = __builtin_popcount(bits);
+        int incl = n;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int t = __shfl_up(incl, off);
+            if (lane >= off) incl += t;
+        }
+        if (lane == 63) s_wave[wave] = incl;
+        __syncthreads();
+        int woff = 0, total = 0;
+#pragma unroll
+        for (int w = 0; w < SCAN_THREADS / 64; w++) {
+            const int v = s_wave[w];
+            if (w < wave) woff += v;
+            total += v;
+        }
+        if (col < p.Lk) {
+            int run = base + woff + incl - n;
+            int32_t cv[SCAN_KEYS];
+#pragma unroll
+            for (int e = 0; e < SCAN_KEYS; e++) {
+                if (bits & (1u << e)) irow[run++] = col + e;
+                cv[e] = run;
+            }
+#pragma unroll
+            for (int q = 0; q < SCAN_KEYS / 4; q++) {
+                u32x4_t w = {(uint32_t)cv[4 * q], (uint32_t)cv[4 * q + 1], (uint32_t)cv[4 * q + 2], (uint32_t)cv[4 * q + 3]};
+                *(u32x4_t *)(crow + col + 4 * q) = w;  // ld is a multiple of 16: the row has room
+            }
+        }
+        base += total;
+        __syncthreads();
+    }
+    if (tid == 0) count[pair] = base;
+}
+
+// orig: the caller's tensors.  kc / vc: dense [B*Hk, Lk, d] destinations.
+template <typename T>
+__global__ void __launch_bounds__(256) compact_gather_kernel(const FwdParams p, const int32_t *idx, const int32_t *count,
+                                                              float *fb, uint16_t *kc, uint16_t *vc, int ld, int Hfb) {
+    using E = Elem<T>;
+    const int pair = blockIdx.y, b = pair / p.Hk, hk = pair % p.Hk;
+    const int n = count[pair];
+    const int c0 = blockIdx.x * GATHER_KEYS;
+    if (c0 >= n) return;
+    __shared__ int s_src[GATHER_KEYS];
+    const int tid = threadIdx.x;
+    if (tid < GATHER_KEYS) s_src[tid] = (c0 + tid < n) ? idx[(size_t)pair * ld + c0 + tid] : -1;
+    __syncthreads();
+    const int CH = p.d / 8;
+    const uint16_t *kb = (const uint16_t *)p.k + b * p.k_b + hk * p.k_h;
+    const uint16_t *vb = (const uint16_t *)p.v + b * p.v_b + hk * p.v_h;
+    uint16_t *kd = kc + ((size_t)pair * p.Lk + c0) * p.d;
+    uint16_t *vd = vc + ((size_t)pair * p.Lk + c0) * p.d;
+    for (int it = tid; it < GATHER_KEYS * CH; it += 256) {
+        const int rr = it / CH, ch = it - rr * CH;
+        const int src = s_src[rr];
+        if (src >= 0) {
+            const u32x4_t kv = *(const u32x4_t *)(kb + (int64_t)src * p.k_r + ch * 8);
+            const u32x4_t vv = *(const u32x4_t *)(vb + (int64_t)src * p.v_r + ch * 8);
+            *(u32x4_t *)(kd + (size_t)rr * p.d + ch * 8) = kv;
+            *(u32x4_t *)(vd + (size_t)rr * p.d + ch * 8) = vv;
+        }
+    }
+    // fused bias of the compacted keys, one vector per bias class of this kv head
+    const int G = p.H / p.Hk;
+    const int nfb = Hfb == p.H ? G : 1;
+    for (int it = tid; it < GATHER_KEYS * nfb; it += 256) {
+        const int gi = it / GATHER_KEYS, rr = it - gi * GATHER_KEYS;
+        const int src = s_src[rr];
+        if (src < 0) continue;
+        const int hfb = Hfb == p.H ? hk * G + gi : hk;
+        float v = 0.f;
+        if (p.bias) {
+            const int hb = p.Hb == p.H ? hfb : (p.Hb == 1 ? 0 : hk);
+            v = E::lo((uint32_t)((const uint16_t *)p.bias)[b * p.bi_b + hb * p.bi_h + src]) * kLog2e;
+        }
+        fb[((size_t)b * Hfb + hfb) * ld + c0 + rr] = v;
+    }
+}
+
+// Gradient rows (dK, dV) and columns (dBias) of dropped keys: no workgroup of the compacted backward
+// owns them, and the operator's contract is that they come back as zeros.
+__global__ void __launch_bounds__(256) compact_zero_kernel(const BwdParams p, const uint8_t *mask, int64_t m_b, int64_t m_h,
+                                                            int Hm, bool dbias_direct) {
+    const FwdParams &f = p.f;
+    const int pair = blockIdx.y, b = pair / f.Hk, hk = pair % f.Hk;
+    const int hm = Hm == 1 ? 0 : hk;
+    const uint8_t *mrow = mask + b * m_b + hm * m_h;
+    const int c0 = blockIdx.x * GATHER_KEYS;
+    const int tid = threadIdx.x;
+    const int CH = f.d / 8;
+    uint16_t *dkb = (uint16_t *)p.dk + b * p.dk_b + hk * p.dk_h;
+    uint16_t *dvb = (uint16_t *)p.dv + b * p.dv_b + hk * p.dv_h;
+    const u32x4_t z = {0, 0, 0, 0};
+    for (int it = tid; it < GATHER_KEYS * CH; it += 256) {
+        const int rr = it / CH, ch = it - rr * CH;
+        const int key = c0 + rr;
+        if (key < f.Lk && !mrow[key]) {
+            *(u32x4_t *)(dkb + (int64_t)key * p.dk_r + ch * 8) = z;
+            *(u32x4_t *)(dvb + (int64_t)key * p.dv_r + ch * 8) = z;
+        }
+    }
+    if (dbias_direct) {
+        const int G = f.H / f.Hk;
+        const int nh = f.Hb == f.H ? G : 1;
+        for (int it = tid; it < GATHER_KEYS * nh; it += 256) {
+            const int gi = it / GATHER_KEYS, key = c0 + (it - gi * GATHER_KEYS);
+            if (key < f.Lk && !mrow[key]) {
+                const int hb = f.Hb == f.H ? hk * G + gi : (f.Hb == 1 ? 0 : hk);
+                ((uint16_t *)p.dbias)[b * p.db_b + hb * p.db_h + key] = 0;
+            }
+        }
+    }
+}
+
+bool compaction_enabled() {
+    static const bool on = [] {
+        const char *e = getenv("FDMA_COMPACT");
+        return !(e && e[0] == '0');
+    }();
+    return on;
+}
+
+}  // namespace
+
+bool use_compact(const FwdParams &p) {
+    if (!compaction_enabled() || !p.mask || p.m_r != 0) return false;
+    if (p.bias && p.bi_r != 0) return false;
+    if (!(p.Hm == 1 || p.Hm == p.Hk)) return false;
+    // the pre-pass costs about one copy of K and V; it pays once a pair has a few query tiles
+    return p.Lq >= 128 && p.Lk >= 128 && (int64_t)p.Lk * p.d < (int64_t)1 << 31;
+}
+
+size_t compact_bytes(const FwdParams &p) { return layout_of(p).total; }
+
+hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream) {
+    const Layout l = layout_of(p);
+    char *w = static_cast<char *>(ws);
+    int32_t *idx = (int32_t *)(w + l.off_idx), *cnt = (int32_t *)(w + l.off_cnt), *count = (int32_t *)(w + l.off_count);
+    float *fb = (float *)(w + l.off_fb);
+    uint16_t *kc = (uint16_t *)(w + l.off_k), *vc = (uint16_t *)(w + l.off_v);
+    const int pairs = p.B * p.Hk;
+    hipLaunchKernelGGL(compact_scan_kernel, dim3(pairs), dim3(SCAN_THREADS), 0, stream, p, idx, cnt, count, l.ld);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    const dim3 grid((p.Lk + GATHER_KEYS - 1) / GATHER_KEYS, pairs);
+    if (dtype == 0)
+        hipLaunchKernelGGL((compact_gather_kernel<bf16_tag>), grid, dim3(256), 0, stream, p, idx, count, fb, kc, vc, l.ld, l.Hfb);
+    else
+        hipLaunchKernelGGL((compact_gather_kernel<fp16_tag>), grid, dim3(256), 0, stream, p, idx, count, fb, kc, vc, l.ld, l.Hfb);
+    if ((e = hipGetLastError()) != hipSuccess) return e;
+    p.k = kc;
+    p.v = vc;
+    p.k_r = p.v_r = p.d;
+    p.k_h = p.v_h = (int64_t)p.Lk * p.d;
+    p.k_b = p.v_b = (int64_t)p.Hk * p.Lk * p.d;
+    p.cmp.idx = idx;
+    p.cmp.cnt = cnt;
+    p.cmp.count = count;
+    p.cmp.fb = fb;
+    p.cmp.ld = l.ld;
+    p.cmp.Hfb = l.Hfb;
+    p.cmp.on = 1;
+    return hipSuccess;
+}
+
+hipError_t compact_zero_dropped(const BwdParams &p, const FwdParams &orig, hipStream_t stream) {
+    const dim3 grid((orig.Lk + GATHER_KEYS - 1) / GATHER_KEYS, orig.B * orig.Hk);
+    const bool dbias_direct = p.dbias != nullptr && p.dbias_accum == nullptr;
+    hipLaunchKernelGGL(compact_zero_kernel, grid, dim3(256), 0, stream, p, orig.mask, orig.m_b, orig.m_h, orig.Hm, dbias_direct);
+    return hipGetLastError();
+}
+
+}  // namespace fdma

@@ -40,7 +40,10 @@ template <int D, int BN> struct CmSmem {
     static constexpr int TOTAL = OFF_BITS + MAX_TILES / 8;
 };
 
-template <typename T, int D, int NQ, int BN, bool CAUSAL, int NW>
+// CMP: K / V are the compacted copies of the kept columns (see fdma_compact.hip).  The key axis then has
+// `count` columns, all kept; the fused bias vector comes pre-gathered, and the causal limit of a query row
+// is the number of kept columns at or below its diagonal instead of the column index itself.
+template <typename T, int D, int NQ, int BN, bool CAUSAL, int NW, bool CMP>
 __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(const FwdParams p) {
     constexpr int NTHREADS = 64 * NW;
     // with 8 waves the staging work is split by role: waves 0-3 stage V, waves 4-7 stage K and bias
@@ -103,17 +106,28 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
     const uint16_t *kbase = (const uint16_t *)p.k + b * p.k_b + hk * p.k_h;
     const uint16_t *vbase = (const uint16_t *)p.v + b * p.v_b + hk * p.v_h;
 
-    int n_end = (p.Lk + BN - 1) / BN;
+    // key columns this workgroup iterates over, and the number of them a query row may see
+    const int Lk = CMP ? p.cmp.count[b * p.Hk + hk] : p.Lk;
+    const int32_t *ccnt = CMP ? p.cmp.cnt + (int64_t)(b * p.Hk + hk) * p.cmp.ld : nullptr;
+    const float *fbrow = CMP ? p.cmp.fb + (int64_t)(b * p.cmp.Hfb + (p.cmp.Hfb == p.H ? h : hk)) * p.cmp.ld : nullptr;
+    auto visible = [&](int row) -> int {  // columns [0, visible(row)) pass the causal test for `row`
+        if (row >= p.Lq) row = p.Lq - 1;
+        int c = row + shift;
+        if (!CMP) return c + 1;
+        if (c < 0) return 0;
+        return ccnt[c < p.Lk ? c : p.Lk - 1];
+    };
+
+    int n_end = (Lk + BN - 1) / BN;
     if (CAUSAL) {
-        int lim = m0 + BM + shift;
-        if (lim > p.Lq + shift) lim = p.Lq + shift;  // rows beyond Lq do not exist
+        int lim = visible(m0 + BM - 1);
         if (lim < 0) lim = 0;
         int ne = (lim + BN - 1) / BN;
         if (ne < n_end) n_end = ne;
     }
 
     // ---- active-tile bitmap
-    for (int base = 0; base < n_end; base += NTHREADS) {
+    for (int base = 0; !CMP && base < n_end; base += NTHREADS) {
         const int j = base + tid;
         bool act = false;
         if (j < n_end) {
@@ -142,6 +156,7 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
     __syncthreads();
 
     auto next_active = [&](int j) -> int {  // smallest active tile >= j, or n_end
+        if (CMP) return j < n_end ? j : n_end;
         while (j < n_end) {
             uint32_t w = sBits[j >> 5] >> (j & 31);
             if (w) {
@@ -206,7 +221,7 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
         if (!k_role) return;
         const int n0 = j * BN;
         const char *tb = (const char *)kbase + (int64_t)n0 * p.k_r * 2;
-        if (n0 + BN <= p.Lk) {
+        if (n0 + BN <= Lk) {
 #pragma unroll
             for (int it = 0; it < K_IT; it++) kreg[it] = *(const u32x4_t *)(tb + koff[it]);
             if (!d_full) {
@@ -219,14 +234,16 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
             for (int it = 0; it < K_IT; it++) {
                 const int key = n0 + kr0 + it * K_RPP;
                 u32x4_t kv = {0, 0, 0, 0};
-                if (key < p.Lk && k_dvalid) kv = *(const u32x4_t *)(tb + koff[it]);
+                if (key < Lk && k_dvalid) kv = *(const u32x4_t *)(tb + koff[it]);
                 kreg[it] = kv;
             }
         }
         if (ktid < BN) {
             const int col = n0 + ktid;
             float v = -INFINITY;
-            if (col < p.Lk && (!mrow || mrow[col])) {
+            if (CMP) {
+                if (col < Lk) v = fbrow[col];
+            } else if (col < Lk && (!mrow || mrow[col])) {
                 v = 0.f;
                 if (brow) v = E::lo((uint32_t)brow[col]) * kLog2e;
             }
@@ -245,7 +262,7 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
         const int n0 = j * BN;
         const char *tb = (const char *)vbase + (int64_t)n0 * p.v_r * 2;
         if (v_role && tid < V_ITEMS) {
-            if (n0 + BN <= p.Lk) {
+            if (n0 + BN <= Lk) {
 #pragma unroll
                 for (int i = 0; i < 4; i++) vreg[i] = *(const u32x4_t *)(tb + voff[i]);
                 if (!d_full) {
@@ -258,7 +275,7 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
                 for (int i = 0; i < 4; i++) {
                     const int key = n0 + 4 * vkg + i;
                     u32x4_t vv = {0, 0, 0, 0};
-                    if (key < p.Lk && v_dvalid) vv = *(const u32x4_t *)(tb + voff[i]);
+                    if (key < Lk && v_dvalid) vv = *(const u32x4_t *)(tb + voff[i]);
                     vreg[i] = vv;
                 }
             }
@@ -280,6 +297,15 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
     };
 
     const int a_row = pi_row(r);
+
+    // causal limits: columns below vis_lane[nb] are visible to this lane's query row, and a tile that ends at
+    // or below vis_wave[nb] (the limit of the block's first row) needs no masking at all
+    int vis_lane[NQ], vis_wave[NQ];
+#pragma unroll
+    for (int nb = 0; nb < NQ; nb++) {
+        vis_lane[nb] = CAUSAL ? visible(wrow0 + nb * 32 + r) : 0;
+        vis_wave[nb] = CAUSAL ? visible(wrow0 + nb * 32) : 0;
+    }
 
     auto qk = [&](f32x16_t (&s)[NQ][MB], int buf) {
         const char *sK = smem + SM::OFF_K + buf * SM::K_BYTES;
@@ -334,9 +360,8 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
         uint32_t pk[NQ][8 * MB];
 #pragma unroll
         for (int nb = 0; nb < NQ; nb++) {
-            const int qrow = wrow0 + nb * 32 + r;
             // diagonal tile for this 32-row block? (wave-uniform)
-            const bool diag = CAUSAL && (n0 + BN - 1 > wrow0 + nb * 32 + shift);
+            const bool diag = CAUSAL && (n0 + BN > vis_wave[nb]);
             float tmax = -INFINITY;
 #pragma unroll
             for (int mb = 0; mb < MB; mb++)
@@ -344,7 +369,7 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
                 for (int i = 0; i < 16; i++) s[nb][mb][i] = fmaf(s[nb][mb][i], p.scale_log2, bl2[16 * mb + i]);
             if (diag) {
                 asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch: only diagonal tiles pay
-                const int lim = qrow + shift - n0 - 8 * g;  // local column limit for this lane
+                const int lim = vis_lane[nb] - 1 - n0 - 8 * g;  // local column limit for this lane
 #pragma unroll
                 for (int mb = 0; mb < MB; mb++)
 #pragma unroll
@@ -464,10 +489,10 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
     }
 }
 
-template <typename T, int D, int NQ, int BN, bool CAUSAL, int NW = 4>
+template <typename T, int D, int NQ, int BN, bool CAUSAL, bool CMP, int NW = 4>
 hipError_t launch_one(const FwdParams &p, hipStream_t stream) {
     constexpr int BM = 32 * NQ * NW;
-    auto kern = fwd_colmask_kernel<T, D, NQ, BN, CAUSAL, NW>;
+    auto kern = fwd_colmask_kernel<T, D, NQ, BN, CAUSAL, NW, CMP>;
     const int smem = CmSmem<D, BN>::TOTAL;
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
@@ -482,7 +507,8 @@ hipError_t launch_one(const FwdParams &p, hipStream_t stream) {
 template <typename T, int D>
 hipError_t launch_d(const FwdParams &p, int variant, hipStream_t stream) {
     (void)variant;
-    return p.causal ? launch_one<T, D, 1, 64, true>(p, stream) : launch_one<T, D, 1, 64, false>(p, stream);
+    if (p.cmp.on) return p.causal ? launch_one<T, D, 1, 64, true, true>(p, stream) : launch_one<T, D, 1, 64, false, true>(p, stream);
+    return p.causal ? launch_one<T, D, 1, 64, true, false>(p, stream) : launch_one<T, D, 1, 64, false, false>(p, stream);
 }
 
 }  // namespace

@@ -8,6 +8,20 @@
 
 namespace fdma {
 
+// Column compaction for keep-masks that are broadcast over queries: the kept keys of every
+// (batch, kv head) pair are gathered, in ascending column order, into dense copies of K and V, and the
+// main kernels then run over `count` keys instead of Lk.  Causal masking compares against the number of
+// kept columns a query can see (`cnt`), and gradients are written back through `idx`.
+struct Compact {
+    const int32_t *idx;    // (B*Hk, ld): original column of compacted key c, c < count
+    const int32_t *cnt;    // (B*Hk, ld): kept keys among the original columns 0..j (inclusive)
+    const int32_t *count;  // (B*Hk): kept keys
+    const float *fb;       // (B*Hfb, ld): bias * log2(e) of compacted key c (0 without a bias)
+    int32_t ld;            // row stride of the arrays above (Lk rounded up to 16)
+    int32_t Hfb;           // heads of fb: Hk, or H when the bias differs per query head
+    int32_t on;            // 0 = no compaction: k / v are the caller's tensors
+};
+
 struct FwdParams {
     const void *q, *k, *v;
     const uint8_t *mask;  // nullptr = absent
@@ -28,6 +42,7 @@ struct FwdParams {
     float *o_part;      // (splits, B, H, Lq, d) fp32
     float *lse_part;    // (splits, B, H, Lq) fp32, natural log, -inf for an empty split
     int32_t splits;
+    Compact cmp;        // when cmp.on, k / v (and their strides) describe the compacted copies
 };
 
 struct BwdParams {
@@ -56,6 +71,14 @@ hipError_t launch_bwd(const BwdParams &p, int dtype, hipStream_t stream);
 bool bwd_colmask_applicable(const BwdParams &p);
 hipError_t launch_bwd_dkdv_colmask(const BwdParams &p, int dtype, hipStream_t stream);
 hipError_t launch_bwd_dq_colmask(const BwdParams &p, int dtype, hipStream_t stream);
+
+// Column compaction: use_compact() decides from the problem alone (no device data), compact_bytes() is
+// the scratch it needs, compact_setup() launches the gather pre-pass into `ws` and rewrites p.k / p.v /
+// p.cmp; compact_zero_dropped() zero-fills the gradient rows / columns of dropped keys.
+bool use_compact(const FwdParams &p);
+size_t compact_bytes(const FwdParams &p);
+hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream);
+hipError_t compact_zero_dropped(const BwdParams &p, const FwdParams &orig, hipStream_t stream);
 
 // number of KV splits the decode path uses for this shape (1 = no workspace needed)
 int decode_num_splits(int B, int Hk, int Lk);

@@ -67,6 +67,14 @@ SMALL_CASES = {
     "head_dim_96": (1, 256, 256, 2, 1, 96, (1, 1, 1, 256), (1, 1, 1, 256), 128, True),
     "head_dim_32": (1, 192, 256, 2, 1, 32, (1, 1, 1, 256), (1, 1, 1, 256), 128, False),
     "tiny": (1, 3, 5, 2, 1, 8, (1, 1, 3, 5), (1, 1, 3, 5), 2, True),
+    # query-broadcast masks long enough for the column-compaction path (gathered K / V, scattered grads)
+    "compact_gqa_bias_per_qhead": (2, 300, 300, 4, 2, 64, (2, 4, 1, 300), (2, 2, 1, 300), 77, True),
+    "compact_lq_lt_lk_shared_mask": (1, 160, 400, 4, 2, 128, (1, 2, 1, 400), (1, 1, 1, 400), 90, True),
+    "compact_lq_gt_lk_empty_rows": (1, 400, 200, 2, 2, 64, (1, 2, 1, 200), (1, 2, 1, 200), 50, True),
+    "compact_noncausal_mask_only": (2, 257, 391, 4, 4, 128, None, (2, 4, 1, 391), 100, False),
+    "compact_batch_broadcast_bias": (2, 256, 256, 4, 2, 64, (1, 2, 1, 256), (2, 2, 1, 256), 64, True),
+    "compact_head_dim_96_dense_mask": (1, 200, 200, 2, 1, 96, (1, 1, 1, 200), (1, 1, 1, 200), 200, True),
+    "colmask_per_query_head_gqa": (1, 256, 256, 4, 2, 64, (1, 4, 1, 256), (1, 4, 1, 256), 64, True),
 }
 
 
@@ -160,6 +168,28 @@ def test_fully_masked_tiles_are_skipped_and_rows_without_keys_give_zero():
     for g, r, n in ((dq, rdq, "dq"), (dk, rdk, "dk"), (dv, rdv, "dv"), (db, rdb, "dbias")):
         assert_grad_close(g.cpu(), r, n)
     assert torch.equal(dk[:, :64].cpu(), torch.zeros(B, 64, Hk, D, dtype=torch.bfloat16))  # keys nobody keeps
+
+
+def test_column_mask_with_an_all_dropped_pair_and_late_first_key():
+    """Query-broadcast mask whose (batch 0, kv head 1) row keeps nothing and whose other rows keep no key
+    before column 150: that pair's outputs and gradients are exactly zero, rows that see no kept key give
+    O = 0 / LSE = +inf, and everything else matches the oracle."""
+    B, L, H, Hk, D = 2, 320, 4, 2, 64
+    q, k, v, mask, bias = make_inputs(B, L, L, H, Hk, D, (B, Hk, 1, L), (B, Hk, 1, L), 60, seed=5)
+    mask[..., :150] = False
+    mask[0, 1] = False
+    dout = torch.randn(B, L, H, D, generator=torch.Generator().manual_seed(6)).to(torch.bfloat16)
+    out, lse, (dq, dk, dv, db) = _run_fwd_bwd(q, k, v, mask, bias, True, dout=dout)
+    ro, rl = c_oracle.forward(q, k, v, mask, bias, None, True)
+    assert_out_close(out.cpu(), ro)
+    _check_lse(lse.cpu(), rl)
+    assert torch.isinf(lse[0, 2:]).all() and torch.isinf(lse[:, :, :150]).all()
+    assert not out[0, :, 2:].any() and not dq[0, :, 2:].any()
+    assert not dk[0, :, 1].any() and not dv[0, :, 1].any() and not db[0, 1].any()
+    assert not dk[:, :150].any() and not dv[:, :150].any() and not db[..., :150].any()
+    rdq, rdk, rdv, rdb = c_oracle.backward(q, k, v, dout, mask, bias, None, True)
+    for g, r, n in ((dq, rdq, "dq"), (dk, rdk, "dk"), (dv, rdv, "dv"), (db, rdb, "dbias")):
+        assert_grad_close(g.cpu(), r, n)
 
 
 def test_seqlen_k_zero_and_no_grad_path():
@@ -272,6 +302,12 @@ def test_direct_c_abi_call_without_the_python_operator():
     lse = torch.empty(1, 2, 128, dtype=torch.float32, device=DEV)
     a = _cabi.FwdArgs()
     _cabi.fill_fwd(a, qd, kd, vd, md, bd, out, lse, 0.125, True, 0.0)
+    need = _cabi.lib.fdma_fwd_workspace_bytes(a)
+    if need:  # a caller that ignores the scratch request gets an error code and a message, not a fault
+        assert _cabi.lib.fdma_fwd(a, _cabi.current_stream(qd.device)) == -3
+        assert "workspace too small" in _cabi.last_error()
+        ws = torch.empty(need, dtype=torch.uint8, device=DEV)
+        a.workspace, a.workspace_bytes = ws.data_ptr(), need
     assert _cabi.lib.fdma_fwd(a, _cabi.current_stream(qd.device)) == 0, _cabi.last_error()
     torch.cuda.synchronize()
     ro, rl = c_oracle.forward(q, k, v, mask, bias, 0.125, True)
