@@ -31,8 +31,9 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch of the forward kernel on the headline workload, from two rocprofv3 --pmc runs of
 # this script (FETCH_SIZE, WRITE_SIZE; each scaled by what the counter reads for a 256 MiB device copy,
-# see --calib-copy): 143 MiB read + 65 MiB written.  Override with --traffic-bytes after re-measuring.
-MEASURED_FWD_TRAFFIC_BYTES = 208.0 * 1024 * 1024
+# see --calib-copy): compacted kernel 79 MiB read + 65 MiB written, tile-skipping kernel 143 + 65 MiB.
+# Override with --traffic-bytes after re-measuring.
+MEASURED_FWD_TRAFFIC_BYTES = {True: 144.0 * 1024 * 1024, False: 208.0 * 1024 * 1024}
 
 CONFIGS = {
     # name: B, Lq, Lk, H, Hk, D, bias shape, window, causal, passes
@@ -152,9 +153,10 @@ def time_gpu(fn, steps, warmup):
     return e0.elapsed_time(e1) / steps
 
 
-def run_config(name, steps, warmup, device):
+def run_config(name, steps, warmup, device, compact=True, backward=True):
     from flash_sparse_attn import flash_sparse_attn_func
 
+    os.environ["FDMA_COMPACT"] = "1" if compact else "0"  # the library reads it on every call
     c = CONFIGS[name]
     q, k, v, mask, bias = make_case(c, device)
     scale = c["scale"]
@@ -187,7 +189,7 @@ def run_config(name, steps, warmup, device):
         blocks = int(m.view(m.shape[0], m.shape[1], -1, 64).any(-1).sum().item())
         res["tile64_bytes"] = 2.0 * blocks * 64 * c["D"] * 2 + side
         res["hbm_gbs_tile64"] = res["tile64_bytes"] / ms_fwd / 1e6
-    if c["bwd"]:
+    if c["bwd"] and backward:
         qg, kg, vg = [t.clone().requires_grad_(True) for t in (q, k, v)]
         bg = bias.clone().requires_grad_(True)
 
@@ -249,11 +251,17 @@ def main():
         sys.exit(1)
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
-    if args.no_compact:
-        os.environ["FDMA_COMPACT"] = "0"  # read once by the library, which is loaded on first use below
-
-    main_res = run_config("cfg2", args.steps, args.warmup, device)
+    compact = not args.no_compact
+    main_res = run_config("cfg2", args.steps, args.warmup, device, compact)
     c = CONFIGS["cfg2"]
+    if main_res["compacted"]:
+        kernel = ("fdma::fwd_colmask_kernel<bf16, 128, causal, compacted>, with its pre-pass (compact_scan_kernel, "
+                  "compact_gather_kernel) in the same call: the duration is that of the whole forward call")
+        flops_model = ("4*64*64*d per executed 64x64 tile on the compacted key axis (kept columns packed to the front per "
+                       "(batch, kv head)); a 64-row query block executes ceil(visible kept columns / 64) tiles")
+    else:
+        kernel = "fdma::fwd_colmask_kernel<bf16, 128, causal> (tile skipping on the original key axis)"
+        flops_model = "4*64*64*d per 64x64 tile of the original layout that holds a kept, causally visible element"
     out = {
         "metric": "fwd effective TFLOP/s on executed 64x64 tiles (L=8192, W=2048, d=128, bf16, GQA 4:1, mask+bias+causal)",
         "value": main_res["tflops_fwd"],
@@ -269,7 +277,11 @@ def main():
         "data": "synthetic",
         "config": {"workload": "cfg2: B=1 Lq=Lk=8192 H=32 Hkv=8 d=128 bias[1,8,1,8192] top-2048 ∩ causal, forward",
                    "mask_form": main_res["mask_form"], "n_exec_tiles": main_res["n_exec"],
-                   "tile_occupancy": main_res["tile_occupancy"]},
+                   "column_compaction": main_res["compacted"], "flops_model": flops_model,
+                   "n_exec_tiles_original_layout": main_res.get("n_exec_original_layout", main_res["n_exec"]),
+                   "tile_occupancy_original_layout": main_res["tile_occupancy"]},
+        "tflops_fwd_elementwise": main_res["tflops_fwd_elementwise"],
+        "tflops_fwd_original_layout_tiles": main_res.get("tflops_fwd_original_layout_tiles", main_res["tflops_fwd"]),
         "ms_fwd": main_res["ms_fwd"],
         "ms_fwd_bwd": main_res.get("ms_fwd_bwd"),
         "tflops_fwd_bwd": main_res.get("tflops_fwd_bwd"),
@@ -279,11 +291,18 @@ def main():
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": main_res["tflops_fwd"] / PEAK_BF16_TFLOPS,
-            "traffic": MEASURED_FWD_TRAFFIC_BYTES,
-            "kernel": "fdma::fwd_kernel<bf16, 128, causal>",
+            "traffic": MEASURED_FWD_TRAFFIC_BYTES[bool(main_res["compacted"])],
+            "kernel": kernel,
             "flops_per_launch": 4.0 * 64 * 64 * c["D"] * main_res["n_exec"],
+            "duration_ms": main_res["ms_fwd"],
         },
     }
+    if compact:
+        # the same workload through the tile-skipping kernel alone (one kernel per call, no pre-pass)
+        ts = run_config("cfg2", max(3, args.steps // 2), max(1, args.warmup // 2), device, compact=False, backward=False)
+        out["tile_skip_path"] = {"ms_fwd": ts["ms_fwd"], "n_exec_tiles": ts["n_exec"], "tflops_fwd": ts["tflops_fwd"],
+                                 "frac_of_peak": ts["tflops_fwd"] / PEAK_BF16_TFLOPS,
+                                 "kernel": "fdma::fwd_colmask_kernel<bf16, 128, causal> (FDMA_COMPACT=0)"}
     if args.traffic_bytes is not None:
         out["roofline"]["traffic"] = args.traffic_bytes
     if args.calib_copy:
@@ -292,7 +311,7 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
     if args.all:
-        out["other_configs"] = [run_config(n, max(3, args.steps // 4), max(1, args.warmup // 2), device)
+        out["other_configs"] = [run_config(n, max(3, args.steps // 4), max(1, args.warmup // 2), device, compact)
                                 for n in ("cfg1", "cfg3", "cfg4", "cfg5")]
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline("cfg2", groups=1)

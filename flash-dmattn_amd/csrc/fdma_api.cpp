@@ -122,7 +122,7 @@ size_t fdma_fwd_workspace_bytes(const fdma_fwd_args *a) {
     if (!fdma::use_decode_path(a->seqlen_q, a->num_heads, a->num_heads_k)) {
         fdma::FwdParams p;
         fill_fwd_params(a, p);
-        return fdma::use_compact(p) ? fdma::compact_bytes(p) : 0;
+        return fdma::use_compact(p) ? fdma::compact_bytes(p, false) : 0;
     }
     const int splits = fdma::decode_num_splits(a->batch, a->num_heads_k, a->seqlen_k);
     if (splits <= 1) return 0;
@@ -153,7 +153,7 @@ int fdma_fwd(const fdma_fwd_args *a, void *hip_stream) {
     } else {
         // seqlen_k == 0 falls out of the kernel as O = 0, LSE = +inf (flash_api.cpp:535-539)
         if (fdma::use_compact(p)) {
-            const size_t need = fdma::compact_bytes(p);
+            const size_t need = fdma::compact_bytes(p, false);
             if (!a->workspace || a->workspace_bytes < need)
                 return fail(FDMA_ERR_WORKSPACE, "forward workspace too small: need %zu bytes, got %zu", need, a->workspace_bytes);
             if ((e = fdma::compact_setup(p, a->workspace, a->dtype, stream)) != hipSuccess)
@@ -210,7 +210,7 @@ size_t fdma_bwd_workspace_bytes(const fdma_bwd_args *a) {
     if (!a) return 0;
     fdma::FwdParams p;
     fill_fwd_params(&a->f, p);
-    return dbias_accum_bytes(a) + (fdma::use_compact(p) ? fdma::compact_bytes(p) : 0);
+    return dbias_accum_bytes(a) + (fdma::use_compact(p) ? fdma::compact_bytes(p, true) : 0);
 }
 
 int fdma_bwd(const fdma_bwd_args *a, void *hip_stream) {
@@ -242,7 +242,7 @@ int fdma_bwd(const fdma_bwd_args *a, void *hip_stream) {
     hipError_t e;
     if (a->f.seqlen_q > 0 && fdma::use_compact(p.f)) {
         const fdma::FwdParams orig = p.f;
-        e = fdma::compact_setup(p.f, static_cast<char *>(a->workspace) + dbias_accum_bytes(a), a->f.dtype, stream);
+        e = fdma::compact_setup(p.f, static_cast<char *>(a->workspace) + dbias_accum_bytes(a), a->f.dtype, stream, &p);
         if (e == hipSuccess) e = fdma::compact_zero_dropped(p, orig, stream);
         if (e != hipSuccess) return fail(FDMA_ERR_LAUNCH, "backward launch failed: %s", hipGetErrorString(e));
     }

@@ -77,19 +77,54 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
     const FwdParams &f = p.f;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 31, g = lane >> 5;
     const int G = f.H / f.Hk;
-    const int n_nb = (f.Lk + KV_BN - 1) / KV_BN;
-    const XcdMap wm = xcd_map(blockIdx.x, f.B * f.Hk, n_nb, 1);
-    if (!wm.valid) return;
-    const int n_block = wm.unit;  // low key blocks are seen by the most queries under causal: heaviest first
-    const int b = wm.pair / f.Hk, hk = wm.pair % f.Hk;
+    // work item: a 128-key block of one (batch, kv head) pair, over query heads [g_lo, g_hi) and segment
+    // `seg` of `Sm` of the query range; `slot` >= 0 when the block is shared by several workgroups
+    int pair, n_block, g_lo = 0, g_hi = G, seg = 0, Sm = 1, Q = 1 << 30, slot = -1;
+    if (CMP) {
+        const int32_t *plan = f.cmp.plan;
+        const int Gs = plan[1];
+        Sm = plan[2];
+        Q = plan[4];
+        const int per = Gs * Sm;
+        // unit lists per XCD (see DkdvPlan); within a list all units of one split index sit side by side:
+        // neighbours in time then stream the same Q / dO tiles through that XCD's L2
+        const int P = f.B * f.Hk, k = dkdv_lists_per_pair(P);
+        const int list_len = plan[3];
+        if (list_len == 0) return;
+        const int x = blockIdx.x % 8, l = blockIdx.x / 8;
+        const int span = list_len * per;
+        const int ls = l / span, within = l % span;
+        if (ls >= P * k / 8) return;
+        // Consecutive workgroups of an XCD go to its shader engines in turn; unit weights fall with the unit
+        // index, so the start of the unit order is rotated with the split index -- otherwise one engine would
+        // receive the heavy unit of every group and the others would idle behind it.
+        const int sub = within / list_len, pos = (within % list_len + sub) % list_len;
+        const int vlist = x + 8 * ls, fold = vlist % k;
+        pair = vlist / k;
+        n_block = 2 * k * (pos >> 1) + ((pos & 1) ? 2 * k - 1 - fold : fold);
+        if (n_block >= plan[DKDV_PLAN_HDR + pair + 1] - plan[DKDV_PLAN_HDR + pair]) return;
+        const int unit = plan[DKDV_PLAN_HDR + pair] + n_block;
+        const int gper = G / Gs;
+        g_lo = (sub / Sm) * gper;
+        g_hi = g_lo + gper;
+        seg = sub % Sm;
+        if (per > 1) slot = unit * per + sub;
+    } else {
+        const int n_nb = (f.Lk + KV_BN - 1) / KV_BN;
+        const XcdMap wm = xcd_map(blockIdx.x, f.B * f.Hk, n_nb, 1);
+        if (!wm.valid) return;
+        n_block = wm.unit;  // low key blocks are seen by the most queries under causal: heaviest first
+        pair = wm.pair;
+    }
+    const int b = pair / f.Hk, hk = pair % f.Hk;
     const int n0 = n_block * KV_BN;
-    const int Lk = CMP ? f.cmp.count[wm.pair] : f.Lk;  // key columns on this pair's (possibly compacted) key axis
+    const int Lk = CMP ? f.cmp.count[pair] : f.Lk;  // key columns on this pair's (possibly compacted) key axis
     if (CMP && n0 >= Lk) return;
     const int key = n0 + wave * 32 + r;  // the key column this lane owns
     const int key_c = key < Lk ? key : Lk - 1;
     const int shift = f.Lk - f.Lq;
     // original column indices: of this lane's key, of the workgroup's first key and of the wave's last key
-    const int32_t *cidx = CMP ? f.cmp.idx + (int64_t)wm.pair * f.cmp.ld : nullptr;
+    const int32_t *cidx = CMP ? f.cmp.idx + (int64_t)pair * f.cmp.ld : nullptr;
     const int okey = CMP ? cidx[key_c] : key;
     const int okey_first = CMP ? cidx[n0] : n0;
     const int okey_wlast = CMP ? cidx[n0 + wave * 32 + 31 < Lk ? n0 + wave * 32 + 31 : Lk - 1] : n0 + wave * 32 + 31;
@@ -116,17 +151,22 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
         for (int i = 0; i < 16; i++) { dk[db][i] = 0.f; dv[db][i] = 0.f; }
 
     const int M_blocks = (f.Lq + KV_BM - 1) / KV_BM;
-    int m_start = 0;
-    if (CAUSAL) {
-        const int first_q = okey_first - shift;  // first query row that sees the workgroup's first key
-        if (first_q > 0) m_start = first_q / KV_BM;
-        if (m_start > M_blocks) m_start = M_blocks;
+    // query blocks that see the workgroup's first key: [m_start, M_blocks)
+    const int m_start = M_blocks - dkdv_query_blocks(f.Lq, f.Lk, CAUSAL, okey_first);
+    // this workgroup's query blocks [m_lo, m_hi): all of them, or one of the unit's equal segments
+    int m_lo = m_start, m_hi = M_blocks;
+    if (slot >= 0) {
+        const int n_seg = dkdv_segments(M_blocks - m_start, Q, Sm);
+        if (seg >= n_seg) return;  // the reduce kernel knows that this slot stays unwritten
+        const int len = (M_blocks - m_start + n_seg - 1) / n_seg;
+        m_lo = m_start + seg * len;
+        m_hi = m_lo + len < M_blocks ? m_lo + len : M_blocks;
     }
-    const int n_m = M_blocks - m_start;
-    // (g outer, m inner); the query blocks are walked from the LAST one down to m_start, so that the
+    const int n_m = m_hi > m_lo ? m_hi - m_lo : 0;
+    // (g outer, m inner); the query blocks are walked from the LAST one down, so that the
     // workgroups of one (batch, kv head) pair, which run side by side on an XCD, all begin at the same
     // Q / dO tile and stream the same tiles at the same time (L2 hits instead of re-fetches)
-    const int n_steps = n_m * G;
+    const int n_steps = n_m * (g_hi - g_lo);
 
     const bool has_bias = f.bias != nullptr;
     const bool use_accum = p.dbias_accum != nullptr;
@@ -152,7 +192,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
     u32x4_t qreg[Q_IT], doreg[Q_IT];
     float lreg = INFINITY, dreg = 0.f;
     auto load_step = [&](int step) {
-        const int gi = step / n_m, mi = M_blocks - 1 - step % n_m;  // last query block first: see below
+        const int gi = g_lo + step / n_m, mi = m_hi - 1 - step % n_m;  // last query block first: see below
         const int h = hk * G + gi, m0 = mi * KV_BM;
         const uint16_t *qbase = (const uint16_t *)f.q + b * f.q_b + h * f.q_h + qcol;
         const uint16_t *dobase = (const uint16_t *)p.dout + b * p.do_b + h * p.do_h + qcol;
@@ -204,7 +244,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
     }
 
     for (int step = 0; step < n_steps; step++) {
-        const int gi = step / n_m, mi = M_blocks - 1 - step % n_m;  // last query block first: see below
+        const int gi = g_lo + step / n_m, mi = m_hi - 1 - step % n_m;  // last query block first: see below
         const int h = hk * G + gi;
         const int m0 = mi * KV_BM;
         const int buf = step & 1;
@@ -302,10 +342,12 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
         // ---- dBias column sum: flush when the bias head changes
         if (has_bias) {
             const bool last_m = (step % n_m) == n_m - 1;
-            if (last_m && (f.Hb == f.H || gi == G - 1)) {
+            if (last_m && (slot >= 0 || f.Hb == f.H || gi == G - 1)) {
                 const float tot = xhalf_sum(colsum);
                 const int hb = f.Hb == f.H ? h : (f.Hb == 1 ? 0 : hk);
-                if (g == 0 && key < Lk) {
+                if (slot >= 0) {  // per-head partial column sums; the reduce kernel folds them
+                    if (g == 0) p.db_part[((int64_t)slot * G + (gi - g_lo)) * KV_BN + (key - n0)] = tot;
+                } else if (g == 0 && key < Lk) {
                     if (use_accum) atomicAdd(p.dbias_accum + b * p.dba_b + hb * p.dba_h + okey, tot);
                     else ((uint16_t *)p.dbias)[b * p.db_b + hb * p.db_h + okey] = (uint16_t)(E::pack2(tot, 0.f) & 0xffffu);
                 }
@@ -318,12 +360,29 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
     }
 
     // a key block that no query can see still owns its dbias column
-    if (has_bias && n_steps == 0 && !use_accum && g == 0 && key < Lk) {
+    if (has_bias && n_steps == 0 && slot >= 0 && g == 0) {
+        for (int gl = 0; gl < g_hi - g_lo; gl++) p.db_part[((int64_t)slot * G + gl) * KV_BN + (key - n0)] = 0.f;
+    }
+    if (has_bias && n_steps == 0 && slot < 0 && !use_accum && g == 0 && key < Lk) {
         const int ngh = (f.Hb == f.H) ? G : 1;
         for (int gh = 0; gh < ngh; gh++) {
             const int hb = f.Hb == f.H ? hk * G + gh : (f.Hb == 1 ? 0 : hk);
             ((uint16_t *)p.dbias)[b * p.db_b + hb * p.db_h + okey] = 0;
         }
+    }
+
+    // ---- shared block: fp32 partial dK^T / dV^T, [which][d][key] so that a wave writes 128-byte runs
+    if (slot >= 0) {
+        float *pk = p.dkv_part + (int64_t)slot * 2 * D * KV_BN + (key - n0);
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int i = 0; i < 16; i++) {
+                const int dcol = 32 * db + 16 * (i >> 3) + 8 * g + (i & 7);
+                pk[dcol * KV_BN] = dk[db][i];
+                pk[(D + dcol) * KV_BN] = dv[db][i];
+            }
+        return;
     }
 
     // ---- store dK (scaled) and dV
@@ -349,6 +408,93 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
     }
 }
 
+// Sums the partial results of the blocks that the compacted dK/dV kernel split over several workgroups, in a
+// fixed order, and writes dK (scaled), dV and dBias to the original rows / columns of the kept keys.
+template <typename T, int D>
+__global__ void __launch_bounds__(NTHREADS) bwd_dkdv_reduce_kernel(const BwdParams p) {
+    using E = Elem<T>;
+    const FwdParams &f = p.f;
+    const int32_t *plan = f.cmp.plan;
+    const int U = plan[0], Gs = plan[1], Sm = plan[2], Q = plan[4], per = Gs * Sm;
+    const int unit = blockIdx.x;
+    if (per == 1 || unit >= U) return;
+    int lo = 0, hi = f.B * f.Hk;
+    while (hi - lo > 1) {
+        const int mid = (lo + hi) >> 1;
+        if (plan[DKDV_PLAN_HDR + mid] <= unit) lo = mid;
+        else hi = mid;
+    }
+    const int pair = lo, b = pair / f.Hk, hk = pair % f.Hk;
+    const int n0 = (unit - plan[DKDV_PLAN_HDR + pair]) * KV_BN;
+    const int Lk = f.cmp.count[pair];
+    const int G = f.H / f.Hk;
+    const int tid = threadIdx.x, kk = tid % KV_BN, half = tid / KV_BN;
+    const bool live = n0 + kk < Lk;
+    const int okey = live ? f.cmp.idx[(int64_t)pair * f.cmp.ld + n0 + kk] : 0;
+    // segments of this unit that were written (same rule as in the main kernel)
+    const int n_seg = dkdv_segments(dkdv_query_blocks(f.Lq, f.Lk, f.causal, f.cmp.idx[(int64_t)pair * f.cmp.ld + n0]), Q, Sm);
+    const float *base = p.dkv_part + (int64_t)unit * per * 2 * D * KV_BN + kk;
+    // blockIdx.y picks a pair of 8-wide head-dim chunks, so that few units still give many workgroups
+    for (int c = 2 * blockIdx.y + half; c == 2 * (int)blockIdx.y + half && c * 8 < f.d; c += NTHREADS / KV_BN) {
+        float ak[8], av[8];
+#pragma unroll
+        for (int e = 0; e < 8; e++) { ak[e] = 0.f; av[e] = 0.f; }
+        // written slots in a fixed order, two at a time so that more loads are in flight
+        const int n_w = Gs * n_seg;
+        for (int j = 0; j < n_w; j += 2) {
+            const bool two = j + 1 < n_w;
+            const int j1 = two ? j + 1 : j;
+            const float *p0 = base + (int64_t)((j / n_seg) * Sm + j % n_seg) * 2 * D * KV_BN;
+            const float *p1 = base + (int64_t)((j1 / n_seg) * Sm + j1 % n_seg) * 2 * D * KV_BN;
+            float k0[8], v0[8], k1[8], v1[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                k0[e] = p0[(c * 8 + e) * KV_BN];
+                v0[e] = p0[(D + c * 8 + e) * KV_BN];
+                k1[e] = p1[(c * 8 + e) * KV_BN];
+                v1[e] = p1[(D + c * 8 + e) * KV_BN];
+            }
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                ak[e] += k0[e];
+                av[e] += v0[e];
+                if (two) { ak[e] += k1[e]; av[e] += v1[e]; }
+            }
+        }
+        if (live) {
+            u32x4_t wk, wv;
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                wk[e] = E::pack2(ak[2 * e] * f.scale, ak[2 * e + 1] * f.scale);
+                wv[e] = E::pack2(av[2 * e], av[2 * e + 1]);
+            }
+            *(u32x4_t *)((uint16_t *)p.dk + b * p.dk_b + (int64_t)okey * p.dk_r + hk * p.dk_h + c * 8) = wk;
+            *(u32x4_t *)((uint16_t *)p.dv + b * p.dv_b + (int64_t)okey * p.dv_r + hk * p.dv_h + c * 8) = wv;
+        }
+    }
+    if (f.bias && live && blockIdx.y == 0) {
+        const int gper = G / Gs;
+        const float *dbp = p.db_part + (int64_t)unit * per * G * KV_BN + kk;  // [part][local head][key]
+        auto emit = [&](int hb, float tot) {
+            if (p.dbias_accum) atomicAdd(p.dbias_accum + b * p.dba_b + hb * p.dba_h + okey, tot);
+            else ((uint16_t *)p.dbias)[b * p.db_b + hb * p.db_h + okey] = (uint16_t)(E::pack2(tot, 0.f) & 0xffffu);
+        };
+        if (f.Hb == f.H) {
+            for (int gi = half; gi < G; gi += NTHREADS / KV_BN) {
+                float tot = 0.f;
+                for (int sg = 0; sg < n_seg; sg++) tot += dbp[((int64_t)((gi / gper) * Sm + sg) * G + gi % gper) * KV_BN];
+                emit(hk * G + gi, tot);
+            }
+        } else if (half == 0) {
+            float tot = 0.f;
+            for (int gs = 0; gs < Gs; gs++)
+                for (int sg = 0; sg < n_seg; sg++)
+                    for (int gl = 0; gl < gper; gl++) tot += dbp[((int64_t)(gs * Sm + sg) * G + gl) * KV_BN];
+            emit(f.Hb == 1 ? 0 : hk, tot);
+        }
+    }
+}
+
 template <typename T, int D, bool CAUSAL, bool CMP>
 hipError_t launch_dkdv_c(const BwdParams &p, hipStream_t stream) {
     const FwdParams &f = p.f;
@@ -356,6 +502,15 @@ hipError_t launch_dkdv_c(const BwdParams &p, hipStream_t stream) {
     const int smem = KvcSmem<D>::TOTAL;
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
+    const int units_max = f.B * f.Hk * ((f.Lk + KV_BN - 1) / KV_BN);
+    if (CMP) {
+        int grid, slots;
+        dkdv_split_bounds(f.B * f.Hk, (f.Lk + KV_BN - 1) / KV_BN, f.H / f.Hk, grid, slots);
+        hipLaunchKernelGGL(kern, dim3(grid), dim3(NTHREADS), smem, stream, p);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        hipLaunchKernelGGL((bwd_dkdv_reduce_kernel<T, D>), dim3(units_max, D / 16), dim3(NTHREADS), 0, stream, p);
+        return hipGetLastError();
+    }
     dim3 grid(xcd_grid(f.B * f.Hk, (f.Lk + KV_BN - 1) / KV_BN, 1));
     hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, stream, p);
     return hipGetLastError();

@@ -30,11 +30,11 @@ constexpr int GATHER_KEYS = 64;                        // compacted keys per gat
 inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 struct Layout {
-    size_t off_idx, off_cnt, off_count, off_fb, off_k, off_v, total;
+    size_t off_idx, off_cnt, off_count, off_fb, off_k, off_v, off_plan, off_part_kv, off_part_db, total;
     int ld, Hfb;
 };
 
-Layout layout_of(const FwdParams &p) {
+Layout layout_of(const FwdParams &p, bool backward) {
     Layout l;
     l.ld = (p.Lk + 15) / 16 * 16;
     l.Hfb = (p.bias && p.Hb == p.H) ? p.H : p.Hk;
@@ -46,6 +46,15 @@ Layout layout_of(const FwdParams &p) {
     l.off_fb = o;    o += align256((size_t)p.B * l.Hfb * l.ld * 4);
     l.off_k = o;     o += align256(pairs * p.Lk * p.d * 2);
     l.off_v = o;     o += align256(pairs * p.Lk * p.d * 2);
+    l.off_plan = l.off_part_kv = l.off_part_db = o;
+    if (backward) {
+        int grid, slots;
+        dkdv_split_bounds((int)pairs, (p.Lk + 127) / 128, p.H / p.Hk, grid, slots);
+        const int dpad = p.d <= 64 ? 64 : 128;
+        l.off_plan = o;    o += align256((DKDV_PLAN_HDR + pairs + 1) * 4);
+        l.off_part_kv = o; o += align256((size_t)slots * 2 * dpad * 128 * 4);
+        l.off_part_db = o; o += align256((size_t)slots * (p.H / p.Hk) * 128 * 4);
+    }
     l.total = o;
     return l;
 }
@@ -187,28 +196,109 @@ __global__ void __launch_bounds__(256) compact_zero_kernel(const BwdParams p, co
     }
 }
 
-bool compaction_enabled() {
-    static const bool on = [] {
-        const char *e = getenv("FDMA_COMPACT");
-        return !(e && e[0] == '0');
-    }();
-    return on;
+// One workgroup: prefix of 128-key units over the pairs and the split the dK/dV kernel will use.
+__global__ void __launch_bounds__(256) compact_plan_kernel(const int32_t *count, const int32_t *idx, int ld, int32_t *plan,
+                                                            int pairs, int G, int Lq, int Lk, int causal) {
+    __shared__ int s_sum, s_max;
+    const int tid = threadIdx.x;
+    if (tid == 0) {
+        int u = 0, n_max = 0;
+        for (int i = 0; i < pairs; i++) {
+            plan[DKDV_PLAN_HDR + i] = u;
+            const int n = (count[i] + 127) / 128;
+            u += n;
+            n_max = n > n_max ? n : n_max;
+        }
+        plan[DKDV_PLAN_HDR + pairs] = u;
+        plan[0] = u;
+        plan[3] = dkdv_list_len(n_max, dkdv_lists_per_pair(pairs));
+        s_sum = 0;
+        s_max = 0;
+    }
+    __syncthreads();
+    // query blocks per unit: their sum sizes the parts, their maximum the number of segment slots
+    int sum = 0, mx = 0;
+    for (int i = 0; i < pairs; i++) {
+        const int n = (count[i] + 127) / 128;
+        for (int u = tid; u < n; u += 256) {
+            const int nt = dkdv_query_blocks(Lq, Lk, causal, idx[(size_t)i * ld + u * 128]);
+            sum += nt;
+            mx = nt > mx ? nt : mx;
+        }
+    }
+    atomicAdd(&s_sum, sum);
+    atomicMax(&s_max, mx);
+    __syncthreads();
+    if (tid == 0) {
+        int Gs, Sm;
+        dkdv_split(plan[0], G, Gs, Sm);
+        int Q = 1 << 30;
+        if (Sm > 1) {
+            const int64_t even = ((int64_t)G * s_sum + DKDV_TARGET_PARTS - 1) / DKDV_TARGET_PARTS;
+            const int fit = (s_max + Sm - 1) / Sm;  // Sm slots must cover the longest unit
+            Q = (int)(even > fit ? even : fit);
+            if (Q < 1) Q = 1;
+            Sm = dkdv_segments(s_max, Q, Sm);
+            if (Sm < 1) Sm = 1;
+        }
+        plan[1] = Gs;
+        plan[2] = Sm;
+        plan[4] = Q;
+    }
+}
+
+// FDMA_COMPACT: 0 = never, 2 = whenever the mask form allows it, anything else / unset = when it also pays.
+// Read on every call, so that one process can time both paths.
+int compaction_mode() {
+    const char *e = getenv("FDMA_COMPACT");
+    return (e && e[0] == '0') ? 0 : ((e && e[0] == '2') ? 2 : 1);
 }
 
 }  // namespace
 
 bool use_compact(const FwdParams &p) {
-    if (!compaction_enabled() || !p.mask || p.m_r != 0) return false;
+    const int mode = compaction_mode();
+    if (mode == 0 || !p.mask || p.m_r != 0) return false;
     if (p.bias && p.bi_r != 0) return false;
     if (!(p.Hm == 1 || p.Hm == p.Hk)) return false;
-    // the pre-pass costs about one copy of K and V; it pays once a pair has a few query tiles
-    return p.Lq >= 128 && p.Lk >= 128 && (int64_t)p.Lk * p.d < (int64_t)1 << 31;
+    if (p.Lq < 2 || p.Lk < 1 || (int64_t)p.Lk * p.d >= (int64_t)1 << 31) return false;
+    if (mode == 2) return true;
+    // the pre-pass costs about one copy of K and V plus three small launches; it pays once the attention
+    // itself is a few million (query, key) pairs per kv head
+    return p.Lq >= 128 && p.Lk >= 128 && (int64_t)p.Lq * (p.H / p.Hk) * p.Lk >= (int64_t)1 << 21;
 }
 
-size_t compact_bytes(const FwdParams &p) { return layout_of(p).total; }
+size_t compact_bytes(const FwdParams &p, bool backward) { return layout_of(p, backward).total; }
 
-hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream) {
-    const Layout l = layout_of(p);
+void dkdv_split_bounds(int pairs, int n_max, int G, int &grid, int &slots) {
+    const int k = dkdv_lists_per_pair(pairs);
+    const int lists_per_xcd = pairs * k / 8;
+    // n = units of the largest pair; the total U is then between n and pairs * n, and the split factor does
+    // not grow with U: the split of U = n bounds the workgroups, U * split(U) bounds the partial slots
+    int64_t items = 1, sl = 1;
+    for (int n = 1; n <= n_max; n++) {
+        int Gs, Sm;
+        dkdv_split(n, G, Gs, Sm);
+        const int64_t it = (int64_t)dkdv_list_len(n, k) * Gs * Sm;
+        if (it > items) items = it;
+        if (n >= DKDV_ENOUGH_UNITS) {  // no split from here on: the bound grows with n alone
+            const int64_t last = dkdv_list_len(n_max, k);
+            if (last > items) items = last;
+            break;
+        }
+    }
+    const int U_max = pairs * n_max < DKDV_ENOUGH_UNITS ? pairs * n_max : DKDV_ENOUGH_UNITS - 1;
+    for (int U = 1; U <= U_max; U++) {
+        int Gs, Sm;
+        dkdv_split(U, G, Gs, Sm);
+        if (Gs * Sm > 1 && (int64_t)U * Gs * Sm > sl) sl = (int64_t)U * Gs * Sm;
+    }
+    grid = (int)(8 * lists_per_xcd * items);
+    slots = (int)sl;
+}
+
+hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, BwdParams *bp) {
+    const Layout l = layout_of(p, bp != nullptr);
     char *w = static_cast<char *>(ws);
     int32_t *idx = (int32_t *)(w + l.off_idx), *cnt = (int32_t *)(w + l.off_cnt), *count = (int32_t *)(w + l.off_count);
     float *fb = (float *)(w + l.off_fb);
@@ -223,6 +313,15 @@ hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream) 
     else
         hipLaunchKernelGGL((compact_gather_kernel<fp16_tag>), grid, dim3(256), 0, stream, p, idx, count, fb, kc, vc, l.ld, l.Hfb);
     if ((e = hipGetLastError()) != hipSuccess) return e;
+    if (bp) {
+        int32_t *plan = (int32_t *)(w + l.off_plan);
+        hipLaunchKernelGGL(compact_plan_kernel, dim3(1), dim3(256), 0, stream, count, idx, l.ld, plan, pairs, p.H / p.Hk, p.Lq,
+                           p.Lk, p.causal);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        p.cmp.plan = plan;
+        bp->dkv_part = (float *)(w + l.off_part_kv);
+        bp->db_part = (float *)(w + l.off_part_db);
+    }
     p.k = kc;
     p.v = vc;
     p.k_r = p.v_r = p.d;

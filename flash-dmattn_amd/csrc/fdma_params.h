@@ -17,10 +17,65 @@ struct Compact {
     const int32_t *cnt;    // (B*Hk, ld): kept keys among the original columns 0..j (inclusive)
     const int32_t *count;  // (B*Hk): kept keys
     const float *fb;       // (B*Hfb, ld): bias * log2(e) of compacted key c (0 without a bias)
+    const int32_t *plan;   // backward only: work split of the dK/dV kernel, see DkdvPlan
     int32_t ld;            // row stride of the arrays above (Lk rounded up to 16)
     int32_t Hfb;           // heads of fb: Hk, or H when the bias differs per query head
     int32_t on;            // 0 = no compaction: k / v are the caller's tensors
 };
+
+// Work split of the compacted dK/dV kernel, made on the device once the kept-key counts are known.
+// A unit is one 128-key block of one (batch, kv head) pair; U = number of units.  With few units the
+// chip would idle (the kernel keeps K / V stationary and loops over query heads and query blocks), so
+// every unit is split over `Gs` groups of query heads and, once every head has its own group, over
+// segments of at most `Q` query blocks (a unit that fewer queries see gets fewer segments, so that parts
+// are of similar size); each part writes fp32 partial results that a reduce kernel sums in a fixed order.
+// Units go to the 8 XCDs (workgroup id % 8) pair by pair so that workgroups sharing an L2 stream the same
+// Q / dO tiles; with fewer than 8 pairs (or a pair count that 8 does not divide) a pair is folded into
+// k = 8 / gcd(pairs, 8) lists, unit u going to list snake(u mod 2k) -- low key blocks see the most queries
+// under a causal mask, and the fold gives every list the same mix of heavy and light units.
+//   plan[0] = U, plan[1] = Gs, plan[2] = Sm (segment slots per unit and head group), plan[3] = list length
+//   bound (units), plan[4] = Q, plan[8 + i] = first unit of pair i (i = 0..pairs)
+constexpr int DKDV_PLAN_HDR = 8;
+#ifndef FDMA_DKDV_TARGET
+#define FDMA_DKDV_TARGET 1024
+#endif
+constexpr int DKDV_TARGET_PARTS = FDMA_DKDV_TARGET;   // parts wanted in flight (4 per CU)
+constexpr int DKDV_ENOUGH_UNITS = 384;    // from here on the units alone fill the chip
+__host__ __device__ inline void dkdv_split(int U, int G, int &Gs, int &Sm) {
+    Gs = 1;
+    Sm = 1;
+    if (U <= 0 || U >= DKDV_ENOUGH_UNITS) return;
+    const int want = (DKDV_TARGET_PARTS + U - 1) / U;
+    for (int c = 2; c <= G && c <= want; c++)
+        if (G % c == 0) Gs = c;  // query heads first: largest divisor of G not above `want`
+    if (Gs == G) {  // upper bound of the segments per unit: twice the even split, units differ in length
+        Sm = 2 * want / G;
+        Sm = Sm < 1 ? 1 : (Sm > 16 ? 16 : Sm);
+    }
+}
+// query blocks (of 64 rows) that see a key block whose first key sits at original column `okey_first`
+__host__ __device__ inline int dkdv_query_blocks(int Lq, int Lk, int causal, int okey_first) {
+    const int M_blocks = (Lq + 63) / 64;
+    int m_start = 0;
+    if (causal) {
+        const int first_q = okey_first - (Lk - Lq);
+        if (first_q > 0) m_start = first_q / 64;
+        if (m_start > M_blocks) m_start = M_blocks;
+    }
+    return M_blocks - m_start;
+}
+// segments a unit with n_tot query blocks is cut into
+__host__ __device__ inline int dkdv_segments(int n_tot, int Q, int Sm) {
+    const int s = (n_tot + Q - 1) / Q;
+    return s < Sm ? s : Sm;
+}
+
+__host__ __device__ inline int dkdv_lists_per_pair(int pairs) {
+    return pairs % 8 == 0 ? 1 : (pairs % 4 == 0 ? 2 : (pairs % 2 == 0 ? 4 : 8));
+}
+__host__ __device__ inline int dkdv_list_len(int units_in_largest_pair, int k) {
+    return 2 * ((units_in_largest_pair + 2 * k - 1) / (2 * k));
+}
 
 struct FwdParams {
     const void *q, *k, *v;
@@ -58,6 +113,9 @@ struct BwdParams {
     int32_t Lq_rounded;
     float *dbias_accum;        // fp32 scratch at the dbias shape when several workgroups share an element
     int64_t dba_b, dba_h, dba_r;
+    // compacted dK/dV kernel, split mode: per part [2][Dpad][128] fp32 (dK^T, dV^T) and [G][128] fp32 (dBias)
+    float *dkv_part;
+    float *db_part;
 };
 
 // dtype: 0 = bf16, 1 = fp16.  All launches are asynchronous on `stream`; return hipError_t.
@@ -76,9 +134,13 @@ hipError_t launch_bwd_dq_colmask(const BwdParams &p, int dtype, hipStream_t stre
 // the scratch it needs, compact_setup() launches the gather pre-pass into `ws` and rewrites p.k / p.v /
 // p.cmp; compact_zero_dropped() zero-fills the gradient rows / columns of dropped keys.
 bool use_compact(const FwdParams &p);
-size_t compact_bytes(const FwdParams &p);
-hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream);
+size_t compact_bytes(const FwdParams &p, bool backward);
+// bp != nullptr: backward -- also plans the dK/dV split and sets bp->dkv_part / bp->db_part
+hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, BwdParams *bp = nullptr);
 hipError_t compact_zero_dropped(const BwdParams &p, const FwdParams &orig, hipStream_t stream);
+// host-side bounds over every possible unit count 1..U_max: workgroups to launch, partial slots to hold
+// (n_max = units of one pair at most)
+void dkdv_split_bounds(int pairs, int n_max, int G, int &grid, int &slots);
 
 // number of KV splits the decode path uses for this shape (1 = no workspace needed)
 int decode_num_splits(int B, int Hk, int Lk);

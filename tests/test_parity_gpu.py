@@ -8,6 +8,9 @@ compared with the oracle on identical seeded inputs:
 Tolerances (bf16 compute): max-abs error of the output <= 2e-2; gradients within rtol 5e-2 as
 defined in _util.assert_grad_close.
 """
+import functools
+import os
+
 import pytest
 import torch
 
@@ -25,6 +28,15 @@ def _op():
 
 def _to_dev(*ts):
     return [t.to(DEV) if t is not None else None for t in ts]
+
+
+@pytest.fixture(autouse=True)
+def _default_compaction_mode():
+    """FDMA_COMPACT picks the path for query-broadcast masks (0 = tile skipping, 2 = column compaction whenever
+    the mask form allows it, unset = the library's own cost rule); the library reads it on every call."""
+    os.environ.pop("FDMA_COMPACT", None)
+    yield
+    os.environ.pop("FDMA_COMPACT", None)
 
 
 def _run_fwd_bwd(q, k, v, mask, bias, causal, scale=None, dout=None, need_grad=True):
@@ -78,17 +90,35 @@ SMALL_CASES = {
 }
 
 
-@pytest.mark.parametrize("name", list(SMALL_CASES))
-def test_forward_backward_vs_c_oracle(name):
+@functools.lru_cache(maxsize=None)
+def _small_case(name):
     B, Lq, Lk, H, Hk, D, bshape, mshape, W, causal = SMALL_CASES[name]
     q, k, v, mask, bias = make_inputs(B, Lq, Lk, H, Hk, D, bshape, mshape, W, seed=0)
     dout = torch.randn(B, Lq, H, D, generator=torch.Generator().manual_seed(1)).to(torch.bfloat16)
+    fwd = c_oracle.forward(q, k, v, mask, bias, None, causal)
+    bwd = c_oracle.backward(q, k, v, dout, mask, bias, None, causal)
+    return (q, k, v, mask, bias, dout), fwd, bwd
+
+
+def _eligible_for_compaction(name):
+    mshape, Hk = SMALL_CASES[name][7], SMALL_CASES[name][4]
+    bshape = SMALL_CASES[name][6]
+    return (mshape is not None and mshape[2] == 1 and mshape[1] in (1, Hk) and (bshape is None or bshape[2] == 1)
+            and SMALL_CASES[name][1] > 1)
+
+
+@pytest.mark.parametrize("compact", ["0", "2"])
+@pytest.mark.parametrize("name", list(SMALL_CASES))
+def test_forward_backward_vs_c_oracle(name, compact):
+    if compact == "2" and not _eligible_for_compaction(name):
+        pytest.skip("mask form has no column-compaction path; covered by the other mode")
+    os.environ["FDMA_COMPACT"] = compact
+    B, Lq, Lk, H, Hk, D, bshape, mshape, W, causal = SMALL_CASES[name]
+    (q, k, v, mask, bias, dout), (ro, rl), (rdq, rdk, rdv, rdb) = _small_case(name)
     out, lse, (dq, dk, dv, db) = _run_fwd_bwd(q, k, v, mask, bias, causal, dout=dout)
-    ro, rl = c_oracle.forward(q, k, v, mask, bias, None, causal)
     assert out.dtype == torch.bfloat16 and out.shape == q.shape and lse.shape == (B, H, Lq)
     assert_out_close(out.cpu(), ro)
     _check_lse(lse.cpu(), rl)
-    rdq, rdk, rdv, rdb = c_oracle.backward(q, k, v, dout, mask, bias, None, causal)
     assert_grad_close(dq.cpu(), rdq, "dq")
     assert_grad_close(dk.cpu(), rdk, "dk")
     assert_grad_close(dv.cpu(), rdv, "dv")
@@ -97,7 +127,9 @@ def test_forward_backward_vs_c_oracle(name):
         assert_grad_close(db.cpu(), rdb, "dbias")
 
 
-def test_fp16_inputs():
+@pytest.mark.parametrize("compact", ["0", "2"])
+def test_fp16_inputs(compact):
+    os.environ["FDMA_COMPACT"] = compact
     q, k, v, mask, bias = make_inputs(1, 256, 256, 2, 1, 64, (1, 1, 1, 256), (1, 1, 1, 256), 128, seed=0, dtype=torch.float16)
     out, lse, (dq, dk, dv, db) = _run_fwd_bwd(q, k, v, mask, bias, True)
     ro, rl = c_oracle.forward(q, k, v, mask, bias, None, True)
@@ -116,7 +148,8 @@ def test_cfg1_reference_plumbing_config():
     full = colmask.expand(1, 1, 256, 256) & torch.tril(torch.ones(256, 256, dtype=torch.bool))
     ro, rl = c_oracle.forward(q, k, v, full, bias, 0.125, True)
     rdq, rdk, rdv, rdb = c_oracle.backward(q, k, v, torch.ones_like(ro), full, bias, 0.125, True)
-    for m in (full, colmask):
+    for m, compact in ((full, "1"), (colmask, "0"), (colmask, "2")):
+        os.environ["FDMA_COMPACT"] = compact
         out, lse, (dq, dk, dv, db) = _run_fwd_bwd(q, k, v, m, bias, True, scale=0.125)
         assert_out_close(out.cpu(), ro)
         _check_lse(lse.cpu(), rl)
@@ -174,6 +207,7 @@ def test_column_mask_with_an_all_dropped_pair_and_late_first_key():
     """Query-broadcast mask whose (batch 0, kv head 1) row keeps nothing and whose other rows keep no key
     before column 150: that pair's outputs and gradients are exactly zero, rows that see no kept key give
     O = 0 / LSE = +inf, and everything else matches the oracle."""
+    os.environ["FDMA_COMPACT"] = "2"
     B, L, H, Hk, D = 2, 320, 4, 2, 64
     q, k, v, mask, bias = make_inputs(B, L, L, H, Hk, D, (B, Hk, 1, L), (B, Hk, 1, L), 60, seed=5)
     mask[..., :150] = False
@@ -203,8 +237,13 @@ def test_seqlen_k_zero_and_no_grad_path():
     assert o.shape == q2.shape and not o.requires_grad
 
 
-def test_deterministic_rerun_is_bit_identical():
-    q, k, v, mask, bias = make_inputs(2, 384, 384, 4, 2, 64, (2, 2, 384, 384), (2, 2, 384, 384), 96, seed=7)
+@pytest.mark.parametrize("form", ["per_query_mask", "column_mask_compacted"])
+def test_deterministic_rerun_is_bit_identical(form):
+    if form == "per_query_mask":
+        q, k, v, mask, bias = make_inputs(2, 384, 384, 4, 2, 64, (2, 2, 384, 384), (2, 2, 384, 384), 96, seed=7)
+    else:  # dK / dV blocks split over several workgroups, partial sums folded in a fixed order
+        os.environ["FDMA_COMPACT"] = "2"
+        q, k, v, mask, bias = make_inputs(2, 640, 640, 4, 2, 64, (2, 4, 1, 640), (2, 2, 1, 640), 300, seed=7)
     a = _run_fwd_bwd(q, k, v, mask, bias, True)
     b = _run_fwd_bwd(q, k, v, mask, bias, True)
     assert torch.equal(a[0], b[0]) and torch.equal(a[1], b[1])
@@ -302,7 +341,11 @@ def test_direct_c_abi_call_without_the_python_operator():
     lse = torch.empty(1, 2, 128, dtype=torch.float32, device=DEV)
     a = _cabi.FwdArgs()
     _cabi.fill_fwd(a, qd, kd, vd, md, bd, out, lse, 0.125, True, 0.0)
+    os.environ["FDMA_COMPACT"] = "0"
+    assert _cabi.lib.fdma_fwd_workspace_bytes(a) == 0
+    os.environ["FDMA_COMPACT"] = "2"
     need = _cabi.lib.fdma_fwd_workspace_bytes(a)
+    assert need > 0
     if need:  # a caller that ignores the scratch request gets an error code and a message, not a fault
         assert _cabi.lib.fdma_fwd(a, _cabi.current_stream(qd.device)) == -3
         assert "workspace too small" in _cabi.last_error()
