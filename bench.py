@@ -116,9 +116,11 @@ def count_tiles(mask, Lq, Lk, causal, H, tile=64):
 
 def compaction_applies(mask, c):
     """Mirror of the library's rule for taking the column-compaction path (query-broadcast keep-mask with
-    1 or Hkv heads, at least 128 queries and keys, not switched off)."""
-    return (mask.shape[2] == 1 and mask.shape[1] in (1, c["Hk"]) and c["Lq"] >= 128 and c["Lk"] >= 128
-            and os.environ.get("FDMA_COMPACT", "1")[:1] != "0")
+    1 or Hkv heads, a problem large enough for the pre-pass to pay, not switched off)."""
+    mode = os.environ.get("FDMA_COMPACT", "1")[:1]
+    form_ok = mask.shape[2] == 1 and mask.shape[1] in (1, c["Hk"]) and c["Lq"] >= 2
+    pays = c["Lq"] >= 128 and c["Lk"] >= 128 and c["Lq"] * (c["H"] // c["Hk"]) * c["Lk"] >= 1 << 21
+    return mode != "0" and form_ok and (mode == "2" or pays)
 
 
 def count_compacted_tiles(mask, Lq, Lk, causal, H, tile=64):

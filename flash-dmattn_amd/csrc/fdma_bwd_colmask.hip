@@ -139,6 +139,10 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
             const int c = ks * 16 + g * 8;
             u32x4_t kv = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
             if (c < f.d) { kv = *(const u32x4_t *)(kp + c); vv = *(const u32x4_t *)(vp + c); }
+            // K is only used for the scores here: scale it by softmax_scale * log2(e) once, so that the MFMA
+            // accumulates exp2-domain scores on top of the column constant (no multiply per element later)
+#pragma unroll
+            for (int e = 0; e < 4; e++) kv[e] = E::pack2(E::lo(kv[e]) * f.scale_log2, E::hi(kv[e]) * f.scale_log2);
             kf[ks] = kv;
             vf[ks] = vv;
         }
@@ -261,7 +265,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
 #pragma unroll
         for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-            for (int i = 0; i < 16; i++) { s[mb][i] = 0.f; dp[mb][i] = 0.f; }
+            for (int i = 0; i < 16; i++) { s[mb][i] = cconst; dp[mb][i] = 0.f; }
         {
             constexpr int NF = 2 * MB * KS, FR = 8;  // fragment f: (ks, mb, which) with which = 0: Q, 1: dO
             u32x4_t a[NF];
@@ -280,7 +284,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
             }
         }
 
-        // ---- P = exp2(S*scale*log2e + c - LSE*log2e) ; dS = P * (dP - D)
+        // ---- P = exp2(S - LSE*log2e), S already scaled and offset by the column constant ; dS = P * (dP - D)
         // diagonal step: some (query, key) pairs of this wave are above the causal diagonal
         const bool diag = CAUSAL && (okey_wlast > m0 + shift);
         uint32_t ppk[MB * 8], dpk[MB * 8];
@@ -299,8 +303,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
                     const int ii = 8 * blk + e;
                     const float lse2 = e < 4 ? l0[e] : l1[e - 4];
                     const float dd = e < 4 ? d0[e] : d1[e - 4];
-                    const float x = fmaf(s[mb][ii], f.scale_log2, cconst) - lse2;
-                    pv[e] = fast_exp2(x);
+                    pv[e] = fast_exp2(s[mb][ii] - lse2);
                     dsv[e] = dp[mb][ii] - dd;
                 }
                 if (diag) {
@@ -623,10 +626,10 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
         }
     }
     __syncthreads();
-    auto next_active = [&](int j) -> int {
+    auto next_active = [&](int j) -> int {  // wave-uniform: keeps tile bases and loop conditions scalar
         if (CMP) return j < n_end ? j : n_end;
         while (j < n_end) {
-            const uint32_t w = sBits[j >> 5] >> (j & 31);
+            const uint32_t w = __builtin_amdgcn_readfirstlane(sBits[j >> 5]) >> (j & 31);
             if (w) {
                 j += __builtin_ctz(w);
                 return j < n_end ? j : n_end;
@@ -646,6 +649,9 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
             const int c = ks * 16 + g * 8;
             u32x4_t qv = {0, 0, 0, 0}, dv = {0, 0, 0, 0};
             if (qrow < f.Lq && c < f.d) { qv = *(const u32x4_t *)(qp + c); dv = *(const u32x4_t *)(dp + c); }
+            // Q only feeds the scores in this kernel: scale it by softmax_scale * log2(e) once
+#pragma unroll
+            for (int e = 0; e < 4; e++) qv[e] = E::pack2(E::lo(qv[e]) * f.scale_log2, E::hi(qv[e]) * f.scale_log2);
             qf[ks] = qv;
             dof[ks] = dv;
         }
@@ -727,7 +733,17 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
 #pragma unroll
         for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-            for (int ii = 0; ii < 16; ii++) { s[mb][ii] = 0.f; dp[mb][ii] = 0.f; }
+            for (int blk = 0; blk < 2; blk++) {  // the score accumulators start from the fused bias vector
+                const f32x4_t b0 = *(const f32x4_t *)(bs + 32 * mb + 16 * blk);
+                const f32x4_t b1 = *(const f32x4_t *)(bs + 32 * mb + 16 * blk + 4);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    s[mb][8 * blk + e] = b0[e];
+                    s[mb][8 * blk + 4 + e] = b1[e];
+                    dp[mb][8 * blk + e] = 0.f;
+                    dp[mb][8 * blk + 4 + e] = 0.f;
+                }
+            }
         {
             constexpr int NF = 2 * MB * KS, FR = 8;
             u32x4_t a[NF];
@@ -752,14 +768,9 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
         for (int mb = 0; mb < MB; mb++)
 #pragma unroll
             for (int blk = 0; blk < 2; blk++) {
-                const f32x4_t b0 = *(const f32x4_t *)(bs + 32 * mb + 16 * blk);
-                const f32x4_t b1 = *(const f32x4_t *)(bs + 32 * mb + 16 * blk + 4);
                 float pv[8];
 #pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const float bl = e < 4 ? b0[e] : b1[e - 4];
-                    pv[e] = fast_exp2(fmaf(s[mb][8 * blk + e], f.scale_log2, bl) - lse2);
-                }
+                for (int e = 0; e < 8; e++) pv[e] = fast_exp2(s[mb][8 * blk + e] - lse2);
                 if (diag) {
                     asm volatile("" ::: "memory");
                     const int lim = vis_lane - 1 - n0 - 32 * mb - 16 * blk - 8 * g;  // local columns e <= lim are visible

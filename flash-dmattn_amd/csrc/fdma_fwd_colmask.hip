@@ -14,11 +14,14 @@
 //     Lk) staged in LDS, so the score epilogue is a single FMA per element;
 //   * causal masking costs instructions on diagonal tiles only.
 //
-// Pipeline: K tiles are double-buffered in LDS, V tiles are transposed in registers while being
-// staged and double-buffered as V^T, the fused bias vector is triple-buffered.  Global loads for
-// tile i+2 (K, bias) and i+1 (V) are in flight while tile i is computed; LDS fragment reads run a
-// batch ahead of the MFMAs that consume them.  Workgroup ids are remapped so that the workgroups
-// sharing one XCD's L2 also share K / V.
+// Pipeline: K, V^T (V is transposed in registers while being staged) and the fused bias vector are
+// double-buffered in LDS.  Tile i is computed from buffers i&1 while the global loads of tile i+1 are in
+// flight; their LDS stores go to the other buffers after the compute, so one barrier per tile suffices.
+// Q is scaled by softmax_scale*log2(e) once and the score accumulators start from the fused bias vector,
+// so the MFMA result is the exp2-domain score with bias and mask applied and the softmax spends five
+// vector instructions per element (max, sub, exp2, add, half a convert).  LDS fragment reads run a batch
+// ahead of the MFMAs that consume them.  Workgroup ids are remapped so that the workgroups sharing one
+// XCD's L2 also share K / V.
 #include "fdma_common.h"
 #include "fdma_params.h"
 
@@ -36,7 +39,7 @@ template <int D, int BN> struct CmSmem {
     static constexpr int OFF_K = 0;
     static constexpr int OFF_VT = OFF_K + 2 * K_BYTES;
     static constexpr int OFF_BIAS = OFF_VT + 2 * VT_BYTES;
-    static constexpr int OFF_BITS = OFF_BIAS + 3 * BN * 4;
+    static constexpr int OFF_BITS = OFF_BIAS + 2 * BN * 4;
     static constexpr int TOTAL = OFF_BITS + MAX_TILES / 8;
 };
 
@@ -44,11 +47,9 @@ template <int D, int BN> struct CmSmem {
 // `count` columns, all kept; the fused bias vector comes pre-gathered, and the causal limit of a query row
 // is the number of kept columns at or below its diagonal instead of the column index itself.
 template <typename T, int D, int NQ, int BN, bool CAUSAL, int NW, bool CMP>
-__global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(const FwdParams p) {
+__global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_colmask_kernel(const FwdParams p) {
     constexpr int NTHREADS = 64 * NW;
-    // with 8 waves the staging work is split by role: waves 0-3 stage V, waves 4-7 stage K and bias
-    constexpr bool SPLIT_ROLES = NW == 8;
-    constexpr int STHREADS = SPLIT_ROLES ? NTHREADS / 2 : NTHREADS;  // threads staging one operand
+    constexpr int STHREADS = NTHREADS;        // threads staging one operand
     using E = Elem<T>;
     using SM = CmSmem<D, BN>;
     constexpr int MB = BN / 32;               // 32-key blocks per tile
@@ -155,10 +156,12 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
     }
     __syncthreads();
 
-    auto next_active = [&](int j) -> int {  // smallest active tile >= j, or n_end
+    // smallest active tile >= j, or n_end.  The bitmap word comes from LDS; readfirstlane tells the compiler that
+    // the result is wave-uniform, so tile bases, loop conditions and load addresses stay in scalar registers.
+    auto next_active = [&](int j) -> int {
         if (CMP) return j < n_end ? j : n_end;
         while (j < n_end) {
-            uint32_t w = sBits[j >> 5] >> (j & 31);
+            const uint32_t w = __builtin_amdgcn_readfirstlane(sBits[j >> 5]) >> (j & 31);
             if (w) {
                 j += __builtin_ctz(w);
                 return j < n_end ? j : n_end;
@@ -180,6 +183,11 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
             const int c = ks * 16 + g * 8;
             u32x4_t v = {0, 0, 0, 0};
             if (qrow < p.Lq && c < p.d) v = *(const u32x4_t *)(qp + c);
+            // Q is scaled by softmax_scale * log2(e) once, here (the reference also rounds the scaled Q to the
+            // input type, flash_fwd_kernel.h:428-439): the MFMA then accumulates exp2-domain scores directly on
+            // top of the fused bias, with no per-element multiply afterwards
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = E::pack2(E::lo(v[e]) * p.scale_log2, E::hi(v[e]) * p.scale_log2);
             qf[nb][ks] = v;
         }
     }
@@ -199,9 +207,7 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
     // ---- staging helpers (global -> registers -> LDS)
     // Per-thread byte offsets inside a tile are 32-bit and computed once; the per-tile base is
     // wave-uniform, so a full tile costs no vector address arithmetic and no predication.
-    const bool k_role = !SPLIT_ROLES || tid >= STHREADS;
-    const bool v_role = !SPLIT_ROLES || tid < STHREADS;
-    const int ktid = SPLIT_ROLES ? (tid - STHREADS) & (STHREADS - 1) : tid;
+    const int ktid = tid;
     const int kc = ktid % CH, kr0 = ktid / CH;
     const int vkg = tid % KQ, vc = (tid / KQ) % CH;  // V: key quad and d chunk of this thread
     const bool k_dvalid = kc * 8 < p.d, v_dvalid = vc * 8 < p.d;
@@ -211,14 +217,10 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
 #pragma unroll
     for (int i = 0; i < 4; i++) voff[i] = (uint32_t)(((int64_t)(4 * vkg + i) * p.v_r + (v_dvalid ? vc * 8 : 0)) * 2);
     const bool d_full = p.d == D;
-    // staging registers; with split roles a thread stages either K or V, so the two share storage
-    u32x4_t stage_regs[SPLIT_ROLES ? 4 : K_IT + 4];
-    u32x4_t *kreg = stage_regs;
-    u32x4_t *vreg = stage_regs + (SPLIT_ROLES ? 0 : K_IT);
+    u32x4_t kreg[K_IT], vreg[4];  // staging registers
     float breg = 0.f;
 
     auto load_k = [&](int j) {
-        if (!k_role) return;
         const int n0 = j * BN;
         const char *tb = (const char *)kbase + (int64_t)n0 * p.k_r * 2;
         if (n0 + BN <= Lk) {
@@ -251,7 +253,6 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
         }
     };
     auto store_k = [&](int buf, int slot) {
-        if (!k_role) return;
         char *sK = smem + SM::OFF_K + buf * SM::K_BYTES;
 #pragma unroll
         for (int it = 0; it < K_IT; it++)
@@ -261,7 +262,7 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
     auto load_v = [&](int j) {
         const int n0 = j * BN;
         const char *tb = (const char *)vbase + (int64_t)n0 * p.v_r * 2;
-        if (v_role && tid < V_ITEMS) {
+        if (tid < V_ITEMS) {
             if (n0 + BN <= Lk) {
 #pragma unroll
                 for (int i = 0; i < 4; i++) vreg[i] = *(const u32x4_t *)(tb + voff[i]);
@@ -283,7 +284,7 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
     };
     auto store_v = [&](int buf) {  // transpose 4 keys x 8 d in registers, write V^T[d][key quad]
         char *sVt = smem + SM::OFF_VT + buf * SM::VT_BYTES;
-        if (v_role && tid < V_ITEMS) {
+        if (tid < V_ITEMS) {
 #pragma unroll
             for (int dd = 0; dd < 8; dd++) {
                 const int w = dd >> 1;
@@ -307,14 +308,24 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
         vis_wave[nb] = CAUSAL ? visible(wrow0 + nb * 32) : 0;
     }
 
-    auto qk = [&](f32x16_t (&s)[NQ][MB], int buf) {
+    auto qk = [&](f32x16_t (&s)[NQ][MB], int buf, int slot) {
         const char *sK = smem + SM::OFF_K + buf * SM::K_BYTES;
+        // the accumulators start from the fused bias vector (bias * log2e, -inf for dropped keys) of the tile
+        const float *bs = sBias + slot * BN + 8 * g;
 #pragma unroll
-        for (int nb = 0; nb < NQ; nb++)
+        for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-            for (int mb = 0; mb < MB; mb++)
+            for (int blk = 0; blk < 2; blk++) {
+                const f32x4_t b0 = *(const f32x4_t *)(bs + 32 * mb + 16 * blk);
+                const f32x4_t b1 = *(const f32x4_t *)(bs + 32 * mb + 16 * blk + 4);
 #pragma unroll
-                for (int i = 0; i < 16; i++) s[nb][mb][i] = 0.f;
+                for (int nb = 0; nb < NQ; nb++)
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        s[nb][mb][8 * blk + e] = b0[e];
+                        s[nb][mb][8 * blk + 4 + e] = b1[e];
+                    }
+            }
         // fragment reads run FR ahead of the MFMAs that consume them, so the LDS latency is paid once
         // per batch instead of once per MFMA; (ks, mb) order alternates accumulators
         constexpr int NF = MB * KS, FR = NF < 8 ? NF : 8;
@@ -332,7 +343,7 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
 #pragma unroll
             for (int nb = 0; nb < NQ; nb++) s[nb][mb] = E::mfma(a[f], qf[nb][ks], s[nb][mb]);
         }
-        __builtin_amdgcn_sched_group_barrier(0x100, FR, 0);
+        __builtin_amdgcn_sched_group_barrier(0x100, FR + 4 * MB, 0);
 #pragma unroll
         for (int f = 0; f < NF - FR; f++) {
             __builtin_amdgcn_sched_group_barrier(0x008, NQ, 0);
@@ -341,32 +352,14 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
         __builtin_amdgcn_sched_group_barrier(0x008, FR * NQ, 0);
     };
 
-    auto softmax_pv = [&](f32x16_t (&s)[NQ][MB], int j, int slot, int vbuf) {
+    // softmax of one tile: scores in `s` (exp2 domain, bias and mask already in) -> packed probabilities `pk`
+    auto softmax = [&](f32x16_t (&s)[NQ][MB], int j, uint32_t (&pk)[NQ][8 * MB]) {
         const int n0 = j * BN;
-        const float *bs = sBias + slot * BN;
-        float bl2[16 * MB];
-#pragma unroll
-        for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-            for (int blk = 0; blk < 2; blk++) {
-                const f32x4_t b0 = *(const f32x4_t *)(bs + 32 * mb + 16 * blk + 8 * g);
-                const f32x4_t b1 = *(const f32x4_t *)(bs + 32 * mb + 16 * blk + 8 * g + 4);
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    bl2[16 * mb + 8 * blk + e] = b0[e];
-                    bl2[16 * mb + 8 * blk + 4 + e] = b1[e];
-                }
-            }
-        uint32_t pk[NQ][8 * MB];
 #pragma unroll
         for (int nb = 0; nb < NQ; nb++) {
             // diagonal tile for this 32-row block? (wave-uniform)
             const bool diag = CAUSAL && (n0 + BN > vis_wave[nb]);
             float tmax = -INFINITY;
-#pragma unroll
-            for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-                for (int i = 0; i < 16; i++) s[nb][mb][i] = fmaf(s[nb][mb][i], p.scale_log2, bl2[16 * mb + i]);
             if (diag) {
                 asm volatile("" ::: "memory");  // keep this a real (wave-uniform) branch: only diagonal tiles pay
                 const int lim = vis_lane[nb] - 1 - n0 - 8 * g;  // local column limit for this lane
@@ -407,6 +400,9 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
                 }
             row_sum[nb] += psum;
         }
+    };
+    // O^T += V^T P^T for one tile
+    auto pv = [&](const uint32_t (&pk)[NQ][8 * MB], int vbuf) {
         const char *sVt = smem + SM::OFF_VT + vbuf * SM::VT_BYTES;
         {
             constexpr int NF = KB * DB, FR = NF < 8 ? NF : 8;
@@ -430,33 +426,34 @@ __global__ void __launch_bounds__(64 * NW, NQ == 1 ? 2 : 1) fwd_colmask_kernel(c
         }
     };
 
-    // ---- prologue: tiles t0 (K, bias, V) and t1 (K, bias)
-    int j0 = next_active(0);
-    if (j0 < n_end) {
-        int j1 = next_active(j0 + 1);
-        load_k(j0);
-        load_v(j0);
+    // ---- main loop: tile i is computed from LDS buffers i&1 while tile i+1 travels global -> registers; its LDS
+    // stores go to the other buffers (last read in iteration i-1) after the compute, one barrier per tile
+    int jc = next_active(0);
+    if (jc < n_end) {
+        load_k(jc);
+        load_v(jc);
         store_k(0, 0);
         store_v(0);
-        if (j1 < n_end) {
-            load_k(j1);
-            store_k(1, 1);
-        }
         __syncthreads();
 
         f32x16_t sa[NQ][MB];
-        int i = 0, jc = j0, jn1 = j1;
+        int i = 0;
         while (jc < n_end) {
-            const int jn2 = jn1 < n_end ? next_active(jn1 + 1) : n_end;
-            if (jn2 < n_end) load_k(jn2);
-            if (jn1 < n_end) load_v(jn1);
-            qk(sa, i & 1);
-            softmax_pv(sa, jc, i % 3, i & 1);
-            __syncthreads();  // every wave is done with K buffer i&1 before it is refilled
-            if (jn2 < n_end) store_k(i & 1, (i + 2) % 3);
-            if (jn1 < n_end) store_v((i + 1) & 1);
+            const int jn = next_active(jc + 1);
+            if (jn < n_end) {
+                load_k(jn);
+                load_v(jn);
+            }
+            qk(sa, i & 1, i & 1);
+            uint32_t pk[NQ][8 * MB];
+            softmax(sa, jc, pk);
+            pv(pk, i & 1);
+            if (jn < n_end) {
+                store_k((i + 1) & 1, (i + 1) & 1);
+                store_v((i + 1) & 1);
+            }
             __syncthreads();
-            i++; jc = jn1; jn1 = jn2;
+            i++; jc = jn;
         }
     }
 

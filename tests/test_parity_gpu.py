@@ -287,10 +287,15 @@ def test_cfg2_full_size_forward_properties():
     nonempty = torch.isfinite(lse).transpose(1, 2)[..., None].expand_as(ones)  # (B, L, H, 1)
     assert torch.equal(ones[nonempty], torch.ones_like(ones[nonempty]))
     assert torch.equal(ones[~nonempty], torch.zeros_like(ones[~nonempty]))
-    shifted, lse_s, _ = f(qd, kd, vd, md, bd + 2.0, None, True, None, None, True)
-    assert (shifted.float() - out.float()).abs().max().item() <= 2e-2
-    fin = torch.isfinite(lse)
-    assert (lse_s[fin] - lse[fin] - 2.0).abs().max().item() <= 2e-2
+    # the shift must not itself be rounded: quantise the bias to multiples of 1/32 inside (-2, 2), so that bias and
+    # bias + 2 are both exact in bf16 and the two calls see the same scores up to the constant
+    bq = (torch.round(bd.float() * 32) / 32).clamp_(-1.96875, 1.96875).to(bd.dtype)
+    base, lse_b, _ = f(qd, kd, vd, md, bq, None, True, None, None, True)
+    shifted, lse_s, _ = f(qd, kd, vd, md, bq + 2.0, None, True, None, None, True)
+    assert torch.equal((bq + 2.0).float(), bq.float() + 2.0)
+    assert (shifted.float() - base.float()).abs().max().item() <= 2e-2
+    fin = torch.isfinite(lse_b)
+    assert (lse_s[fin] - lse_b[fin] - 2.0).abs().max().item() <= 2e-2
     ro, rl = eager.attention_forward(qd[:, :, :4], kd[:, :, :1], vd[:, :, :1], md[:, :1], bd[:, :1], None, True)
     assert_out_close(out[:, :, :4], ro)
     _check_lse(lse[:, :4], rl)
