@@ -1,21 +1,28 @@
-// Forward dynamic-mask attention for gfx950.
+// Forward dynamic-mask attention for gfx950, general form: mask and / or bias vary per query row.
 //
 // Replaces compute_attn_1rowblock (csrc/flash_sparse_attn/src/flash_fwd_kernel.h:53-804) with its
 // online softmax (src/softmax.h:127-221), masking (src/mask.h:94-161) and mask-tile OR skip
 // (src/utils.h:339-352) of the reference.  Same math:
 //     S = Q K^T * scale + bias ; S[~mask or non-causal] = -inf ; P = softmax(S) ; O = P V
 // with the causal mask aligned bottom-right, O = 0 and LSE = +inf for rows with no visible key.
+// (Mask and bias that are absent or broadcast over queries take the kernels of fdma_fwd_colmask.hip.)
 //
-// One workgroup = 4 waves = BM (128) query rows of one (batch, head); each wave owns 32 rows.
-// The wave computes the TRANSPOSED score tile S^T = K Q^T with K rows as the MFMA A operand read
-// from LDS and its Q rows held in registers as the B operand, so a lane owns one query row and
-// the row max / row sum are in-lane reductions plus one cross-half swap.  P^T then feeds
-// O^T = V^T P^T straight from the accumulator registers; V^T comes from the row-major V tile in
-// LDS through transposing LDS reads.
+// One workgroup = 4 waves = 128 query rows of one (batch, head); each wave owns 32 rows and computes the
+// TRANSPOSED score tile S^T = K Q^T (K rows from LDS as the MFMA A operand, its pre-scaled Q rows in
+// registers as the B operand), so a lane owns one query row and row max / row sum are in-lane reductions
+// plus one cross-half swap.  P^T feeds O^T = V^T P^T straight from the accumulator registers.
+//
+// With a [Lq, Lk] bias (2 B) and mask (1 B) per score this path is bound by HBM, not by the matrix pipe, so the
+// kernel is built around the mask / bias stream:
+//   * every 128 x 64 mask and bias tile is fetched with coalesced 8- / 16-byte loads (a row's 64 keys are
+//     contiguous), fused in registers into one 16-bit tile (bias where kept, -inf where dropped or beyond Lk) and
+//     parked in LDS; the score accumulators then START from that tile, so bias and mask cost nothing later;
+//   * everything is double-buffered and fetched a tile ahead, the mask two tiles ahead: the workgroup-wide OR
+//     of the next tile's mask is known before that tile's bias / K / V loads are issued, and a tile without
+//     any kept element costs its mask bytes only (no bias, K, V traffic, no MFMA work);
+//   * one barrier per tile: the OR reduction is that barrier.
 #include "fdma_common.h"
 #include "fdma_params.h"
-
-#include <cstdlib>
 
 namespace fdma {
 
@@ -26,54 +33,57 @@ constexpr int BN = 64;
 constexpr int NTHREADS = 256;
 
 template <int D> struct FwdSmem {
-    static constexpr int SK = D + 8;    // K tile row stride (elements): conflict-free 16-byte row reads
-    static constexpr int SV = D + 32;   // V tile row stride: conflict-free transposing reads
+    static constexpr int SK = D + 8;     // K tile row stride (elements): conflict-free 16-byte row reads
+    static constexpr int SVT = BN + 8;   // V^T tile row stride
+    static constexpr int SF = BN + 8;    // fused mask+bias tile row stride
     static constexpr int K_BYTES = BN * SK * 2;
-    static constexpr int V_BYTES = BN * SV * 2;
-    static constexpr int TOTAL = K_BYTES + V_BYTES;
+    static constexpr int VT_BYTES = D * SVT * 2;
+    static constexpr int F_BYTES = BM * SF * 2;
+    static constexpr int STAGE = K_BYTES + VT_BYTES + F_BYTES;
+    static constexpr int TOTAL = 2 * STAGE;
 };
 
-// nonzero bytes of x -> bit k of the result is set iff byte k of x != 0
-__device__ __forceinline__ uint32_t nz_bytes_to_bits(uint32_t x) {
-    uint32_t y = (((x & 0x7f7f7f7fu) + 0x7f7f7f7fu) | x) & 0x80808080u;  // 0x80 per nonzero byte
-    return ((y >> 7) * 0x10204080u) >> 28;
-}
+template <typename T> struct NegInf2;
+template <> struct NegInf2<bf16_tag> { static constexpr uint32_t value = 0xFF80FF80u; };
+template <> struct NegInf2<fp16_tag> { static constexpr uint32_t value = 0xFC00FC00u; };
 
 template <typename T, int D, bool CAUSAL>
-__global__ void __launch_bounds__(NTHREADS, 2) fwd_kernel(const FwdParams p) {
+__global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) fwd_kernel(const FwdParams p) {
     using E = Elem<T>;
     using SM = FwdSmem<D>;
     constexpr int KS = D / 16;  // contraction steps of Q K^T
     constexpr int DB = D / 32;  // 32-wide blocks of the head dimension
+    constexpr int MB = BN / 32, KB = BN / 16, KQ = BN / 4;
+    constexpr int CH = D / 8;               // 16-byte chunks per K row
+    constexpr int K_RPP = NTHREADS / CH;    // K rows staged per pass
+    constexpr int K_IT = BN / K_RPP;
+    constexpr int V_ITEMS = KQ * CH;        // (key quad, d chunk) items of a V tile
+    constexpr int F_IT = BM * (BN / 8) / NTHREADS;  // 8-key chunks of the mask / bias tile per thread (4)
 
-    __shared__ __attribute__((aligned(16))) char smem[SM::TOTAL];
-    char *sK = smem;
-    char *sV = smem + SM::K_BYTES;
+    extern __shared__ __attribute__((aligned(16))) char smem[];
 
-    const int tid = threadIdx.x;
-    const int wave = tid >> 6;
-    const int lane = tid & 63;
-    const int r = lane & 31;
-    const int g = lane >> 5;
-
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 31, g = lane >> 5;
     const int m_block = gridDim.x - 1 - blockIdx.x;  // heaviest (most KV tiles) first under causal
-    const int h = blockIdx.y;
-    const int b = blockIdx.z;
+    const int h = blockIdx.y, b = blockIdx.z;
     const int hk = h / (p.H / p.Hk);
     const int m0 = m_block * BM;
-    const int qrow = m0 + wave * 32 + r;
-    const int qrow_c = qrow < p.Lq ? qrow : p.Lq - 1;
+    const int wrow0 = m0 + wave * 32;
+    const int qrow = wrow0 + r;
     const int shift = p.Lk - p.Lq;  // bottom-right causal alignment
 
-    // ---- Q fragments (B operand of S^T = K Q^T), kept in registers for the whole KV loop
+    // ---- Q fragments (B operand of S^T = K Q^T), scaled by softmax_scale * log2(e) once (the reference also rounds
+    // the scaled Q to the input type, flash_fwd_kernel.h:428-439) and kept in registers for the whole KV loop
     u32x4_t qf[KS];
     {
-        const uint16_t *qp = (const uint16_t *)p.q + b * p.q_b + (int64_t)qrow_c * p.q_r + h * p.q_h;
+        const int qc = qrow < p.Lq ? qrow : p.Lq - 1;
+        const uint16_t *qp = (const uint16_t *)p.q + b * p.q_b + (int64_t)qc * p.q_r + h * p.q_h;
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
-            int c = ks * 16 + g * 8;
+            const int c = ks * 16 + g * 8;
             u32x4_t v = {0, 0, 0, 0};
             if (qrow < p.Lq && c < p.d) v = *(const u32x4_t *)(qp + c);
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[e] = E::pack2(E::lo(v[e]) * p.scale_log2, E::hi(v[e]) * p.scale_log2);
             qf[ks] = v;
         }
     }
@@ -81,8 +91,9 @@ __global__ void __launch_bounds__(NTHREADS, 2) fwd_kernel(const FwdParams p) {
     int n_end = (p.Lk + BN - 1) / BN;
     if (CAUSAL) {
         int lim = m0 + BM + shift;  // first invisible column for the last row of the block
+        if (lim > p.Lq + shift) lim = p.Lq + shift;
         if (lim < 0) lim = 0;
-        int ne = (lim + BN - 1) / BN;
+        const int ne = (lim + BN - 1) / BN;
         if (ne < n_end) n_end = ne;
     }
 
@@ -91,148 +102,252 @@ __global__ void __launch_bounds__(NTHREADS, 2) fwd_kernel(const FwdParams p) {
     for (int db = 0; db < DB; db++)
 #pragma unroll
         for (int i = 0; i < 16; i++) o[db][i] = 0.f;
-    float row_max = -INFINITY;  // log2 domain
+    float row_max = -INFINITY;  // exp2 domain
     float row_sum = 0.f;        // per-lane partial (this lane's half of the keys)
 
     const int hm = p.mask ? (p.Hm == p.H ? h : (p.Hm == 1 ? 0 : h / (p.H / p.Hm))) : 0;
     const int hb = p.bias ? (p.Hb == p.H ? h : (p.Hb == 1 ? 0 : h / (p.H / p.Hb))) : 0;
-    const uint8_t *mrow = p.mask ? p.mask + b * p.m_b + hm * p.m_h + (int64_t)qrow_c * p.m_r : nullptr;
-    const uint16_t *brow = p.bias ? (const uint16_t *)p.bias + b * p.bi_b + hb * p.bi_h + (int64_t)qrow_c * p.bi_r : nullptr;
-
+    const uint8_t *mbase = p.mask ? p.mask + b * p.m_b + hm * p.m_h : nullptr;
+    const uint16_t *bbase = p.bias ? (const uint16_t *)p.bias + b * p.bi_b + hb * p.bi_h : nullptr;
     const uint16_t *kbase = (const uint16_t *)p.k + b * p.k_b + hk * p.k_h;
     const uint16_t *vbase = (const uint16_t *)p.v + b * p.v_b + hk * p.v_h;
 
-    // A-operand row of this lane inside a 32-row block of K
-    const int a_row = pi_row(r);
-    // transposing-read supplier coordinates (see lds_read_tr16)
-    const int tj = lane & 15, te = tj >> 2, tc = tj & 3;
-    const int tcp = (tc == 1) ? 2 : (tc == 2 ? 1 : tc);
-    const int tdh = (lane >> 4) & 1;
-    const uint32_t v_tr_off = (uint32_t)(((8 * g + te) * SM::SV + 16 * tdh + 4 * tcp) * 2);
+    // ---- staging maps
+    const int kc = tid % CH, kr0 = tid / CH;             // K: d chunk, first row
+    const int vkg = tid % KQ, vc = (tid / KQ) % CH;      // V: key quad, d chunk
+    const bool k_dvalid = kc * 8 < p.d, v_dvalid = vc * 8 < p.d;
+    const int fc = tid & 7, fr0 = tid >> 3;              // mask / bias: 8-key chunk, first row (rows fr0 + 32 it)
+    u32x4_t kreg[K_IT], vreg[4], breg[F_IT];
+    u32x2_t mreg[F_IT], mnext[F_IT];
 
-    for (int j = 0; j < n_end; j++) {
+    // All tile loads are unconditional, from clamped (always valid) addresses, so that they can be issued early and
+    // stay in flight; what a clamped load fetched in place of a missing element is neutralised later: the mask
+    // words are ANDed with a validity pattern when they are consumed, rows of K / V beyond Lk and head-dim chunks
+    // beyond d are finite duplicates that meet a -inf score or a zero Q fragment.
+    const int kcol = k_dvalid ? kc * 8 : 0, vcol = v_dvalid ? vc * 8 : 0;
+    auto load_mask = [&](int j, u32x2_t (&dst)[F_IT]) {
+        if (!mbase) return;
+        int kk = j * BN + 8 * fc;
+        kk = kk < p.Lk ? kk : 0;
+#pragma unroll
+        for (int it = 0; it < F_IT; it++) {
+            int row = m0 + fr0 + 32 * it;
+            row = row < p.Lq ? row : p.Lq - 1;
+            dst[it] = *(const u32x2_t *)(mbase + (int64_t)row * p.m_r + kk);
+        }
+    };
+    // validity of the chunks (rows < Lq, keys < Lk, not entirely above the causal diagonal) applied to the loaded
+    // mask words; returns "any element kept"
+    auto finish_mask = [&](int j, u32x2_t (&dst)[F_IT]) -> bool {
+        const int kk = j * BN + 8 * fc;
+        uint32_t any = 0;
+#pragma unroll
+        for (int it = 0; it < F_IT; it++) {
+            const int row = m0 + fr0 + 32 * it;
+            u32x2_t mv = mbase ? dst[it] : u32x2_t{0x01010101u, 0x01010101u};
+            const bool ok = row < p.Lq && kk < p.Lk && !(CAUSAL && kk > row + shift);
+            uint64_t keepm = ok ? ~0ull : 0ull;
+            if (kk + 8 > p.Lk && kk < p.Lk) keepm = (1ull << (8 * (p.Lk - kk))) - 1ull;  // chunk straddles the end of the keys
+            mv[0] &= (uint32_t)keepm;
+            mv[1] &= (uint32_t)(keepm >> 32);
+            dst[it] = mv;
+            any |= mv[0] | mv[1];
+        }
+        return any != 0;
+    };
+    // bias, K and V of tile j into registers
+    auto load_rest = [&](int j) {
         const int n0 = j * BN;
-        // ---- keep bits of this lane's 32 score elements: bit 16*mb + i  <->  key n0 + 32mb + 16(i/8) + 8g + i%8
-        uint32_t keep = 0;
+        if (bbase) {
+            int kk = n0 + 8 * fc;
+            kk = kk < p.Lk ? kk : 0;
 #pragma unroll
-        for (int mb = 0; mb < 2; mb++)
-#pragma unroll
-            for (int blk = 0; blk < 2; blk++) {
-                int c0 = n0 + 32 * mb + 16 * blk + 8 * g;
-                uint32_t bits = 0xffu;
-                if (mrow) {
-                    bits = 0;
-                    if (c0 < p.Lk) {
-                        u32x2_t mv = *(const u32x2_t *)(mrow + c0);
-                        bits = nz_bytes_to_bits(mv[0]) | (nz_bytes_to_bits(mv[1]) << 4);
-                    }
-                }
-                int lim = p.Lk;
-                if (CAUSAL) { int cl = qrow + 1 + shift; lim = cl < lim ? cl : lim; }
-                int nvis = lim - c0;  // columns c0 .. c0+nvis-1 visible
-                uint32_t vis = nvis >= 8 ? 0xffu : (nvis <= 0 ? 0u : ((1u << nvis) - 1u));
-                bits &= vis;
-                if (qrow >= p.Lq) bits = 0;
-                keep |= bits << (16 * mb + 8 * blk);
+            for (int it = 0; it < F_IT; it++) {
+                int row = m0 + fr0 + 32 * it;
+                row = row < p.Lq ? row : p.Lq - 1;
+                breg[it] = *(const u32x4_t *)(bbase + (int64_t)row * p.bi_r + kk);
             }
-        // workgroup-uniform activity; the barrier also fences LDS reuse from the previous tile
-        const int active = __syncthreads_or(keep != 0);
-        if (!active) continue;
-
-        // ---- stage K and V tiles into LDS (rows beyond Lk are zero-filled)
-        {
-            constexpr int CH = D / 8;           // 16-byte chunks per row
-            constexpr int RPP = NTHREADS / CH;  // rows per pass
-            const int c = tid % CH;
-            const int r0 = tid / CH;
+        } else {
 #pragma unroll
-            for (int it = 0; it < BN / RPP; it++) {
-                int row = r0 + it * RPP;
-                int key = n0 + row;
-                u32x4_t kv = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
-                if (key < p.Lk && c * 8 < p.d) {
-                    kv = *(const u32x4_t *)(kbase + (int64_t)key * p.k_r + c * 8);
-                    vv = *(const u32x4_t *)(vbase + (int64_t)key * p.v_r + c * 8);
-                }
-                *(u32x4_t *)(sK + (row * SM::SK + c * 8) * 2) = kv;
-                *(u32x4_t *)(sV + (row * SM::SV + c * 8) * 2) = vv;
+            for (int it = 0; it < F_IT; it++) breg[it] = u32x4_t{0, 0, 0, 0};
+        }
+#pragma unroll
+        for (int it = 0; it < K_IT; it++) {
+            int key = n0 + kr0 + it * K_RPP;
+            key = key < p.Lk ? key : p.Lk - 1;
+            kreg[it] = *(const u32x4_t *)(kbase + (int64_t)key * p.k_r + kcol);
+        }
+        if (tid < V_ITEMS) {
+#pragma unroll
+            for (int i = 0; i < 4; i++) {
+                int key = n0 + 4 * vkg + i;
+                key = key < p.Lk ? key : p.Lk - 1;
+                vreg[i] = *(const u32x4_t *)(vbase + (int64_t)key * p.v_r + vcol);
             }
         }
-        // bias fragment for this lane (log2 domain), fetched while the tile lands
-        float bl2[32];
+    };
+    // registers -> LDS stage `buf`: K rows, V transposed, mask and bias fused (bias where kept, -inf elsewhere)
+    auto store_stage = [&](int buf, const u32x2_t (&mv)[F_IT]) {
+        char *sK = smem + buf * SM::STAGE;
+        char *sVt = sK + SM::K_BYTES;
+        char *sF = sVt + SM::VT_BYTES;
 #pragma unroll
-        for (int mb = 0; mb < 2; mb++)
+        for (int it = 0; it < K_IT; it++)
+            *(u32x4_t *)(sK + ((kr0 + it * K_RPP) * SM::SK + kc * 8) * 2) = kreg[it];
+        if (tid < V_ITEMS) {
+#pragma unroll
+            for (int dd = 0; dd < 8; dd++) {
+                const int w = dd >> 1;
+                const uint32_t sel = (dd & 1) ? 0x07060302u : 0x05040100u;
+                u32x2_t out;
+                out[0] = __builtin_amdgcn_perm(vreg[1][w], vreg[0][w], sel);
+                out[1] = __builtin_amdgcn_perm(vreg[3][w], vreg[2][w], sel);
+                *(u32x2_t *)(sVt + ((vc * 8 + dd) * SM::SVT + 4 * vkg) * 2) = out;
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < F_IT; it++) {
+            u32x4_t bv = breg[it];
+#pragma unroll
+            for (int hlf = 0; hlf < 2; hlf++) {
+                uint32_t x = mv[it][hlf];
+                x = ((((x & 0x7f7f7f7fu) + 0x7f7f7f7fu) | x) >> 7) & 0x01010101u;  // nonzero byte -> 0x01
+                const uint32_t z = (x << 8) - x;                                      // 0x01 -> 0xFF per byte
+                const uint32_t m0w = __builtin_amdgcn_perm(0, z, 0x01010000u);        // [b0 b0 b1 b1]
+                const uint32_t m1w = __builtin_amdgcn_perm(0, z, 0x03030202u);        // [b2 b2 b3 b3]
+                bv[2 * hlf] = (bv[2 * hlf] & m0w) | (NegInf2<T>::value & ~m0w);
+                bv[2 * hlf + 1] = (bv[2 * hlf + 1] & m1w) | (NegInf2<T>::value & ~m1w);
+            }
+            *(u32x4_t *)(sF + ((fr0 + 32 * it) * SM::SF + 8 * fc) * 2) = bv;
+        }
+    };
+
+    const int a_row = pi_row(r);
+
+    // ---- one tile from LDS stage `buf`
+    auto compute = [&](int j, int buf) {
+        const int n0 = j * BN;
+        const char *sK = smem + buf * SM::STAGE;
+        const char *sVt = sK + SM::K_BYTES;
+        const char *sF = sVt + SM::VT_BYTES + ((wave * 32 + r) * SM::SF + 8 * g) * 2;
+        // scores start from the fused mask+bias tile (exp2 domain)
+        f32x16_t s[MB];
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
 #pragma unroll
             for (int blk = 0; blk < 2; blk++) {
-                int c0 = n0 + 32 * mb + 16 * blk + 8 * g;
-                u32x4_t bv = {0, 0, 0, 0};
-                if (brow && c0 < p.Lk) bv = *(const u32x4_t *)(brow + c0);
+                const u32x4_t fv = *(const u32x4_t *)(sF + (32 * mb + 16 * blk) * 2);
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    bl2[16 * mb + 8 * blk + 2 * e] = E::lo(bv[e]) * kLog2e;
-                    bl2[16 * mb + 8 * blk + 2 * e + 1] = E::hi(bv[e]) * kLog2e;
+                    s[mb][8 * blk + 2 * e] = E::lo(fv[e]) * kLog2e;
+                    s[mb][8 * blk + 2 * e + 1] = E::hi(fv[e]) * kLog2e;
                 }
             }
-        __syncthreads();
-
-        // ---- S^T = K Q^T
-        f32x16_t s[2];
+        {
+            constexpr int NF = MB * KS, FR = NF < 8 ? NF : 8;
+            u32x4_t a[NF];
+            auto frag = [&](int f) {
+                const int ks = f / MB, mb = f % MB;
+                return *(const u32x4_t *)(sK + ((32 * mb + a_row) * SM::SK + ks * 16 + g * 8) * 2);
+            };
 #pragma unroll
-        for (int mb = 0; mb < 2; mb++) {
+            for (int f = 0; f < FR; f++) a[f] = frag(f);
 #pragma unroll
-            for (int i = 0; i < 16; i++) s[mb][i] = 0.f;
-#pragma unroll
-            for (int ks = 0; ks < KS; ks++) {
-                u32x4_t a = *(const u32x4_t *)(sK + ((32 * mb + a_row) * SM::SK + ks * 16 + g * 8) * 2);
-                s[mb] = E::mfma(a, qf[ks], s[mb]);
+            for (int f = 0; f < NF; f++) {
+                if (f + FR < NF) a[f + FR] = frag(f + FR);
+                s[f % MB] = E::mfma(a[f], qf[f / MB], s[f % MB]);
             }
         }
-
-        // ---- scale, bias, mask, online softmax (log2 domain)
+        // causal selects on diagonal tiles only (wave-uniform branch)
+        if (CAUSAL && n0 + BN - 1 > wrow0 + shift) {
+            asm volatile("" ::: "memory");
+            const int lim = qrow + shift - n0 - 8 * g;  // local column limit for this lane
+#pragma unroll
+            for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) {
+                    const int lc = 32 * mb + 16 * (i >> 3) + (i & 7);
+                    s[mb][i] = lc <= lim ? s[mb][i] : -INFINITY;
+                }
+        }
         float tmax = -INFINITY;
 #pragma unroll
-        for (int mb = 0; mb < 2; mb++)
+        for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-            for (int i = 0; i < 16; i++) {
-                float x = fmaf(s[mb][i], p.scale_log2, bl2[16 * mb + i]);
-                x = ((keep >> (16 * mb + i)) & 1u) ? x : -INFINITY;
-                s[mb][i] = x;
-                tmax = fmaxf(tmax, x);
-            }
+            for (int i = 0; i < 16; i++) tmax = fmaxf(tmax, s[mb][i]);
         tmax = xhalf_max(tmax);
-        const float new_max = fmaxf(row_max, tmax);
-        const float safe_max = new_max == -INFINITY ? 0.f : new_max;
-        const float alpha = fast_exp2(row_max - safe_max);  // row_max = -inf -> 0
-        row_max = new_max;
-        float psum = 0.f;
-        uint32_t pk[16];
+        if (__any(tmax > row_max)) {
+            const float new_max = fmaxf(row_max, tmax);
+            const float safe = new_max == -INFINITY ? 0.f : new_max;
+            const float alpha = fast_exp2(row_max - safe);
+            row_max = new_max;
+            row_sum *= alpha;
 #pragma unroll
-        for (int mb = 0; mb < 2; mb++)
+            for (int db = 0; db < DB; db++)
+#pragma unroll
+                for (int i = 0; i < 16; i++) o[db][i] *= alpha;
+        }
+        const float m_use = row_max == -INFINITY ? 0.f : row_max;
+        float psum = 0.f;
+        uint32_t pk[8 * MB];
+#pragma unroll
+        for (int mb = 0; mb < MB; mb++)
 #pragma unroll
             for (int i = 0; i < 16; i += 2) {
-                float p0 = fast_exp2(s[mb][i] - safe_max);
-                float p1 = fast_exp2(s[mb][i + 1] - safe_max);
+                const float p0 = fast_exp2(s[mb][i] - m_use);
+                const float p1 = fast_exp2(s[mb][i + 1] - m_use);
                 psum += p0 + p1;
                 pk[8 * mb + i / 2] = E::pack2(p0, p1);
             }
-        row_sum = row_sum * alpha + psum;
+        row_sum += psum;
+        {
+            constexpr int NF = KB * DB, FR = NF < 8 ? NF : 8;
+            u32x4_t a[NF];
+            auto frag = [&](int f) {
+                const int kb = f / DB, db = f % DB;
+                return *(const u32x4_t *)(sVt + ((32 * db + a_row) * SM::SVT + 16 * kb + 8 * g) * 2);
+            };
 #pragma unroll
-        for (int db = 0; db < DB; db++)
+            for (int f = 0; f < FR; f++) a[f] = frag(f);
 #pragma unroll
-            for (int i = 0; i < 16; i++) o[db][i] *= alpha;
-
-        // ---- O^T += V^T P^T
-#pragma unroll
-        for (int kb = 0; kb < 4; kb++) {
-            u32x4_t bop = {pk[4 * kb], pk[4 * kb + 1], pk[4 * kb + 2], pk[4 * kb + 3]};
-#pragma unroll
-            for (int db = 0; db < DB; db++) {
-                uint32_t off = v_tr_off + (uint32_t)((16 * kb * SM::SV + 32 * db) * 2);
-                u32x2_t lo = lds_read_tr16(sV, off);
-                u32x2_t hi = lds_read_tr16(sV, off + 4 * SM::SV * 2);
-                u32x4_t a = {lo[0], lo[1], hi[0], hi[1]};
-                o[db] = E::mfma(a, bop, o[db]);
+            for (int f = 0; f < NF; f++) {
+                if (f + FR < NF) a[f + FR] = frag(f + FR);
+                const int kb = f / DB, db = f % DB;
+                const u32x4_t bop = {pk[4 * kb], pk[4 * kb + 1], pk[4 * kb + 2], pk[4 * kb + 3]};
+                o[db] = E::mfma(a[f], bop, o[db]);
             }
+        }
+    };
+
+    // ---- main loop.  At the top of iteration j: tile j sits in LDS stage j&1 if it is active, `mreg` holds
+    // the mask of tile j+1 and `act_next` says whether that tile has any kept element.
+    if (n_end > 0) {
+        load_mask(0, mreg);
+        if (n_end > 1) load_mask(1, mnext);
+        bool act_cur = __syncthreads_or(finish_mask(0, mreg));
+        if (act_cur) {
+            load_rest(0);
+            store_stage(0, mreg);
+        }
+        bool act_next = __syncthreads_or(n_end > 1 && finish_mask(1, mnext));
+        // one iteration; `m_next` holds the (finished) mask of tile j+1, `m_new` receives the mask of tile j+2.
+        // The scheduling barriers keep the loads at the top and their first use below the compute: their
+        // latency is then covered by the MFMA work instead of being waited for right away.
+        auto step = [&](int j, u32x2_t (&m_next)[F_IT], u32x2_t (&m_new)[F_IT]) {
+            const bool have_next = j + 1 < n_end && act_next;
+            if (have_next) load_rest(j + 1);
+            if (j + 2 < n_end) load_mask(j + 2, m_new);
+            __builtin_amdgcn_sched_barrier(0);
+            if (act_cur) compute(j, j & 1);
+            __builtin_amdgcn_sched_barrier(0);
+            if (have_next) store_stage((j + 1) & 1, m_next);
+            const bool act_nn = __syncthreads_or(j + 2 < n_end && finish_mask(j + 2, m_new));
+            act_cur = have_next;
+            act_next = act_nn;
+        };
+        for (int j = 0; j < n_end; j += 2) {
+            step(j, mnext, mreg);
+            if (j + 1 < n_end) step(j + 1, mreg, mnext);
         }
     }
 
@@ -245,7 +360,7 @@ __global__ void __launch_bounds__(NTHREADS, 2) fwd_kernel(const FwdParams p) {
         for (int db = 0; db < DB; db++)
 #pragma unroll
             for (int blk = 0; blk < 2; blk++) {
-                int c = 32 * db + 16 * blk + 8 * g;
+                const int c = 32 * db + 16 * blk + 8 * g;
                 if (c < p.d) {
                     u32x4_t w;
 #pragma unroll
@@ -255,30 +370,33 @@ __global__ void __launch_bounds__(NTHREADS, 2) fwd_kernel(const FwdParams p) {
                 }
             }
         if (g == 0) {
-            float lse = total > 0.f ? (row_max + __builtin_amdgcn_logf(total)) * kLn2 : INFINITY;
+            const float lse = total > 0.f ? (row_max + __builtin_amdgcn_logf(total)) * kLn2 : INFINITY;
             p.lse[((int64_t)b * p.H + h) * p.Lq + qrow] = lse;
         }
     }
 }
 
+template <typename T, int D, bool CAUSAL>
+hipError_t launch_fwd_c(const FwdParams &p, hipStream_t stream) {
+    auto kern = fwd_kernel<T, D, CAUSAL>;
+    const int smem = FwdSmem<D>::TOTAL;
+    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    if (e != hipSuccess) return e;
+    dim3 grid((p.Lq + BM - 1) / BM, p.H, p.B);
+    hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, stream, p);
+    return hipGetLastError();
+}
+
 template <typename T, int D>
 hipError_t launch_fwd_t(const FwdParams &p, hipStream_t stream) {
-    dim3 grid((p.Lq + BM - 1) / BM, p.H, p.B);
-    dim3 block(NTHREADS);
-    if (p.causal)
-        hipLaunchKernelGGL((fwd_kernel<T, D, true>), grid, block, 0, stream, p);
-    else
-        hipLaunchKernelGGL((fwd_kernel<T, D, false>), grid, block, 0, stream, p);
-    return hipGetLastError();
+    return p.causal ? launch_fwd_c<T, D, true>(p, stream) : launch_fwd_c<T, D, false>(p, stream);
 }
 
 }  // namespace
 
 hipError_t launch_fwd(const FwdParams &p, int dtype, hipStream_t stream) {
     if (p.Lq <= 0 || p.B <= 0) return hipSuccess;
-    if (fwd_colmask_applicable(p)) {
-        return launch_fwd_colmask(p, dtype, 1, stream);
-    }
+    if (fwd_colmask_applicable(p)) return launch_fwd_colmask(p, dtype, 1, stream);
     const bool d64 = p.d <= 64;
     if (dtype == 0) return d64 ? launch_fwd_t<bf16_tag, 64>(p, stream) : launch_fwd_t<bf16_tag, 128>(p, stream);
     return d64 ? launch_fwd_t<fp16_tag, 64>(p, stream) : launch_fwd_t<fp16_tag, 128>(p, stream);
