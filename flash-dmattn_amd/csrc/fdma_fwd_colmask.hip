@@ -205,81 +205,84 @@ __global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_col
     }
 
     // ---- staging helpers (global -> registers -> LDS)
-    // Per-thread byte offsets inside a tile are 32-bit and computed once; the per-tile base is
-    // wave-uniform, so a full tile costs no vector address arithmetic and no predication.
+    // Every load is unconditional, from an always valid address: rows beyond the end of the keys are clamped to
+    // the last row (their fused bias is -inf, so the duplicate never counts) and head-dim chunks beyond d to chunk
+    // 0 (they meet zero Q fragments / columns of O that are not stored).  That keeps the loads free of branches,
+    // so that they can be issued one by one between the MFMAs of the tile being computed.
     const int ktid = tid;
     const int kc = ktid % CH, kr0 = ktid / CH;
     const int vkg = tid % KQ, vc = (tid / KQ) % CH;  // V: key quad and d chunk of this thread
-    const bool k_dvalid = kc * 8 < p.d, v_dvalid = vc * 8 < p.d;
-    uint32_t koff[K_IT], voff[4];
-#pragma unroll
-    for (int it = 0; it < K_IT; it++) koff[it] = (uint32_t)(((int64_t)(kr0 + it * K_RPP) * p.k_r + (k_dvalid ? kc * 8 : 0)) * 2);
-#pragma unroll
-    for (int i = 0; i < 4; i++) voff[i] = (uint32_t)(((int64_t)(4 * vkg + i) * p.v_r + (v_dvalid ? vc * 8 : 0)) * 2);
-    const bool d_full = p.d == D;
+    const uint32_t k_r2 = (uint32_t)(p.k_r * 2), v_r2 = (uint32_t)(p.v_r * 2);  // bytes per row
+    const uint32_t kcolb = (kc * 8 < p.d ? kc * 16 : 0), vcolb = (vc * 8 < p.d ? vc * 16 : 0);
     u32x4_t kreg[K_IT], vreg[4];  // staging registers
-    float breg = 0.f;
+    uint32_t braw = 0, mraw = 0;  // raw bias / mask of this thread's column of the tile in flight
+    // an absent mask / bias is read from K instead (any valid address) and ignored when the value is used
+    const uint8_t *mrow_ld = mrow ? mrow : (const uint8_t *)kbase;
+    const uint16_t *brow_ld = brow ? brow : kbase;
+    bool bcol_ok = false;
+    int bias_col = 0;
+    const char *ktb = nullptr, *vtb = nullptr;  // base of the tile in flight
+    int last_row = 0;                           // its last valid row
 
-    auto load_k = [&](int j) {
+    auto begin_tile = [&](int j) {
         const int n0 = j * BN;
-        const char *tb = (const char *)kbase + (int64_t)n0 * p.k_r * 2;
-        if (n0 + BN <= Lk) {
-#pragma unroll
-            for (int it = 0; it < K_IT; it++) kreg[it] = *(const u32x4_t *)(tb + koff[it]);
-            if (!d_full) {
-#pragma unroll
-                for (int it = 0; it < K_IT; it++)
-                    if (!k_dvalid) kreg[it] = u32x4_t{0, 0, 0, 0};
-            }
-        } else {
-#pragma unroll
-            for (int it = 0; it < K_IT; it++) {
-                const int key = n0 + kr0 + it * K_RPP;
-                u32x4_t kv = {0, 0, 0, 0};
-                if (key < Lk && k_dvalid) kv = *(const u32x4_t *)(tb + koff[it]);
-                kreg[it] = kv;
-            }
-        }
+        ktb = (const char *)kbase + (int64_t)n0 * p.k_r * 2;
+        vtb = (const char *)vbase + (int64_t)n0 * p.v_r * 2;
+        last_row = (Lk - n0 < BN ? Lk - n0 : BN) - 1;
+        bias_col = n0 + ktid;
+    };
+    // fused bias of the tile's columns: only the raw loads here -- the values are looked at in store_k, after the
+    // compute.  Issued after the scores, not at the top of the iteration: with loads in flight there, the waits the
+    // compiler places in front of the first LDS fragment reads (it cannot prove that the registers they overwrite
+    // have no load pending from the previous iteration) would stall on them.
+    auto load_bias_raw = [&]() {
         if (ktid < BN) {
-            const int col = n0 + ktid;
-            float v = -INFINITY;
+            const int col = bias_col;
+            const int cc = col < Lk ? col : 0;
+            bcol_ok = col < Lk;
+            // (unconditional loads: a load in one arm of a select would have to be waited for right here)
             if (CMP) {
-                if (col < Lk) v = fbrow[col];
-            } else if (col < Lk && (!mrow || mrow[col])) {
-                v = 0.f;
-                if (brow) v = E::lo((uint32_t)brow[col]) * kLog2e;
+                braw = __float_as_uint(fbrow[cc]);
+            } else {
+                mraw = mrow_ld[cc];
+                braw = brow_ld[cc];
             }
-            breg = v;
         }
+    };
+    auto load_k_item = [&](int it) {
+        int row = kr0 + it * K_RPP;
+        row = row < last_row ? row : last_row;
+        kreg[it] = *(const u32x4_t *)(ktb + (uint32_t)row * k_r2 + kcolb);
+    };
+    auto load_v_item = [&](int i) {
+        int row = 4 * vkg + i;
+        row = row < last_row ? row : last_row;
+        vreg[i] = *(const u32x4_t *)(vtb + (uint32_t)row * v_r2 + vcolb);
+    };
+    auto load_k = [&](int j) {
+        begin_tile(j);
+        load_bias_raw();
+#pragma unroll
+        for (int it = 0; it < K_IT; it++) load_k_item(it);
+    };
+    auto load_v = [&](int j) {
+        (void)j;
+#pragma unroll
+        for (int i = 0; i < 4; i++) load_v_item(i);
     };
     auto store_k = [&](int buf, int slot) {
         char *sK = smem + SM::OFF_K + buf * SM::K_BYTES;
 #pragma unroll
         for (int it = 0; it < K_IT; it++)
             *(u32x4_t *)(sK + ((kr0 + it * K_RPP) * SM::SK + kc * 8) * 2) = kreg[it];
-        if (ktid < BN) sBias[slot * BN + ktid] = breg;
-    };
-    auto load_v = [&](int j) {
-        const int n0 = j * BN;
-        const char *tb = (const char *)vbase + (int64_t)n0 * p.v_r * 2;
-        if (tid < V_ITEMS) {
-            if (n0 + BN <= Lk) {
-#pragma unroll
-                for (int i = 0; i < 4; i++) vreg[i] = *(const u32x4_t *)(tb + voff[i]);
-                if (!d_full) {
-#pragma unroll
-                    for (int i = 0; i < 4; i++)
-                        if (!v_dvalid) vreg[i] = u32x4_t{0, 0, 0, 0};
-                }
-            } else {
-#pragma unroll
-                for (int i = 0; i < 4; i++) {
-                    const int key = n0 + 4 * vkg + i;
-                    u32x4_t vv = {0, 0, 0, 0};
-                    if (key < Lk && v_dvalid) vv = *(const u32x4_t *)(tb + voff[i]);
-                    vreg[i] = vv;
-                }
+        if (ktid < BN) {
+            float v = -INFINITY;
+            if (CMP) {
+                if (bcol_ok) v = __uint_as_float(braw);
+            } else if (bcol_ok && (!mrow || mraw)) {
+                v = brow ? E::lo(braw) * kLog2e : 0.f;
             }
+            sBias[slot * BN + ktid] = v;
         }
     };
     auto store_v = [&](int buf) {  // transpose 4 keys x 8 d in registers, write V^T[d][key quad]
@@ -308,6 +311,7 @@ __global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_col
         vis_wave[nb] = CAUSAL ? visible(wrow0 + nb * 32) : 0;
     }
 
+    // `prefetch`: the K loads of the tile in flight are issued between the MFMAs
     auto qk = [&](f32x16_t (&s)[NQ][MB], int buf, int slot) {
         const char *sK = smem + SM::OFF_K + buf * SM::K_BYTES;
         // the accumulators start from the fused bias vector (bias * log2e, -inf for dropped keys) of the tile
@@ -342,6 +346,7 @@ __global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_col
             const int ks = f / MB, mb = f % MB;
 #pragma unroll
             for (int nb = 0; nb < NQ; nb++) s[nb][mb] = E::mfma(a[f], qf[nb][ks], s[nb][mb]);
+            if (f % (NF / K_IT) == 0) load_k_item(f / (NF / K_IT));
         }
         __builtin_amdgcn_sched_group_barrier(0x100, FR + 4 * MB, 0);
 #pragma unroll
@@ -440,14 +445,19 @@ __global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_col
         int i = 0;
         while (jc < n_end) {
             const int jn = next_active(jc + 1);
-            if (jn < n_end) {
-                load_k(jn);
-                load_v(jn);
-            }
+            // the loads of the next tile are spread over the MFMAs of this one (after the last tile the current
+            // one is simply fetched again and dropped): eight waves issuing all their loads at once right after
+            // the barrier would queue up at the CU's address unit while the matrix pipe idles
+            begin_tile(jn < n_end ? jn : jc);
+            __builtin_amdgcn_sched_barrier(0);
             qk(sa, i & 1, i & 1);
+            load_bias_raw();
+            load_v(jc);  // V of the tile in flight: issued before the softmax so that softmax and PV cover the latency
+            __builtin_amdgcn_sched_barrier(0);
             uint32_t pk[NQ][8 * MB];
             softmax(sa, jc, pk);
             pv(pk, i & 1);
+            __builtin_amdgcn_sched_barrier(0);
             if (jn < n_end) {
                 store_k((i + 1) & 1, (i + 1) & 1);
                 store_v((i + 1) & 1);
