@@ -175,19 +175,27 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
     const bool has_bias = f.bias != nullptr;
     const bool use_accum = p.dbias_accum != nullptr;
 
-    // fused per-lane column constant for query head h: bias*log2e, or -inf when the column is dropped
-    auto column_const = [&](int h) -> float {
+    // Fused per-lane column constant for query head h: bias*log2e, or -inf when the column is dropped.  It travels
+    // with the prefetch of the step that needs it: raw, unconditional loads (an absent mask / bias is read from K,
+    // any valid address, and ignored) issued first in load_step, turned into the constant after the compute.
+    uint32_t cm_raw = 1, cb_raw = 0;
+    const uint8_t *mask_ld = f.mask ? f.mask : (const uint8_t *)f.k;
+    const uint16_t *bias_ld = has_bias ? (const uint16_t *)f.bias : (const uint16_t *)f.k;
+    auto column_const_load = [&](int h) {
+        if (CMP) {
+            cb_raw = __float_as_uint(f.cmp.fb[(int64_t)(b * f.cmp.Hfb + (f.cmp.Hfb == f.H ? h : hk)) * f.cmp.ld + key_c]);
+        } else {
+            const int hm = f.mask ? (f.Hm == f.H ? h : (f.Hm == 1 ? 0 : hk)) : 0;
+            const int hb = has_bias ? (f.Hb == f.H ? h : (f.Hb == 1 ? 0 : hk)) : 0;
+            cm_raw = mask_ld[f.mask ? b * f.m_b + hm * f.m_h + key_c : 0];
+            cb_raw = bias_ld[has_bias ? b * f.bi_b + hb * f.bi_h + key_c : 0];
+        }
+    };
+    auto column_const_value = [&]() -> float {
         if (key >= Lk) return -INFINITY;
-        if (CMP) return f.cmp.fb[(int64_t)(b * f.cmp.Hfb + (f.cmp.Hfb == f.H ? h : hk)) * f.cmp.ld + key];
-        if (f.mask) {
-            const int hm = f.Hm == f.H ? h : (f.Hm == 1 ? 0 : hk);
-            if (!f.mask[b * f.m_b + hm * f.m_h + key]) return -INFINITY;
-        }
-        if (has_bias) {
-            const int hb = f.Hb == f.H ? h : (f.Hb == 1 ? 0 : hk);
-            return E::lo((uint32_t)((const uint16_t *)f.bias)[b * f.bi_b + hb * f.bi_h + key]) * kLog2e;
-        }
-        return 0.f;
+        if (CMP) return __uint_as_float(cb_raw);
+        if (f.mask && !cm_raw) return -INFINITY;
+        return has_bias ? E::lo(cb_raw) * kLog2e : 0.f;
     };
 
     // ---- staging of Q / dO / LSE / D for one step (global -> registers -> LDS)
@@ -195,9 +203,11 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
     const int qcol = (qc * 8 < f.d) ? qc * 8 : 0;  // head-dim chunks beyond d: re-read chunk 0 (K/V fragments there are zero)
     u32x4_t qreg[Q_IT], doreg[Q_IT];
     float lreg = INFINITY, dreg = 0.f;
+    bool stat_ok = false;
     auto load_step = [&](int step) {
         const int gi = g_lo + step / n_m, mi = m_hi - 1 - step % n_m;  // last query block first: see below
         const int h = hk * G + gi, m0 = mi * KV_BM;
+        column_const_load(h);
         const uint16_t *qbase = (const uint16_t *)f.q + b * f.q_b + h * f.q_h + qcol;
         const uint16_t *dobase = (const uint16_t *)p.dout + b * p.do_b + h * p.do_h + qcol;
 #pragma unroll
@@ -207,14 +217,14 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
             qreg[it] = *(const u32x4_t *)(qbase + (int64_t)qq * f.q_r);
             doreg[it] = *(const u32x4_t *)(dobase + (int64_t)qq * p.do_r);
         }
-        if (tid < KV_BM) {
-            const int qq = m0 + tid;
-            lreg = INFINITY;
-            dreg = 0.f;
-            if (qq < f.Lq) {
-                lreg = f.lse[((int64_t)b * f.H + h) * f.Lq + qq] * kLog2e;
-                dreg = p.softmax_d[((int64_t)b * f.H + h) * p.Lq_rounded + qq];
-            }
+        // row statistics: raw, unconditional loads from a clamped row (nothing may look at a loaded value here, or the
+        // wait for it would also cover the tile loads above); range check and scaling happen in store_step
+        {
+            const int qq = m0 + (tid & (KV_BM - 1));
+            stat_ok = qq < f.Lq;
+            const int qc = stat_ok ? qq : f.Lq - 1;
+            lreg = f.lse[((int64_t)b * f.H + h) * f.Lq + qc];
+            dreg = p.softmax_d[((int64_t)b * f.H + h) * p.Lq_rounded + qc];
         }
     };
     auto store_step = [&](int buf) {
@@ -226,8 +236,8 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
             *(u32x4_t *)(base + SM::Q_BYTES + off) = doreg[it];
         }
         if (tid < KV_BM) {
-            ((float *)(base + 2 * SM::Q_BYTES))[tid] = lreg;
-            ((float *)(base + 2 * SM::Q_BYTES + KV_BM * 4))[tid] = dreg;
+            ((float *)(base + 2 * SM::Q_BYTES))[tid] = stat_ok ? lreg * kLog2e : INFINITY;
+            ((float *)(base + 2 * SM::Q_BYTES + KV_BM * 4))[tid] = stat_ok ? dreg : 0.f;
         }
     };
 
@@ -244,6 +254,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
     if (n_steps > 0) {
         load_step(0);
         store_step(0);
+        cconst = column_const_value();
         __syncthreads();
     }
 
@@ -252,9 +263,6 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
         const int h = hk * G + gi;
         const int m0 = mi * KV_BM;
         const int buf = step & 1;
-        if (step % n_m == 0) cconst = column_const(h);
-        if (step + 1 < n_steps) load_step(step + 1);
-
         const char *sQ = smem + buf * SM::STAGE;
         const char *sDO = sQ + SM::Q_BYTES;
         const float *sLSE = (const float *)(sQ + 2 * SM::Q_BYTES);
@@ -266,6 +274,9 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
         for (int mb = 0; mb < MB; mb++)
 #pragma unroll
             for (int i = 0; i < 16; i++) { s[mb][i] = cconst; dp[mb][i] = 0.f; }
+        // global loads of the next step: in flight behind all the matrix work of this one
+        if (step + 1 < n_steps) load_step(step + 1);
+        __builtin_amdgcn_sched_barrier(0);
         {
             constexpr int NF = 2 * MB * KS, FR = 8;  // fragment f: (ks, mb, which) with which = 0: Q, 1: dO
             u32x4_t a[NF];
@@ -326,19 +337,33 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
         colsum += part;
 
         // ---- dV^T += dO^T P ; dK^T += Q^T dS   (M = d, N = key, contraction = query)
-#pragma unroll
-        for (int qb = 0; qb < KV_BM / 16; qb++) {
-            const u32x4_t pb = {ppk[4 * qb], ppk[4 * qb + 1], ppk[4 * qb + 2], ppk[4 * qb + 3]};
-            const u32x4_t sb = {dpk[4 * qb], dpk[4 * qb + 1], dpk[4 * qb + 2], dpk[4 * qb + 3]};
-#pragma unroll
-            for (int db = 0; db < DB; db++) {
+        {   // the transposing fragment reads run one (query block, d block) pair ahead of the MFMAs that use them
+            constexpr int NP = (KV_BM / 16) * DB;
+            u32x4_t a1[2], a2[2];
+            auto frag = [&](int idx, int slot) {
+                const int qb = idx / DB, db = idx % DB;
                 const uint32_t off = tr_off + (uint32_t)((16 * qb * SM::S + 32 * db) * 2);
                 const u32x2_t lo = lds_read_tr16(sDO, off), hi = lds_read_tr16(sDO, off + 4 * SM::S * 2);
                 const u32x2_t lo2 = lds_read_tr16(sQ, off), hi2 = lds_read_tr16(sQ, off + 4 * SM::S * 2);
-                const u32x4_t a1 = {lo[0], lo[1], hi[0], hi[1]};
-                const u32x4_t a2 = {lo2[0], lo2[1], hi2[0], hi2[1]};
-                dv[db] = E::mfma(a1, pb, dv[db]);
-                dk[db] = E::mfma(a2, sb, dk[db]);
+                a1[slot] = u32x4_t{lo[0], lo[1], hi[0], hi[1]};
+                a2[slot] = u32x4_t{lo2[0], lo2[1], hi2[0], hi2[1]};
+            };
+            frag(0, 0);
+#pragma unroll
+            for (int idx = 0; idx < NP; idx++) {
+                if (idx + 1 < NP) frag(idx + 1, (idx + 1) & 1);
+                const int qb = idx / DB, db = idx % DB;
+                const u32x4_t pb = {ppk[4 * qb], ppk[4 * qb + 1], ppk[4 * qb + 2], ppk[4 * qb + 3]};
+                const u32x4_t sb = {dpk[4 * qb], dpk[4 * qb + 1], dpk[4 * qb + 2], dpk[4 * qb + 3]};
+                dv[db] = E::mfma(a1[idx & 1], pb, dv[db]);
+                dk[db] = E::mfma(a2[idx & 1], sb, dk[db]);
+            }
+            // pin the order: reads of pair idx+1, then the two MFMAs of pair idx
+            __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+#pragma unroll
+            for (int idx = 0; idx < NP; idx++) {
+                if (idx + 1 < NP) __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
+                __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
             }
         }
 
@@ -358,7 +383,10 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
             }
         }
 
-        if (step + 1 < n_steps) store_step(buf ^ 1);
+        if (step + 1 < n_steps) {
+            store_step(buf ^ 1);
+            cconst = column_const_value();  // of the next step
+        }
         __syncthreads();
     }
 
