@@ -15,7 +15,7 @@
 //   2. bwd_dkdv_kernel  : one workgroup per (key block, batch, KV head); K/V stationary, loops over the
 //                         query heads of the group and over query blocks; dK, dV and dBias complete in
 //                         registers (S is computed un-transposed so a lane owns one key column);
-//   3. bwd_dq_kernel    : one workgroup per (query block, batch, head); loops over key blocks exactly like
+//   3. bwd_dq_kernel    : (fdma_bwd_dq.hip) one workgroup per (query block, batch, head); loops over key blocks like
 //                         the forward kernel (transposed scores, a lane owns one query row).
 // Work is therefore 7 tile GEMMs instead of 5, in exchange for a deterministic result and no
 // read-modify-write traffic.
@@ -460,203 +460,6 @@ __global__ void __launch_bounds__(NTHREADS, 1) bwd_dkdv_kernel(const BwdParams p
 }
 
 // ------------------------------------------------------------------------------------------------
-// 3. dQ
-// ------------------------------------------------------------------------------------------------
-constexpr int Q_BM = 128;
-constexpr int Q_BN = 64;
-
-template <int D> struct DqSmem {
-    static constexpr int S = D + 8;
-    static constexpr int K_BYTES = Q_BN * S * 2;
-    static constexpr int TOTAL = 2 * K_BYTES;
-};
-
-template <typename T, int D, bool CAUSAL>
-__global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_kernel(const BwdParams p) {
-    using E = Elem<T>;
-    using SM = DqSmem<D>;
-    constexpr int KS = D / 16;
-    constexpr int DB = D / 32;
-
-    __shared__ __attribute__((aligned(16))) char smem[SM::TOTAL];
-    char *sK = smem, *sV = smem + SM::K_BYTES;
-
-    const FwdParams &f = p.f;
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 31, g = lane >> 5;
-    const int m_block = gridDim.x - 1 - blockIdx.x;
-    const int h = blockIdx.y, b = blockIdx.z;
-    const int hk = h / (f.H / f.Hk);
-    const int m0 = m_block * Q_BM;
-    const int qrow = m0 + wave * 32 + r;
-    const int qrow_c = qrow < f.Lq ? qrow : f.Lq - 1;
-    const int shift = f.Lk - f.Lq;
-
-    u32x4_t qf[KS], dof[KS];
-    {
-        const uint16_t *qp = (const uint16_t *)f.q + b * f.q_b + (int64_t)qrow_c * f.q_r + h * f.q_h;
-        const uint16_t *dp = (const uint16_t *)p.dout + b * p.do_b + (int64_t)qrow_c * p.do_r + h * p.do_h;
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-            int c = ks * 16 + g * 8;
-            u32x4_t qv = {0, 0, 0, 0}, dv = {0, 0, 0, 0};
-            if (qrow < f.Lq && c < f.d) { qv = *(const u32x4_t *)(qp + c); dv = *(const u32x4_t *)(dp + c); }
-            qf[ks] = qv;
-            dof[ks] = dv;
-        }
-    }
-    float lse2 = INFINITY, dd = 0.f;
-    if (qrow < f.Lq) {
-        lse2 = f.lse[((int64_t)b * f.H + h) * f.Lq + qrow] * kLog2e;
-        dd = p.softmax_d[((int64_t)b * f.H + h) * p.Lq_rounded + qrow];
-    }
-
-    int n_end = (f.Lk + Q_BN - 1) / Q_BN;
-    if (CAUSAL) {
-        int lim = m0 + Q_BM + shift;
-        if (lim < 0) lim = 0;
-        int ne = (lim + Q_BN - 1) / Q_BN;
-        if (ne < n_end) n_end = ne;
-    }
-
-    f32x16_t dq[DB];
-#pragma unroll
-    for (int db = 0; db < DB; db++)
-#pragma unroll
-        for (int i = 0; i < 16; i++) dq[db][i] = 0.f;
-
-    const int hm = f.mask ? (f.Hm == f.H ? h : (f.Hm == 1 ? 0 : h / (f.H / f.Hm))) : 0;
-    const int hb = f.bias ? (f.Hb == f.H ? h : (f.Hb == 1 ? 0 : h / (f.H / f.Hb))) : 0;
-    const uint8_t *mrow = f.mask ? f.mask + b * f.m_b + hm * f.m_h + (int64_t)qrow_c * f.m_r : nullptr;
-    const uint16_t *brow = f.bias ? (const uint16_t *)f.bias + b * f.bi_b + hb * f.bi_h + (int64_t)qrow_c * f.bi_r : nullptr;
-    const uint16_t *kbase = (const uint16_t *)f.k + b * f.k_b + hk * f.k_h;
-    const uint16_t *vbase = (const uint16_t *)f.v + b * f.v_b + hk * f.v_h;
-
-    const int a_row = pi_row(r);
-    const int tj = lane & 15, te = tj >> 2, tc = tj & 3;
-    const int tcp = (tc == 1) ? 2 : (tc == 2 ? 1 : tc);
-    const int tdh = (lane >> 4) & 1;
-    const uint32_t tr_off = (uint32_t)(((8 * g + te) * SM::S + 16 * tdh + 4 * tcp) * 2);
-
-    for (int j = 0; j < n_end; j++) {
-        const int n0 = j * Q_BN;
-        uint32_t keep = 0;
-#pragma unroll
-        for (int mb = 0; mb < 2; mb++)
-#pragma unroll
-            for (int blk = 0; blk < 2; blk++) {
-                int c0 = n0 + 32 * mb + 16 * blk + 8 * g;
-                uint32_t bits = 0xffu;
-                if (mrow) {
-                    bits = 0;
-                    if (c0 < f.Lk) {
-                        u32x2_t mv = *(const u32x2_t *)(mrow + c0);
-                        bits = nz_bytes_to_bits(mv[0]) | (nz_bytes_to_bits(mv[1]) << 4);
-                    }
-                }
-                int lim = f.Lk;
-                if (CAUSAL) { int cl = qrow + 1 + shift; lim = cl < lim ? cl : lim; }
-                int nvis = lim - c0;
-                uint32_t vis = nvis >= 8 ? 0xffu : (nvis <= 0 ? 0u : ((1u << nvis) - 1u));
-                bits &= vis;
-                if (qrow >= f.Lq) bits = 0;
-                keep |= bits << (16 * mb + 8 * blk);
-            }
-        const int active = __syncthreads_or(keep != 0);
-        if (!active) continue;
-
-        {
-            constexpr int CH = D / 8, RPP = NTHREADS / CH;
-            const int c = tid % CH, r0 = tid / CH;
-#pragma unroll
-            for (int it = 0; it < Q_BN / RPP; it++) {
-                int row = r0 + it * RPP, kk = n0 + row;
-                u32x4_t kv = {0, 0, 0, 0}, vv = {0, 0, 0, 0};
-                if (kk < f.Lk && c * 8 < f.d) {
-                    kv = *(const u32x4_t *)(kbase + (int64_t)kk * f.k_r + c * 8);
-                    vv = *(const u32x4_t *)(vbase + (int64_t)kk * f.v_r + c * 8);
-                }
-                *(u32x4_t *)(sK + (row * SM::S + c * 8) * 2) = kv;
-                *(u32x4_t *)(sV + (row * SM::S + c * 8) * 2) = vv;
-            }
-        }
-        float bl2[32];
-#pragma unroll
-        for (int mb = 0; mb < 2; mb++)
-#pragma unroll
-            for (int blk = 0; blk < 2; blk++) {
-                int c0 = n0 + 32 * mb + 16 * blk + 8 * g;
-                u32x4_t bv = {0, 0, 0, 0};
-                if (brow && c0 < f.Lk) bv = *(const u32x4_t *)(brow + c0);
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    bl2[16 * mb + 8 * blk + 2 * e] = E::lo(bv[e]) * kLog2e;
-                    bl2[16 * mb + 8 * blk + 2 * e + 1] = E::hi(bv[e]) * kLog2e;
-                }
-            }
-        __syncthreads();
-
-        // ---- S^T = K Q^T, dP^T = V dO^T
-        f32x16_t s[2], dp[2];
-#pragma unroll
-        for (int mb = 0; mb < 2; mb++) {
-#pragma unroll
-            for (int i = 0; i < 16; i++) { s[mb][i] = 0.f; dp[mb][i] = 0.f; }
-#pragma unroll
-            for (int ks = 0; ks < KS; ks++) {
-                u32x4_t ka = *(const u32x4_t *)(sK + ((32 * mb + a_row) * SM::S + ks * 16 + g * 8) * 2);
-                u32x4_t va = *(const u32x4_t *)(sV + ((32 * mb + a_row) * SM::S + ks * 16 + g * 8) * 2);
-                s[mb] = E::mfma(ka, qf[ks], s[mb]);
-                dp[mb] = E::mfma(va, dof[ks], dp[mb]);
-            }
-        }
-        uint32_t dpk[16];
-#pragma unroll
-        for (int mb = 0; mb < 2; mb++)
-#pragma unroll
-            for (int i = 0; i < 16; i += 2) {
-                float d2[2];
-#pragma unroll
-                for (int e = 0; e < 2; e++) {
-                    const int ii = i + e;
-                    float x = fmaf(s[mb][ii], f.scale_log2, bl2[16 * mb + ii]) - lse2;
-                    float pe = ((keep >> (16 * mb + ii)) & 1u) ? fast_exp2(x) : 0.f;
-                    d2[e] = pe * (dp[mb][ii] - dd);
-                }
-                dpk[8 * mb + i / 2] = E::pack2(d2[0], d2[1]);
-            }
-        // ---- dQ^T += K^T dS^T
-#pragma unroll
-        for (int kb = 0; kb < 4; kb++) {
-            u32x4_t bop = {dpk[4 * kb], dpk[4 * kb + 1], dpk[4 * kb + 2], dpk[4 * kb + 3]};
-#pragma unroll
-            for (int db = 0; db < DB; db++) {
-                uint32_t off = tr_off + (uint32_t)((16 * kb * SM::S + 32 * db) * 2);
-                u32x2_t lo = lds_read_tr16(sK, off), hi = lds_read_tr16(sK, off + 4 * SM::S * 2);
-                u32x4_t a = {lo[0], lo[1], hi[0], hi[1]};
-                dq[db] = E::mfma(a, bop, dq[db]);
-            }
-        }
-    }
-
-    if (qrow < f.Lq) {
-        uint16_t *dqp = (uint16_t *)p.dq + b * p.dq_b + (int64_t)qrow * p.dq_r + h * p.dq_h;
-#pragma unroll
-        for (int db = 0; db < DB; db++)
-#pragma unroll
-            for (int blk = 0; blk < 2; blk++) {
-                int c = 32 * db + 16 * blk + 8 * g;
-                if (c < f.d) {
-                    u32x4_t w;
-#pragma unroll
-                    for (int e = 0; e < 4; e++)
-                        w[e] = E::pack2(dq[db][8 * blk + 2 * e] * f.scale, dq[db][8 * blk + 2 * e + 1] * f.scale);
-                    *(u32x4_t *)(dqp + c) = w;
-                }
-            }
-    }
-}
-
-// ------------------------------------------------------------------------------------------------
 // fp32 dbias accumulator helpers (only when several workgroups share a dbias element)
 // ------------------------------------------------------------------------------------------------
 __global__ void fill_zero_kernel(float *ptr, size_t n) {
@@ -724,12 +527,7 @@ hipError_t launch_bwd_t(const BwdParams &p, hipStream_t stream) {
     if (colmask) {
         if ((e = launch_bwd_dq_colmask(p, dtype_code, stream)) != hipSuccess) return e;
     } else {
-        dim3 grid((f.Lq + Q_BM - 1) / Q_BM, f.H, f.B);
-        if (f.causal)
-            hipLaunchKernelGGL((bwd_dq_kernel<T, D, true>), grid, dim3(NTHREADS), 0, stream, p);
-        else
-            hipLaunchKernelGGL((bwd_dq_kernel<T, D, false>), grid, dim3(NTHREADS), 0, stream, p);
-        if ((e = hipGetLastError()) != hipSuccess) return e;
+        if ((e = launch_bwd_dq(p, dtype_code, stream)) != hipSuccess) return e;
     }
     return hipSuccess;
 }

@@ -129,6 +129,8 @@ hipError_t launch_bwd(const BwdParams &p, int dtype, hipStream_t stream);
 bool bwd_colmask_applicable(const BwdParams &p);
 hipError_t launch_bwd_dkdv_colmask(const BwdParams &p, int dtype, hipStream_t stream);
 hipError_t launch_bwd_dq_colmask(const BwdParams &p, int dtype, hipStream_t stream);
+// general dQ kernel (mask / bias per query row), fdma_bwd_dq.hip
+hipError_t launch_bwd_dq(const BwdParams &p, int dtype, hipStream_t stream);
 
 // Column compaction: use_compact() decides from the problem alone (no device data), compact_bytes() is
 // the scratch it needs, compact_setup() launches the gather pre-pass into `ws` and rewrites p.k / p.v /
