@@ -167,8 +167,15 @@ __global__ void __launch_bounds__(NTHREADS, 1) bwd_dkdv_kernel(const BwdParams p
     const int qc = tid % CH, qr0 = tid / CH;
     const int qcol = (qc * 8 < f.d) ? qc * 8 : 0;
     const int bc = tid & 15, br0 = tid >> 4;  // fused-bias tile: 8-key chunk and first row of this thread
-    u32x4_t qreg[Q_IT], doreg[Q_IT], fbreg[4];
+    u32x4_t qreg[Q_IT], doreg[Q_IT], braw[4];
+    u32x2_t mraw[4];
     float lreg = INFINITY, dreg = 0.f;
+    bool stat_ok = false;
+    // Every load of a step is unconditional and raw (clamped rows / keys; an absent mask or bias is read from K, any
+    // valid address, and ignored later): a conditional load or a value that is looked at right away would make the
+    // wait for it -- and for every load issued before it -- land in front of the matrix work instead of behind it.
+    const uint8_t *mask_ld = f.mask ? f.mask : (const uint8_t *)f.k;
+    const uint16_t *bias_ld = has_bias ? (const uint16_t *)f.bias : (const uint16_t *)f.k;
     auto step_head = [&](int step, int &gi, int &mi) {
         gi = m_outer ? step % G : step / n_m;
         mi = M_blocks - 1 - (m_outer ? step / G : step % n_m);
@@ -186,48 +193,26 @@ __global__ void __launch_bounds__(NTHREADS, 1) bwd_dkdv_kernel(const BwdParams p
             qreg[it] = *(const u32x4_t *)(qbase + (int64_t)qq * f.q_r);
             doreg[it] = *(const u32x4_t *)(dobase + (int64_t)qq * p.do_r);
         }
-        if (tid < KV_BM) {
-            const int qq = m0 + tid;
-            lreg = INFINITY;
-            dreg = 0.f;
-            if (qq < f.Lq) {
-                lreg = f.lse[((int64_t)b * f.H + h) * f.Lq + qq] * kLog2e;
-                dreg = p.softmax_d[((int64_t)b * f.H + h) * p.Lq_rounded + qq];
-            }
+        {
+            const int qq = m0 + (tid & (KV_BM - 1));
+            stat_ok = qq < f.Lq;
+            const int qc = stat_ok ? qq : f.Lq - 1;
+            lreg = f.lse[((int64_t)b * f.H + h) * f.Lq + qc];
+            dreg = p.softmax_d[((int64_t)b * f.H + h) * p.Lq_rounded + qc];
         }
-        // fused bias chunks: rows br0 + 16*it, keys n0 + 8*bc .. +8
+        // mask / bias chunks: rows br0 + 16*it, keys n0 + 8*bc .. +8
         const int hm = f.mask ? (f.Hm == f.H ? h : (f.Hm == 1 ? 0 : hk)) : 0;
         const int hb = has_bias ? (f.Hb == f.H ? h : (f.Hb == 1 ? 0 : hk)) : 0;
         const int kk = n0 + 8 * bc;
+        const int kk_c = kk < f.Lk ? kk : 0;
+        const int64_t moff = f.mask ? b * f.m_b + hm * f.m_h + kk_c : 0;
+        const int64_t boff = has_bias ? b * f.bi_b + hb * f.bi_h + kk_c : 0;
 #pragma unroll
         for (int it = 0; it < 4; it++) {
             int qq = m0 + br0 + 16 * it;
             qq = qq < f.Lq ? qq : f.Lq - 1;
-            u32x4_t bv = {0, 0, 0, 0};
-            u32x2_t mv = {0x01010101u, 0x01010101u};
-            if (kk < f.Lk) {
-                if (has_bias) bv = *(const u32x4_t *)((const uint16_t *)f.bias + b * f.bi_b + hb * f.bi_h + (int64_t)qq * f.bi_r + kk);
-                if (f.mask) mv = *(const u32x2_t *)(f.mask + b * f.m_b + hm * f.m_h + (int64_t)qq * f.m_r + kk);
-            } else {
-                mv = u32x2_t{0, 0};
-            }
-            if (kk + 8 > f.Lk && kk < f.Lk) {  // chunk straddles the end of the keys
-                const int nv = f.Lk - kk;       // 1..7 valid keys
-                const uint64_t keepm = (1ull << (8 * nv)) - 1ull;
-                mv[0] &= (uint32_t)keepm;
-                mv[1] &= (uint32_t)(keepm >> 32);
-            }
-#pragma unroll
-            for (int hlf = 0; hlf < 2; hlf++) {
-                uint32_t x = mv[hlf];
-                x = ((((x & 0x7f7f7f7fu) + 0x7f7f7f7fu) | x) >> 7) & 0x01010101u;  // nonzero byte -> 0x01
-                const uint32_t z = (x << 8) - x;                                      // 0x01 -> 0xFF per byte
-                const uint32_t m0w = __builtin_amdgcn_perm(0, z, 0x01010000u);        // [b0 b0 b1 b1]
-                const uint32_t m1w = __builtin_amdgcn_perm(0, z, 0x03030202u);        // [b2 b2 b3 b3]
-                bv[2 * hlf] = (bv[2 * hlf] & m0w) | (NegInfPair<T>::value & ~m0w);
-                bv[2 * hlf + 1] = (bv[2 * hlf + 1] & m1w) | (NegInfPair<T>::value & ~m1w);
-            }
-            fbreg[it] = bv;
+            braw[it] = *(const u32x4_t *)(bias_ld + boff + (has_bias ? (int64_t)qq * f.bi_r : 0));
+            mraw[it] = *(const u32x2_t *)(mask_ld + moff + (f.mask ? (int64_t)qq * f.m_r : 0));
         }
     };
     auto store_step = [&](int buf) {
@@ -239,12 +224,32 @@ __global__ void __launch_bounds__(NTHREADS, 1) bwd_dkdv_kernel(const BwdParams p
             *(u32x4_t *)(base + SM::Q_BYTES + off) = doreg[it];
         }
         if (tid < KV_BM) {
-            ((float *)(base + 2 * SM::Q_BYTES))[tid] = lreg;
-            ((float *)(base + 2 * SM::Q_BYTES + KV_BM * 4))[tid] = dreg;
+            ((float *)(base + 2 * SM::Q_BYTES))[tid] = stat_ok ? lreg * kLog2e : INFINITY;
+            ((float *)(base + 2 * SM::Q_BYTES + KV_BM * 4))[tid] = stat_ok ? dreg : 0.f;
         }
+        // fuse mask and bias: bias where kept, -inf where dropped or beyond Lk
         char *fb = base + 2 * SM::Q_BYTES + 2 * KV_BM * 4;
+        const int kk = n0 + 8 * bc;
 #pragma unroll
-        for (int it = 0; it < 4; it++) *(u32x4_t *)(fb + ((br0 + 16 * it) * SM::SB + 8 * bc) * 2) = fbreg[it];
+        for (int it = 0; it < 4; it++) {
+            u32x4_t bv = has_bias ? braw[it] : u32x4_t{0, 0, 0, 0};
+            u32x2_t mv = f.mask ? mraw[it] : u32x2_t{0x01010101u, 0x01010101u};
+            uint64_t keepm = kk < f.Lk ? ~0ull : 0ull;
+            if (kk + 8 > f.Lk && kk < f.Lk) keepm = (1ull << (8 * (f.Lk - kk))) - 1ull;  // chunk straddles the end of the keys
+            mv[0] &= (uint32_t)keepm;
+            mv[1] &= (uint32_t)(keepm >> 32);
+#pragma unroll
+            for (int hlf = 0; hlf < 2; hlf++) {
+                uint32_t x = mv[hlf];
+                x = ((((x & 0x7f7f7f7fu) + 0x7f7f7f7fu) | x) >> 7) & 0x01010101u;  // nonzero byte -> 0x01
+                const uint32_t z = (x << 8) - x;                                      // 0x01 -> 0xFF per byte
+                const uint32_t m0w = __builtin_amdgcn_perm(0, z, 0x01010000u);        // [b0 b0 b1 b1]
+                const uint32_t m1w = __builtin_amdgcn_perm(0, z, 0x03030202u);        // [b2 b2 b3 b3]
+                bv[2 * hlf] = (bv[2 * hlf] & m0w) | (NegInfPair<T>::value & ~m0w);
+                bv[2 * hlf + 1] = (bv[2 * hlf + 1] & m1w) | (NegInfPair<T>::value & ~m1w);
+            }
+            *(u32x4_t *)(fb + ((br0 + 16 * it) * SM::SB + 8 * bc) * 2) = bv;
+        }
     };
 
     const int a_row = pi_row(r);
@@ -275,7 +280,6 @@ __global__ void __launch_bounds__(NTHREADS, 1) bwd_dkdv_kernel(const BwdParams p
         const int m0 = mi * KV_BM;
         const int buf = step & 1;
         const int hb = has_bias ? (f.Hb == f.H ? h : (f.Hb == 1 ? 0 : hk)) : 0;
-        if (step + 1 < n_steps) load_step(step + 1);
 
         const char *sQ = smem + buf * SM::STAGE;
         const char *sDO = sQ + SM::Q_BYTES;
@@ -306,6 +310,13 @@ __global__ void __launch_bounds__(NTHREADS, 1) bwd_dkdv_kernel(const BwdParams p
                 else s[mb] = E::mfma(a[fi], kf[ks], s[mb]);
             }
         }
+        // Global loads of the next step: issued here, behind the first GEMM pair, not at the top of the step -- the
+        // compiler puts a wait for all outstanding loads in front of the first MFMA (it cannot prove that the
+        // registers involved have no load pending from the previous trip), which is free only while nothing is in
+        // flight.  The softmax and the dK / dV GEMMs below cover the latency.
+        __builtin_amdgcn_sched_barrier(0);
+        if (step + 1 < n_steps) load_step(step + 1);
+        __builtin_amdgcn_sched_barrier(0);
 
         // ---- P = exp2((S*scale + fused)*log2e - LSE*log2e) ; dS = P * (dP - D)
         const bool diag = CAUSAL && (n0 + wave * 32 + 31 > m0 + shift);
