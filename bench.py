@@ -31,9 +31,9 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch of the forward kernel on the headline workload, from two rocprofv3 --pmc runs of
 # this script (FETCH_SIZE, WRITE_SIZE; each scaled by what the counter reads for a 256 MiB device copy,
-# see --calib-copy): compacted kernel 79 MiB read + 65 MiB written, tile-skipping kernel 143 + 65 MiB.
+# see --calib-copy): compacted kernel 77 MiB read + 65 MiB written, tile-skipping kernel 151 + 65 MiB.
 # Override with --traffic-bytes after re-measuring.
-MEASURED_FWD_TRAFFIC_BYTES = {True: 144.0 * 1024 * 1024, False: 208.0 * 1024 * 1024}
+MEASURED_FWD_TRAFFIC_BYTES = {True: 142.0 * 1024 * 1024, False: 216.0 * 1024 * 1024}
 
 CONFIGS = {
     # name: B, Lq, Lk, H, Hk, D, bias shape, window, causal, passes
@@ -227,7 +227,8 @@ def cpu_baseline(device_cfg="cfg2", groups=1):
     tfl = 4.0 * 64 * 64 * c["D"] * n_exec / dt / 1e12
     return {"value": tfl, "unit": "TFLOP/s", "cores": cores, "kind": "port",
             "sample": f"{groups} of {c['Hk']} KV groups ({G * groups} query heads) of {device_cfg} forward, fp32 eager on host, "
-                      f"{dt:.2f} s; same executed-tile FLOP count as the GPU figure",
+                      f"{dt:.2f} s; FLOPs counted on the executed 64x64 tiles of the original layout, as in tile_skip_path "
+                      f"(the host computes dense masked attention)",
             "ms_scaled_to_full": dt * 1e3 * c["Hk"] / groups}
 
 
