@@ -163,3 +163,37 @@ def test_product_package_never_imports_the_oracle():
             if fn.endswith((".py", ".cpp", ".hip", ".h")):
                 text = open(os.path.join(dirpath, fn)).read()
                 assert "oracle" not in text.lower(), f"{fn} mentions the oracle"
+
+
+def test_compaction_workspace_rule(monkeypatch):
+    """fdma_*_workspace_bytes is pure host arithmetic: the column-compaction path asks for scratch exactly when the
+    mask is query-broadcast with 1 or Hkv heads and FDMA_COMPACT allows it (0 = never, 2 = whenever the form allows)."""
+    import torch
+    from flash_sparse_attn import _cabi
+
+    def args(Lq, Lk, H, Hk, Hm, mask_rows):
+        B, D = 1, 64
+        q = torch.empty(B, Lq, H, D, dtype=torch.bfloat16)
+        k = torch.empty(B, Lk, Hk, D, dtype=torch.bfloat16)
+        mask = torch.empty(B, Hm, mask_rows, Lk, dtype=torch.bool)
+        bias = torch.empty(B, Hk, 1, Lk, dtype=torch.bfloat16)
+        lse = torch.empty(B, H, Lq, dtype=torch.float32)
+        a = _cabi.FwdArgs()
+        _cabi.fill_fwd(a, q, k, k, mask, bias, torch.empty_like(q), lse, 0.125, True, 0.0)
+        return a
+
+    small = args(256, 256, 4, 2, 2, 1)
+    big = args(4096, 4096, 4, 2, 2, 1)
+    per_query = args(4096, 4096, 4, 2, 2, 4096)
+    per_qhead = args(4096, 4096, 4, 2, 4, 1)
+    monkeypatch.setenv("FDMA_COMPACT", "0")
+    assert _cabi.lib.fdma_fwd_workspace_bytes(big) == 0
+    monkeypatch.setenv("FDMA_COMPACT", "2")
+    assert _cabi.lib.fdma_fwd_workspace_bytes(small) > 0
+    assert _cabi.lib.fdma_fwd_workspace_bytes(per_query) == 0
+    assert _cabi.lib.fdma_fwd_workspace_bytes(per_qhead) == 0
+    monkeypatch.delenv("FDMA_COMPACT")
+    assert _cabi.lib.fdma_fwd_workspace_bytes(small) == 0       # too small for the pre-pass to pay
+    need = _cabi.lib.fdma_fwd_workspace_bytes(big)
+    kv_bytes = 2 * 4096 * 2 * 64 * 2
+    assert kv_bytes <= need <= 2 * kv_bytes                      # dense K / V copies plus index lists
