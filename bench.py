@@ -141,7 +141,17 @@ def count_compacted_tiles(mask, Lq, Lk, causal, H, tile=64):
     return int(((vis + tile - 1) // tile).sum().item()) * (H // Hm)
 
 
+RAMP_SECONDS = 0.25  # busy time before the warm-up steps: an idle MI355X takes that long to reach its running clocks
+
+
 def time_gpu(fn, steps, warmup):
+    """`warmup` untimed steps, then exactly `steps` timed ones between two events on the current stream.  Before
+    both, the same step runs for RAMP_SECONDS so that a cold device (power state, clocks) does not dominate a
+    timed region of a few milliseconds."""
+    t0 = time.perf_counter()
+    while time.perf_counter() - t0 < RAMP_SECONDS:
+        fn()
+        torch.cuda.synchronize()
     for _ in range(warmup):
         fn()
     torch.cuda.synchronize()

@@ -396,7 +396,7 @@ hipError_t launch_fwd_t(const FwdParams &p, hipStream_t stream) {
 
 hipError_t launch_fwd(const FwdParams &p, int dtype, hipStream_t stream) {
     if (p.Lq <= 0 || p.B <= 0) return hipSuccess;
-    if (fwd_colmask_applicable(p)) return launch_fwd_colmask(p, dtype, 1, stream);
+    if (fwd_colmask_applicable(p)) return launch_fwd_colmask(p, dtype, stream);
     const bool d64 = p.d <= 64;
     if (dtype == 0) return d64 ? launch_fwd_t<bf16_tag, 64>(p, stream) : launch_fwd_t<bf16_tag, 128>(p, stream);
     return d64 ? launch_fwd_t<fp16_tag, 64>(p, stream) : launch_fwd_t<fp16_tag, 128>(p, stream);

@@ -15,13 +15,16 @@
 //   * causal masking costs instructions on diagonal tiles only.
 //
 // Pipeline: K, V^T (V is transposed in registers while being staged) and the fused bias vector are
-// double-buffered in LDS.  Tile i is computed from buffers i&1 while the global loads of tile i+1 are in
-// flight; their LDS stores go to the other buffers after the compute, so one barrier per tile suffices.
+// double-buffered in LDS.  Tile i is computed from buffers i&1; the registers hold tile i+1, whose LDS stores go
+// to the other buffers between the scores and the softmax of tile i (the LDS port is idle there), and the global
+// loads of tile i+2 are then issued between the PV MFMAs, each a single instruction (scalar tile base + a
+// loop-invariant per-thread offset).  One barrier per tile.  Workgroups have 256 rows (8 waves: four stage V,
+// four stage K and the bias) when the grid stays large enough, else 128 rows (4 waves doing both).
 // Q is scaled by softmax_scale*log2(e) once and the score accumulators start from the fused bias vector,
 // so the MFMA result is the exp2-domain score with bias and mask applied and the softmax spends five
-// vector instructions per element (max, sub, exp2, add, half a convert).  LDS fragment reads run a batch
-// ahead of the MFMAs that consume them.  Workgroup ids are remapped so that the workgroups sharing one
-// XCD's L2 also share K / V.
+// vector instructions per element (max, sub, exp2, add, half a convert); the running maximum moves only when a
+// score exceeds it by 2^8, so the rescale of O is rare.  LDS fragment reads run a batch ahead of the MFMAs that
+// consume them.  Workgroup ids are remapped so that the workgroups sharing one XCD's L2 also share K / V.
 #include "fdma_common.h"
 #include "fdma_params.h"
 
@@ -49,7 +52,9 @@ template <int D, int BN> struct CmSmem {
 template <typename T, int D, int NQ, int BN, bool CAUSAL, int NW, bool CMP>
 __global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_colmask_kernel(const FwdParams p) {
     constexpr int NTHREADS = 64 * NW;
-    constexpr int STHREADS = NTHREADS;        // threads staging one operand
+    constexpr int STHREADS = 256;             // threads staging one operand
+    constexpr bool SPLIT = NW == 8;           // 8 waves: the first four stage V, the last four K and the bias
+    static_assert(NW == 4 || NW == 8, "staging maps are written for 256 or 512 threads");
     using E = Elem<T>;
     using SM = CmSmem<D, BN>;
     constexpr int MB = BN / 32;               // 32-key blocks per tile
@@ -62,6 +67,9 @@ __global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_col
     constexpr int K_RPP = STHREADS / CH;      // K rows staged per pass
     constexpr int K_IT = BN / K_RPP;          // passes (registers) per K tile
     constexpr int V_ITEMS = KQ * CH;          // (key quad, d chunk) items of a V tile
+    constexpr int NL = SPLIT ? 4 : K_IT + 4;  // 16-byte loads per thread and tile
+    constexpr int VB = SPLIT ? 0 : K_IT;      // first V staging register
+    static_assert(!SPLIT || K_IT == 4, "the role split assumes four loads per thread for either operand");
 
     extern __shared__ __attribute__((aligned(16))) char smem[];
     float *sBias = (float *)(smem + SM::OFF_BIAS);
@@ -204,39 +212,66 @@ __global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_col
             for (int i = 0; i < 16; i++) o[nb][db][i] = 0.f;
     }
 
-    // ---- staging helpers (global -> registers -> LDS)
-    // Every load is unconditional, from an always valid address: rows beyond the end of the keys are clamped to
-    // the last row (their fused bias is -inf, so the duplicate never counts) and head-dim chunks beyond d to chunk
-    // 0 (they meet zero Q fragments / columns of O that are not stored).  That keeps the loads free of branches,
-    // so that they can be issued one by one between the MFMAs of the tile being computed.
-    const int ktid = tid;
-    const int kc = ktid % CH, kr0 = ktid / CH;
-    const int vkg = tid % KQ, vc = (tid / KQ) % CH;  // V: key quad and d chunk of this thread
+    // ---- staging (global -> registers -> LDS).  A tile is BN * CH 16-byte chunks of K plus V_ITEMS (key quad, d chunk)
+    // items of V with four loads each (V is transposed in registers on its way to LDS).  Every load is unconditional,
+    // from an always valid address: rows beyond the end of the keys are clamped to the last row (their fused bias is
+    // -inf, so the duplicate never counts) and head-dim chunks beyond d to chunk 0 (they meet zero Q fragments /
+    // columns of O that are not stored).  The per-thread byte offsets are loop invariants -- one set for full tiles,
+    // one for the (only) partial tile at the end of the keys -- so a load is one instruction with a scalar tile base,
+    // and the loads of a tile can be issued one by one between the MFMAs of the tile being computed.
+    const bool role_v = !SPLIT || wave < 4, role_k = !SPLIT || wave >= 4;  // wave-uniform
+    const int kt = tid & (STHREADS - 1);
+    const int kc = kt % CH, kr0 = kt / CH;
+    const int vkg = kt % KQ, vc = (kt / KQ) % CH;  // V: key quad and d chunk of this thread
     const uint32_t k_r2 = (uint32_t)(p.k_r * 2), v_r2 = (uint32_t)(p.v_r * 2);  // bytes per row
     const uint32_t kcolb = (kc * 8 < p.d ? kc * 16 : 0), vcolb = (vc * 8 < p.d ? vc * 16 : 0);
-    u32x4_t kreg[K_IT], vreg[4];  // staging registers
+    const int j_last = Lk > 0 ? (Lk - 1) / BN : 0, last_row = Lk > 0 ? (Lk - 1) % BN : 0;
+    uint32_t soff[NL], soff_l[NL];  // byte offsets of this thread's loads inside a full / the last tile
+#pragma unroll
+    for (int n = 0; n < NL; n++) {
+        const bool is_v = SPLIT ? role_v : n >= K_IT;
+        const int item = SPLIT ? n : (n >= K_IT ? n - K_IT : n);
+        const int row = is_v ? 4 * vkg + item : kr0 + item * K_RPP;
+        const uint32_t r2 = is_v ? v_r2 : k_r2, colb = is_v ? vcolb : kcolb;
+        soff[n] = (uint32_t)row * r2 + colb;
+        soff_l[n] = (uint32_t)(row < last_row ? row : last_row) * r2 + colb;
+    }
+    u32x4_t sreg[NL];             // staging registers
     uint32_t braw = 0, mraw = 0;  // raw bias / mask of this thread's column of the tile in flight
     // an absent mask / bias is read from K instead (any valid address) and ignored when the value is used
     const uint8_t *mrow_ld = mrow ? mrow : (const uint8_t *)kbase;
     const uint16_t *brow_ld = brow ? brow : kbase;
     bool bcol_ok = false;
     int bias_col = 0;
-    const char *ktb = nullptr, *vtb = nullptr;  // base of the tile in flight
-    int last_row = 0;                           // its last valid row
+    typedef const __attribute__((address_space(1))) char *gptr_t;  // global address space survives the integer round trip
+    gptr_t tb_k = nullptr, tb_v = nullptr;        // tile bases (wave-uniform, in scalar registers)
+    bool t_last = false;                          // the tile in flight is the partial one
 
-    auto begin_tile = [&](int j) {
-        const int n0 = j * BN;
-        ktb = (const char *)kbase + (int64_t)n0 * p.k_r * 2;
-        vtb = (const char *)vbase + (int64_t)n0 * p.v_r * 2;
-        last_row = (Lk - n0 < BN ? Lk - n0 : BN) - 1;
-        bias_col = n0 + ktid;
+    auto uniform_ptr = [](const char *ptr) -> gptr_t {
+        const uint64_t v = (uint64_t)ptr;
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+        return (gptr_t)(((uint64_t)hi << 32) | lo);
     };
-    // fused bias of the tile's columns: only the raw loads here -- the values are looked at in store_k, after the
-    // compute.  Issued after the scores, not at the top of the iteration: with loads in flight there, the waits the
-    // compiler places in front of the first LDS fragment reads (it cannot prove that the registers they overwrite
-    // have no load pending from the previous iteration) would stall on them.
+    auto set_tile = [&](int j) {
+        const int n0 = j * BN;
+        const char *tk = (const char *)kbase + (int64_t)n0 * p.k_r * 2;
+        const char *tv = (const char *)vbase + (int64_t)n0 * p.v_r * 2;
+        if (SPLIT) {
+            tb_k = tb_v = uniform_ptr(role_v ? tv : tk);
+        } else {
+            tb_k = uniform_ptr(tk);
+            tb_v = uniform_ptr(tv);
+        }
+        t_last = j == j_last;
+        bias_col = n0 + kt;
+    };
+    auto issue_load = [&](int n) {
+        const gptr_t base = (SPLIT || n < K_IT) ? tb_k : tb_v;
+        sreg[n] = *(const __attribute__((address_space(1))) u32x4_t *)(base + (t_last ? soff_l[n] : soff[n]));
+    };
+    // fused bias of the tile's columns: only the raw loads here -- the values are looked at when they are stored
     auto load_bias_raw = [&]() {
-        if (ktid < BN) {
+        if (role_k && kt < BN) {
             const int col = bias_col;
             const int cc = col < Lk ? col : 0;
             bcol_ok = col < Lk;
@@ -249,52 +284,37 @@ __global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_col
             }
         }
     };
-    auto load_k_item = [&](int it) {
-        int row = kr0 + it * K_RPP;
-        row = row < last_row ? row : last_row;
-        kreg[it] = *(const u32x4_t *)(ktb + (uint32_t)row * k_r2 + kcolb);
-    };
-    auto load_v_item = [&](int i) {
-        int row = 4 * vkg + i;
-        row = row < last_row ? row : last_row;
-        vreg[i] = *(const u32x4_t *)(vtb + (uint32_t)row * v_r2 + vcolb);
-    };
-    auto load_k = [&](int j) {
-        begin_tile(j);
+    auto load_tile = [&](int j) {
+        set_tile(j);
         load_bias_raw();
 #pragma unroll
-        for (int it = 0; it < K_IT; it++) load_k_item(it);
+        for (int n = 0; n < NL; n++) issue_load(n);
     };
-    auto load_v = [&](int j) {
-        (void)j;
+    auto store_stage = [&](int buf, int slot) {
+        if (role_k) {
+            char *sK = smem + SM::OFF_K + buf * SM::K_BYTES;
 #pragma unroll
-        for (int i = 0; i < 4; i++) load_v_item(i);
-    };
-    auto store_k = [&](int buf, int slot) {
-        char *sK = smem + SM::OFF_K + buf * SM::K_BYTES;
-#pragma unroll
-        for (int it = 0; it < K_IT; it++)
-            *(u32x4_t *)(sK + ((kr0 + it * K_RPP) * SM::SK + kc * 8) * 2) = kreg[it];
-        if (ktid < BN) {
-            float v = -INFINITY;
-            if (CMP) {
-                if (bcol_ok) v = __uint_as_float(braw);
-            } else if (bcol_ok && (!mrow || mraw)) {
-                v = brow ? E::lo(braw) * kLog2e : 0.f;
+            for (int it = 0; it < K_IT; it++)
+                *(u32x4_t *)(sK + ((kr0 + it * K_RPP) * SM::SK + kc * 8) * 2) = sreg[it];
+            if (kt < BN) {
+                float v = -INFINITY;
+                if (CMP) {
+                    if (bcol_ok) v = __uint_as_float(braw);
+                } else if (bcol_ok && (!mrow || mraw)) {
+                    v = brow ? E::lo(braw) * kLog2e : 0.f;
+                }
+                sBias[slot * BN + kt] = v;
             }
-            sBias[slot * BN + ktid] = v;
         }
-    };
-    auto store_v = [&](int buf) {  // transpose 4 keys x 8 d in registers, write V^T[d][key quad]
-        char *sVt = smem + SM::OFF_VT + buf * SM::VT_BYTES;
-        if (tid < V_ITEMS) {
+        if (role_v && kt < V_ITEMS) {  // transpose 4 keys x 8 d in registers, write V^T[d][key quad]
+            char *sVt = smem + SM::OFF_VT + buf * SM::VT_BYTES;
 #pragma unroll
             for (int dd = 0; dd < 8; dd++) {
                 const int w = dd >> 1;
                 const uint32_t sel = (dd & 1) ? 0x07060302u : 0x05040100u;
                 u32x2_t out;
-                out[0] = __builtin_amdgcn_perm(vreg[1][w], vreg[0][w], sel);
-                out[1] = __builtin_amdgcn_perm(vreg[3][w], vreg[2][w], sel);
+                out[0] = __builtin_amdgcn_perm(sreg[VB + 1][w], sreg[VB + 0][w], sel);
+                out[1] = __builtin_amdgcn_perm(sreg[VB + 3][w], sreg[VB + 2][w], sel);
                 *(u32x2_t *)(sVt + ((vc * 8 + dd) * SM::SVT + 4 * vkg) * 2) = out;
             }
         }
@@ -311,7 +331,6 @@ __global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_col
         vis_wave[nb] = CAUSAL ? visible(wrow0 + nb * 32) : 0;
     }
 
-    // `prefetch`: the K loads of the tile in flight are issued between the MFMAs
     auto qk = [&](f32x16_t (&s)[NQ][MB], int buf, int slot) {
         const char *sK = smem + SM::OFF_K + buf * SM::K_BYTES;
         // the accumulators start from the fused bias vector (bias * log2e, -inf for dropped keys) of the tile
@@ -346,7 +365,6 @@ __global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_col
             const int ks = f / MB, mb = f % MB;
 #pragma unroll
             for (int nb = 0; nb < NQ; nb++) s[nb][mb] = E::mfma(a[f], qf[nb][ks], s[nb][mb]);
-            if (f % (NF / K_IT) == 0) load_k_item(f / (NF / K_IT));
         }
         __builtin_amdgcn_sched_group_barrier(0x100, FR + 4 * MB, 0);
 #pragma unroll
@@ -381,7 +399,11 @@ __global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_col
 #pragma unroll
                 for (int i = 0; i < 16; i++) tmax = fmaxf(tmax, s[nb][mb][i]);
             tmax = xhalf_max(tmax);
-            if (__any(tmax > row_max[nb])) {
+            // Lazy rescale: the running maximum is only a reference point of the exp2 (any value gives the same
+            // softmax), so it is moved -- and O and the row sums rescaled -- only when a score exceeds it by more
+            // than 2^8; below that the probabilities stay far inside the range of the 16-bit operand and of the fp32
+            // sums, and almost every tile skips the rescale.
+            if (__any(tmax > row_max[nb] + 8.f)) {
                 const float new_max = fmaxf(row_max[nb], tmax);
                 const float safe = new_max == -INFINITY ? 0.f : new_max;
                 const float alpha = fast_exp2(row_max[nb] - safe);
@@ -406,7 +428,8 @@ __global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_col
             row_sum[nb] += psum;
         }
     };
-    // O^T += V^T P^T for one tile
+    // O^T += V^T P^T for one tile; the global loads of the tile two ahead are issued between the MFMAs (a burst of
+    // loads from every wave right after a barrier would queue up at the CU's address unit with the matrix pipe idle)
     auto pv = [&](const uint32_t (&pk)[NQ][8 * MB], int vbuf) {
         const char *sVt = smem + SM::OFF_VT + vbuf * SM::VT_BYTES;
         {
@@ -427,43 +450,40 @@ __global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_col
                     u32x4_t bop = {pk[nb][4 * kb], pk[nb][4 * kb + 1], pk[nb][4 * kb + 2], pk[nb][4 * kb + 3]};
                     o[nb][db] = E::mfma(a[f], bop, o[nb][db]);
                 }
+#pragma unroll
+                for (int n = f * NL / NF; n < (f + 1) * NL / NF; n++) issue_load(n);  // spread evenly over the MFMAs
             }
         }
     };
 
-    // ---- main loop: tile i is computed from LDS buffers i&1 while tile i+1 travels global -> registers; its LDS
-    // stores go to the other buffers (last read in iteration i-1) after the compute, one barrier per tile
-    int jc = next_active(0);
-    if (jc < n_end) {
-        load_k(jc);
-        load_v(jc);
-        store_k(0, 0);
-        store_v(0);
+    // ---- main loop.  Tile i is computed from LDS buffers i&1.  The registers hold tile i+1 (loaded during the PV
+    // MFMAs of the previous iteration); its LDS stores go to the other buffers -- last read before the previous
+    // barrier -- between the scores and the softmax, when the LDS port is idle; the loads of tile i+2 then reuse the
+    // registers during the PV MFMAs.  One barrier per tile.
+    const int j0 = next_active(0);
+    if (j0 < n_end) {
+        const int j1 = next_active(j0 + 1);
+        load_tile(j0);
+        store_stage(0, 0);
+        load_tile(j1 < n_end ? j1 : j0);
         __syncthreads();
 
         f32x16_t sa[NQ][MB];
-        int i = 0;
+        int i = 0, jc = j0, jn1 = j1;
         while (jc < n_end) {
-            const int jn = next_active(jc + 1);
-            // the loads of the next tile are spread over the MFMAs of this one (after the last tile the current
-            // one is simply fetched again and dropped): eight waves issuing all their loads at once right after
-            // the barrier would queue up at the CU's address unit while the matrix pipe idles
-            begin_tile(jn < n_end ? jn : jc);
-            __builtin_amdgcn_sched_barrier(0);
+            const int jn2 = jn1 < n_end ? next_active(jn1 + 1) : n_end;
             qk(sa, i & 1, i & 1);
-            load_bias_raw();
-            load_v(jc);  // V of the tile in flight: issued before the softmax so that softmax and PV cover the latency
             __builtin_amdgcn_sched_barrier(0);
+            if (jn1 < n_end) store_stage((i + 1) & 1, (i + 1) & 1);
             uint32_t pk[NQ][8 * MB];
             softmax(sa, jc, pk);
-            pv(pk, i & 1);
             __builtin_amdgcn_sched_barrier(0);
-            if (jn < n_end) {
-                store_k((i + 1) & 1, (i + 1) & 1);
-                store_v((i + 1) & 1);
-            }
+            set_tile(jn2 < n_end ? jn2 : jc);  // (after the last tile an existing one is fetched again and dropped)
+            pv(pk, i & 1);
+            load_bias_raw();
+            __builtin_amdgcn_sched_barrier(0);
             __syncthreads();
-            i++; jc = jn;
+            i++; jc = jn1; jn1 = jn2;
         }
     }
 
@@ -512,8 +532,14 @@ hipError_t launch_one(const FwdParams &p, hipStream_t stream) {
 }
 
 template <typename T, int D>
-hipError_t launch_d(const FwdParams &p, int variant, hipStream_t stream) {
-    (void)variant;
+hipError_t launch_d(const FwdParams &p, hipStream_t stream) {
+    // 256-row workgroups (8 waves, one workgroup per CU) stage every K / V tile once for twice the rows and win
+    // whenever the grid still has a few workgroups per CU; smaller problems keep 128-row workgroups, two per CU
+    const int64_t groups256 = (int64_t)p.B * p.H * ((p.Lq + 255) / 256);
+    if constexpr (D == 128) if (groups256 >= 512) {
+        if (p.cmp.on) return p.causal ? launch_one<T, D, 1, 64, true, true, 8>(p, stream) : launch_one<T, D, 1, 64, false, true, 8>(p, stream);
+        return p.causal ? launch_one<T, D, 1, 64, true, false, 8>(p, stream) : launch_one<T, D, 1, 64, false, false, 8>(p, stream);
+    }
     if (p.cmp.on) return p.causal ? launch_one<T, D, 1, 64, true, true>(p, stream) : launch_one<T, D, 1, 64, false, true>(p, stream);
     return p.causal ? launch_one<T, D, 1, 64, true, false>(p, stream) : launch_one<T, D, 1, 64, false, false>(p, stream);
 }
@@ -526,10 +552,10 @@ bool fwd_colmask_applicable(const FwdParams &p) {
     return mask_ok && bias_ok && (p.Lk + 31) / 32 <= MAX_TILES;
 }
 
-hipError_t launch_fwd_colmask(const FwdParams &p, int dtype, int nq, hipStream_t stream) {
+hipError_t launch_fwd_colmask(const FwdParams &p, int dtype, hipStream_t stream) {
     const bool d64 = p.d <= 64;
-    if (dtype == 0) return d64 ? launch_d<bf16_tag, 64>(p, nq, stream) : launch_d<bf16_tag, 128>(p, nq, stream);
-    return d64 ? launch_d<fp16_tag, 64>(p, nq, stream) : launch_d<fp16_tag, 128>(p, nq, stream);
+    if (dtype == 0) return d64 ? launch_d<bf16_tag, 64>(p, stream) : launch_d<bf16_tag, 128>(p, stream);
+    return d64 ? launch_d<fp16_tag, 64>(p, stream) : launch_d<fp16_tag, 128>(p, stream);
 }
 
 }  // namespace fdma

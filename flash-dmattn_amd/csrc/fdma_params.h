@@ -122,7 +122,7 @@ struct BwdParams {
 hipError_t launch_fwd(const FwdParams &p, int dtype, hipStream_t stream);
 // column-mask specialisation (mask / bias absent or broadcast over queries); nq = 32-row blocks per wave
 bool fwd_colmask_applicable(const FwdParams &p);
-hipError_t launch_fwd_colmask(const FwdParams &p, int dtype, int nq, hipStream_t stream);
+hipError_t launch_fwd_colmask(const FwdParams &p, int dtype, hipStream_t stream);
 hipError_t launch_fwd_decode(const FwdParams &p, int dtype, hipStream_t stream);
 hipError_t launch_bwd(const BwdParams &p, int dtype, hipStream_t stream);
 // column-mask specialisations of the two main backward kernels
