@@ -204,18 +204,43 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
     u32x4_t qreg[Q_IT], doreg[Q_IT];
     float lreg = INFINITY, dreg = 0.f;
     bool stat_ok = false;
-    auto load_step = [&](int step) {
+    // Byte offsets of this thread's loads inside a 64-row block are loop invariants -- one set for full blocks, one
+    // for the (only) partial block at the end of the queries, whose rows beyond Lq are clamped to the last row
+    // (finite duplicates, cancelled by LSE = +inf) -- so a load is one instruction with a scalar block base.
+    typedef const __attribute__((address_space(1))) char *gptr_t;
+    auto uniform_ptr = [](const void *ptr) -> gptr_t {
+        const uint64_t v = (uint64_t)ptr;
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+        return (gptr_t)(((uint64_t)hi << 32) | lo);
+    };
+    const int m_last = (f.Lq - 1) / KV_BM, row_last = (f.Lq - 1) % KV_BM;
+    uint32_t qoff[Q_IT], qoff_l[Q_IT], dooff[Q_IT], dooff_l[Q_IT];
+#pragma unroll
+    for (int it = 0; it < Q_IT; it++) {
+        const int row = qr0 + it * RPP, row_c = row < row_last ? row : row_last;
+        qoff[it] = (uint32_t)(row * f.q_r + qcol) * 2;
+        qoff_l[it] = (uint32_t)(row_c * f.q_r + qcol) * 2;
+        dooff[it] = (uint32_t)(row * p.do_r + qcol) * 2;
+        dooff_l[it] = (uint32_t)(row_c * p.do_r + qcol) * 2;
+    }
+    gptr_t ld_qbase = nullptr, ld_dobase = nullptr;  // block bases of the step being fetched (scalar registers)
+    bool ld_partial = false;
+    // tile load `n` of the step being fetched: 0 .. Q_IT-1 are Q rows, Q_IT .. 2*Q_IT-1 dO rows
+    auto load_item = [&](int n) {
+        if (n < Q_IT) qreg[n] = *(const __attribute__((address_space(1))) u32x4_t *)(ld_qbase + (ld_partial ? qoff_l[n] : qoff[n]));
+        else doreg[n - Q_IT] = *(const __attribute__((address_space(1))) u32x4_t *)(ld_dobase + (ld_partial ? dooff_l[n - Q_IT] : dooff[n - Q_IT]));
+    };
+    // everything of a step's fetch except the tile loads: block bases, column constant, row statistics
+    auto load_step = [&](int step, bool with_tiles) {
         const int gi = g_lo + step / n_m, mi = m_hi - 1 - step % n_m;  // last query block first: see below
         const int h = hk * G + gi, m0 = mi * KV_BM;
         column_const_load(h);
-        const uint16_t *qbase = (const uint16_t *)f.q + b * f.q_b + h * f.q_h + qcol;
-        const uint16_t *dobase = (const uint16_t *)p.dout + b * p.do_b + h * p.do_h + qcol;
+        ld_qbase = uniform_ptr((const uint16_t *)f.q + b * f.q_b + h * f.q_h + (int64_t)m0 * f.q_r);
+        ld_dobase = uniform_ptr((const uint16_t *)p.dout + b * p.do_b + h * p.do_h + (int64_t)m0 * p.do_r);
+        ld_partial = mi == m_last;
+        if (with_tiles) {
 #pragma unroll
-        for (int it = 0; it < Q_IT; it++) {
-            int qq = m0 + qr0 + it * RPP;
-            qq = qq < f.Lq ? qq : f.Lq - 1;  // rows beyond Lq: finite duplicates, cancelled by LSE = +inf
-            qreg[it] = *(const u32x4_t *)(qbase + (int64_t)qq * f.q_r);
-            doreg[it] = *(const u32x4_t *)(dobase + (int64_t)qq * p.do_r);
+            for (int n = 0; n < 2 * Q_IT; n++) load_item(n);
         }
         // row statistics: raw, unconditional loads from a clamped row (nothing may look at a loaded value here, or the
         // wait for it would also cover the tile loads above); range check and scaling happen in store_step
@@ -252,7 +277,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
     float cconst = 0.f;
 
     if (n_steps > 0) {
-        load_step(0);
+        load_step(0, true);
         store_step(0);
         cconst = column_const_value();
         __syncthreads();
@@ -274,8 +299,10 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
         for (int mb = 0; mb < MB; mb++)
 #pragma unroll
             for (int i = 0; i < 16; i++) { s[mb][i] = cconst; dp[mb][i] = 0.f; }
-        // global loads of the next step: in flight behind all the matrix work of this one
-        if (step + 1 < n_steps) load_step(step + 1);
+        // Global loads of the next step: in flight behind all the matrix work of this one.  The tile loads are issued
+        // one by one between the MFMAs below: all of them at once, from every wave at the same moment, queue up at the
+        // CU's address unit while the matrix pipe idles.  (After the last step the same tiles are fetched again and dropped.)
+        load_step(step + 1 < n_steps ? step + 1 : step, false);
         __builtin_amdgcn_sched_barrier(0);
         {
             constexpr int NF = 2 * MB * KS, FR = 8;  // fragment f: (ks, mb, which) with which = 0: Q, 1: dO
@@ -292,6 +319,8 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
                 const int which = fi & 1, mb = (fi >> 1) % MB, ks = (fi >> 1) / MB;
                 if (which) dp[mb] = E::mfma(a[fi], vf[ks], dp[mb]);
                 else s[mb] = E::mfma(a[fi], kf[ks], s[mb]);
+#pragma unroll
+                for (int n = fi * 2 * Q_IT / NF; n < (fi + 1) * 2 * Q_IT / NF; n++) load_item(n);
             }
         }
 
