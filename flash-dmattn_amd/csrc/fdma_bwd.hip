@@ -71,28 +71,31 @@ __global__ void __launch_bounds__(256) bwd_dot_kernel(const BwdParams p) {
 // bias tile through LDS: fused[q][k] = bias[q][k] where (mask[q][k] and k < Lk), else -inf, built from
 // coalesced 16-byte bias / 8-byte mask loads (broadcast dims simply have stride 0).  exp2(-inf) = 0 does
 // the masking.  dS goes back through an LDS tile so that dBias is written with coalesced 16-byte stores
-// at the bias's own shape; over the query heads of a group it is summed in registers first.
+// at the bias's own shape.  GSUM: a per-query bias with fewer heads than queries -- dS is summed over the
+// query heads of the group in registers first and leaves through a tile of its own.  Otherwise every lane
+// writes its dS over the fused-bias elements it has just read (same rows, its own column), which saves the
+// extra tile and 64 registers: at d <= 64 two workgroups then fit on a CU and cover each other's phases.
 constexpr int KV_BM = 64;   // query rows per step
 constexpr int KV_BN = 128;  // key columns per workgroup (32 per wave)
 
-template <int D> struct KvSmem {
+template <int D, bool GSUM> struct KvSmem {
     static constexpr int S = D + 8;          // Q / dO row stride (elements)
     static constexpr int SB = KV_BN + 8;     // fused-bias / dS tile row stride (elements)
     static constexpr int Q_BYTES = KV_BM * S * 2;
     static constexpr int FB_BYTES = KV_BM * SB * 2;
     static constexpr int STAGE = 2 * Q_BYTES + 2 * KV_BM * 4 + FB_BYTES;  // Q, dO, LSE, D, fused bias
     static constexpr int OFF_DS = 2 * STAGE;
-    static constexpr int TOTAL = OFF_DS + FB_BYTES;
+    static constexpr int TOTAL = OFF_DS + (GSUM ? FB_BYTES : 0);
 };
 
 template <typename T> struct NegInfPair;
 template <> struct NegInfPair<bf16_tag> { static constexpr uint32_t value = 0xFF80FF80u; };
 template <> struct NegInfPair<fp16_tag> { static constexpr uint32_t value = 0xFC00FC00u; };
 
-template <typename T, int D, bool CAUSAL>
-__global__ void __launch_bounds__(NTHREADS, 1) bwd_dkdv_kernel(const BwdParams p) {
+template <typename T, int D, bool CAUSAL, bool GSUM>
+__global__ void __launch_bounds__(NTHREADS, (D <= 64 && !GSUM) ? 2 : 1) bwd_dkdv_kernel(const BwdParams p) {
     using E = Elem<T>;
-    using SM = KvSmem<D>;
+    using SM = KvSmem<D, GSUM>;
     constexpr int KS = D / 16;
     constexpr int DB = D / 32;
     constexpr int MB = KV_BM / 32;
@@ -258,14 +261,15 @@ __global__ void __launch_bounds__(NTHREADS, 1) bwd_dkdv_kernel(const BwdParams p
     const int tdh = (lane >> 4) & 1;
     const uint32_t tr_off = (uint32_t)(((8 * g + te) * SM::S + 16 * tdh + 4 * tcp) * 2);
     const uint32_t a_off = (uint32_t)((a_row * SM::S + g * 8) * 2);
-    uint16_t *sDS = (uint16_t *)(smem + SM::OFF_DS);
 
     float colsum = 0.f;       // row-broadcast dbias: sum over queries of dS for this lane's key
-    f32x16_t dsum[MB];        // per-query dbias with bias heads < H: sum over the group
+    f32x16_t dsum[GSUM ? MB : 1];  // per-query dbias with bias heads < H: sum over the group
+    if (GSUM) {
 #pragma unroll
-    for (int mb = 0; mb < MB; mb++)
+        for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-        for (int i = 0; i < 16; i++) dsum[mb][i] = 0.f;
+            for (int i = 0; i < 16; i++) dsum[mb][i] = 0.f;
+    }
 
     if (n_steps > 0) {
         load_step(0);
@@ -285,7 +289,8 @@ __global__ void __launch_bounds__(NTHREADS, 1) bwd_dkdv_kernel(const BwdParams p
         const char *sDO = sQ + SM::Q_BYTES;
         const float *sLSE = (const float *)(sQ + 2 * SM::Q_BYTES);
         const float *sDD = sLSE + KV_BM;
-        const uint16_t *sFB = (const uint16_t *)(sDD + KV_BM) + wave * 32 + r;  // this lane's column
+        uint16_t *sFB = (uint16_t *)(smem + buf * SM::STAGE + 2 * SM::Q_BYTES + 2 * KV_BM * 4) + wave * 32 + r;  // this lane's column
+        uint16_t *sDS = GSUM ? (uint16_t *)(smem + SM::OFF_DS) : (uint16_t *)(smem + buf * SM::STAGE + 2 * SM::Q_BYTES + 2 * KV_BM * 4);
 
         // ---- S = Q K^T and dP = dO V^T
         f32x16_t s[MB], dp[MB];
@@ -294,7 +299,7 @@ __global__ void __launch_bounds__(NTHREADS, 1) bwd_dkdv_kernel(const BwdParams p
 #pragma unroll
             for (int i = 0; i < 16; i++) { s[mb][i] = 0.f; dp[mb][i] = 0.f; }
         {
-            constexpr int NF = 2 * MB * KS, FR = 8;
+            constexpr int NF = 2 * MB * KS, FR = (D <= 64 && !GSUM) ? 4 : 8;  // (two workgroups per CU cover the rest of the LDS latency)
             u32x4_t a[NF];
             auto frag = [&](int fi) {
                 const int which = fi & 1, mb = (fi >> 1) % MB, ks = (fi >> 1) / MB;
@@ -315,13 +320,16 @@ __global__ void __launch_bounds__(NTHREADS, 1) bwd_dkdv_kernel(const BwdParams p
         // registers involved have no load pending from the previous trip), which is free only while nothing is in
         // flight.  The softmax and the dK / dV GEMMs below cover the latency.
         __builtin_amdgcn_sched_barrier(0);
-        if (step + 1 < n_steps) load_step(step + 1);
-        __builtin_amdgcn_sched_barrier(0);
+        if (GSUM || D > 64) {
+            if (step + 1 < n_steps) load_step(step + 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
 
         // ---- P = exp2((S*scale + fused)*log2e - LSE*log2e) ; dS = P * (dP - D)
         const bool diag = CAUSAL && (n0 + wave * 32 + 31 > m0 + shift);
         uint32_t ppk[MB * 8], dpk[MB * 8];
-        f32x16_t ds[MB];
+        f32x16_t ds[GSUM ? MB : 1];
+        float part = 0.f;
 #pragma unroll
         for (int mb = 0; mb < MB; mb++)
 #pragma unroll
@@ -349,15 +357,32 @@ __global__ void __launch_bounds__(NTHREADS, 1) bwd_dkdv_kernel(const BwdParams p
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
                     dsv[e] *= pv[e];
-                    ds[mb][8 * blk + e] = dsv[e];
+                    if (GSUM) ds[mb][8 * blk + e] = dsv[e];
+                    else part += dsv[e];
                 }
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     ppk[mb * 8 + blk * 4 + e] = E::pack2(pv[2 * e], pv[2 * e + 1]);
                     dpk[mb * 8 + blk * 4 + e] = E::pack2(dsv[2 * e], dsv[2 * e + 1]);
                 }
+                if (!GSUM && bias_rows && !use_accum) {
+                    // dS replaces the fused-bias elements this lane has just read: same rows, its own column
+#pragma unroll
+                    for (int e = 0; e < 4; e++) {
+                        const uint32_t w = dpk[mb * 8 + blk * 4 + e];
+                        sFB[(q0l + 2 * e) * SM::SB] = (uint16_t)(w & 0xffffu);
+                        sFB[(q0l + 2 * e + 1) * SM::SB] = (uint16_t)(w >> 16);
+                    }
+                }
             }
 
+        // (two workgroups per CU: the staging registers of the next step would not fit next to the softmax's, so its
+        // loads are issued here, behind the softmax; the other workgroup covers what the GEMMs below do not)
+        if (!GSUM && D <= 64) {
+            __builtin_amdgcn_sched_barrier(0);
+            if (step + 1 < n_steps) load_step(step + 1);
+            __builtin_amdgcn_sched_barrier(0);
+        }
         // ---- dV^T += dO^T P ; dK^T += Q^T dS
 #pragma unroll
         for (int qb = 0; qb < KV_BM / 16; qb++) {
@@ -379,11 +404,12 @@ __global__ void __launch_bounds__(NTHREADS, 1) bwd_dkdv_kernel(const BwdParams p
         bool tile_out = false;  // this step leaves a dS tile in LDS to be stored (uniform)
         if (has_bias) {
             if (!bias_rows) {
-                float part = 0.f;
+                if (GSUM) {
 #pragma unroll
-                for (int mb = 0; mb < MB; mb++)
+                    for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-                    for (int i = 0; i < 16; i++) part += ds[mb][i];
+                        for (int i = 0; i < 16; i++) part += ds[mb][i];
+                }
                 colsum += part;
                 const bool last_m = (step % n_m) == n_m - 1;
                 if (last_m && (f.Hb == f.H || gi == G - 1)) {
@@ -393,6 +419,22 @@ __global__ void __launch_bounds__(NTHREADS, 1) bwd_dkdv_kernel(const BwdParams p
                         else ((uint16_t *)p.dbias)[b * p.db_b + hb * p.db_h + key] = (uint16_t)(E::pack2(tot, 0.f) & 0xffffu);
                     }
                     colsum = 0.f;
+                }
+            } else if (!GSUM) {
+                // every step owns its dbias tile (bias per query head, or one query head per bias head)
+                if (use_accum) {
+#pragma unroll
+                    for (int mb = 0; mb < MB; mb++)
+#pragma unroll
+                        for (int i = 0; i < 16; i++) {
+                            const int qq = m0 + 32 * mb + 16 * (i >> 3) + 8 * g + (i & 7);
+                            const uint32_t w = dpk[mb * 8 + (i >> 3) * 4 + ((i & 7) >> 1)];
+                            const float v = (i & 1) ? E::hi(w) : E::lo(w);
+                            if (qq < f.Lq && key < f.Lk)
+                                atomicAdd(p.dbias_accum + b * p.dba_b + hb * p.dba_h + (int64_t)qq * p.dba_r + key, v);
+                        }
+                } else {
+                    tile_out = true;
                 }
             } else {
                 const bool per_head = f.Hb == f.H;
@@ -518,17 +560,17 @@ hipError_t launch_bwd_t(const BwdParams &p, hipStream_t stream) {
         if ((e = launch_bwd_dkdv_colmask(p, dtype_code, stream)) != hipSuccess) return e;
     } else if (f.Lk > 0) {
         dim3 grid((f.Lk + KV_BN - 1) / KV_BN, f.Hk, f.B);
-        const size_t smem = KvSmem<D>::TOTAL;
-        if (f.causal) {
-            auto kern = bwd_dkdv_kernel<T, D, true>;
-            if ((e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem)) != hipSuccess) return e;
+        // a per-query bias shared by several query heads: dS is summed over the group before it is written
+        const bool gsum = f.bias != nullptr && f.bi_r != 0 && f.Hb != f.H && f.H / f.Hk > 1;
+        auto launch = [&](auto kern, size_t smem) -> hipError_t {
+            hipError_t e2 = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+            if (e2 != hipSuccess) return e2;
             hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, stream, p);
-        } else {
-            auto kern = bwd_dkdv_kernel<T, D, false>;
-            if ((e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem)) != hipSuccess) return e;
-            hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, stream, p);
-        }
-        if ((e = hipGetLastError()) != hipSuccess) return e;
+            return hipGetLastError();
+        };
+        if (gsum) e = f.causal ? launch(bwd_dkdv_kernel<T, D, true, true>, KvSmem<D, true>::TOTAL) : launch(bwd_dkdv_kernel<T, D, false, true>, KvSmem<D, true>::TOTAL);
+        else e = f.causal ? launch(bwd_dkdv_kernel<T, D, true, false>, KvSmem<D, false>::TOTAL) : launch(bwd_dkdv_kernel<T, D, false, false>, KvSmem<D, false>::TOTAL);
+        if (e != hipSuccess) return e;
     }
     if (p.dbias_accum) {
         hipLaunchKernelGGL((dbias_convert_kernel<T>), dim3(1024), dim3(256), 0, stream, p, nb, f.Hb, nr, f.Lk);
