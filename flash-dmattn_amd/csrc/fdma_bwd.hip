@@ -421,21 +421,9 @@ __global__ void __launch_bounds__(NTHREADS, (D <= 64 && !GSUM) ? 2 : 1) bwd_dkdv
                     colsum = 0.f;
                 }
             } else if (!GSUM) {
-                // every step owns its dbias tile (bias per query head, or one query head per bias head)
-                if (use_accum) {
-#pragma unroll
-                    for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-                        for (int i = 0; i < 16; i++) {
-                            const int qq = m0 + 32 * mb + 16 * (i >> 3) + 8 * g + (i & 7);
-                            const uint32_t w = dpk[mb * 8 + (i >> 3) * 4 + ((i & 7) >> 1)];
-                            const float v = (i & 1) ? E::hi(w) : E::lo(w);
-                            if (qq < f.Lq && key < f.Lk)
-                                atomicAdd(p.dbias_accum + b * p.dba_b + hb * p.dba_h + (int64_t)qq * p.dba_r + key, v);
-                        }
-                } else {
-                    tile_out = true;
-                }
+                // every step owns its dbias tile (bias per query head, or one query head per bias head); dbias
+                // elements shared between workgroups take the GSUM variant and its fp32 atomics
+                tile_out = true;
             } else {
                 const bool per_head = f.Hb == f.H;
 #pragma unroll
@@ -560,8 +548,9 @@ hipError_t launch_bwd_t(const BwdParams &p, hipStream_t stream) {
         if ((e = launch_bwd_dkdv_colmask(p, dtype_code, stream)) != hipSuccess) return e;
     } else if (f.Lk > 0) {
         dim3 grid((f.Lk + KV_BN - 1) / KV_BN, f.Hk, f.B);
-        // a per-query bias shared by several query heads: dS is summed over the group before it is written
-        const bool gsum = f.bias != nullptr && f.bi_r != 0 && f.Hb != f.H && f.H / f.Hk > 1;
+        // a per-query bias shared by several query heads: dS is summed over the group before it is written; one
+        // shared by several workgroups (broadcast over the batch or over kv heads) is accumulated with fp32 atomics
+        const bool gsum = f.bias != nullptr && f.bi_r != 0 && ((f.Hb != f.H && f.H / f.Hk > 1) || p.dbias_accum != nullptr);
         auto launch = [&](auto kern, size_t smem) -> hipError_t {
             hipError_t e2 = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
             if (e2 != hipSuccess) return e2;

@@ -73,6 +73,7 @@ SMALL_CASES = {
     "full_mask_full_bias": (2, 200, 264, 4, 2, 64, (2, 4, 200, 264), (2, 4, 200, 264), 64, True),
     "full_bias_kv_heads": (2, 200, 264, 4, 2, 64, (2, 2, 200, 264), (2, 1, 200, 264), 64, True),
     "full_bias_batch_broadcast": (2, 200, 264, 4, 2, 64, (1, 2, 200, 264), (2, 1, 200, 264), 64, True),
+    "full_bias_per_head_batch_broadcast": (2, 200, 264, 4, 2, 64, (1, 4, 200, 264), (2, 4, 200, 264), 64, True),
     "row_bias_single_head": (2, 200, 264, 4, 2, 64, (2, 1, 1, 264), (2, 1, 1, 264), 64, False),
     "lq_lt_lk_bottom_right": (1, 100, 333, 2, 2, 128, (1, 2, 1, 333), (1, 1, 100, 333), 100, True),
     "lq_gt_lk_empty_rows": (1, 333, 100, 2, 2, 128, (1, 2, 1, 100), (1, 1, 333, 100), 50, True),
