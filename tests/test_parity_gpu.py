@@ -273,19 +273,29 @@ def test_mid_size_vs_eager_fp32(name):
         assert_grad_close(g, r, n)
 
 
+LARGE_GRID_CASES = {
+    # name: (B, Lq, Lk, H, Hk, D, window, causal, dtype) -- batch * heads * ceil(Lq / 256) >= 512 and d = 128
+    "bf16_causal_ragged": (4, 1000, 1090, 32, 8, 128, 300, True, torch.bfloat16),
+    "fp16_noncausal_lq_lt_lk": (6, 520, 1090, 32, 8, 128, 200, False, torch.float16),
+    "bf16_causal_lq_gt_lk_empty_rows": (4, 1024, 700, 32, 4, 128, 150, True, torch.bfloat16),
+}
+
+
 @pytest.mark.parametrize("compact", ["0", "2"])
-def test_large_grid_256_row_workgroups_vs_eager_fp32(compact):
-    """A d = 128 problem whose grid is large enough (batch * heads * ceil(Lq / 256) >= 512) for the forward to take
-    its 256-row, 8-wave workgroups (split K / V staging roles), on the original and on the compacted key axis;
-    ragged lengths so that the last query block and the last key tile are partial."""
+@pytest.mark.parametrize("name", list(LARGE_GRID_CASES))
+def test_large_grid_256_row_workgroups_vs_eager_fp32(name, compact):
+    """d = 128 problems whose grid is large enough for the forward to take its 256-row, 8-wave workgroups (split
+    K / V staging roles), on the original and on the compacted key axis; ragged lengths so that the last query
+    block and the last key tile are partial, both dtypes, causal with empty rows and non-causal."""
     os.environ["FDMA_COMPACT"] = compact
-    B, Lq, Lk, H, Hk, D, W = 4, 1000, 1090, 32, 8, 128, 300
+    B, Lq, Lk, H, Hk, D, W, causal, dtype = LARGE_GRID_CASES[name]
     q, k, v, mask, bias = make_inputs(B, Lq, Lk, H, Hk, D, (B, Hk, 1, Lk), (B, Hk, 1, Lk), W, seed=5)
-    out, lse, (dq, dk, dv, db) = _run_fwd_bwd(q, k, v, mask, bias, True)
+    q, k, v, bias = [t.to(dtype) for t in (q, k, v, bias)]
+    out, lse, (dq, dk, dv, db) = _run_fwd_bwd(q, k, v, mask, bias, causal)
     qd, kd, vd, md, bd = _to_dev(q, k, v, mask, bias)
-    ro, rdq, rdk, rdv, rdb = eager.attention_forward_backward(qd, kd, vd, md, bd, None, True)
+    ro, rdq, rdk, rdv, rdb = eager.attention_forward_backward(qd, kd, vd, md, bd, None, causal)
     assert_out_close(out, ro)
-    _, rl = eager.attention_forward(qd, kd, vd, md, bd, None, True)
+    _, rl = eager.attention_forward(qd, kd, vd, md, bd, None, causal)
     _check_lse(lse, rl)
     for g, r, n in ((dq, rdq, "dq"), (dk, rdk, "dk"), (dv, rdv, "dv"), (db, rdb, "dbias")):
         assert_grad_close(g, r, n)
