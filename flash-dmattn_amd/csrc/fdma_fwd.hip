@@ -276,7 +276,9 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) fwd_kernel(const Fw
 #pragma unroll
             for (int i = 0; i < 16; i++) tmax = fmaxf(tmax, s[mb][i]);
         tmax = xhalf_max(tmax);
-        if (__any(tmax > row_max)) {
+        // lazy rescale: the running maximum is only the reference point of the exp2, so it moves (and O and the row
+        // sums are rescaled) only when a score exceeds it by more than 2^8 -- rare after the first tiles
+        if (__any(tmax > row_max + 8.f)) {
             const float new_max = fmaxf(row_max, tmax);
             const float safe = new_max == -INFINITY ? 0.f : new_max;
             const float alpha = fast_exp2(row_max - safe);
