@@ -51,26 +51,35 @@ inline int xcd_grid(int pairs, int n_units, int per_unit) {
 // ------------------------------------------------------------------------------------------------
 // dK / dV / dBias
 // ------------------------------------------------------------------------------------------------
-constexpr int KV_BM = 64;   // query rows per step
+constexpr int KV_BM = 64;   // query rows per planning block (the work split counts these)
 constexpr int KV_BN = 128;  // key columns per workgroup (32 per wave)
 
+// Query rows per step.  At d = 128 the stationary K / V fragments and the dK / dV accumulators alone take 192 registers
+// per lane; with 32-row steps and V parked in LDS (every lane re-reads its own row: a private spill, no sharing) the
+// kernel fits in 256 registers and 70 KB of LDS, so that two workgroups share a CU and fill each other's stalls.
 template <int D> struct KvcSmem {
+    static constexpr int BM = D > 64 ? 32 : 64;
+    static constexpr bool V_LDS = D > 64;
     static constexpr int S = D + 8;
-    static constexpr int Q_BYTES = KV_BM * S * 2;
-    static constexpr int STAGE = 2 * Q_BYTES + 2 * KV_BM * 4;  // Q, dO, LSE, D
-    static constexpr int TOTAL = 2 * STAGE;
+    static constexpr int Q_BYTES = BM * S * 2;
+    static constexpr int STAGE = 2 * Q_BYTES + 2 * BM * 4;  // Q, dO, LSE, D
+    static constexpr int OFF_V = 2 * STAGE;
+    static constexpr int TOTAL = OFF_V + (V_LDS ? KV_BN * S * 2 : 0);
 };
 
 // CMP: the key axis is the compacted list of kept columns (fdma_compact.hip); a lane still owns one key,
 // reads it from the dense copies, and writes its gradients to the key's original row / column.
 template <typename T, int D, bool CAUSAL, bool CMP>
-__global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_kernel(const BwdParams p) {
+__global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const BwdParams p) {
     using E = Elem<T>;
     using SM = KvcSmem<D>;
+    constexpr int BM = SM::BM;       // query rows per step
+    constexpr int SUB = KV_BM / BM;  // steps per planning block
+    constexpr bool V_LDS = SM::V_LDS;
     constexpr int KS = D / 16;
     constexpr int DB = D / 32;
-    constexpr int MB = KV_BM / 32;
-    constexpr int CH = D / 8, RPP = NTHREADS / CH, Q_IT = KV_BM / RPP;
+    constexpr int MB = BM / 32;
+    constexpr int CH = D / 8, RPP = NTHREADS / CH, Q_IT = BM / RPP;
 
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
@@ -130,7 +139,8 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
     const int okey_wlast = CMP ? cidx[n0 + wave * 32 + 31 < Lk ? n0 + wave * 32 + 31 : Lk - 1] : n0 + wave * 32 + 31;
 
     // ---- stationary K / V fragments (B operands): lane holds K[key][16ks + 8g .. +8]
-    u32x4_t kf[KS], vf[KS];
+    u32x4_t kf[KS], vf[V_LDS ? 1 : KS];
+    char *sVrow = smem + SM::OFF_V + ((wave * 32 + r) * SM::S + g * 8) * 2;  // V_LDS: this lane's V row, its chunks
     {
         const uint16_t *kp = (const uint16_t *)f.k + b * f.k_b + (int64_t)key_c * f.k_r + hk * f.k_h;
         const uint16_t *vp = (const uint16_t *)f.v + b * f.v_b + (int64_t)key_c * f.v_r + hk * f.v_h;
@@ -144,7 +154,8 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
 #pragma unroll
             for (int e = 0; e < 4; e++) kv[e] = E::pack2(E::lo(kv[e]) * f.scale_log2, E::hi(kv[e]) * f.scale_log2);
             kf[ks] = kv;
-            vf[ks] = vv;
+            if (V_LDS) *(u32x4_t *)(sVrow + ks * 32) = vv;
+            else vf[ks] = vv;
         }
     }
 
@@ -166,7 +177,10 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
         m_lo = m_start + seg * len;
         m_hi = m_lo + len < M_blocks ? m_lo + len : M_blocks;
     }
-    const int n_m = m_hi > m_lo ? m_hi - m_lo : 0;
+    // the planning blocks [m_lo, m_hi) in steps of BM rows: [s_lo, s_hi), without steps entirely beyond Lq
+    const int S_blocks = (f.Lq + BM - 1) / BM;
+    const int s_lo = m_lo * SUB, s_hi = m_hi * SUB < S_blocks ? m_hi * SUB : S_blocks;
+    const int n_m = s_hi > s_lo ? s_hi - s_lo : 0;
     // (g outer, m inner); the query blocks are walked from the LAST one down, so that the
     // workgroups of one (batch, kv head) pair, which run side by side on an XCD, all begin at the same
     // Q / dO tile and stream the same tiles at the same time (L2 hits instead of re-fetches)
@@ -213,7 +227,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
         const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
         return (gptr_t)(((uint64_t)hi << 32) | lo);
     };
-    const int m_last = (f.Lq - 1) / KV_BM, row_last = (f.Lq - 1) % KV_BM;
+    const int m_last = (f.Lq - 1) / BM, row_last = (f.Lq - 1) % BM;
     uint32_t qoff[Q_IT], qoff_l[Q_IT], dooff[Q_IT], dooff_l[Q_IT];
 #pragma unroll
     for (int it = 0; it < Q_IT; it++) {
@@ -232,8 +246,8 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
     };
     // everything of a step's fetch except the tile loads: block bases, column constant, row statistics
     auto load_step = [&](int step, bool with_tiles) {
-        const int gi = g_lo + step / n_m, mi = m_hi - 1 - step % n_m;  // last query block first: see below
-        const int h = hk * G + gi, m0 = mi * KV_BM;
+        const int gi = g_lo + step / n_m, mi = s_hi - 1 - step % n_m;  // last query block first: see below
+        const int h = hk * G + gi, m0 = mi * BM;
         column_const_load(h);
         ld_qbase = uniform_ptr((const uint16_t *)f.q + b * f.q_b + h * f.q_h + (int64_t)m0 * f.q_r);
         ld_dobase = uniform_ptr((const uint16_t *)p.dout + b * p.do_b + h * p.do_h + (int64_t)m0 * p.do_r);
@@ -245,7 +259,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
         // row statistics: raw, unconditional loads from a clamped row (nothing may look at a loaded value here, or the
         // wait for it would also cover the tile loads above); range check and scaling happen in store_step
         {
-            const int qq = m0 + (tid & (KV_BM - 1));
+            const int qq = m0 + (tid & (BM - 1));
             stat_ok = qq < f.Lq;
             const int qc = stat_ok ? qq : f.Lq - 1;
             lreg = f.lse[((int64_t)b * f.H + h) * f.Lq + qc];
@@ -260,9 +274,9 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
             *(u32x4_t *)(base + off) = qreg[it];
             *(u32x4_t *)(base + SM::Q_BYTES + off) = doreg[it];
         }
-        if (tid < KV_BM) {
+        if (tid < BM) {
             ((float *)(base + 2 * SM::Q_BYTES))[tid] = stat_ok ? lreg * kLog2e : INFINITY;
-            ((float *)(base + 2 * SM::Q_BYTES + KV_BM * 4))[tid] = stat_ok ? dreg : 0.f;
+            ((float *)(base + 2 * SM::Q_BYTES + BM * 4))[tid] = stat_ok ? dreg : 0.f;
         }
     };
 
@@ -284,14 +298,14 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
     }
 
     for (int step = 0; step < n_steps; step++) {
-        const int gi = g_lo + step / n_m, mi = m_hi - 1 - step % n_m;  // last query block first: see below
+        const int gi = g_lo + step / n_m, mi = s_hi - 1 - step % n_m;  // last query block first: see below
         const int h = hk * G + gi;
-        const int m0 = mi * KV_BM;
+        const int m0 = mi * BM;
         const int buf = step & 1;
         const char *sQ = smem + buf * SM::STAGE;
         const char *sDO = sQ + SM::Q_BYTES;
         const float *sLSE = (const float *)(sQ + 2 * SM::Q_BYTES);
-        const float *sDD = sLSE + KV_BM;
+        const float *sDD = sLSE + BM;
 
         // ---- S = Q K^T and dP = dO V^T (M = query, N = key); fragment reads run a batch ahead
         f32x16_t s[MB], dp[MB];
@@ -305,7 +319,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
         load_step(step + 1 < n_steps ? step + 1 : step, false);
         __builtin_amdgcn_sched_barrier(0);
         {
-            constexpr int NF = 2 * MB * KS, FR = 8;  // fragment f: (ks, mb, which) with which = 0: Q, 1: dO
+            constexpr int NF = 2 * MB * KS, FR = D > 64 ? 4 : 8;  // fragment f: (ks, mb, which) with which = 0: Q, 1: dO
             u32x4_t a[NF];
             auto frag = [&](int fi) {
                 const int which = fi & 1, mb = (fi >> 1) % MB, ks = (fi >> 1) / MB;
@@ -317,7 +331,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
             for (int fi = 0; fi < NF; fi++) {
                 if (fi + FR < NF) a[fi + FR] = frag(fi + FR);
                 const int which = fi & 1, mb = (fi >> 1) % MB, ks = (fi >> 1) / MB;
-                if (which) dp[mb] = E::mfma(a[fi], vf[ks], dp[mb]);
+                if (which) dp[mb] = E::mfma(a[fi], V_LDS ? *(const u32x4_t *)(sVrow + ks * 32) : vf[V_LDS ? 0 : ks], dp[mb]);
                 else s[mb] = E::mfma(a[fi], kf[ks], s[mb]);
 #pragma unroll
                 for (int n = fi * 2 * Q_IT / NF; n < (fi + 1) * 2 * Q_IT / NF; n++) load_item(n);
@@ -367,7 +381,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dkdv_colmask_ke
 
         // ---- dV^T += dO^T P ; dK^T += Q^T dS   (M = d, N = key, contraction = query)
         {   // the transposing fragment reads run one (query block, d block) pair ahead of the MFMAs that use them
-            constexpr int NP = (KV_BM / 16) * DB;
+            constexpr int NP = (BM / 16) * DB;
             u32x4_t a1[2], a2[2];
             auto frag = [&](int idx, int slot) {
                 const int qb = idx / DB, db = idx % DB;
