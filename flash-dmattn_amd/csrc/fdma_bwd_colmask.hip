@@ -290,10 +290,16 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
     float colsum = 0.f;
     float cconst = 0.f;
 
+    // Pipeline: step i is computed from LDS stage i & 1.  The registers hold step i+1 (fetched during the dK / dV
+    // MFMAs of step i-1, a whole step earlier -- these tiles come from HBM, not from a cache); they go to the other
+    // stage between the first GEMM pair and the softmax of step i, and the loads of step i+2 then reuse them, issued
+    // one by one between the dK / dV MFMAs (all at once, from every wave at the same moment, they would queue up at the
+    // CU's address unit while the matrix pipe idles).
     if (n_steps > 0) {
         load_step(0, true);
         store_step(0);
         cconst = column_const_value();
+        load_step(n_steps > 1 ? 1 : 0, true);
         __syncthreads();
     }
 
@@ -313,11 +319,6 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
         for (int mb = 0; mb < MB; mb++)
 #pragma unroll
             for (int i = 0; i < 16; i++) { s[mb][i] = cconst; dp[mb][i] = 0.f; }
-        // Global loads of the next step: in flight behind all the matrix work of this one.  The tile loads are issued
-        // one by one between the MFMAs below: all of them at once, from every wave at the same moment, queue up at the
-        // CU's address unit while the matrix pipe idles.  (After the last step the same tiles are fetched again and dropped.)
-        load_step(step + 1 < n_steps ? step + 1 : step, false);
-        __builtin_amdgcn_sched_barrier(0);
         {
             constexpr int NF = 2 * MB * KS, FR = D > 64 ? 4 : 8;  // fragment f: (ks, mb, which) with which = 0: Q, 1: dO
             u32x4_t a[NF];
@@ -333,10 +334,16 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
                 const int which = fi & 1, mb = (fi >> 1) % MB, ks = (fi >> 1) / MB;
                 if (which) dp[mb] = E::mfma(a[fi], V_LDS ? *(const u32x4_t *)(sVrow + ks * 32) : vf[V_LDS ? 0 : ks], dp[mb]);
                 else s[mb] = E::mfma(a[fi], kf[ks], s[mb]);
-#pragma unroll
-                for (int n = fi * 2 * Q_IT / NF; n < (fi + 1) * 2 * Q_IT / NF; n++) load_item(n);
             }
         }
+        // the registers (step i+1) go to the other LDS stage, whose readers finished before the last barrier
+        __builtin_amdgcn_sched_barrier(0);
+        float cconst_next = cconst;
+        if (step + 1 < n_steps) {
+            store_step(buf ^ 1);
+            cconst_next = column_const_value();
+        }
+        __builtin_amdgcn_sched_barrier(0);
 
         // ---- P = exp2(S - LSE*log2e), S already scaled and offset by the column constant ; dS = P * (dP - D)
         // diagonal step: some (query, key) pairs of this wave are above the causal diagonal
@@ -380,6 +387,8 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
         colsum += part;
 
         // ---- dV^T += dO^T P ; dK^T += Q^T dS   (M = d, N = key, contraction = query)
+        // (after the last steps an existing tile is fetched again and dropped)
+        load_step(step + 2 < n_steps ? step + 2 : step, false);
         {   // the transposing fragment reads run one (query block, d block) pair ahead of the MFMAs that use them
             constexpr int NP = (BM / 16) * DB;
             u32x4_t a1[2], a2[2];
@@ -400,6 +409,8 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
                 const u32x4_t sb = {dpk[4 * qb], dpk[4 * qb + 1], dpk[4 * qb + 2], dpk[4 * qb + 3]};
                 dv[db] = E::mfma(a1[idx & 1], pb, dv[db]);
                 dk[db] = E::mfma(a2[idx & 1], sb, dk[db]);
+#pragma unroll
+                for (int n = idx * 2 * Q_IT / NP; n < (idx + 1) * 2 * Q_IT / NP; n++) load_item(n);
             }
             // pin the order: reads of pair idx+1, then the two MFMAs of pair idx
             __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
@@ -426,10 +437,7 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
             }
         }
 
-        if (step + 1 < n_steps) {
-            store_step(buf ^ 1);
-            cconst = column_const_value();  // of the next step
-        }
+        cconst = cconst_next;
         __syncthreads();
     }
 
