@@ -31,9 +31,9 @@ PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
 # HBM bytes per launch of the forward kernel on the headline workload, from two rocprofv3 --pmc runs of
 # this script (FETCH_SIZE, WRITE_SIZE; each scaled by what the counter reads for a 256 MiB device copy,
-# see --calib-copy): compacted kernel 77 MiB read + 65 MiB written, tile-skipping kernel 151 + 65 MiB.
+# see --calib-copy): compacted kernel 82 MiB read + 65 MiB written, tile-skipping kernel 141 + 65 MiB.
 # Override with --traffic-bytes after re-measuring.
-MEASURED_FWD_TRAFFIC_BYTES = {True: 142.0 * 1024 * 1024, False: 216.0 * 1024 * 1024}
+MEASURED_FWD_TRAFFIC_BYTES = {True: 147.0 * 1024 * 1024, False: 206.0 * 1024 * 1024}
 
 CONFIGS = {
     # name: B, Lq, Lk, H, Hk, D, bias shape, window, causal, passes
@@ -216,24 +216,28 @@ def run_config(name, steps, warmup, device, compact=True, backward=True):
     return res
 
 
-def cpu_baseline(device_cfg="cfg2", groups=1):
+def cpu_baseline(device_cfg="cfg2", groups=8, chunk=2):
     """The fp32 safe-eager restatement (oracle/eager.py, a port of the reference's eager formula) timed
     on the host cores for a bounded sample of the headline workload: `groups` KV groups (each with its
-    4 query heads) of the 8, full sequence length."""
+    4 query heads) of the 8, full sequence length, `chunk` groups at a time (the eager formula materialises
+    the [heads, Lq, Lk] fp32 score tensor: 2 groups are 2 GiB per temporary)."""
     from oracle import eager
 
     c = dict(CONFIGS[device_cfg])
     q, k, v, mask, bias = make_case(c, "cpu")
     G = c["H"] // c["Hk"]
-    qs, ks, vs = q[:, :, : G * groups].float(), k[:, :, :groups].float(), v[:, :, :groups].float()
-    ms_, bs = mask[:, :groups], bias[:, :groups].float()
     cores = os.cpu_count() or 1
     torch.set_num_threads(cores)
+    dt, n_exec = 0.0, 0
     with torch.no_grad():
-        t0 = time.perf_counter()
-        eager.attention_forward(qs, ks, vs, ms_, bs, c["scale"], c["causal"])
-        dt = time.perf_counter() - t0
-    n_exec, _, _ = count_tiles(ms_, c["Lq"], c["Lk"], c["causal"], G * groups)
+        for g0 in range(0, groups, chunk):
+            g1 = min(groups, g0 + chunk)
+            qs, ks, vs = q[:, :, G * g0:G * g1].float(), k[:, :, g0:g1].float(), v[:, :, g0:g1].float()
+            ms_, bs = mask[:, g0:g1], bias[:, g0:g1].float()
+            t0 = time.perf_counter()
+            eager.attention_forward(qs, ks, vs, ms_, bs, c["scale"], c["causal"])
+            dt += time.perf_counter() - t0
+            n_exec += count_tiles(ms_, c["Lq"], c["Lk"], c["causal"], G * (g1 - g0))[0]
     tfl = 4.0 * 64 * 64 * c["D"] * n_exec / dt / 1e12
     return {"value": tfl, "unit": "TFLOP/s", "cores": cores, "kind": "port",
             "sample": f"{groups} of {c['Hk']} KV groups ({G * groups} query heads) of {device_cfg} forward, fp32 eager on host, "
@@ -327,7 +331,7 @@ def main():
         out["other_configs"] = [run_config(n, max(3, args.steps // 4), max(1, args.warmup // 2), device, compact)
                                 for n in ("cfg1", "cfg3", "cfg4", "cfg5")]
     if not args.no_cpu:
-        out["cpu_baseline"] = cpu_baseline("cfg2", groups=1)
+        out["cpu_baseline"] = cpu_baseline("cfg2", groups=8)
     print(json.dumps(out))
 
 
