@@ -105,7 +105,10 @@ __global__ void __launch_bounds__(NTHREADS, (D <= 64 && !GSUM) ? 2 : 1) bwd_dkdv
 
     const FwdParams &f = p.f;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 31, g = lane >> 5;
-    const int n_block = blockIdx.x, hk = blockIdx.y, b = blockIdx.z;
+    // linear workgroup id -> (key block, kv head, batch), key block OUTERMOST and ascending: under causal masking the low
+    // key blocks are seen by the most queries, so the heaviest workgroups of every head start first
+    const int hb_count = f.Hk * f.B;
+    const int n_block = (int)blockIdx.x / hb_count, hk = ((int)blockIdx.x % hb_count) % f.Hk, b = ((int)blockIdx.x % hb_count) / f.Hk;
     const int G = f.H / f.Hk;
     const int n0 = n_block * KV_BN;
     const int key = n0 + wave * 32 + r;  // the key column this lane owns
@@ -547,7 +550,7 @@ hipError_t launch_bwd_t(const BwdParams &p, hipStream_t stream) {
     if (f.Lk > 0 && colmask) {
         if ((e = launch_bwd_dkdv_colmask(p, dtype_code, stream)) != hipSuccess) return e;
     } else if (f.Lk > 0) {
-        dim3 grid((f.Lk + KV_BN - 1) / KV_BN, f.Hk, f.B);
+        dim3 grid(((f.Lk + KV_BN - 1) / KV_BN) * f.Hk * f.B);
         // a per-query bias shared by several query heads: dS is summed over the group before it is written; one
         // shared by several workgroups (broadcast over the batch or over kv heads) is accumulated with fp32 atomics
         const bool gsum = f.bias != nullptr && f.bi_r != 0 && ((f.Hb != f.H && f.H / f.Hk > 1) || p.dbias_accum != nullptr);

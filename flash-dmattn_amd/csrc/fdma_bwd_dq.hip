@@ -49,8 +49,11 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dq_kernel(const
 
     const FwdParams &f = p.f;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 31, g = lane >> 5;
-    const int m_block = gridDim.x - 1 - blockIdx.x;  // heaviest first under causal
-    const int h = blockIdx.y, b = blockIdx.z;
+    // linear workgroup id -> (query block, head, batch) with the query block OUTERMOST and descending: under causal
+    // masking the blocks with the most KV tiles of every head start first, the light ones fill the tail
+    const int hb_count = f.H * f.B;
+    const int m_block = (int)gridDim.x / hb_count - 1 - (int)blockIdx.x / hb_count;
+    const int h = ((int)blockIdx.x % hb_count) % f.H, b = ((int)blockIdx.x % hb_count) / f.H;
     const int hk = h / (f.H / f.Hk);
     const int m0 = m_block * BM;
     const int wrow0 = m0 + wave * 32;
@@ -330,7 +333,7 @@ hipError_t launch_dq_c(const BwdParams &p, hipStream_t stream) {
     const int smem = DqSmem<D>::TOTAL;
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    dim3 grid((p.f.Lq + BM - 1) / BM, p.f.H, p.f.B);
+    dim3 grid(((p.f.Lq + BM - 1) / BM) * p.f.H * p.f.B);
     hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, stream, p);
     return hipGetLastError();
 }

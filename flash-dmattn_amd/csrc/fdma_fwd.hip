@@ -63,8 +63,11 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) fwd_kernel(const Fw
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 31, g = lane >> 5;
-    const int m_block = gridDim.x - 1 - blockIdx.x;  // heaviest (most KV tiles) first under causal
-    const int h = blockIdx.y, b = blockIdx.z;
+    // linear workgroup id -> (query block, head, batch) with the query block OUTERMOST and descending: under causal
+    // masking the blocks with the most KV tiles of every head start first, the light ones fill the tail
+    const int hb_count = p.H * p.B;
+    const int m_block = (int)gridDim.x / hb_count - 1 - (int)blockIdx.x / hb_count;
+    const int h = ((int)blockIdx.x % hb_count) % p.H, b = ((int)blockIdx.x % hb_count) / p.H;
     const int hk = h / (p.H / p.Hk);
     const int m0 = m_block * BM;
     const int wrow0 = m0 + wave * 32;
@@ -384,7 +387,7 @@ hipError_t launch_fwd_c(const FwdParams &p, hipStream_t stream) {
     const int smem = FwdSmem<D>::TOTAL;
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
-    dim3 grid((p.Lq + BM - 1) / BM, p.H, p.B);
+    dim3 grid(((p.Lq + BM - 1) / BM) * p.H * p.B);
     hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, stream, p);
     return hipGetLastError();
 }
