@@ -751,27 +751,56 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
     const int kc = tid % CH, kr0 = tid / CH;
     const int kcol = (kc * 8 < f.d) ? kc * 8 : 0;
     u32x4_t kreg[K_IT], vreg[K_IT];
-    float breg = 0.f;
-    auto load_tile = [&](int j) {
-        const int n0 = j * BN;
+    // Byte offsets of this thread's loads inside a tile are loop invariants -- one set for full tiles, one for the
+    // (only) partial tile at the end of the keys -- so a load is one instruction with a scalar tile base, and the
+    // loads of the next tile can be issued one by one between the MFMAs of the current one.  The bias / mask of the
+    // thread's column travel as raw, unconditional loads (an absent one is read from K and ignored) and are looked
+    // at when they are stored.
+    typedef const __attribute__((address_space(1))) char *gptr_t;
+    auto uniform_ptr = [](const void *ptr) -> gptr_t {
+        const uint64_t v = (uint64_t)ptr;
+        const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
+        return (gptr_t)(((uint64_t)hi << 32) | lo);
+    };
+    const int j_last = Lk > 0 ? (Lk - 1) / BN : 0, last_row = Lk > 0 ? (Lk - 1) % BN : 0;
+    uint32_t koff[K_IT], koff_l[K_IT], voff[K_IT], voff_l[K_IT];
 #pragma unroll
-        for (int it = 0; it < K_IT; it++) {
-            int key = n0 + kr0 + it * RPP;
-            key = key < Lk ? key : Lk - 1;
-            kreg[it] = *(const u32x4_t *)(kbase + (int64_t)key * f.k_r + kcol);
-            vreg[it] = *(const u32x4_t *)(vbase + (int64_t)key * f.v_r + kcol);
-        }
+    for (int it = 0; it < K_IT; it++) {
+        const int row = kr0 + it * RPP, row_c = row < last_row ? row : last_row;
+        koff[it] = (uint32_t)(row * f.k_r + kcol) * 2;
+        koff_l[it] = (uint32_t)(row_c * f.k_r + kcol) * 2;
+        voff[it] = (uint32_t)(row * f.v_r + kcol) * 2;
+        voff_l[it] = (uint32_t)(row_c * f.v_r + kcol) * 2;
+    }
+    gptr_t tb_k = nullptr, tb_v = nullptr;
+    bool t_last = false, bcol_ok = false;
+    uint32_t braw = 0, mraw = 0;
+    const uint8_t *mrow_ld = mrow ? mrow : (const uint8_t *)kbase;
+    const uint16_t *brow_ld = brow ? brow : kbase;
+    auto set_tile = [&](int j) {
+        tb_k = uniform_ptr(kbase + (int64_t)j * BN * f.k_r);
+        tb_v = uniform_ptr(vbase + (int64_t)j * BN * f.v_r);
+        t_last = j == j_last;
         if (tid < BN) {
-            const int col = n0 + tid;
-            float v = -INFINITY;
+            const int col = j * BN + tid;
+            bcol_ok = col < Lk;
+            const int cc = bcol_ok ? col : 0;
             if (CMP) {
-                if (col < Lk) v = fbrow[col];
-            } else if (col < Lk && (!mrow || mrow[col])) {
-                v = 0.f;
-                if (brow) v = E::lo((uint32_t)brow[col]) * kLog2e;
+                braw = __float_as_uint(fbrow[cc]);
+            } else {
+                mraw = mrow_ld[cc];
+                braw = brow_ld[cc];
             }
-            breg = v;
         }
+    };
+    auto load_item = [&](int n) {  // 0 .. K_IT-1: K rows, K_IT .. 2*K_IT-1: V rows
+        if (n < K_IT) kreg[n] = *(const __attribute__((address_space(1))) u32x4_t *)(tb_k + (t_last ? koff_l[n] : koff[n]));
+        else vreg[n - K_IT] = *(const __attribute__((address_space(1))) u32x4_t *)(tb_v + (t_last ? voff_l[n - K_IT] : voff[n - K_IT]));
+    };
+    auto load_tile = [&](int j) {
+        set_tile(j);
+#pragma unroll
+        for (int n = 0; n < 2 * K_IT; n++) load_item(n);
     };
     auto store_tile = [&](int buf, int slot) {
         char *sK = smem + SM::OFF_K + buf * SM::K_BYTES;
@@ -782,7 +811,15 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
             *(u32x4_t *)(sK + off) = kreg[it];
             *(u32x4_t *)(sV + off) = vreg[it];
         }
-        if (tid < BN) sBias[slot * BN + tid] = breg;
+        if (tid < BN) {
+            float v = -INFINITY;
+            if (CMP) {
+                if (bcol_ok) v = __uint_as_float(braw);
+            } else if (bcol_ok && (!mrow || mraw)) {
+                v = brow ? E::lo(braw) * kLog2e : 0.f;
+            }
+            sBias[slot * BN + tid] = v;
+        }
     };
 
     const int a_row = pi_row(r);
@@ -801,7 +838,7 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
     int i = 0;
     while (jc < n_end) {
         const int jn = next_active(jc + 1);
-        if (jn < n_end) load_tile(jn);
+        set_tile(jn < n_end ? jn : jc);  // (after the last tile the current one is fetched again and dropped)
         const int n0 = jc * BN;
         const char *sK = smem + SM::OFF_K + (i & 1) * SM::K_BYTES;
         const char *sV = smem + SM::OFF_V + (i & 1) * SM::K_BYTES;
@@ -838,6 +875,8 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
                 const int which = fi & 1, mb = (fi >> 1) % MB, ks = (fi >> 1) / MB;
                 if (which) dp[mb] = E::mfma(a[fi], dof[ks], dp[mb]);
                 else s[mb] = E::mfma(a[fi], qf[ks], s[mb]);
+#pragma unroll
+                for (int n = fi * 2 * K_IT / NF; n < (fi + 1) * 2 * K_IT / NF; n++) load_item(n);
             }
         }
         // ---- dS^T = P^T * (dP^T - D)
