@@ -205,9 +205,11 @@ def run_config(name, steps, warmup, device, compact=True, backward=True):
         qg, kg, vg = [t.clone().requires_grad_(True) for t in (q, k, v)]
         bg = bias.clone().requires_grad_(True)
 
+        dout = torch.ones_like(q)  # upstream gradient, resident like the other inputs
+
         def step():
             out = flash_sparse_attn_func(qg, kg, vg, mask, bg, scale, c["causal"])
-            out.backward(torch.ones_like(out))
+            out.backward(dout)
             qg.grad = kg.grad = vg.grad = bg.grad = None
 
         ms_fb = time_gpu(step, max(2, steps // 2), max(1, warmup // 2))
