@@ -10,10 +10,10 @@
 //   * dBias is the column sum of dS, accumulated in a register and written once;
 //   * in the dQ kernel the fused vector is staged per tile exactly as in the forward kernel and
 //     fully masked 64-key tiles are skipped through the same LDS bitmap.
-// K and V are stationary in registers in the dK/dV kernel (B operands), Q / dO tiles and the row
-// statistics stream through double-buffered LDS with the next step's global loads in flight during
-// the current step.  Workgroup ids are remapped so that workgroups sharing an XCD's L2 share the
-// streamed operands.
+// K and V are stationary in the dK/dV kernel (B operands: in registers, except V at d = 128, which every
+// lane parks in LDS as a private spill so that two workgroups fit on a CU); Q / dO tiles and the row
+// statistics stream through double-buffered LDS, fetched two steps ahead of their use.  Workgroup ids
+// are remapped so that workgroups sharing an XCD's L2 share the streamed operands.
 #include "fdma_common.h"
 #include "fdma_params.h"
 
