@@ -19,6 +19,8 @@ namespace {
 
 thread_local char g_err[512] = "";
 
+constexpr int64_t kMaxRowStride = (int64_t)1 << 24;  // elements
+
 int fail(int code, const char *fmt, ...) {
     va_list ap;
     va_start(ap, fmt);
@@ -72,6 +74,9 @@ int validate_common(const fdma_fwd_args *a, bool backward) {
     if (!aligned16(a->q) || !aligned16(a->k) || !aligned16(a->v) || !aligned16(a->out) || !strides_ok(a->q_strides, 8) ||
         !strides_ok(a->k_strides, 8) || !strides_ok(a->v_strides, 8) || !strides_ok(a->o_strides, 8))
         return fail(FDMA_ERR_INVALID, "q, k, v, out must be 16-byte aligned with strides that are multiples of 8 elements");
+    // the kernels address the rows of a tile with 32-bit byte offsets from a 64-bit tile base
+    if (a->q_strides[1] >= kMaxRowStride || a->k_strides[1] >= kMaxRowStride || a->v_strides[1] >= kMaxRowStride)
+        return fail(FDMA_ERR_UNSUPPORTED, "q, k, v row strides of 2^24 elements or more are not supported");
     if (a->softcap != 0.f) return fail(FDMA_ERR_UNSUPPORTED, "softcap is not supported by this build");
     if (a->head_dim > 128) return fail(FDMA_ERR_UNSUPPORTED, "head dimensions above 128 are not built yet (got %d)", a->head_dim);
     if (!std::isfinite(a->softmax_scale)) return fail(FDMA_ERR_INVALID, "softmax_scale must be finite");
@@ -177,6 +182,8 @@ int fdma_bwd_validate(const fdma_bwd_args *a) {
     if (!aligned16(a->dout) || !aligned16(a->dq) || !aligned16(a->dk) || !aligned16(a->dv) || !strides_ok(a->do_strides, 8) ||
         !strides_ok(a->dq_strides, 8) || !strides_ok(a->dk_strides, 8) || !strides_ok(a->dv_strides, 8))
         return fail(FDMA_ERR_INVALID, "dout, dq, dk, dv must be 16-byte aligned with strides that are multiples of 8 elements");
+    if (a->do_strides[1] >= kMaxRowStride)
+        return fail(FDMA_ERR_UNSUPPORTED, "dout row strides of 2^24 elements or more are not supported");
     if (a->dbias) {
         if (!aligned16(a->dbias) || !strides_ok(a->dbias_strides, 8))
             return fail(FDMA_ERR_INVALID, "dbias must be 16-byte aligned with strides that are multiples of 8");

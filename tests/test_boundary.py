@@ -69,6 +69,7 @@ def test_validation_accepts_a_good_call_and_needs_no_gpu():
         (lambda a: (setattr(a, "bias", 0x2000), setattr(a, "num_heads_bias", 5)), "Number of heads in bias must be 1, h_k or h"),
         (lambda a: setattr(a, "q", 0x1004), "16-byte aligned"),
         (lambda a: setattr(a, "softcap", 30.0), "softcap"),
+        (lambda a: a.k_strides.__setitem__(1, 1 << 24), "row strides of 2^24 elements or more"),
     ],
 )
 def test_validation_errors(mutate, needle):
