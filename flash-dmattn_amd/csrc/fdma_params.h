@@ -37,9 +37,9 @@ struct Compact {
 //   bound (units), plan[4] = Q, plan[8 + i] = first unit of pair i (i = 0..pairs)
 constexpr int DKDV_PLAN_HDR = 8;
 #ifndef FDMA_DKDV_TARGET
-#define FDMA_DKDV_TARGET 1024
+#define FDMA_DKDV_TARGET 768
 #endif
-constexpr int DKDV_TARGET_PARTS = FDMA_DKDV_TARGET;   // parts wanted in flight (4 per CU)
+constexpr int DKDV_TARGET_PARTS = FDMA_DKDV_TARGET;   // parts wanted (3 per CU, two of them resident at a time: measured best)
 constexpr int DKDV_ENOUGH_UNITS = 384;    // from here on the units alone fill the chip
 __host__ __device__ inline void dkdv_split(int U, int G, int &Gs, int &Sm) {
     Gs = 1;
