@@ -28,11 +28,12 @@ namespace fdma {
 
 namespace {
 
-constexpr int BM = 128;
+// Workgroups have 4 waves (128 query rows; two per CU at d <= 64) or, at d = 128 on grids that stay large enough,
+// 8 waves (256 rows): at d = 128 only one workgroup fits on a CU, and with a single wave per SIMD nothing hides the
+// in-order issue of that wave -- a second wave per SIMD does.
 constexpr int BN = 64;
-constexpr int NTHREADS = 256;
 
-template <int D> struct FwdSmem {
+template <int D, int BM> struct FwdSmem {
     static constexpr int SK = D + 8;     // K tile row stride (elements): conflict-free 16-byte row reads
     static constexpr int SVT = BN + 8;   // V^T tile row stride
     static constexpr int SF = BN + 8;    // fused mask+bias tile row stride
@@ -47,10 +48,12 @@ template <typename T> struct NegInf2;
 template <> struct NegInf2<bf16_tag> { static constexpr uint32_t value = 0xFF80FF80u; };
 template <> struct NegInf2<fp16_tag> { static constexpr uint32_t value = 0xFC00FC00u; };
 
-template <typename T, int D, bool CAUSAL>
-__global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) fwd_kernel(const FwdParams p) {
+template <typename T, int D, bool CAUSAL, int NW>
+__global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) fwd_kernel(const FwdParams p) {
+    constexpr int NTHREADS = 64 * NW, BM = 32 * NW;
+    constexpr int F_RPP = NTHREADS / 8;     // mask / bias rows staged per pass (8 threads cover the 64 keys of a row)
     using E = Elem<T>;
-    using SM = FwdSmem<D>;
+    using SM = FwdSmem<D, BM>;
     constexpr int KS = D / 16;  // contraction steps of Q K^T
     constexpr int DB = D / 32;  // 32-wide blocks of the head dimension
     constexpr int MB = BN / 32, KB = BN / 16, KQ = BN / 4;
@@ -119,7 +122,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) fwd_kernel(const Fw
     const int kc = tid % CH, kr0 = tid / CH;             // K: d chunk, first row
     const int vkg = tid % KQ, vc = (tid / KQ) % CH;      // V: key quad, d chunk
     const bool k_dvalid = kc * 8 < p.d, v_dvalid = vc * 8 < p.d;
-    const int fc = tid & 7, fr0 = tid >> 3;              // mask / bias: 8-key chunk, first row (rows fr0 + 32 it)
+    const int fc = tid & 7, fr0 = tid >> 3;              // mask / bias: 8-key chunk, first row (rows fr0 + F_RPP it)
     u32x4_t kreg[K_IT], vreg[4], breg[F_IT];
     u32x2_t mreg[F_IT], mnext[F_IT];
 
@@ -134,7 +137,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) fwd_kernel(const Fw
         kk = kk < p.Lk ? kk : 0;
 #pragma unroll
         for (int it = 0; it < F_IT; it++) {
-            int row = m0 + fr0 + 32 * it;
+            int row = m0 + fr0 + F_RPP * it;
             row = row < p.Lq ? row : p.Lq - 1;
             dst[it] = *(const u32x2_t *)(mbase + (int64_t)row * p.m_r + kk);
         }
@@ -146,7 +149,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) fwd_kernel(const Fw
         uint32_t any = 0;
 #pragma unroll
         for (int it = 0; it < F_IT; it++) {
-            const int row = m0 + fr0 + 32 * it;
+            const int row = m0 + fr0 + F_RPP * it;
             u32x2_t mv = mbase ? dst[it] : u32x2_t{0x01010101u, 0x01010101u};
             const bool ok = row < p.Lq && kk < p.Lk && !(CAUSAL && kk > row + shift);
             uint64_t keepm = ok ? ~0ull : 0ull;
@@ -166,7 +169,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) fwd_kernel(const Fw
             kk = kk < p.Lk ? kk : 0;
 #pragma unroll
             for (int it = 0; it < F_IT; it++) {
-                int row = m0 + fr0 + 32 * it;
+                int row = m0 + fr0 + F_RPP * it;
                 row = row < p.Lq ? row : p.Lq - 1;
                 breg[it] = *(const u32x4_t *)(bbase + (int64_t)row * p.bi_r + kk);
             }
@@ -221,7 +224,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) fwd_kernel(const Fw
                 bv[2 * hlf] = (bv[2 * hlf] & m0w) | (NegInf2<T>::value & ~m0w);
                 bv[2 * hlf + 1] = (bv[2 * hlf + 1] & m1w) | (NegInf2<T>::value & ~m1w);
             }
-            *(u32x4_t *)(sF + ((fr0 + 32 * it) * SM::SF + 8 * fc) * 2) = bv;
+            *(u32x4_t *)(sF + ((fr0 + F_RPP * it) * SM::SF + 8 * fc) * 2) = bv;
         }
     };
 
@@ -381,10 +384,11 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) fwd_kernel(const Fw
     }
 }
 
-template <typename T, int D, bool CAUSAL>
+template <typename T, int D, bool CAUSAL, int NW>
 hipError_t launch_fwd_c(const FwdParams &p, hipStream_t stream) {
-    auto kern = fwd_kernel<T, D, CAUSAL>;
-    const int smem = FwdSmem<D>::TOTAL;
+    constexpr int BM = 32 * NW, NTHREADS = 64 * NW;
+    auto kern = fwd_kernel<T, D, CAUSAL, NW>;
+    const int smem = FwdSmem<D, BM>::TOTAL;
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
     dim3 grid(((p.Lq + BM - 1) / BM) * p.H * p.B);
@@ -394,7 +398,12 @@ hipError_t launch_fwd_c(const FwdParams &p, hipStream_t stream) {
 
 template <typename T, int D>
 hipError_t launch_fwd_t(const FwdParams &p, hipStream_t stream) {
-    return p.causal ? launch_fwd_c<T, D, true>(p, stream) : launch_fwd_c<T, D, false>(p, stream);
+    if constexpr (D > 64) {
+        // 256-row workgroups while the grid still covers the chip about twice
+        if ((int64_t)p.B * p.H * ((p.Lq + 255) / 256) >= 512)
+            return p.causal ? launch_fwd_c<T, D, true, 8>(p, stream) : launch_fwd_c<T, D, false, 8>(p, stream);
+    }
+    return p.causal ? launch_fwd_c<T, D, true, 4>(p, stream) : launch_fwd_c<T, D, false, 4>(p, stream);
 }
 
 }  // namespace
