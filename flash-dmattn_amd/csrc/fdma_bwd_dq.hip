@@ -18,11 +18,11 @@ namespace fdma {
 
 namespace {
 
-constexpr int BM = 128;
-constexpr int BN = 64;
-constexpr int NTHREADS = 256;
-
-template <int D> struct DqSmem {
+// Workgroups have 4 waves (128 query rows; two per CU at d <= 64) or, at d = 128 on grids that stay large enough,
+// 8 waves (256 rows): one workgroup fits on a CU there, and a second wave per SIMD hides what a single wave's
+// in-order issue cannot.  Key tiles have 64 keys with 4 waves and 32 with 8 (the 64-key tile's score and dP accumulators
+// do not fit next to dQ and the Q / dO fragments in the 256 registers a wave has when two share a SIMD).
+template <int D, int BM, int BN> struct DqSmem {
     static constexpr int S = D + 8;      // K / V tile row stride (elements)
     static constexpr int SF = BN + 8;    // fused mask+bias tile row stride
     static constexpr int K_BYTES = BN * S * 2;
@@ -35,15 +35,18 @@ template <typename T> struct NegInf2;
 template <> struct NegInf2<bf16_tag> { static constexpr uint32_t value = 0xFF80FF80u; };
 template <> struct NegInf2<fp16_tag> { static constexpr uint32_t value = 0xFC00FC00u; };
 
-template <typename T, int D, bool CAUSAL>
-__global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dq_kernel(const BwdParams p) {
+template <typename T, int D, bool CAUSAL, int NW>
+__global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) bwd_dq_kernel(const BwdParams p) {
+    constexpr int NTHREADS = 64 * NW, BM = 32 * NW, BN = NW == 8 ? 32 : 64;
+    constexpr int FCH = BN / 8;             // 8-key chunks per mask / bias row of a tile
+    constexpr int F_RPP = NTHREADS / FCH;   // mask / bias rows staged per pass
     using E = Elem<T>;
-    using SM = DqSmem<D>;
+    using SM = DqSmem<D, BM, BN>;
     constexpr int KS = D / 16, DB = D / 32, MB = BN / 32, KB = BN / 16;
     constexpr int CH = D / 8;               // 16-byte chunks per K / V row
     constexpr int K_RPP = NTHREADS / CH;    // rows staged per pass
     constexpr int K_IT = BN / K_RPP;
-    constexpr int F_IT = BM * (BN / 8) / NTHREADS;  // 8-key chunks of the mask / bias tile per thread (4)
+    constexpr int F_IT = BM * FCH / NTHREADS;  // 8-key chunks of the mask / bias tile per thread
 
     extern __shared__ __attribute__((aligned(16))) char smem[];
 
@@ -110,7 +113,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dq_kernel(const
     // words are ANDed with a validity pattern when they are consumed
     const int kc = tid % CH, kr0 = tid / CH;
     const int kcol = kc * 8 < f.d ? kc * 8 : 0;
-    const int fc = tid & 7, fr0 = tid >> 3;  // mask / bias: 8-key chunk, first row (rows fr0 + 32 it)
+    const int fc = tid % FCH, fr0 = tid / FCH;  // mask / bias: 8-key chunk, first row (rows fr0 + F_RPP it)
     u32x4_t kreg[K_IT], vreg[K_IT], breg[F_IT];
     u32x2_t mreg[F_IT], mnext[F_IT];
 
@@ -120,7 +123,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dq_kernel(const
         kk = kk < f.Lk ? kk : 0;
 #pragma unroll
         for (int it = 0; it < F_IT; it++) {
-            int row = m0 + fr0 + 32 * it;
+            int row = m0 + fr0 + F_RPP * it;
             row = row < f.Lq ? row : f.Lq - 1;
             dst[it] = *(const u32x2_t *)(mbase + (int64_t)row * f.m_r + kk);
         }
@@ -130,7 +133,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dq_kernel(const
         uint32_t any = 0;
 #pragma unroll
         for (int it = 0; it < F_IT; it++) {
-            const int row = m0 + fr0 + 32 * it;
+            const int row = m0 + fr0 + F_RPP * it;
             u32x2_t mv = mbase ? dst[it] : u32x2_t{0x01010101u, 0x01010101u};
             const bool ok = row < f.Lq && kk < f.Lk && !(CAUSAL && kk > row + shift);
             uint64_t keepm = ok ? ~0ull : 0ull;
@@ -149,7 +152,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dq_kernel(const
             kk = kk < f.Lk ? kk : 0;
 #pragma unroll
             for (int it = 0; it < F_IT; it++) {
-                int row = m0 + fr0 + 32 * it;
+                int row = m0 + fr0 + F_RPP * it;
                 row = row < f.Lq ? row : f.Lq - 1;
                 breg[it] = *(const u32x4_t *)(bbase + (int64_t)row * f.bi_r + kk);
             }
@@ -188,7 +191,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dq_kernel(const
                 bv[2 * hlf] = (bv[2 * hlf] & m0w) | (NegInf2<T>::value & ~m0w);
                 bv[2 * hlf + 1] = (bv[2 * hlf + 1] & m1w) | (NegInf2<T>::value & ~m1w);
             }
-            *(u32x4_t *)(sF + ((fr0 + 32 * it) * SM::SF + 8 * fc) * 2) = bv;
+            *(u32x4_t *)(sF + ((fr0 + F_RPP * it) * SM::SF + 8 * fc) * 2) = bv;
         }
     };
 
@@ -327,15 +330,25 @@ __global__ void __launch_bounds__(NTHREADS, D <= 64 ? 2 : 1) bwd_dq_kernel(const
     }
 }
 
-template <typename T, int D, bool CAUSAL>
-hipError_t launch_dq_c(const BwdParams &p, hipStream_t stream) {
-    auto kern = bwd_dq_kernel<T, D, CAUSAL>;
-    const int smem = DqSmem<D>::TOTAL;
+template <typename T, int D, bool CAUSAL, int NW>
+hipError_t launch_dq_n(const BwdParams &p, hipStream_t stream) {
+    constexpr int BM = 32 * NW, NTHREADS = 64 * NW, BN = NW == 8 ? 32 : 64;
+    auto kern = bwd_dq_kernel<T, D, CAUSAL, NW>;
+    const int smem = DqSmem<D, BM, BN>::TOTAL;
     hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
     if (e != hipSuccess) return e;
     dim3 grid(((p.f.Lq + BM - 1) / BM) * p.f.H * p.f.B);
     hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, stream, p);
     return hipGetLastError();
+}
+
+template <typename T, int D, bool CAUSAL>
+hipError_t launch_dq_c(const BwdParams &p, hipStream_t stream) {
+    if constexpr (D > 64) {
+        // 256-row workgroups while the grid still covers the chip about twice
+        if ((int64_t)p.f.B * p.f.H * ((p.f.Lq + 255) / 256) >= 512) return launch_dq_n<T, D, CAUSAL, 8>(p, stream);
+    }
+    return launch_dq_n<T, D, CAUSAL, 4>(p, stream);
 }
 
 }  // namespace
