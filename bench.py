@@ -147,7 +147,10 @@ RAMP_SECONDS = 0.25  # busy time before the warm-up steps: an idle MI355X takes 
 def time_gpu(fn, steps, warmup):
     """`warmup` untimed steps, then exactly `steps` timed ones between two events on the current stream.  Before
     both, the same step runs for RAMP_SECONDS so that a cold device (power state, clocks) does not dominate a
-    timed region of a few milliseconds."""
+    timed region of a few milliseconds.  The first call (library and code-object loading on the host) is made
+    before the ramp clock starts: it can take longer than RAMP_SECONDS with the device idle."""
+    fn()
+    torch.cuda.synchronize()
     t0 = time.perf_counter()
     while time.perf_counter() - t0 < RAMP_SECONDS:
         fn()
