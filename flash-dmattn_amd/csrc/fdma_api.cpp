@@ -106,6 +106,74 @@ void fill_fwd_params(const fdma_fwd_args *a, fdma::FwdParams &p) {
     p.scale = a->softmax_scale;
     p.scale_log2 = a->softmax_scale * 1.4426950408889634f;
     p.splits = 1;
+    p.lse_b = (int64_t)a->num_heads * a->seqlen_q;
+    p.lse_h = a->seqlen_q;
+}
+
+// Ragged batch: rules of flash_api.cpp:583-660 (forward), shared by backward (:1090-1150).
+int validate_varlen(const fdma_varlen_fwd_args *a, bool backward) {
+    if (!a) return fail(FDMA_ERR_INVALID, "args must not be NULL");
+    if (a->dtype != FDMA_DTYPE_BF16 && a->dtype != FDMA_DTYPE_FP16)
+        return fail(FDMA_ERR_INVALID, "FlashSparseAttention only support fp16 and bf16 data type");
+    if (a->batch <= 0) return fail(FDMA_ERR_INVALID, "batch size must be positive");
+    if (a->total_q < 0 || a->total_k < 0 || a->max_seqlen_q < 0 || a->max_seqlen_k < 0)
+        return fail(FDMA_ERR_INVALID, "sequence lengths must be non-negative");
+    if (a->num_heads <= 0 || a->num_heads_k <= 0) return fail(FDMA_ERR_INVALID, "number of heads must be positive");
+    if (a->head_dim > 256)
+        return fail(FDMA_ERR_INVALID, "FlashSparseAttention %s only supports head dimension at most 256", backward ? "backward" : "forward");
+    if (a->head_dim <= 0 || a->head_dim % 8 != 0)
+        return fail(FDMA_ERR_INVALID, backward ? "head_size should be a multiple of 8"
+                                               : "query, key, value, and out_ must have a head_size that is a multiple of 8");
+    if (a->num_heads % a->num_heads_k != 0)
+        return fail(FDMA_ERR_INVALID, "Number of heads in key/value must divide number of heads in query");
+    if (!a->cu_seqlens_q || !a->cu_seqlens_k) return fail(FDMA_ERR_INVALID, "cu_seqlens_q and cu_seqlens_k must be device pointers");
+    if ((reinterpret_cast<uintptr_t>(a->cu_seqlens_q) | reinterpret_cast<uintptr_t>(a->cu_seqlens_k)) & 3)
+        return fail(FDMA_ERR_INVALID, "cu_seqlens_q and cu_seqlens_k must be 4-byte aligned int32 arrays");
+    if ((!a->q && a->total_q > 0) || ((!a->k || !a->v) && a->total_k > 0)) return fail(FDMA_ERR_INVALID, "q, k, v must be device pointers");
+    if (a->total_q > 0 && !a->out) return fail(FDMA_ERR_INVALID, "out must be a device pointer");
+    if (a->total_q > 0 && !a->lse) return fail(FDMA_ERR_INVALID, "softmax_lse must be a device pointer");
+    const int64_t *st[4] = {a->q_strides, a->k_strides, a->v_strides, a->o_strides};
+    for (int i = 0; i < 4; i++)
+        if (st[i][0] % 8 != 0 || st[i][1] % 8 != 0)
+            return fail(FDMA_ERR_INVALID, "q, k, v, out must be 16-byte aligned with strides that are multiples of 8 elements");
+    if (!aligned16(a->q) || !aligned16(a->k) || !aligned16(a->v) || !aligned16(a->out))
+        return fail(FDMA_ERR_INVALID, "q, k, v, out must be 16-byte aligned with strides that are multiples of 8 elements");
+    if (a->q_strides[0] >= kMaxRowStride || a->k_strides[0] >= kMaxRowStride || a->v_strides[0] >= kMaxRowStride)
+        return fail(FDMA_ERR_UNSUPPORTED, "q, k, v row strides of 2^24 elements or more are not supported");
+    if (a->softcap != 0.f) return fail(FDMA_ERR_UNSUPPORTED, "softcap is not supported by this build");
+    if (a->head_dim > 128) return fail(FDMA_ERR_UNSUPPORTED, "head dimensions above 128 are not built yet (got %d)", a->head_dim);
+    if (!std::isfinite(a->softmax_scale)) return fail(FDMA_ERR_INVALID, "softmax_scale must be finite");
+    return FDMA_OK;
+}
+
+// The ragged batch runs through the column-mask kernels (no mask, no bias): batch strides 0, per-entry first rows
+// and lengths from cu_seqlens on the device, grids sized by the longest sequences.
+int fill_varlen_params(const fdma_varlen_fwd_args *a, fdma::FwdParams &p) {
+    std::memset(&p, 0, sizeof(p));
+    p.q = a->q; p.k = a->k; p.v = a->v;
+    p.o = a->out;
+    p.lse = a->lse;
+    p.q_r = a->q_strides[0]; p.q_h = a->q_strides[1];
+    p.k_r = a->k_strides[0]; p.k_h = a->k_strides[1];
+    p.v_r = a->v_strides[0]; p.v_h = a->v_strides[1];
+    p.o_r = a->o_strides[0]; p.o_h = a->o_strides[1];
+    p.B = a->batch;
+    p.Lq = a->max_seqlen_q < a->total_q ? a->max_seqlen_q : a->total_q;
+    p.Lk = a->max_seqlen_k < a->total_k ? a->max_seqlen_k : a->total_k;
+    p.H = a->num_heads; p.Hk = a->num_heads_k;
+    p.Hm = 1; p.Hb = 1;
+    p.d = a->head_dim;
+    p.causal = (a->is_causal && a->max_seqlen_q != 1) ? 1 : 0;  // flash_api.cpp:628
+    p.scale = a->softmax_scale;
+    p.scale_log2 = a->softmax_scale * 1.4426950408889634f;
+    p.splits = 1;
+    p.lse_b = 0;
+    p.lse_h = a->total_q;
+    p.cu_q = a->cu_seqlens_q; p.cu_k = a->cu_seqlens_k;
+    p.total_q = a->total_q; p.total_k = a->total_k;
+    if (!fdma::fwd_colmask_applicable(p))
+        return fail(FDMA_ERR_UNSUPPORTED, "ragged batches with sequences of more than 2^19 keys are not supported (max_seqlen_k = %d)", a->max_seqlen_k);
+    return FDMA_OK;
 }
 
 }  // namespace
@@ -234,6 +302,8 @@ int fdma_bwd(const fdma_bwd_args *a, void *hip_stream) {
     if (a->dbias) { p.db_b = a->dbias_strides[0]; p.db_h = a->dbias_strides[1]; p.db_r = a->dbias_strides[2]; }
     p.softmax_d = a->softmax_d;
     p.Lq_rounded = (int32_t)round_up(a->f.seqlen_q, 128);
+    p.sd_b = (int64_t)a->f.num_heads * p.Lq_rounded;
+    p.sd_h = p.Lq_rounded;
     const size_t need = fdma_bwd_workspace_bytes(a);
     if (need && (!a->workspace || a->workspace_bytes < need))
         return fail(FDMA_ERR_WORKSPACE, "backward workspace too small: need %zu bytes, got %zu", need, a->workspace_bytes);
@@ -254,6 +324,71 @@ int fdma_bwd(const fdma_bwd_args *a, void *hip_stream) {
         if (e != hipSuccess) return fail(FDMA_ERR_LAUNCH, "backward launch failed: %s", hipGetErrorString(e));
     }
     e = fdma::launch_bwd(p, a->f.dtype, stream);
+    if (e != hipSuccess) return fail(FDMA_ERR_LAUNCH, "backward launch failed: %s", hipGetErrorString(e));
+    return FDMA_OK;
+}
+
+size_t fdma_sizeof_varlen_fwd_args(void) { return sizeof(fdma_varlen_fwd_args); }
+size_t fdma_sizeof_varlen_bwd_args(void) { return sizeof(fdma_varlen_bwd_args); }
+
+int fdma_varlen_fwd_validate(const fdma_varlen_fwd_args *a) {
+    g_err[0] = 0;
+    return validate_varlen(a, false);
+}
+
+int fdma_varlen_fwd(const fdma_varlen_fwd_args *a, void *hip_stream) {
+    g_err[0] = 0;
+    int rc = validate_varlen(a, false);
+    if (rc != FDMA_OK) return rc;
+    fdma::FwdParams p;
+    if ((rc = fill_varlen_params(a, p)) != FDMA_OK) return rc;
+    if (a->total_q == 0 || p.Lq == 0) return FDMA_OK;
+    const hipError_t e = fdma::launch_fwd_colmask(p, a->dtype, static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(FDMA_ERR_LAUNCH, "forward launch failed: %s", hipGetErrorString(e));
+    return FDMA_OK;
+}
+
+int fdma_varlen_bwd_validate(const fdma_varlen_bwd_args *a) {
+    g_err[0] = 0;
+    if (!a) return fail(FDMA_ERR_INVALID, "args must not be NULL");
+    int rc = validate_varlen(&a->f, true);
+    if (rc != FDMA_OK) return rc;
+    if ((a->f.total_q > 0 && (!a->dout || !a->dq)) || (a->f.total_k > 0 && (!a->dk || !a->dv)))
+        return fail(FDMA_ERR_INVALID, "dout, dq, dk, dv must be device pointers");
+    if (a->f.total_q > 0 && !a->softmax_d) return fail(FDMA_ERR_INVALID, "softmax_d must be a device pointer");
+    const int64_t *st[4] = {a->do_strides, a->dq_strides, a->dk_strides, a->dv_strides};
+    for (int i = 0; i < 4; i++)
+        if (st[i][0] % 8 != 0 || st[i][1] % 8 != 0)
+            return fail(FDMA_ERR_INVALID, "dout, dq, dk, dv must be 16-byte aligned with strides that are multiples of 8 elements");
+    if (!aligned16(a->dout) || !aligned16(a->dq) || !aligned16(a->dk) || !aligned16(a->dv))
+        return fail(FDMA_ERR_INVALID, "dout, dq, dk, dv must be 16-byte aligned with strides that are multiples of 8 elements");
+    if (a->do_strides[0] >= kMaxRowStride)
+        return fail(FDMA_ERR_UNSUPPORTED, "dout row strides of 2^24 elements or more are not supported");
+    return FDMA_OK;
+}
+
+int fdma_varlen_bwd(const fdma_varlen_bwd_args *a, void *hip_stream) {
+    int rc = fdma_varlen_bwd_validate(a);
+    if (rc != FDMA_OK) return rc;
+    fdma::BwdParams p;
+    std::memset(&p, 0, sizeof(p));
+    if ((rc = fill_varlen_params(&a->f, p.f)) != FDMA_OK) return rc;
+    p.dout = a->dout; p.dq = a->dq; p.dk = a->dk; p.dv = a->dv;
+    p.do_r = a->do_strides[0]; p.do_h = a->do_strides[1];
+    p.dq_r = a->dq_strides[0]; p.dq_h = a->dq_strides[1];
+    p.dk_r = a->dk_strides[0]; p.dk_h = a->dk_strides[1];
+    p.dv_r = a->dv_strides[0]; p.dv_h = a->dv_strides[1];
+    p.softmax_d = a->softmax_d;
+    p.Lq_rounded = p.f.Lq;
+    p.sd_b = 0;
+    p.sd_h = a->f.total_q;
+    // Key rows no query can see get zero dK / dV from the dK/dV kernel itself; with no query rows at all, or no
+    // key rows at all, one of the two grids is empty and the other kernel still writes its (zero) outputs.
+    if (p.f.Lq == 0 && p.f.Lk == 0) return FDMA_OK;
+    if (!fdma::bwd_colmask_applicable(p))
+        return fail(FDMA_ERR_UNSUPPORTED, "ragged batches with sequences of more than 2^19 keys are not supported (max_seqlen_k = %d)", a->f.max_seqlen_k);
+    hipStream_t stream = static_cast<hipStream_t>(hip_stream);
+    const hipError_t e = p.f.Lq == 0 ? fdma::launch_bwd_dkdv_colmask(p, a->f.dtype, stream) : fdma::launch_bwd(p, a->f.dtype, stream);
     if (e != hipSuccess) return fail(FDMA_ERR_LAUNCH, "backward launch failed: %s", hipGetErrorString(e));
     return FDMA_OK;
 }

@@ -48,8 +48,10 @@ __global__ void __launch_bounds__(256) bwd_dot_kernel(const BwdParams p) {
     const int sub = threadIdx.x % lanes;
     const int row = blockIdx.x * rows_per_block + threadIdx.x / lanes;
     const int h = blockIdx.y, b = blockIdx.z;
+    // a ragged batch is one run of total_q rows (its batch strides are 0 and the grid has one batch entry)
+    const int n_rows = p.f.cu_q ? p.f.total_q : p.f.Lq, n_out = p.f.cu_q ? p.f.total_q : p.Lq_rounded;
     float acc = 0.f;
-    if (row < p.f.Lq) {
+    if (row < n_rows) {
         const uint16_t *op = (const uint16_t *)p.f.o + b * p.f.o_b + (int64_t)row * p.f.o_r + h * p.f.o_h;
         const uint16_t *dp = (const uint16_t *)p.dout + b * p.do_b + (int64_t)row * p.do_r + h * p.do_h;
         for (int c = sub; c < CH; c += lanes) {
@@ -60,7 +62,7 @@ __global__ void __launch_bounds__(256) bwd_dot_kernel(const BwdParams p) {
         }
     }
     for (int off = lanes / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
-    if (sub == 0 && row < p.Lq_rounded) p.softmax_d[((int64_t)b * p.f.H + h) * p.Lq_rounded + row] = acc;
+    if (sub == 0 && row < n_out) p.softmax_d[b * p.sd_b + h * p.sd_h + row] = acc;
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -534,7 +536,7 @@ hipError_t launch_bwd_t(const BwdParams &p, hipStream_t stream) {
     // 1. D = rowsum(dO * O)
     {
         const int CH = (f.d + 7) / 8, lanes = CH <= 8 ? 8 : 16, rpb = 256 / lanes;
-        dim3 grid((p.Lq_rounded + rpb - 1) / rpb, f.H, f.B);
+        dim3 grid(((f.cu_q ? f.total_q : p.Lq_rounded) + rpb - 1) / rpb, f.H, f.cu_q ? 1 : f.B);
         hipLaunchKernelGGL((bwd_dot_kernel<T>), grid, dim3(256), 0, stream, p);
         if ((e = hipGetLastError()) != hipSuccess) return e;
     }

@@ -127,11 +127,13 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
     }
     const int b = pair / f.Hk, hk = pair % f.Hk;
     const int n0 = n_block * KV_BN;
-    const int Lk = CMP ? f.cmp.count[pair] : f.Lk;  // key columns on this pair's (possibly compacted) key axis
-    if (CMP && n0 >= Lk) return;
+    const SeqInfo sq = seq_info(f, b);  // this batch entry's lengths and first rows (ragged batch: from cu_seqlens)
+    const int LqS = sq.Lq, LkS = sq.Lk;
+    const int Lk = CMP ? f.cmp.count[pair] : LkS;  // key columns on this pair's (possibly compacted) key axis
+    if (n0 >= Lk) return;  // the compacted list, or a shorter sequence of a ragged batch, ends before this block
     const int key = n0 + wave * 32 + r;  // the key column this lane owns
     const int key_c = key < Lk ? key : Lk - 1;
-    const int shift = f.Lk - f.Lq;
+    const int shift = LkS - LqS;
     // original column indices: of this lane's key, of the workgroup's first key and of the wave's last key
     const int32_t *cidx = CMP ? f.cmp.idx + (int64_t)pair * f.cmp.ld : nullptr;
     const int okey = CMP ? cidx[key_c] : key;
@@ -142,8 +144,8 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
     u32x4_t kf[KS], vf[V_LDS ? 1 : KS];
     char *sVrow = smem + SM::OFF_V + ((wave * 32 + r) * SM::S + g * 8) * 2;  // V_LDS: this lane's V row, its chunks
     {
-        const uint16_t *kp = (const uint16_t *)f.k + b * f.k_b + (int64_t)key_c * f.k_r + hk * f.k_h;
-        const uint16_t *vp = (const uint16_t *)f.v + b * f.v_b + (int64_t)key_c * f.v_r + hk * f.v_h;
+        const uint16_t *kp = (const uint16_t *)f.k + b * f.k_b + (sq.k0 + key_c) * f.k_r + hk * f.k_h;
+        const uint16_t *vp = (const uint16_t *)f.v + b * f.v_b + (sq.k0 + key_c) * f.v_r + hk * f.v_h;
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
             const int c = ks * 16 + g * 8;
@@ -165,9 +167,9 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
 #pragma unroll
         for (int i = 0; i < 16; i++) { dk[db][i] = 0.f; dv[db][i] = 0.f; }
 
-    const int M_blocks = (f.Lq + KV_BM - 1) / KV_BM;
+    const int M_blocks = (LqS + KV_BM - 1) / KV_BM;
     // query blocks that see the workgroup's first key: [m_start, M_blocks)
-    const int m_start = M_blocks - dkdv_query_blocks(f.Lq, f.Lk, CAUSAL, okey_first);
+    const int m_start = M_blocks - dkdv_query_blocks(LqS, LkS, CAUSAL, okey_first);
     // this workgroup's query blocks [m_lo, m_hi): all of them, or one of the unit's equal segments
     int m_lo = m_start, m_hi = M_blocks;
     if (slot >= 0) {
@@ -178,7 +180,7 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
         m_hi = m_lo + len < M_blocks ? m_lo + len : M_blocks;
     }
     // the planning blocks [m_lo, m_hi) in steps of BM rows: [s_lo, s_hi), without steps entirely beyond Lq
-    const int S_blocks = (f.Lq + BM - 1) / BM;
+    const int S_blocks = (LqS + BM - 1) / BM;
     const int s_lo = m_lo * SUB, s_hi = m_hi * SUB < S_blocks ? m_hi * SUB : S_blocks;
     const int n_m = s_hi > s_lo ? s_hi - s_lo : 0;
     // (g outer, m inner); the query blocks are walked from the LAST one down, so that the
@@ -227,7 +229,7 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
         const uint32_t lo = __builtin_amdgcn_readfirstlane((uint32_t)v), hi = __builtin_amdgcn_readfirstlane((uint32_t)(v >> 32));
         return (gptr_t)(((uint64_t)hi << 32) | lo);
     };
-    const int m_last = (f.Lq - 1) / BM, row_last = (f.Lq - 1) % BM;
+    const int m_last = (LqS - 1) / BM, row_last = (LqS - 1) % BM;
     uint32_t qoff[Q_IT], qoff_l[Q_IT], dooff[Q_IT], dooff_l[Q_IT];
 #pragma unroll
     for (int it = 0; it < Q_IT; it++) {
@@ -249,8 +251,8 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
         const int gi = g_lo + step / n_m, mi = s_hi - 1 - step % n_m;  // last query block first: see below
         const int h = hk * G + gi, m0 = mi * BM;
         column_const_load(h);
-        ld_qbase = uniform_ptr((const uint16_t *)f.q + b * f.q_b + h * f.q_h + (int64_t)m0 * f.q_r);
-        ld_dobase = uniform_ptr((const uint16_t *)p.dout + b * p.do_b + h * p.do_h + (int64_t)m0 * p.do_r);
+        ld_qbase = uniform_ptr((const uint16_t *)f.q + b * f.q_b + h * f.q_h + (sq.q0 + m0) * f.q_r);
+        ld_dobase = uniform_ptr((const uint16_t *)p.dout + b * p.do_b + h * p.do_h + (sq.q0 + m0) * p.do_r);
         ld_partial = mi == m_last;
         if (with_tiles) {
 #pragma unroll
@@ -260,10 +262,10 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
         // wait for it would also cover the tile loads above); range check and scaling happen in store_step
         {
             const int qq = m0 + (tid & (BM - 1));
-            stat_ok = qq < f.Lq;
-            const int qc = stat_ok ? qq : f.Lq - 1;
-            lreg = f.lse[((int64_t)b * f.H + h) * f.Lq + qc];
-            dreg = p.softmax_d[((int64_t)b * f.H + h) * p.Lq_rounded + qc];
+            stat_ok = qq < LqS;
+            const int qc = stat_ok ? qq : LqS - 1;
+            lreg = f.lse[b * f.lse_b + h * f.lse_h + sq.q0 + qc];
+            dreg = p.softmax_d[b * p.sd_b + h * p.sd_h + sq.q0 + qc];
         }
     };
     auto store_step = [&](int buf) {
@@ -469,8 +471,8 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
 
     // ---- store dK (scaled) and dV
     if (key < Lk) {
-        uint16_t *dkp = (uint16_t *)p.dk + b * p.dk_b + (int64_t)okey * p.dk_r + hk * p.dk_h;
-        uint16_t *dvp = (uint16_t *)p.dv + b * p.dv_b + (int64_t)okey * p.dv_r + hk * p.dv_h;
+        uint16_t *dkp = (uint16_t *)p.dk + b * p.dk_b + (sq.k0 + okey) * p.dk_r + hk * p.dk_h;
+        uint16_t *dvp = (uint16_t *)p.dv + b * p.dv_b + (sq.k0 + okey) * p.dv_r + hk * p.dv_h;
 #pragma unroll
         for (int db = 0; db < DB; db++)
 #pragma unroll
@@ -644,27 +646,30 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
     const int b = wm.pair / f.Hk, hk = wm.pair % f.Hk;
     const int h = hk * G + (blockIdx.x / 8) % G;
     const int m0 = m_block * Q_BM;
+    const SeqInfo sq = seq_info(f, b);  // this batch entry's lengths and first rows (ragged batch: from cu_seqlens)
+    const int LqS = sq.Lq, LkS = sq.Lk;
+    if (m0 >= LqS) return;
     const int qrow = m0 + wave * 32 + r;
-    const int qrow_c = qrow < f.Lq ? qrow : f.Lq - 1;
-    const int shift = f.Lk - f.Lq;
+    const int qrow_c = qrow < LqS ? qrow : LqS - 1;
+    const int shift = LkS - LqS;
 
     const int hm = f.mask ? (f.Hm == f.H ? h : (f.Hm == 1 ? 0 : hk)) : 0;
     const int hb = f.bias ? (f.Hb == f.H ? h : (f.Hb == 1 ? 0 : hk)) : 0;
     const uint8_t *mrow = f.mask ? f.mask + b * f.m_b + hm * f.m_h : nullptr;
     const uint16_t *brow = f.bias ? (const uint16_t *)f.bias + b * f.bi_b + hb * f.bi_h : nullptr;
-    const uint16_t *kbase = (const uint16_t *)f.k + b * f.k_b + hk * f.k_h;
-    const uint16_t *vbase = (const uint16_t *)f.v + b * f.v_b + hk * f.v_h;
+    const uint16_t *kbase = (const uint16_t *)f.k + b * f.k_b + sq.k0 * f.k_r + hk * f.k_h;
+    const uint16_t *vbase = (const uint16_t *)f.v + b * f.v_b + sq.k0 * f.v_r + hk * f.v_h;
 
     // key columns this workgroup iterates over (the compacted list with CMP), and how many a row may see
-    const int Lk = CMP ? f.cmp.count[wm.pair] : f.Lk;
+    const int Lk = CMP ? f.cmp.count[wm.pair] : LkS;
     const int32_t *ccnt = CMP ? f.cmp.cnt + (int64_t)wm.pair * f.cmp.ld : nullptr;
     const float *fbrow = CMP ? f.cmp.fb + (int64_t)(b * f.cmp.Hfb + (f.cmp.Hfb == f.H ? h : hk)) * f.cmp.ld : nullptr;
     auto visible = [&](int row) -> int {  // columns [0, visible(row)) pass the causal test for `row`
-        if (row >= f.Lq) row = f.Lq - 1;
+        if (row >= LqS) row = LqS - 1;
         const int c = row + shift;
         if (!CMP) return c + 1;
         if (c < 0) return 0;
-        return ccnt[c < f.Lk ? c : f.Lk - 1];
+        return ccnt[c < LkS ? c : LkS - 1];
     };
     const int vis_lane = CAUSAL ? visible(qrow) : 0;
     const int vis_wave = CAUSAL ? visible(m0 + wave * 32) : 0;
@@ -687,7 +692,7 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
 #pragma unroll
                 for (int c = 0; c < BN / 16; c++) {
                     const int col = j * BN + c * 16;
-                    if (col < f.Lk) {
+                    if (col < LkS) {
                         const u32x4_t mv = *(const u32x4_t *)(mrow + col);
                         any |= mv[0] | mv[1] | mv[2] | mv[3];
                     }
@@ -721,13 +726,13 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
     // ---- Q and dO fragments (B operands), row statistics
     u32x4_t qf[KS], dof[KS];
     {
-        const uint16_t *qp = (const uint16_t *)f.q + b * f.q_b + (int64_t)qrow_c * f.q_r + h * f.q_h;
-        const uint16_t *dp = (const uint16_t *)p.dout + b * p.do_b + (int64_t)qrow_c * p.do_r + h * p.do_h;
+        const uint16_t *qp = (const uint16_t *)f.q + b * f.q_b + (sq.q0 + qrow_c) * f.q_r + h * f.q_h;
+        const uint16_t *dp = (const uint16_t *)p.dout + b * p.do_b + (sq.q0 + qrow_c) * p.do_r + h * p.do_h;
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
             const int c = ks * 16 + g * 8;
             u32x4_t qv = {0, 0, 0, 0}, dv = {0, 0, 0, 0};
-            if (qrow < f.Lq && c < f.d) { qv = *(const u32x4_t *)(qp + c); dv = *(const u32x4_t *)(dp + c); }
+            if (qrow < LqS && c < f.d) { qv = *(const u32x4_t *)(qp + c); dv = *(const u32x4_t *)(dp + c); }
             // Q only feeds the scores in this kernel: scale it by softmax_scale * log2(e) once
 #pragma unroll
             for (int e = 0; e < 4; e++) qv[e] = E::pack2(E::lo(qv[e]) * f.scale_log2, E::hi(qv[e]) * f.scale_log2);
@@ -736,9 +741,9 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
         }
     }
     float lse2 = INFINITY, dd = 0.f;
-    if (qrow < f.Lq) {
-        lse2 = f.lse[((int64_t)b * f.H + h) * f.Lq + qrow] * kLog2e;
-        dd = p.softmax_d[((int64_t)b * f.H + h) * p.Lq_rounded + qrow];
+    if (qrow < LqS) {
+        lse2 = f.lse[b * f.lse_b + h * f.lse_h + sq.q0 + qrow] * kLog2e;
+        dd = p.softmax_d[b * p.sd_b + h * p.sd_h + sq.q0 + qrow];
     }
 
     f32x16_t dq[DB];
@@ -920,8 +925,8 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
         jc = jn;
     }
 
-    if (qrow < f.Lq) {
-        uint16_t *dqp = (uint16_t *)p.dq + b * p.dq_b + (int64_t)qrow * p.dq_r + h * p.dq_h;
+    if (qrow < LqS) {
+        uint16_t *dqp = (uint16_t *)p.dq + b * p.dq_b + (sq.q0 + qrow) * p.dq_r + h * p.dq_h;
 #pragma unroll
         for (int db = 0; db < DB; db++)
 #pragma unroll

@@ -88,7 +88,7 @@ __global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_col
     // multiple-of-8 lists are dealt to the XCDs, and an XCD walks its lists one after the other,
     // heaviest query block first, the G query heads of a block side by side.  Re-reads of K / V
     // tiles then hit in that XCD's L2, and every XCD gets the same amount of work.
-    const int n_mb = (p.Lq + BM - 1) / BM;
+    const int n_mb = (p.Lq + BM - 1) / BM;  // p.Lq, p.Lk: the longest sequence of a ragged batch
     const int G = p.H / p.Hk;
     const int pairs = p.B * p.Hk;
     const int gcd8 = (pairs % 8 == 0) ? 8 : ((pairs % 4 == 0) ? 4 : ((pairs % 2 == 0) ? 2 : 1));
@@ -105,26 +105,29 @@ __global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_col
     const int h = (pair % p.Hk) * G + pos % G;
     const int hk = h / (p.H / p.Hk);
     const int m0 = m_block * BM;
-    const int shift = p.Lk - p.Lq;
+    const SeqInfo sq = seq_info(p, b);  // this batch entry's lengths and first rows (ragged batch: from cu_seqlens)
+    const int LqS = sq.Lq, LkS = sq.Lk;
+    if (m0 >= LqS) return;
+    const int shift = LkS - LqS;
     const int wrow0 = m0 + wave * 32 * NQ;  // first query row of this wave
 
     const int hm = p.mask ? (p.Hm == p.H ? h : (p.Hm == 1 ? 0 : h / (p.H / p.Hm))) : 0;
     const int hb = p.bias ? (p.Hb == p.H ? h : (p.Hb == 1 ? 0 : h / (p.H / p.Hb))) : 0;
     const uint8_t *mrow = p.mask ? p.mask + b * p.m_b + hm * p.m_h : nullptr;
     const uint16_t *brow = p.bias ? (const uint16_t *)p.bias + b * p.bi_b + hb * p.bi_h : nullptr;
-    const uint16_t *kbase = (const uint16_t *)p.k + b * p.k_b + hk * p.k_h;
-    const uint16_t *vbase = (const uint16_t *)p.v + b * p.v_b + hk * p.v_h;
+    const uint16_t *kbase = (const uint16_t *)p.k + b * p.k_b + sq.k0 * p.k_r + hk * p.k_h;
+    const uint16_t *vbase = (const uint16_t *)p.v + b * p.v_b + sq.k0 * p.v_r + hk * p.v_h;
 
     // key columns this workgroup iterates over, and the number of them a query row may see
-    const int Lk = CMP ? p.cmp.count[b * p.Hk + hk] : p.Lk;
+    const int Lk = CMP ? p.cmp.count[b * p.Hk + hk] : LkS;
     const int32_t *ccnt = CMP ? p.cmp.cnt + (int64_t)(b * p.Hk + hk) * p.cmp.ld : nullptr;
     const float *fbrow = CMP ? p.cmp.fb + (int64_t)(b * p.cmp.Hfb + (p.cmp.Hfb == p.H ? h : hk)) * p.cmp.ld : nullptr;
     auto visible = [&](int row) -> int {  // columns [0, visible(row)) pass the causal test for `row`
-        if (row >= p.Lq) row = p.Lq - 1;
+        if (row >= LqS) row = LqS - 1;
         int c = row + shift;
         if (!CMP) return c + 1;
         if (c < 0) return 0;
-        return ccnt[c < p.Lk ? c : p.Lk - 1];
+        return ccnt[c < LkS ? c : LkS - 1];
     };
 
     int n_end = (Lk + BN - 1) / BN;
@@ -145,7 +148,7 @@ __global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_col
 #pragma unroll
                 for (int c = 0; c < BN / 16; c++) {
                     const int col = j * BN + c * 16;
-                    if (col < p.Lk) {
+                    if (col < LkS) {
                         u32x4_t mv = *(const u32x4_t *)(mrow + col);
                         any |= mv[0] | mv[1] | mv[2] | mv[3];
                     }
@@ -184,13 +187,13 @@ __global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_col
 #pragma unroll
     for (int nb = 0; nb < NQ; nb++) {
         const int qrow = wrow0 + nb * 32 + r;
-        const int qc = qrow < p.Lq ? qrow : p.Lq - 1;
-        const uint16_t *qp = (const uint16_t *)p.q + b * p.q_b + (int64_t)qc * p.q_r + h * p.q_h;
+        const int qc = qrow < LqS ? qrow : LqS - 1;
+        const uint16_t *qp = (const uint16_t *)p.q + b * p.q_b + (sq.q0 + qc) * p.q_r + h * p.q_h;
 #pragma unroll
         for (int ks = 0; ks < KS; ks++) {
             const int c = ks * 16 + g * 8;
             u32x4_t v = {0, 0, 0, 0};
-            if (qrow < p.Lq && c < p.d) v = *(const u32x4_t *)(qp + c);
+            if (qrow < LqS && c < p.d) v = *(const u32x4_t *)(qp + c);
             // Q is scaled by softmax_scale * log2(e) once, here (the reference also rounds the scaled Q to the
             // input type, flash_fwd_kernel.h:428-439): the MFMA then accumulates exp2-domain scores directly on
             // top of the fused bias, with no per-element multiply afterwards
@@ -493,8 +496,8 @@ __global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_col
         const int qrow = wrow0 + nb * 32 + r;
         const float total = xhalf_sum(row_sum[nb]);
         const float inv = total > 0.f ? 1.f / total : 0.f;
-        if (qrow < p.Lq) {
-            uint16_t *op = (uint16_t *)p.o + b * p.o_b + (int64_t)qrow * p.o_r + h * p.o_h;
+        if (qrow < LqS) {
+            uint16_t *op = (uint16_t *)p.o + b * p.o_b + (sq.q0 + qrow) * p.o_r + h * p.o_h;
 #pragma unroll
             for (int db = 0; db < DB; db++)
 #pragma unroll
@@ -510,7 +513,7 @@ __global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_col
                 }
             if (g == 0) {
                 const float lse = total > 0.f ? (row_max[nb] + __builtin_amdgcn_logf(total)) * kLn2 : INFINITY;
-                p.lse[((int64_t)b * p.H + h) * p.Lq + qrow] = lse;
+                p.lse[b * p.lse_b + h * p.lse_h + sq.q0 + qrow] = lse;
             }
         }
     }

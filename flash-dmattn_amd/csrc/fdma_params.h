@@ -82,7 +82,13 @@ struct FwdParams {
     const uint8_t *mask;  // nullptr = absent
     const void *bias;     // nullptr = absent
     void *o;
-    float *lse;           // (B, H, Lq)
+    float *lse;           // element (b, h, row) at b * lse_b + h * lse_h + first row of b + row
+    int64_t lse_b, lse_h; // (B, H, Lq): H * Lq, Lq; ragged batch (H, total_q): 0, total_q
+    // Ragged batch (the reference's "varlen" layout, csrc/flash_sparse_attn/flash_api.cpp:556-790): q / k / v hold the
+    // sequences back to back, (total rows, heads, d), batch entry b owns rows cu[b] .. cu[b + 1] - 1 and the batch
+    // strides are 0.  Lq / Lk below are then the longest sequences (they size the grids).  nullptr = fixed lengths.
+    const int32_t *cu_q, *cu_k;
+    int32_t total_q, total_k;  // rows of the ragged q / k tensors
     int64_t q_b, q_r, q_h;
     int64_t k_b, k_r, k_h;
     int64_t v_b, v_r, v_h;
@@ -100,6 +106,28 @@ struct FwdParams {
     Compact cmp;        // when cmp.on, k / v (and their strides) describe the compacted copies
 };
 
+// lengths and first rows of batch entry b
+struct SeqInfo {
+    int32_t Lq, Lk;
+    int64_t q0, k0;
+};
+__device__ inline SeqInfo seq_info(const FwdParams &p, int b) {
+    SeqInfo s;
+    if (p.cu_q) {
+        const int32_t q0 = p.cu_q[b], k0 = p.cu_k[b];
+        s.q0 = q0;
+        s.k0 = k0;
+        s.Lq = p.cu_q[b + 1] - q0;
+        s.Lk = p.cu_k[b + 1] - k0;
+    } else {
+        s.q0 = 0;
+        s.k0 = 0;
+        s.Lq = p.Lq;
+        s.Lk = p.Lk;
+    }
+    return s;
+}
+
 struct BwdParams {
     FwdParams f;  // f.o = forward output (read), f.lse = forward LSE (read)
     const void *dout;
@@ -109,7 +137,8 @@ struct BwdParams {
     int64_t dk_b, dk_r, dk_h;
     int64_t dv_b, dv_r, dv_h;
     int64_t db_b, db_h, db_r;  // dbias strides (batch, head, row); 0 = broadcast
-    float *softmax_d;          // (B, H, Lq_rounded)
+    float *softmax_d;          // laid out like lse: b * sd_b + h * sd_h + first row of b + row
+    int64_t sd_b, sd_h;        // (B, H, Lq_rounded): H * Lq_rounded, Lq_rounded; ragged batch: 0, total_q
     int32_t Lq_rounded;
     float *dbias_accum;        // fp32 scratch at the dbias shape when several workgroups share an element
     int64_t dba_b, dba_h, dba_r;

@@ -48,10 +48,39 @@ class BwdArgs(ctypes.Structure):
     ]
 
 
+class VarlenFwdArgs(ctypes.Structure):
+    _fields_ = [
+        ("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p),
+        ("out", ctypes.c_void_p), ("lse", ctypes.c_void_p),
+        ("cu_seqlens_q", ctypes.c_void_p), ("cu_seqlens_k", ctypes.c_void_p),
+        ("q_strides", ctypes.c_int64 * 2), ("k_strides", ctypes.c_int64 * 2),
+        ("v_strides", ctypes.c_int64 * 2), ("o_strides", ctypes.c_int64 * 2),
+        ("batch", ctypes.c_int32), ("total_q", ctypes.c_int32), ("total_k", ctypes.c_int32),
+        ("max_seqlen_q", ctypes.c_int32), ("max_seqlen_k", ctypes.c_int32),
+        ("num_heads", ctypes.c_int32), ("num_heads_k", ctypes.c_int32), ("head_dim", ctypes.c_int32),
+        ("dtype", ctypes.c_int32), ("is_causal", ctypes.c_int32),
+        ("softmax_scale", ctypes.c_float), ("softcap", ctypes.c_float),
+    ]
+
+
+class VarlenBwdArgs(ctypes.Structure):
+    _fields_ = [
+        ("f", VarlenFwdArgs),
+        ("dout", ctypes.c_void_p),
+        ("dq", ctypes.c_void_p), ("dk", ctypes.c_void_p), ("dv", ctypes.c_void_p),
+        ("do_strides", ctypes.c_int64 * 2), ("dq_strides", ctypes.c_int64 * 2),
+        ("dk_strides", ctypes.c_int64 * 2), ("dv_strides", ctypes.c_int64 * 2),
+        ("softmax_d", ctypes.c_void_p),
+        ("deterministic", ctypes.c_int32),
+    ]
+
+
 EXPORTS = (
     "fdma_fwd", "fdma_bwd", "fdma_fwd_workspace_bytes", "fdma_bwd_workspace_bytes",
     "fdma_fwd_validate", "fdma_bwd_validate", "fdma_last_error", "fdma_abi_version",
     "fdma_sizeof_fwd_args", "fdma_sizeof_bwd_args",
+    "fdma_varlen_fwd", "fdma_varlen_bwd", "fdma_varlen_fwd_validate", "fdma_varlen_bwd_validate",
+    "fdma_sizeof_varlen_fwd_args", "fdma_sizeof_varlen_bwd_args",
 )
 
 
@@ -87,9 +116,21 @@ def _load() -> ctypes.CDLL:
     lib.fdma_abi_version.restype = ctypes.c_int
     lib.fdma_sizeof_fwd_args.restype = ctypes.c_size_t
     lib.fdma_sizeof_bwd_args.restype = ctypes.c_size_t
-    if lib.fdma_abi_version() != 1:
-        raise ImportError(f"{path}: ABI version {lib.fdma_abi_version()} != 1")
-    if lib.fdma_sizeof_fwd_args() != ctypes.sizeof(FwdArgs) or lib.fdma_sizeof_bwd_args() != ctypes.sizeof(BwdArgs):
+    if lib.fdma_abi_version() != 2:
+        raise ImportError(f"{path}: ABI version {lib.fdma_abi_version()} != 2")
+    lib.fdma_varlen_fwd.argtypes = [ctypes.POINTER(VarlenFwdArgs), ctypes.c_void_p]
+    lib.fdma_varlen_fwd.restype = ctypes.c_int
+    lib.fdma_varlen_bwd.argtypes = [ctypes.POINTER(VarlenBwdArgs), ctypes.c_void_p]
+    lib.fdma_varlen_bwd.restype = ctypes.c_int
+    lib.fdma_varlen_fwd_validate.argtypes = [ctypes.POINTER(VarlenFwdArgs)]
+    lib.fdma_varlen_fwd_validate.restype = ctypes.c_int
+    lib.fdma_varlen_bwd_validate.argtypes = [ctypes.POINTER(VarlenBwdArgs)]
+    lib.fdma_varlen_bwd_validate.restype = ctypes.c_int
+    lib.fdma_sizeof_varlen_fwd_args.restype = ctypes.c_size_t
+    lib.fdma_sizeof_varlen_bwd_args.restype = ctypes.c_size_t
+    sizes = ((lib.fdma_sizeof_fwd_args(), FwdArgs), (lib.fdma_sizeof_bwd_args(), BwdArgs),
+             (lib.fdma_sizeof_varlen_fwd_args(), VarlenFwdArgs), (lib.fdma_sizeof_varlen_bwd_args(), VarlenBwdArgs))
+    if any(n != ctypes.sizeof(t) for n, t in sizes):
         raise ImportError(f"{path}: argument block size differs from the Python mirror")
     return lib
 
@@ -152,6 +193,24 @@ def fill_fwd(a: FwdArgs, q, k, v, mask, bias, out, lse, softmax_scale, is_causal
         head_dim, dtype_code(q), int(bool(is_causal)),
         float(softmax_scale), float(softcap), 0, 0,
     )
+
+
+def fill_varlen_fwd(a: VarlenFwdArgs, q, k, v, out, lse, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
+                    softmax_scale, is_causal, softcap) -> None:
+    a.q, a.k, a.v = q.data_ptr(), k.data_ptr(), v.data_ptr()
+    a.out, a.lse = out.data_ptr(), lse.data_ptr()
+    a.cu_seqlens_q, a.cu_seqlens_k = cu_seqlens_q.data_ptr(), cu_seqlens_k.data_ptr()
+    a.q_strides[:] = (q.stride(0), q.stride(1))
+    a.k_strides[:] = (k.stride(0), k.stride(1))
+    a.v_strides[:] = (v.stride(0), v.stride(1))
+    a.o_strides[:] = (out.stride(0), out.stride(1))
+    a.batch = cu_seqlens_q.numel() - 1
+    a.total_q, a.total_k = q.shape[0], k.shape[0]
+    a.max_seqlen_q, a.max_seqlen_k = int(max_seqlen_q), int(max_seqlen_k)
+    a.num_heads, a.num_heads_k, a.head_dim = q.shape[1], k.shape[1], q.shape[2]
+    a.dtype = dtype_code(q)
+    a.is_causal = int(bool(is_causal))
+    a.softmax_scale, a.softcap = float(softmax_scale), float(softcap)
 
 
 def _as_buffer(a):

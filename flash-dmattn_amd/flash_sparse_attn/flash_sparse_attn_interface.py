@@ -446,9 +446,297 @@ def flash_sparse_attn_func(
     )
 
 
-def flash_sparse_attn_varlen_func(*args, **kwargs):
-    """Ragged-batch entry point of the reference (interface.py:687-760).  It takes no mask or bias
-    and is not part of the dynamic-mask hot path; it is not built here."""
-    raise NotImplementedError(
-        "flash_sparse_attn_varlen_func (cu_seqlens path without mask/bias) is not provided by the MI355X build"
+def _check_varlen_inputs(q, k, v, cu_seqlens_q, cu_seqlens_k) -> None:
+    """Checks of mha_varlen_fwd (flash_api.cpp:583-660) that concern torch tensors."""
+    if q.dtype not in (torch.float16, torch.bfloat16):
+        raise RuntimeError("FlashSparseAttention only support fp16 and bf16 data type")
+    if k.dtype != q.dtype:
+        raise RuntimeError("query and key must have the same dtype")
+    if v.dtype != q.dtype:
+        raise RuntimeError("query and value must have the same dtype")
+    for name, t in (("cu_seqlens_q", cu_seqlens_q), ("cu_seqlens_k", cu_seqlens_k)):
+        if t.dtype != torch.int32:
+            raise RuntimeError(f"{name} must have dtype int32")
+        if t.device != q.device:
+            raise RuntimeError(f"{name} must be on the device of q")
+        if not t.is_contiguous():
+            raise RuntimeError(f"{name} must be contiguous")
+    if q.dim() != 3 or k.dim() != 3 or v.dim() != 3:
+        raise RuntimeError("q, k, v must have shape (total, nheads, headdim)")
+    if tuple(k.shape) != tuple(v.shape) or k.shape[2] != q.shape[2]:
+        raise RuntimeError("k and v must have shape (total_k, num_heads_k, head_size)")
+    batch = cu_seqlens_q.numel() - 1
+    if batch <= 0:
+        raise RuntimeError("batch size must be positive")
+    if cu_seqlens_k.numel() != batch + 1:
+        raise RuntimeError("cu_seqlens_k must have shape (batch_size + 1)")
+
+
+@torch.library.custom_op("flash_sparse_attn::_flash_sparse_attn_varlen_forward", mutates_args=(), device_types="cuda")
+def _flash_sparse_attn_varlen_forward(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    cu_seqlens_q: torch.Tensor,
+    cu_seqlens_k: torch.Tensor,
+    max_seqlen_q: int,
+    max_seqlen_k: int,
+    softmax_scale: float,
+    is_causal: bool,
+    softcap: float = 0.0,
+    return_softmax: bool = False,
+    block_table: Optional[torch.Tensor] = None,
+    leftpad_k: Optional[torch.Tensor] = None,
+    seqused_k: Optional[torch.Tensor] = None,
+    zero_tensors: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    """Ragged-batch forward (interface.py:129-167 of the reference).  Rows of `out` / `softmax_lse` that belong to
+    no sequence (beyond cu_seqlens_q[-1]) are zero-filled when `zero_tensors` is set and left unwritten otherwise."""
+    if block_table is not None or leftpad_k is not None or seqused_k is not None:
+        raise RuntimeError("paged KV (block_table), leftpad_k and seqused_k are not supported by this build")
+    _check_varlen_inputs(q, k, v, cu_seqlens_q, cu_seqlens_k)
+    q, k, v = [_aligned(x, 8) for x in (q, k, v)]
+    total_q, num_heads, _ = q.shape
+    out = torch.zeros_like(q, memory_format=torch.contiguous_format) if zero_tensors else torch.empty_like(q, memory_format=torch.contiguous_format)
+    softmax_lse = torch.empty((num_heads, total_q), dtype=torch.float32, device=q.device)
+    if zero_tensors:
+        softmax_lse.fill_(float("-inf"))  # flash_api.cpp:699-702
+    p = torch.empty((0,), dtype=q.dtype, device=q.device)
+    if total_q == 0:
+        return out, softmax_lse, p
+    args = _cabi.VarlenFwdArgs()
+    _cabi.fill_varlen_fwd(args, q, k, v, out, softmax_lse, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
+                          softmax_scale, is_causal, softcap)
+    with torch.cuda.device(q.device):
+        _cabi.check(_cabi.lib.fdma_varlen_fwd(args, _cabi.current_stream(q.device)))
+    return out, softmax_lse, p
+
+
+@torch.library.register_fake("flash_sparse_attn::_flash_sparse_attn_varlen_forward")
+def _flash_sparse_attn_varlen_forward_fake(
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    cu_seqlens_q: torch.Tensor,
+    cu_seqlens_k: torch.Tensor,
+    max_seqlen_q: int,
+    max_seqlen_k: int,
+    softmax_scale: float,
+    is_causal: bool,
+    softcap: float = 0.0,
+    return_softmax: bool = False,
+    block_table: Optional[torch.Tensor] = None,
+    leftpad_k: Optional[torch.Tensor] = None,
+    seqused_k: Optional[torch.Tensor] = None,
+    zero_tensors: bool = False,
+) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
+    total_q, num_heads, _ = q.shape
+    out = torch.empty_like(q, memory_format=torch.contiguous_format)
+    softmax_lse = torch.empty((num_heads, total_q), dtype=torch.float32, device=q.device)
+    p = torch.empty((0,), dtype=q.dtype, device=q.device)
+    return out, softmax_lse, p
+
+
+_wrapped_flash_sparse_attn_varlen_forward = _flash_sparse_attn_varlen_forward
+
+
+@torch.library.custom_op(
+    "flash_sparse_attn::_flash_sparse_attn_varlen_backward", mutates_args=("dq", "dk", "dv"), device_types="cuda"
+)
+def _flash_sparse_attn_varlen_backward(
+    dout: torch.Tensor,
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    out: torch.Tensor,
+    softmax_lse: torch.Tensor,
+    dq: Optional[torch.Tensor],
+    dk: Optional[torch.Tensor],
+    dv: Optional[torch.Tensor],
+    cu_seqlens_q: torch.Tensor,
+    cu_seqlens_k: torch.Tensor,
+    max_seqlen_q: int,
+    max_seqlen_k: int,
+    softmax_scale: float,
+    is_causal: bool,
+    softcap: float,
+    deterministic: bool,
+    zero_tensors: bool = False,
+) -> torch.Tensor:
+    """Ragged-batch backward (interface.py:291-339 of the reference).  Gradient rows that belong to no sequence are
+    zero-filled when `zero_tensors` is set and left unwritten otherwise (flash_api.cpp:1209-1214)."""
+    _check_varlen_inputs(q, k, v, cu_seqlens_q, cu_seqlens_k)
+    if out.dtype != q.dtype:
+        raise RuntimeError("query and out must have the same dtype")
+    if dout.dtype != q.dtype:
+        raise RuntimeError("query and dout must have the same dtype")
+    if tuple(out.shape) != tuple(q.shape) or tuple(dout.shape) != tuple(q.shape):
+        raise RuntimeError("out and dout must have the shape of q")
+    dout, q, k, v, out = [_aligned(x, 8) for x in (dout, q, k, v, out)]
+    softmax_lse = softmax_lse.contiguous()
+    total_q, num_heads, _ = q.shape
+    softmax_d = torch.empty((num_heads, total_q), device=q.device, dtype=torch.float32)
+
+    def staging(t, like, name):
+        if t is None:
+            raise RuntimeError(f"{name} must be provided")
+        if t.dtype != q.dtype:
+            raise RuntimeError(f"{name} must have the same dtype as q")
+        if tuple(t.shape) != tuple(like.shape):
+            raise RuntimeError(f"{name} must have the shape of its input")
+        ok = t.stride(-1) == 1 and t.data_ptr() % 16 == 0 and all(
+            t.size(i) == 1 or t.stride(i) % 8 == 0 for i in range(t.dim() - 1))
+        return t if ok else torch.empty_like(t, memory_format=torch.contiguous_format)
+
+    dq_w, dk_w, dv_w = staging(dq, q, "dq"), staging(dk, k, "dk"), staging(dv, v, "dv")
+    if zero_tensors:
+        for t in (dq_w, dk_w, dv_w, softmax_d):
+            t.zero_()
+    args = _cabi.VarlenBwdArgs()
+    _cabi.fill_varlen_fwd(args.f, q, k, v, out, softmax_lse, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
+                          softmax_scale, is_causal, softcap)
+    args.dout = dout.data_ptr()
+    args.dq, args.dk, args.dv = dq_w.data_ptr(), dk_w.data_ptr(), dv_w.data_ptr()
+    args.do_strides[:] = (dout.stride(0), dout.stride(1))
+    args.dq_strides[:] = (dq_w.stride(0), dq_w.stride(1))
+    args.dk_strides[:] = (dk_w.stride(0), dk_w.stride(1))
+    args.dv_strides[:] = (dv_w.stride(0), dv_w.stride(1))
+    args.softmax_d = softmax_d.data_ptr()
+    args.deterministic = int(bool(deterministic))
+    with torch.cuda.device(q.device):
+        _cabi.check(_cabi.lib.fdma_varlen_bwd(args, _cabi.current_stream(q.device)))
+    for given, work in ((dq, dq_w), (dk, dk_w), (dv, dv_w)):
+        if given is not None and work is not given:
+            given.copy_(work)
+    return softmax_d
+
+
+@torch.library.register_fake("flash_sparse_attn::_flash_sparse_attn_varlen_backward")
+def _flash_sparse_attn_varlen_backward_fake(
+    dout: torch.Tensor,
+    q: torch.Tensor,
+    k: torch.Tensor,
+    v: torch.Tensor,
+    out: torch.Tensor,
+    softmax_lse: torch.Tensor,
+    dq: Optional[torch.Tensor],
+    dk: Optional[torch.Tensor],
+    dv: Optional[torch.Tensor],
+    cu_seqlens_q: torch.Tensor,
+    cu_seqlens_k: torch.Tensor,
+    max_seqlen_q: int,
+    max_seqlen_k: int,
+    softmax_scale: float,
+    is_causal: bool,
+    softcap: float,
+    deterministic: bool,
+    zero_tensors: bool = False,
+) -> torch.Tensor:
+    total_q, num_heads, _ = q.shape
+    return torch.empty((num_heads, total_q), device=q.device, dtype=torch.float32)
+
+
+_wrapped_flash_sparse_attn_varlen_backward = _flash_sparse_attn_varlen_backward
+
+
+class FlashAttnVarlenFunc(torch.autograd.Function):
+    """Autograd node of the ragged-batch path (interface.py:500-608 of the reference): argument defaults, head
+    dimension padded to a multiple of 8, saved tensors, slicing of the padded gradients."""
+
+    @staticmethod
+    def forward(
+        ctx,
+        q: torch.Tensor,
+        k: torch.Tensor,
+        v: torch.Tensor,
+        cu_seqlens_q: torch.Tensor,
+        cu_seqlens_k: torch.Tensor,
+        max_seqlen_q: int,
+        max_seqlen_k: int,
+        softmax_scale: Optional[float],
+        is_causal: Optional[bool],
+        softcap: Optional[float],
+        deterministic: Optional[bool],
+        return_softmax: Optional[bool],
+        block_table: Optional[torch.Tensor],
+        is_grad_enabled: bool = True,
+    ):
+        is_grad = is_grad_enabled and any(x.requires_grad for x in [q, k, v])
+        if softmax_scale is None:
+            softmax_scale = q.shape[-1] ** (-0.5)
+        is_causal = False if is_causal is None else is_causal
+        softcap = 0.0 if softcap is None else softcap
+        deterministic = False if deterministic is None else deterministic
+        return_softmax = False if return_softmax is None else return_softmax
+
+        head_size_og = q.size(2)
+        if head_size_og % 8 != 0:
+            pad = [0, 8 - head_size_og % 8]
+            q, k, v = (torch.nn.functional.pad(t, pad) for t in (q, k, v))
+
+        out_padded, softmax_lse, S_dmask = _wrapped_flash_sparse_attn_varlen_forward(
+            q, k, v, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale,
+            is_causal=is_causal, softcap=softcap, return_softmax=return_softmax, block_table=block_table,
+        )
+        if is_grad:
+            ctx.save_for_backward(q, k, v, out_padded, softmax_lse, cu_seqlens_q, cu_seqlens_k)
+            ctx.max_seqlen_q = max_seqlen_q
+            ctx.max_seqlen_k = max_seqlen_k
+            ctx.softmax_scale = softmax_scale
+            ctx.is_causal = is_causal
+            ctx.softcap = softcap
+            ctx.deterministic = deterministic
+        out = out_padded[..., :head_size_og]
+        return out if not return_softmax else (out, softmax_lse, S_dmask)
+
+    @staticmethod
+    def backward(ctx, dout, *args):
+        q, k, v, out, softmax_lse, cu_seqlens_q, cu_seqlens_k = ctx.saved_tensors
+        dq, dk, dv = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v)
+        head_size_og = dout.size(2)
+        dout_padded = dout
+        if head_size_og % 8 != 0:
+            dout_padded = torch.nn.functional.pad(dout, [0, 8 - head_size_og % 8])
+        _wrapped_flash_sparse_attn_varlen_backward(
+            dout_padded, q, k, v, out, softmax_lse, dq, dk, dv, cu_seqlens_q, cu_seqlens_k,
+            ctx.max_seqlen_q, ctx.max_seqlen_k, ctx.softmax_scale, ctx.is_causal, ctx.softcap, ctx.deterministic,
+        )
+        dq = dq[..., : dout.shape[-1]]
+        dk = dk[..., : dout.shape[-1]]
+        dv = dv[..., : dout.shape[-1]]
+        return dq, dk, dv, None, None, None, None, None, None, None, None, None, None, None
+
+
+def flash_sparse_attn_varlen_func(
+    query: torch.Tensor,
+    key: torch.Tensor,
+    value: torch.Tensor,
+    cu_seqlens_q: torch.Tensor,
+    cu_seqlens_k: torch.Tensor,
+    max_seqlen_q: int,
+    max_seqlen_k: int,
+    softmax_scale: Optional[float] = None,
+    is_causal: Optional[bool] = None,
+    softcap: Optional[float] = None,
+    deterministic: Optional[bool] = None,
+    return_attn_probs: Optional[bool] = None,
+    block_table: Optional[torch.Tensor] = None,
+):
+    """Ragged-batch ("varlen") attention without mask or bias, signature and semantics of the reference's
+    `flash_sparse_attn_varlen_func` (interface.py:687-760).
+
+    query: (total_q, nheads, headdim); key, value: (total_k, nheads_k, headdim); the sequences of the batch lie
+    back to back and `cu_seqlens_q` / `cu_seqlens_k` (int32, batch + 1, on the device) hold their first rows.
+    MQA / GQA through nheads_k < nheads (query head h uses kv head h // (nheads / nheads_k)).  With
+    `is_causal` the mask is aligned to the bottom right corner of every sequence's attention matrix; a row
+    without visible keys gives a zero output.  `max_seqlen_q` / `max_seqlen_k` are upper bounds of the
+    sequence lengths.  The lengths are read on the device only: the call never synchronises.
+
+    Returns out (total_q, nheads, headdim), or (out, softmax_lse (nheads, total_q), S_dmask (empty)) when
+    `return_attn_probs` is set.  Paged KV (`block_table`) and softcapping raise RuntimeError.
+    """
+    return FlashAttnVarlenFunc.apply(
+        query, key, value, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
+        softmax_scale, is_causal, softcap, deterministic, return_attn_probs, block_table,
+        torch.is_grad_enabled(),
     )

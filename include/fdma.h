@@ -9,6 +9,8 @@
  *
  *   fdma_fwd   <-  mha_fwd            csrc/flash_sparse_attn/flash_api.cpp:351-554  (pybind "fwd",  :1272)
  *   fdma_bwd   <-  mha_bwd            csrc/flash_sparse_attn/flash_api.cpp:792-1050 (pybind "bwd",  :1274)
+ *   fdma_varlen_fwd <- mha_varlen_fwd csrc/flash_sparse_attn/flash_api.cpp:556-790  (pybind "varlen_fwd", :1273)
+ *   fdma_varlen_bwd <- mha_varlen_bwd csrc/flash_sparse_attn/flash_api.cpp:1052-1268 (pybind "varlen_bwd", :1275)
  *   fdma_fwd_args / fdma_bwd_args
  *              <-  Flash_fwd_params / Flash_bwd_params   csrc/flash_sparse_attn/src/flash.h:20-198
  *
@@ -41,7 +43,7 @@
 extern "C" {
 #endif
 
-#define FDMA_ABI_VERSION 1
+#define FDMA_ABI_VERSION 2 /* 2: fdma_varlen_* added; everything of version 1 is unchanged */
 
 enum { FDMA_DTYPE_BF16 = 0, FDMA_DTYPE_FP16 = 1 };
 
@@ -99,6 +101,50 @@ size_t fdma_bwd_workspace_bytes(const fdma_bwd_args *args);
 /* Argument validation only (no GPU work, callable on a host without a device). */
 int fdma_fwd_validate(const fdma_fwd_args *args);
 int fdma_bwd_validate(const fdma_bwd_args *args);
+
+/*
+ * Ragged batches ("varlen"): the sequences of a batch lie back to back in q (total_q, num_heads, head_dim)
+ * and k / v (total_k, num_heads_k, head_dim); batch entry i owns query rows cu_seqlens_q[i] .. cu_seqlens_q[i+1]-1
+ * and key rows cu_seqlens_k[i] .. cu_seqlens_k[i+1]-1.  cu_seqlens_* are DEVICE arrays of batch+1 int32, starting
+ * at 0 and non-decreasing (the library never reads them on the host and never synchronises).  As in the
+ * reference this path takes no mask and no bias; the causal mask is aligned bottom-right per sequence.
+ *   lse       : (num_heads, total_q) fp32, contiguous; +inf for rows with no visible key
+ *   softmax_d : (num_heads, total_q) fp32, contiguous
+ * Strides are {row, head} in elements, innermost dimension contiguous.  max_seqlen_* must be upper bounds
+ * of the sequence lengths (they size the launch); rows of sequences longer than that are not computed.
+ * Not built: paged KV (block_table), seqused_k, leftpad_k (flash_api.cpp:564-566).
+ */
+typedef struct fdma_varlen_fwd_args {
+    const void *q, *k, *v;
+    void *out;
+    float *lse;
+    const int32_t *cu_seqlens_q, *cu_seqlens_k;
+    int64_t q_strides[2], k_strides[2], v_strides[2], o_strides[2];
+    int32_t batch, total_q, total_k, max_seqlen_q, max_seqlen_k;
+    int32_t num_heads, num_heads_k, head_dim;
+    int32_t dtype;
+    int32_t is_causal;
+    float softmax_scale;
+    float softcap; /* must be 0 */
+} fdma_varlen_fwd_args;
+
+typedef struct fdma_varlen_bwd_args {
+    fdma_varlen_fwd_args f; /* f.out and f.lse are the forward RESULTS (read) */
+    const void *dout;
+    void *dq, *dk, *dv;
+    int64_t do_strides[2], dq_strides[2], dk_strides[2], dv_strides[2];
+    float *softmax_d; /* out: rowsum(dO * O) */
+    int32_t deterministic;
+} fdma_varlen_bwd_args;
+
+/* Forward / backward over a ragged batch.  No workspace is needed.  Every row of out / lse / dq / dk / dv that
+ * belongs to a sequence is written exactly once. */
+int fdma_varlen_fwd(const fdma_varlen_fwd_args *args, void *hip_stream);
+int fdma_varlen_bwd(const fdma_varlen_bwd_args *args, void *hip_stream);
+int fdma_varlen_fwd_validate(const fdma_varlen_fwd_args *args);
+int fdma_varlen_bwd_validate(const fdma_varlen_bwd_args *args);
+size_t fdma_sizeof_varlen_fwd_args(void);
+size_t fdma_sizeof_varlen_bwd_args(void);
 
 /* Message of the last error raised on the calling thread ("" if none). */
 const char *fdma_last_error(void);

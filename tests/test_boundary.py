@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(_cabi.lib_path())
     for name in declared:
         assert hasattr(lib, name), f"{name} not exported"
-    assert lib.fdma_abi_version() == 1
+    assert lib.fdma_abi_version() == 2
 
 
 def test_struct_mirrors_match_compiled_sizes():
@@ -32,6 +32,8 @@ def test_struct_mirrors_match_compiled_sizes():
 
     assert _cabi.lib.fdma_sizeof_fwd_args() == ctypes.sizeof(_cabi.FwdArgs)
     assert _cabi.lib.fdma_sizeof_bwd_args() == ctypes.sizeof(_cabi.BwdArgs)
+    assert _cabi.lib.fdma_sizeof_varlen_fwd_args() == ctypes.sizeof(_cabi.VarlenFwdArgs)
+    assert _cabi.lib.fdma_sizeof_varlen_bwd_args() == ctypes.sizeof(_cabi.VarlenBwdArgs)
 
 
 def _valid_fwd():
@@ -198,3 +200,74 @@ def test_compaction_workspace_rule(monkeypatch):
     need = _cabi.lib.fdma_fwd_workspace_bytes(big)
     kv_bytes = 2 * 4096 * 2 * 64 * 2
     assert kv_bytes <= need <= 2 * kv_bytes                      # dense K / V copies plus index lists
+
+
+def _valid_varlen_fwd():
+    from flash_sparse_attn import _cabi
+
+    a = _cabi.VarlenFwdArgs()
+    for name in ("q", "k", "v", "out", "lse", "cu_seqlens_q", "cu_seqlens_k"):
+        setattr(a, name, 0x1000)
+    a.batch, a.total_q, a.total_k, a.max_seqlen_q, a.max_seqlen_k = 3, 300, 500, 128, 256
+    a.num_heads, a.num_heads_k, a.head_dim, a.dtype, a.is_causal = 8, 2, 64, 0, 1
+    a.softmax_scale, a.softcap = 0.125, 0.0
+    for s, v in (("q_strides", (8 * 64, 64)), ("k_strides", (2 * 64, 64)), ("v_strides", (2 * 64, 64)),
+                 ("o_strides", (8 * 64, 64))):
+        getattr(a, s)[:] = v
+    return a
+
+
+@pytest.mark.parametrize(
+    "field,value,message",
+    [
+        ("dtype", 7, "only support fp16 and bf16"),
+        ("batch", 0, "batch size must be positive"),
+        ("head_dim", 260, "head dimension at most 256"),
+        ("head_dim", 60, "multiple of 8"),
+        ("num_heads_k", 3, "must divide number of heads in query"),
+        ("cu_seqlens_q", 0, "cu_seqlens_q and cu_seqlens_k must be device pointers"),
+        ("cu_seqlens_k", 0x1002, "4-byte aligned"),
+        ("softcap", 1.0, "softcap is not supported"),
+        ("head_dim", 192, "above 128 are not built"),
+        ("q", 0x1008, "16-byte aligned"),
+    ],
+)
+def test_varlen_validation_rejects(field, value, message):
+    """Ragged-batch argument rules (csrc/flash_sparse_attn/flash_api.cpp:583-660 of the reference), checked
+    without a GPU."""
+    from flash_sparse_attn import _cabi
+
+    a = _valid_varlen_fwd()
+    assert _cabi.lib.fdma_varlen_fwd_validate(a) == 0, _cabi.last_error()
+    setattr(a, field, value)
+    assert _cabi.lib.fdma_varlen_fwd_validate(a) < 0
+    assert message in _cabi.last_error()
+
+
+def test_varlen_backward_validation():
+    from flash_sparse_attn import _cabi
+
+    b = _cabi.VarlenBwdArgs()
+    b.f = _valid_varlen_fwd()
+    for name in ("dout", "dq", "dk", "dv", "softmax_d"):
+        setattr(b, name, 0x2000)
+    for s, v in (("do_strides", (8 * 64, 64)), ("dq_strides", (8 * 64, 64)), ("dk_strides", (2 * 64, 64)),
+                 ("dv_strides", (2 * 64, 64))):
+        getattr(b, s)[:] = v
+    assert _cabi.lib.fdma_varlen_bwd_validate(b) == 0, _cabi.last_error()
+    b.dk = 0
+    assert _cabi.lib.fdma_varlen_bwd_validate(b) < 0
+    assert "dout, dq, dk, dv must be device pointers" in _cabi.last_error()
+    b.dk = 0x2000
+    b.dq_strides[0] = 8 * 64 + 4
+    assert _cabi.lib.fdma_varlen_bwd_validate(b) < 0
+    assert "multiples of 8" in _cabi.last_error()
+
+
+def test_varlen_operator_signature_matches_reference():
+    """flash_sparse_attn_interface.py:687-701 of the reference."""
+    from flash_sparse_attn import flash_sparse_attn_varlen_func
+
+    names = list(inspect.signature(flash_sparse_attn_varlen_func).parameters)
+    assert names == ["query", "key", "value", "cu_seqlens_q", "cu_seqlens_k", "max_seqlen_q", "max_seqlen_k",
+                     "softmax_scale", "is_causal", "softcap", "deterministic", "return_attn_probs", "block_table"]
