@@ -393,4 +393,69 @@ int fdma_varlen_bwd(const fdma_varlen_bwd_args *a, void *hip_stream) {
     return FDMA_OK;
 }
 
+size_t fdma_sizeof_mask_args(void) { return sizeof(fdma_mask_args); }
+
+int fdma_create_mask_validate(const fdma_mask_args *a) {
+    g_err[0] = 0;
+    if (!a) return fail(FDMA_ERR_INVALID, "args must not be NULL");
+    if (a->dtype != FDMA_DTYPE_BF16 && a->dtype != FDMA_DTYPE_FP16)
+        return fail(FDMA_ERR_INVALID, "attention_bias must be fp16 or bf16");
+    if (a->type != FDMA_MASK_TOPK && a->type != FDMA_MASK_RELU)
+        return fail(FDMA_ERR_INVALID, "Unsupported mask type: %d. Supported types are 'topk' and 'relu'.", a->type);
+    if (a->batch < 0 || a->heads < 0 || a->rows < 0 || a->seqlen_k < 0) return fail(FDMA_ERR_INVALID, "mask dimensions must be non-negative");
+    if ((int64_t)a->batch * a->heads * a->rows > 0x7fffffff) return fail(FDMA_ERR_UNSUPPORTED, "more than 2^31 - 1 mask rows");
+    if (a->type == FDMA_MASK_TOPK && a->window < 0) return fail(FDMA_ERR_INVALID, "window_size must be non-negative");
+    if (a->block_size < 0) return fail(FDMA_ERR_INVALID, "block_size must be a positive integer, got %d.", a->block_size);
+    const bool empty = (int64_t)a->batch * a->heads * a->rows * a->seqlen_k == 0;
+    if (!empty && (!a->bias || !a->mask_out)) return fail(FDMA_ERR_INVALID, "bias and mask_out must be device pointers");
+    if (reinterpret_cast<uintptr_t>(a->bias) & 1) return fail(FDMA_ERR_INVALID, "bias must be 2-byte aligned");
+    if (std::isnan(a->min_value)) return fail(FDMA_ERR_INVALID, "min_dtype must not be NaN");
+    return FDMA_OK;
+}
+
+// float -> bits of the bias type, round to nearest even, overflow to infinity
+static uint32_t to_bits16(float x, int dtype) {
+    uint32_t u;
+    std::memcpy(&u, &x, 4);
+    if (dtype == FDMA_DTYPE_BF16) {
+        u += 0x7fffu + ((u >> 16) & 1u);
+        return u >> 16;
+    }
+    const uint32_t sign = (u >> 16) & 0x8000u;
+    const float ax = std::fabs(x);
+    if (!(ax < 65520.f)) return sign | 0x7c00u;
+    if (ax < 6.103515625e-05f) {  // subnormal half: units of 2^-24
+        const float scaled = ax * 16777216.f;
+        const uint32_t m = (uint32_t)std::nearbyintf(scaled);
+        return sign | m;
+    }
+    uint32_t a;
+    std::memcpy(&a, &ax, 4);
+    a += 0xfffu + ((a >> 13) & 1u);  // round the 13 dropped mantissa bits to nearest even
+    const uint32_t e = (a >> 23) - 127 + 15, m = (a >> 13) & 0x3ffu;
+    return sign | (e << 10) | m;
+}
+
+int fdma_create_mask(const fdma_mask_args *a, void *hip_stream) {
+    int rc = fdma_create_mask_validate(a);
+    if (rc != FDMA_OK) return rc;
+    fdma::MaskParams p;
+    std::memset(&p, 0, sizeof(p));
+    p.bias = a->bias;
+    p.mask_in = static_cast<const uint8_t *>(a->mask_in);
+    p.mask_out = static_cast<uint8_t *>(a->mask_out);
+    p.bi_b = a->bias_strides[0]; p.bi_h = a->bias_strides[1]; p.bi_r = a->bias_strides[2];
+    p.mi_b = a->mask_in_strides[0]; p.mi_h = a->mask_in_strides[1]; p.mi_r = a->mask_in_strides[2];
+    p.mo_b = a->mask_out_strides[0]; p.mo_h = a->mask_out_strides[1]; p.mo_r = a->mask_out_strides[2];
+    p.batch = a->batch; p.heads = a->heads; p.rows = a->rows; p.Lk = a->seqlen_k;
+    p.window = a->window;
+    p.block_size = a->block_size;
+    p.type = a->type;
+    p.dtype = a->dtype;
+    p.min_bits = to_bits16(a->min_value, a->dtype);
+    const hipError_t e = fdma::launch_make_mask(p, static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(FDMA_ERR_LAUNCH, "mask launch failed: %s", hipGetErrorString(e));
+    return FDMA_OK;
+}
+
 }  // extern "C"

@@ -147,6 +147,23 @@ struct BwdParams {
     float *db_part;
 };
 
+// Keep-mask builder (fdma_mask.hip): one row of `Lk` 16-bit bias values per (batch, head, row).
+struct MaskParams {
+    const void *bias;
+    const uint8_t *mask_in;  // nullptr = absent; 0 strides broadcast
+    uint8_t *mask_out;
+    int64_t bi_b, bi_h, bi_r;
+    int64_t mi_b, mi_h, mi_r;
+    int64_t mo_b, mo_h, mo_r;
+    int32_t batch, heads, rows, Lk;
+    int32_t window;      // top-k: entries kept per row
+    int32_t block_size;  // > 1: majority vote inside aligned key blocks afterwards
+    int32_t type;        // 0 = top-k, 1 = relu
+    int32_t dtype;       // 0 = bf16, 1 = fp16
+    uint32_t min_bits;   // the fill value for entries the incoming mask excludes, as bits of the bias type
+};
+hipError_t launch_make_mask(const MaskParams &p, hipStream_t stream);
+
 // dtype: 0 = bf16, 1 = fp16.  All launches are asynchronous on `stream`; return hipError_t.
 hipError_t launch_fwd(const FwdParams &p, int dtype, hipStream_t stream);
 // column-mask specialisation (mask / bias absent or broadcast over queries); nq = 32-row blocks per wave

@@ -75,12 +75,24 @@ class VarlenBwdArgs(ctypes.Structure):
     ]
 
 
+class MaskArgs(ctypes.Structure):
+    _fields_ = [
+        ("bias", ctypes.c_void_p), ("mask_in", ctypes.c_void_p), ("mask_out", ctypes.c_void_p),
+        ("bias_strides", ctypes.c_int64 * 3), ("mask_in_strides", ctypes.c_int64 * 3),
+        ("mask_out_strides", ctypes.c_int64 * 3),
+        ("batch", ctypes.c_int32), ("heads", ctypes.c_int32), ("rows", ctypes.c_int32), ("seqlen_k", ctypes.c_int32),
+        ("window", ctypes.c_int32), ("block_size", ctypes.c_int32), ("type", ctypes.c_int32), ("dtype", ctypes.c_int32),
+        ("min_value", ctypes.c_float),
+    ]
+
+
 EXPORTS = (
     "fdma_fwd", "fdma_bwd", "fdma_fwd_workspace_bytes", "fdma_bwd_workspace_bytes",
     "fdma_fwd_validate", "fdma_bwd_validate", "fdma_last_error", "fdma_abi_version",
     "fdma_sizeof_fwd_args", "fdma_sizeof_bwd_args",
     "fdma_varlen_fwd", "fdma_varlen_bwd", "fdma_varlen_fwd_validate", "fdma_varlen_bwd_validate",
     "fdma_sizeof_varlen_fwd_args", "fdma_sizeof_varlen_bwd_args",
+    "fdma_create_mask", "fdma_create_mask_validate", "fdma_sizeof_mask_args",
 )
 
 
@@ -128,7 +140,12 @@ def _load() -> ctypes.CDLL:
     lib.fdma_varlen_bwd_validate.restype = ctypes.c_int
     lib.fdma_sizeof_varlen_fwd_args.restype = ctypes.c_size_t
     lib.fdma_sizeof_varlen_bwd_args.restype = ctypes.c_size_t
-    sizes = ((lib.fdma_sizeof_fwd_args(), FwdArgs), (lib.fdma_sizeof_bwd_args(), BwdArgs),
+    lib.fdma_create_mask.argtypes = [ctypes.POINTER(MaskArgs), ctypes.c_void_p]
+    lib.fdma_create_mask.restype = ctypes.c_int
+    lib.fdma_create_mask_validate.argtypes = [ctypes.POINTER(MaskArgs)]
+    lib.fdma_create_mask_validate.restype = ctypes.c_int
+    lib.fdma_sizeof_mask_args.restype = ctypes.c_size_t
+    sizes = ((lib.fdma_sizeof_mask_args(), MaskArgs), (lib.fdma_sizeof_fwd_args(), FwdArgs), (lib.fdma_sizeof_bwd_args(), BwdArgs),
              (lib.fdma_sizeof_varlen_fwd_args(), VarlenFwdArgs), (lib.fdma_sizeof_varlen_bwd_args(), VarlenBwdArgs))
     if any(n != ctypes.sizeof(t) for n, t in sizes):
         raise ImportError(f"{path}: argument block size differs from the Python mirror")

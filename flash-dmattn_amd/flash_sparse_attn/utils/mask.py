@@ -2,9 +2,15 @@
 
 Same functions, argument meaning and error behaviour as the reference's
 flash_sparse_attn/utils/mask.py (topk_indices :20-44, block_smooth :47-73, topk_mask :76-120,
-relu_mask :123-160, create_mask :164-240).  They are thin host-side tensor programs: on a GPU
-tensor they run as a handful of library kernels whose cost is O(rows * key_len), negligible next to
-the attention they feed.
+relu_mask :123-160, create_mask :164-240).
+
+For a 4-D fp16 / bf16 bias on the GPU, `topk_mask` and `relu_mask` (and so `create_mask`) run as ONE kernel of
+libfdma_hip.so (`fdma_create_mask`: masked fill, radix select of the window largest values per row, exclusion of
+the fill value, block smoothing) instead of masked_fill + topk + zeros + scatter (+ view / sum / copy) through
+the tensor library -- on the benchmark shapes that chain costs as much as the attention it feeds.  Among entries
+equal to the smallest selected value the lowest columns are kept; the reference leaves that choice to
+`torch.topk`, which does not define it.  Every other input (CPU tensors, fp32, other ranks) takes the same tensor
+program as the reference.
 """
 from typing import Optional
 
@@ -42,6 +48,47 @@ def block_smooth(attention_mask: torch.Tensor, key_len: int, block_size: int) ->
     return attention_mask
 
 
+def _native_mask(attention_bias, attention_mask, window_size, min_dtype, block_size, kind) -> Optional[torch.Tensor]:
+    """Device path; None when the inputs are not of the form the kernel takes."""
+    if not (attention_bias.is_cuda and attention_bias.dim() == 4 and attention_bias.dtype in (torch.bfloat16, torch.float16)):
+        return None
+    if attention_mask is not None and not (attention_mask.dim() == 4 and attention_mask.dtype == torch.bool
+                                           and attention_mask.device == attention_bias.device):
+        return None
+    from .. import _cabi
+
+    bias = attention_bias.detach()
+    shape = tuple(bias.shape) if attention_mask is None else tuple(torch.broadcast_shapes(bias.shape, attention_mask.shape))
+    if kind == "topk" and window_size > shape[-1]:
+        return None  # torch.topk raises for k beyond the row length; let it
+    bias = bias.expand(shape)
+    if shape[-1] > 1 and bias.stride(-1) != 1:
+        bias = bias.contiguous()
+    mask_in = None
+    if attention_mask is not None:
+        mask_in = attention_mask.expand(shape)
+        if shape[-1] > 1 and mask_in.stride(-1) != 1:
+            mask_in = mask_in.contiguous()
+    out = torch.empty(shape, dtype=torch.bool, device=bias.device)
+    if out.numel() == 0:
+        return out
+    a = _cabi.MaskArgs()
+    a.bias, a.mask_out = bias.data_ptr(), out.data_ptr()
+    a.mask_in = mask_in.data_ptr() if mask_in is not None else None
+    a.bias_strides[:] = bias.stride()[:3]
+    a.mask_in_strides[:] = mask_in.stride()[:3] if mask_in is not None else (0, 0, 0)
+    a.mask_out_strides[:] = out.stride()[:3]
+    a.batch, a.heads, a.rows, a.seqlen_k = shape
+    a.window = int(window_size) if kind == "topk" else 0
+    a.block_size = int(block_size) if block_size is not None and block_size > 1 else 0  # mask.py:112, 152
+    a.type = 0 if kind == "topk" else 1
+    a.dtype = _cabi.dtype_code(bias)
+    a.min_value = float(min_dtype)
+    with torch.cuda.device(bias.device):
+        _cabi.check(_cabi.lib.fdma_create_mask(a, _cabi.current_stream(bias.device)))
+    return out
+
+
 def _masked_bias(attention_bias: torch.Tensor, attention_mask: Optional[torch.Tensor], min_dtype: float):
     bias = attention_bias.detach()
     if attention_mask is not None:
@@ -63,6 +110,9 @@ def topk_mask(
     entry whose value equals `min_dtype` is not kept, so a row with fewer than `window_size`
     admissible keys keeps only those.
     """
+    keep = _native_mask(attention_bias, attention_mask, window_size, min_dtype, block_size, "topk")
+    if keep is not None:
+        return keep
     bias = _masked_bias(attention_bias, attention_mask, min_dtype)
     values, indices = bias.topk(window_size, dim=-1, largest=True, sorted=False)
     keep = torch.zeros_like(bias, dtype=torch.bool).scatter_(-1, indices, values != min_dtype)
@@ -79,6 +129,9 @@ def relu_mask(
     **kwargs,
 ) -> torch.Tensor:
     """Keep the strictly positive bias entries (mask.py:123-160)."""
+    keep = _native_mask(attention_bias, attention_mask, 0, min_dtype, block_size, "relu")
+    if keep is not None:
+        return keep
     keep = _masked_bias(attention_bias, attention_mask, min_dtype) > 0
     if block_size is not None and block_size > 1:
         keep = block_smooth(keep, keep.shape[-1], block_size)

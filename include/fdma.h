@@ -43,7 +43,7 @@
 extern "C" {
 #endif
 
-#define FDMA_ABI_VERSION 2 /* 2: fdma_varlen_* added; everything of version 1 is unchanged */
+#define FDMA_ABI_VERSION 2 /* 2: fdma_varlen_* and fdma_create_mask added; everything of version 1 is unchanged */
 
 enum { FDMA_DTYPE_BF16 = 0, FDMA_DTYPE_FP16 = 1 };
 
@@ -145,6 +145,36 @@ int fdma_varlen_fwd_validate(const fdma_varlen_fwd_args *args);
 int fdma_varlen_bwd_validate(const fdma_varlen_bwd_args *args);
 size_t fdma_sizeof_varlen_fwd_args(void);
 size_t fdma_sizeof_varlen_bwd_args(void);
+
+/*
+ * Keep-mask builder: topk_mask / relu_mask with the optional block_smooth of the reference's
+ * flash_sparse_attn/utils/mask.py:47-160, one kernel per call.
+ *   bias     : ({batch|1}, {heads}, {rows}, seqlen_k) bf16 / fp16, strides {batch, head, row} in elements
+ *   mask_in  : NULL, or bool (uint8) broadcastable to the bias: strides {batch, head, row} in bytes, 0 = broadcast
+ *   mask_out : bool (uint8), one row of seqlen_k bytes per bias row, strides {batch, head, row} in bytes
+ * type 0 (top-k): per row, entries excluded by mask_in are replaced by min_value, the `window` largest values are
+ * selected (all of them when window >= seqlen_k) and a selected entry is kept unless its value equals min_value.
+ * Among entries equal to the smallest selected value the lowest columns win (the reference leaves this choice to
+ * torch.topk, which does not define it).  type 1 (relu): an entry is kept when its value, after the same
+ * replacement, is > 0.  block_size > 1 then replaces every aligned block of block_size keys by the majority vote
+ * of its entries (strictly more than half; a shorter tail block votes over its own length).
+ */
+enum { FDMA_MASK_TOPK = 0, FDMA_MASK_RELU = 1 };
+typedef struct fdma_mask_args {
+    const void *bias;
+    const void *mask_in;
+    void *mask_out;
+    int64_t bias_strides[3], mask_in_strides[3], mask_out_strides[3];
+    int32_t batch, heads, rows, seqlen_k;
+    int32_t window;
+    int32_t block_size; /* 0 or 1 = no smoothing */
+    int32_t type;
+    int32_t dtype;
+    float min_value;
+} fdma_mask_args;
+int fdma_create_mask(const fdma_mask_args *args, void *hip_stream);
+int fdma_create_mask_validate(const fdma_mask_args *args);
+size_t fdma_sizeof_mask_args(void);
 
 /* Message of the last error raised on the calling thread ("" if none). */
 const char *fdma_last_error(void);

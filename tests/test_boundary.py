@@ -34,6 +34,7 @@ def test_struct_mirrors_match_compiled_sizes():
     assert _cabi.lib.fdma_sizeof_bwd_args() == ctypes.sizeof(_cabi.BwdArgs)
     assert _cabi.lib.fdma_sizeof_varlen_fwd_args() == ctypes.sizeof(_cabi.VarlenFwdArgs)
     assert _cabi.lib.fdma_sizeof_varlen_bwd_args() == ctypes.sizeof(_cabi.VarlenBwdArgs)
+    assert _cabi.lib.fdma_sizeof_mask_args() == ctypes.sizeof(_cabi.MaskArgs)
 
 
 def _valid_fwd():
@@ -271,3 +272,28 @@ def test_varlen_operator_signature_matches_reference():
     names = list(inspect.signature(flash_sparse_attn_varlen_func).parameters)
     assert names == ["query", "key", "value", "cu_seqlens_q", "cu_seqlens_k", "max_seqlen_q", "max_seqlen_k",
                      "softmax_scale", "is_causal", "softcap", "deterministic", "return_attn_probs", "block_table"]
+
+
+def test_mask_builder_validation():
+    """Argument rules of fdma_create_mask (the builder behind flash_sparse_attn.utils.mask), checked without a GPU."""
+    from flash_sparse_attn import _cabi
+
+    def good():
+        a = _cabi.MaskArgs()
+        a.bias, a.mask_out = 0x1000, 0x2000
+        a.batch, a.heads, a.rows, a.seqlen_k = 2, 4, 1, 512
+        a.bias_strides[:] = (4 * 512, 512, 0)
+        a.mask_out_strides[:] = (4 * 512, 512, 512)
+        a.window, a.block_size, a.type, a.dtype, a.min_value = 128, 0, 0, 0, -3.0e38
+        return a
+
+    assert _cabi.lib.fdma_create_mask_validate(good()) == 0, _cabi.last_error()
+    for field, value, message in (("dtype", 3, "fp16 or bf16"), ("type", 2, "Unsupported mask type"),
+                                  ("window", -1, "window_size must be non-negative"),
+                                  ("block_size", -2, "block_size must be a positive integer"),
+                                  ("bias", 0, "device pointers"), ("bias", 0x1001, "2-byte aligned"),
+                                  ("min_value", float("nan"), "must not be NaN")):
+        a = good()
+        setattr(a, field, value)
+        assert _cabi.lib.fdma_create_mask_validate(a) < 0, field
+        assert message in _cabi.last_error()
