@@ -221,6 +221,57 @@ def run_config(name, steps, warmup, device, compact=True, backward=True):
     return res
 
 
+def run_mask_builder(steps, warmup, device):
+    """Keep-mask construction in front of the operator (not part of `value`): flash_sparse_attn.utils.mask.topk_mask
+    through the device kernel, next to the reference's tensor program (masked_fill / topk / zeros / scatter,
+    flash_sparse_attn/utils/mask.py:100-110) on the same device, for the bias rows of the benchmark shapes."""
+    from flash_sparse_attn.utils import mask as M
+
+    res = []
+    for name in ("cfg2", "cfg4", "cfg5"):
+        c = CONFIGS[name]
+        bias = torch.randn(c["B"], c["Hk"], 1, c["Lk"], generator=torch.Generator().manual_seed(1)).to(torch.bfloat16).to(device)
+        lowest = torch.finfo(torch.bfloat16).min
+
+        def program():
+            vals, idx = bias.topk(c["W"], dim=-1, largest=True, sorted=False)
+            return torch.zeros_like(bias, dtype=torch.bool).scatter_(-1, idx, vals != lowest)
+
+        with torch.no_grad():
+            ms_kernel = time_gpu(lambda: M.topk_mask(bias, None, c["W"], lowest), steps, warmup)
+            ms_program = time_gpu(program, steps, warmup)
+        res.append({"rows": "%s: %d x %d, top-%d" % (name, c["B"] * c["Hk"], c["Lk"], c["W"]),
+                    "us_device_kernel": 1e3 * ms_kernel, "us_tensor_program": 1e3 * ms_program})
+    return res
+
+
+def run_ragged_batch(steps, warmup, device):
+    """flash_sparse_attn_varlen_func (no mask, no bias, causal) on a ragged batch of 16384 tokens, H=32, Hkv=8, d=128;
+    FLOPs are the element-exact causal ones, 4 * d * H * sum(n * (n + 1) / 2)."""
+    from flash_sparse_attn import flash_sparse_attn_varlen_func
+
+    lens = [100, 3000, 777, 5000, 64, 2048, 1, 5394]
+    H, Hk, D = 32, 8, 128
+    g = torch.Generator().manual_seed(2)
+    total = sum(lens)
+    q = torch.randn(total, H, D, generator=g).to(torch.bfloat16).to(device).requires_grad_(True)
+    k = torch.randn(total, Hk, D, generator=g).to(torch.bfloat16).to(device).requires_grad_(True)
+    v = torch.randn(total, Hk, D, generator=g).to(torch.bfloat16).to(device).requires_grad_(True)
+    cu = torch.tensor([0] + list(torch.tensor(lens).cumsum(0)), dtype=torch.int32, device=device)
+    dout = torch.ones_like(q)
+    flops = float(sum(4 * D * H * (n * (n + 1) // 2) for n in lens))
+    with torch.no_grad():
+        ms_fwd = time_gpu(lambda: flash_sparse_attn_varlen_func(q, k, v, cu, cu, max(lens), max(lens), None, True), steps, warmup)
+
+    def step():
+        flash_sparse_attn_varlen_func(q, k, v, cu, cu, max(lens), max(lens), None, True).backward(dout)
+        q.grad = k.grad = v.grad = None
+
+    ms_fb = time_gpu(step, max(2, steps // 2), max(1, warmup // 2))
+    return {"seqlens": lens, "heads": H, "kv_heads": Hk, "head_dim": D, "ms_fwd": ms_fwd, "tflops_fwd": flops / ms_fwd / 1e9,
+            "ms_fwd_bwd": ms_fb, "tflops_fwd_bwd": 3.5 * flops / ms_fb / 1e9}
+
+
 def cpu_baseline(device_cfg="cfg2", groups=8, chunk=2):
     """The fp32 safe-eager restatement (oracle/eager.py, a port of the reference's eager formula) timed
     on the host cores for a bounded sample of the headline workload: `groups` KV groups (each with its
@@ -335,6 +386,8 @@ def main():
     if args.all:
         out["other_configs"] = [run_config(n, max(3, args.steps // 4), max(1, args.warmup // 2), device, compact)
                                 for n in ("cfg1", "cfg3", "cfg4", "cfg5")]
+        out["mask_builder"] = run_mask_builder(max(3, args.steps // 2), max(1, args.warmup // 2), device)
+        out["ragged_batch"] = run_ragged_batch(max(3, args.steps // 4), max(1, args.warmup // 2), device)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline("cfg2", groups=8)
     print(json.dumps(out))
