@@ -557,7 +557,8 @@ hipError_t launch_bwd_t(const BwdParams &p, hipStream_t stream) {
         // shared by several workgroups (broadcast over the batch or over kv heads) is accumulated with fp32 atomics
         const bool gsum = f.bias != nullptr && f.bi_r != 0 && ((f.Hb != f.H && f.H / f.Hk > 1) || p.dbias_accum != nullptr);
         auto launch = [&](auto kern, size_t smem) -> hipError_t {
-            hipError_t e2 = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+            static DynSmemLimit smem_limit;  // one per kernel: the lambda is instantiated per kernel type
+            hipError_t e2 = smem_limit.ensure((const void *)kern, (int)smem);
             if (e2 != hipSuccess) return e2;
             hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, stream, p);
             return hipGetLastError();

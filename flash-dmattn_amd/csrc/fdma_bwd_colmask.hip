@@ -584,7 +584,8 @@ hipError_t launch_dkdv_c(const BwdParams &p, hipStream_t stream) {
     const FwdParams &f = p.f;
     auto kern = bwd_dkdv_colmask_kernel<T, D, CAUSAL, CMP>;
     const int smem = KvcSmem<D>::TOTAL;
-    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    static DynSmemLimit smem_limit;
+    hipError_t e = smem_limit.ensure((const void *)kern, (int)smem);
     if (e != hipSuccess) return e;
     const int units_max = f.B * f.Hk * ((f.Lk + KV_BN - 1) / KV_BN);
     if (CMP) {
@@ -949,7 +950,8 @@ hipError_t launch_dq(const BwdParams &p, hipStream_t stream) {
     constexpr int BN = D > 64 ? 32 : 64;  // at d = 128 a 64-key tile would spill registers
     auto kern = p.f.cmp.on ? bwd_dq_colmask_kernel<T, D, BN, CAUSAL, true> : bwd_dq_colmask_kernel<T, D, BN, CAUSAL, false>;
     const int smem = DqcSmem<D, BN>::TOTAL;
-    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    static DynSmemLimit smem_limit;
+    hipError_t e = smem_limit.ensure((const void *)kern, (int)smem);
     if (e != hipSuccess) return e;
     dim3 grid(xcd_grid(f.B * f.Hk, (f.Lq + Q_BM - 1) / Q_BM, f.H / f.Hk));
     hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, stream, p);

@@ -335,7 +335,8 @@ hipError_t launch_dq_n(const BwdParams &p, hipStream_t stream) {
     constexpr int BM = 32 * NW, NTHREADS = 64 * NW, BN = NW == 8 ? 32 : 64;
     auto kern = bwd_dq_kernel<T, D, CAUSAL, NW>;
     const int smem = DqSmem<D, BM, BN>::TOTAL;
-    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    static DynSmemLimit smem_limit;
+    hipError_t e = smem_limit.ensure((const void *)kern, (int)smem);
     if (e != hipSuccess) return e;
     dim3 grid(((p.f.Lq + BM - 1) / BM) * p.f.H * p.f.B);
     hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, stream, p);

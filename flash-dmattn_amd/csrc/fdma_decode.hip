@@ -310,7 +310,8 @@ hipError_t launch_decode_gc(const FwdParams &p, int keys_per_split, hipStream_t 
     dim3 grid(p.splits, p.Hk * chunks, p.B);
     const size_t smem = (size_t)4 * GC * Dpad * sizeof(float);
     auto kern = decode_kernel<T, GC>;
-    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);
+    static DynSmemLimit smem_limit;
+    hipError_t e = smem_limit.ensure((const void *)kern, (int)smem);
     if (e != hipSuccess) return e;
     hipLaunchKernelGGL(kern, grid, dim3(DEC_THREADS), smem, stream, p, keys_per_split, 0);
     return hipGetLastError();

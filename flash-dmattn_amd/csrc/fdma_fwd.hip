@@ -389,7 +389,8 @@ hipError_t launch_fwd_c(const FwdParams &p, hipStream_t stream) {
     constexpr int BM = 32 * NW, NTHREADS = 64 * NW;
     auto kern = fwd_kernel<T, D, CAUSAL, NW>;
     const int smem = FwdSmem<D, BM>::TOTAL;
-    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    static DynSmemLimit smem_limit;
+    hipError_t e = smem_limit.ensure((const void *)kern, (int)smem);
     if (e != hipSuccess) return e;
     dim3 grid(((p.Lq + BM - 1) / BM) * p.H * p.B);
     hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, stream, p);

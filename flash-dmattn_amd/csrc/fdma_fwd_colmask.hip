@@ -524,7 +524,8 @@ hipError_t launch_one(const FwdParams &p, hipStream_t stream) {
     constexpr int BM = 32 * NQ * NW;
     auto kern = fwd_colmask_kernel<T, D, NQ, BN, CAUSAL, NW, CMP>;
     const int smem = CmSmem<D, BN>::TOTAL;
-    hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, smem);
+    static DynSmemLimit smem_limit;
+    hipError_t e = smem_limit.ensure((const void *)kern, (int)smem);
     if (e != hipSuccess) return e;
     const int n_mb = (p.Lq + BM - 1) / BM, G = p.H / p.Hk, pairs = p.B * p.Hk;
     const int gcd8 = (pairs % 8 == 0) ? 8 : ((pairs % 4 == 0) ? 4 : ((pairs % 2 == 0) ? 2 : 1));

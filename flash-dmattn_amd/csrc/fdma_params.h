@@ -6,6 +6,8 @@
 #include <hip/hip_runtime.h>
 #include <stdint.h>
 
+#include <atomic>
+
 namespace fdma {
 
 // Column compaction for keep-masks that are broadcast over queries: the kept keys of every
@@ -163,6 +165,26 @@ struct MaskParams {
     uint32_t min_bits;   // the fill value for entries the incoming mask excludes, as bits of the bias type
 };
 hipError_t launch_make_mask(const MaskParams &p, hipStream_t stream);
+
+// Dynamic-LDS limit of a kernel, raised once per device (and again only for a larger request) instead of on every
+// launch: one `static DynSmemLimit` per launch site.  Later launches make no runtime call besides the launch itself.
+struct DynSmemLimit {
+    static constexpr int kDevices = 16;
+    std::atomic<int> set_bytes[kDevices] = {};
+    hipError_t ensure(const void *kernel, int bytes) {
+        int dev = 0;
+        hipError_t e = hipGetDevice(&dev);
+        if (e != hipSuccess) return e;
+        const bool tracked = dev >= 0 && dev < kDevices;
+        if (tracked && set_bytes[dev].load(std::memory_order_acquire) >= bytes) return hipSuccess;
+        e = hipFuncSetAttribute(kernel, hipFuncAttributeMaxDynamicSharedMemorySize, bytes);
+        if (e == hipSuccess && tracked) {
+            int seen = set_bytes[dev].load(std::memory_order_relaxed);
+            while (seen < bytes && !set_bytes[dev].compare_exchange_weak(seen, bytes, std::memory_order_release)) {}
+        }
+        return e;
+    }
+};
 
 // dtype: 0 = bf16, 1 = fp16.  All launches are asynchronous on `stream`; return hipError_t.
 hipError_t launch_fwd(const FwdParams &p, int dtype, hipStream_t stream);
