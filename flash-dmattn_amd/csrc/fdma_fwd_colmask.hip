@@ -429,6 +429,10 @@ __global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_col
                     pk[nb][8 * mb + i / 2] = E::pack2(p0, p1);
                 }
             row_sum[nb] += psum;
+            // pin the sum here: left alone, the compiler sinks the whole chain of additions below the PV MFMAs (its
+            // result is not needed before the next tile), where nothing hides it, and keeps all 32 probabilities
+            // alive in fp32 until then
+            asm volatile("" : "+v"(row_sum[nb]));
         }
     };
     // O^T += V^T P^T for one tile; the global loads of the tile two ahead are issued between the MFMAs (a burst of
