@@ -197,6 +197,18 @@ def _flash_sparse_attn_backward(
     dq_w, dk_w, dv_w = staging(dq, q, "dq"), staging(dk, k, "dk"), staging(dv, v, "dv")
     dbias_w = staging(dbias, bias, "dbias") if bias is not None else None
 
+    # A bias that is broadcast over the batch (batch > 1) or has one head for several kv heads makes several
+    # workgroups add into the same dbias element; the kernels do that with fp32 atomics, whose order is not fixed.
+    # With deterministic=True every (batch entry, kv head) gets its own slice instead and the slices are summed in
+    # a fixed order afterwards, which is what the reference always does (flash_api.cpp:970-983, 1027-1047).
+    dbias_sum_dims = ()
+    if deterministic and bias is not None:
+        dbias_sum_dims = tuple(d for d, full in ((0, batch), (1, k.size(2))) if bias.size(d) == 1 and full > 1)
+    if dbias_sum_dims:
+        bias = bias.expand(batch if 0 in dbias_sum_dims else bias.size(0), k.size(2) if 1 in dbias_sum_dims else bias.size(1),
+                           -1, -1).contiguous()
+        dbias_final, dbias_w = dbias_w, torch.empty_like(bias)
+
     args = _cabi.BwdArgs()
     _cabi.fill_fwd(args.f, q, k, v, mask, bias, out, softmax_lse, softmax_scale, is_causal, softcap)
     args.dout = dout.data_ptr()
@@ -223,6 +235,9 @@ def _flash_sparse_attn_backward(
             for t in (dk_w, dv_w, dbias_w, softmax_d):
                 if t is not None:
                     t.zero_()
+    if dbias_sum_dims:
+        dbias_final.copy_(dbias_w.sum(dim=dbias_sum_dims, keepdim=True, dtype=torch.float32))
+        dbias_w = dbias_final
     for given, work in ((dq, dq_w), (dk, dk_w), (dv, dv_w), (dbias, dbias_w)):
         if given is not None and work is not given:
             given.copy_(work)
@@ -423,8 +438,10 @@ def flash_sparse_attn_func(
         softmax_scale: scaling of QK^T before the bias is added. Default 1 / sqrt(headdim).
         is_causal: apply the (bottom-right aligned) causal mask.
         softcap: must be None or 0 (soft-capping is not built).
-        deterministic: accepted; the backward pass never uses atomics on dQ/dK/dV and is
-            deterministic regardless.
+        deterministic: dQ, dK and dV never go through atomics and are bit-reproducible regardless.  dBias of a
+            bias that is broadcast over the batch (batch > 1) or shared by several kv heads is accumulated with
+            fp32 atomics unless this flag is set; with it, one slice per (batch entry, kv head) is written and
+            the slices are summed in a fixed order.
         return_attn_probs: also return (softmax_lse, S_dmask); S_dmask is an empty tensor.
     Return:
         out: (batch_size, seqlen, nheads, headdim).

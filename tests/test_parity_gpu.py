@@ -408,6 +408,32 @@ def test_direct_c_abi_call_without_the_python_operator():
     _check_lse(lse.cpu(), rl)
 
 
+@pytest.mark.parametrize("form", ["column_bias_batch_broadcast", "per_query_bias_one_head"])
+def test_deterministic_flag_with_shared_dbias(form):
+    """dBias elements shared by several workgroups (bias broadcast over the batch, or one bias head for several kv
+    heads) are summed in a fixed order when deterministic=True: reruns agree bit for bit, and the values match the
+    oracle like the default (atomic) path."""
+    if form == "column_bias_batch_broadcast":
+        q, k, v, mask, bias = make_inputs(3, 300, 300, 4, 2, 64, (1, 2, 1, 300), (3, 2, 1, 300), 100, seed=31)
+    else:
+        q, k, v, mask, bias = make_inputs(2, 200, 264, 4, 2, 64, (2, 1, 200, 264), (2, 1, 200, 264), 64, seed=32)
+    qd, kd, vd, md, bd = _to_dev(q, k, v, mask, bias)
+    runs = []
+    for _ in range(3):
+        qg, kg, vg, bg = [t.clone().requires_grad_(True) for t in (qd, kd, vd, bd)]
+        out = _op()(qg, kg, vg, md, bg, None, True, None, True)  # deterministic=True
+        out.backward(torch.ones_like(out))
+        torch.cuda.synchronize()
+        runs.append((qg.grad, kg.grad, vg.grad, bg.grad))
+    for other in runs[1:]:
+        for a, b in zip(runs[0], other):
+            assert torch.equal(a, b)
+    assert runs[0][3].shape == bias.shape
+    rdq, rdk, rdv, rdb = c_oracle.backward(q, k, v, torch.ones_like(q), mask, bias, None, True)
+    for g, r, n in zip(runs[0], (rdq, rdk, rdv, rdb), ("dq", "dk", "dv", "dbias")):
+        assert_grad_close(g.cpu(), r, n)
+
+
 def test_two_host_threads_on_two_streams():
     """The library keeps no mutable state besides a thread-local error string: two host threads, each on its own
     stream (default priority), run different problems at the same time and both get the single-threaded result."""
