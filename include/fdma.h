@@ -82,7 +82,7 @@ typedef struct fdma_bwd_args {
     int64_t do_strides[3], dq_strides[3], dk_strides[3], dv_strides[3];
     int64_t dbias_strides[3];
     float *softmax_d; /* out: rowsum(dO * O) */
-    /* Accepted for parity with mha_bwd (flash_api.cpp:812).  dq, dk, dv never depend on it: they are written without
+    /* Accepted for parity with mha_bwd (flash_api.cpp:809).  dq, dk, dv never depend on it: they are written without
      * atomics.  dbias elements that several (batch, kv head) pairs share -- bias strides[0] == 0 with batch > 1, or
      * num_heads_bias == 1 < num_heads_k -- are accumulated with fp32 atomics whatever this says; a caller that needs
      * them bit-reproducible passes a bias / dbias expanded over those dimensions and sums the slices itself, as the
