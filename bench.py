@@ -245,6 +245,40 @@ def run_mask_builder(steps, warmup, device):
     return res
 
 
+def run_bias_producer(steps, warmup, device):
+    """The bias producer in front of the operator (not part of `value`): flash_sparse_attn.utils.bias.dynamic_mask_bias
+    (one kernel forwards, two backwards) next to the tensor program of the reference's Doge caller
+    (examples/modeling/modeling_doge.py:217-222: linear, softplus, multiply, transpose, cast) for the value states of cfg2."""
+    import torch.nn.functional as F
+    from flash_sparse_attn.utils.bias import dynamic_mask_bias
+
+    c = CONFIGS["cfg2"]
+    g = torch.Generator().manual_seed(3)
+    K = c["Hk"] * c["D"]
+    v = torch.randn(c["B"], c["Lk"], c["Hk"], c["D"], generator=g).to(torch.bfloat16).to(device).requires_grad_(True)
+    w = (torch.randn(c["Hk"], K, generator=g) / K ** 0.5).to(torch.bfloat16).to(device).requires_grad_(True)
+    a = torch.ones(c["Hk"]).to(torch.bfloat16).to(device).requires_grad_(True)
+    gout = torch.randn(c["B"], c["Hk"], 1, c["Lk"], generator=g).to(torch.bfloat16).to(device)
+
+    def program(v_, w_, a_):
+        dt = F.linear(v_.reshape(c["B"], c["Lk"], -1), w_)
+        return (a_ * F.softplus(dt)).transpose(-1, -2).unsqueeze(-2).to(v_.dtype)
+
+    def fwd_bwd(fn):
+        def run():
+            fn(v, w, a).backward(gout)
+            v.grad = w.grad = a.grad = None
+        return run
+
+    res = {"shape": "cfg2 value states: %d x %d x %d x %d" % (c["B"], c["Lk"], c["Hk"], c["D"])}
+    with torch.no_grad():
+        res["us_fwd_kernel"] = 1e3 * time_gpu(lambda: dynamic_mask_bias(v, w, a), steps, warmup)
+        res["us_fwd_tensor_program"] = 1e3 * time_gpu(lambda: program(v, w, a), steps, warmup)
+    res["us_fwd_bwd_kernels"] = 1e3 * time_gpu(fwd_bwd(dynamic_mask_bias), steps, warmup)
+    res["us_fwd_bwd_tensor_program"] = 1e3 * time_gpu(fwd_bwd(program), steps, warmup)
+    return res
+
+
 def run_ragged_batch(steps, warmup, device):
     """flash_sparse_attn_varlen_func (no mask, no bias, causal) on a ragged batch of 16384 tokens, H=32, Hkv=8, d=128;
     FLOPs are the element-exact causal ones, 4 * d * H * sum(n * (n + 1) / 2)."""
@@ -387,6 +421,7 @@ def main():
         out["other_configs"] = [run_config(n, max(3, args.steps // 4), max(1, args.warmup // 2), device, compact)
                                 for n in ("cfg1", "cfg3", "cfg4", "cfg5")]
         out["mask_builder"] = run_mask_builder(max(3, args.steps // 2), max(1, args.warmup // 2), device)
+        out["bias_producer"] = run_bias_producer(max(3, args.steps // 2), max(1, args.warmup // 2), device)
         out["ragged_batch"] = run_ragged_batch(max(3, args.steps // 4), max(1, args.warmup // 2), device)
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline("cfg2", groups=8)

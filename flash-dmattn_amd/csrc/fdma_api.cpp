@@ -458,4 +458,72 @@ int fdma_create_mask(const fdma_mask_args *a, void *hip_stream) {
     return FDMA_OK;
 }
 
+size_t fdma_sizeof_dyn_bias_args(void) { return sizeof(fdma_dyn_bias_args); }
+
+int fdma_dyn_bias_validate(const fdma_dyn_bias_args *a, int backward) {
+    g_err[0] = 0;
+    if (!a) return fail(FDMA_ERR_INVALID, "args must not be NULL");
+    if (a->dtype != FDMA_DTYPE_BF16 && a->dtype != FDMA_DTYPE_FP16) return fail(FDMA_ERR_INVALID, "value states must be fp16 or bf16");
+    if (a->batch < 0 || a->seqlen_k < 0) return fail(FDMA_ERR_INVALID, "batch and seqlen_k must be non-negative");
+    if (a->num_heads_k <= 0 || a->num_heads_k > 32) return fail(FDMA_ERR_UNSUPPORTED, "the bias producer is built for 1 to 32 kv heads (got %d)", a->num_heads_k);
+    if (a->head_dim <= 0 || a->head_dim % 8 != 0 || (a->num_heads_k * a->head_dim) % 16 != 0)
+        return fail(FDMA_ERR_UNSUPPORTED, "head_dim must be a multiple of 8 and num_heads_k * head_dim a multiple of 16");
+    const bool empty = (int64_t)a->batch * a->seqlen_k == 0;
+    if (!a->weight || !a->a || (!empty && (!a->value || !a->bias || !a->dt))) return fail(FDMA_ERR_INVALID, "value, weight, a, bias, dt must be device pointers");
+    if (!aligned16(a->value) || !aligned16(a->weight) || !strides_ok(a->value_strides, 8))
+        return fail(FDMA_ERR_INVALID, "value and weight must be 16-byte aligned, value strides multiples of 8 elements");
+    if (backward) {
+        if (!a->dweight || !a->da || (!empty && (!a->dbias || !a->dvalue))) return fail(FDMA_ERR_INVALID, "dbias, dvalue, dweight, da must be device pointers");
+        if ((a->proj_bias != nullptr) != (a->dproj_bias != nullptr)) return fail(FDMA_ERR_INVALID, "dproj_bias must be given exactly when proj_bias is given");
+        if ((reinterpret_cast<uintptr_t>(a->dvalue) & 7) || a->dvalue_strides[0] % 4 || a->dvalue_strides[1] % 4 || a->dvalue_strides[2] % 4)
+            return fail(FDMA_ERR_INVALID, "dvalue must be 8-byte aligned with strides that are multiples of 4 elements");
+    }
+    return FDMA_OK;
+}
+
+static void fill_dyn_bias(const fdma_dyn_bias_args *a, fdma::DynBiasParams &p) {
+    std::memset(&p, 0, sizeof(p));
+    p.v = a->value; p.w = a->weight; p.pb = a->proj_bias; p.a = a->a;
+    p.bias = a->bias; p.dt = a->dt;
+    p.v_b = a->value_strides[0]; p.v_r = a->value_strides[1]; p.v_h = a->value_strides[2];
+    p.bias_b = a->bias_strides[0]; p.bias_h = a->bias_strides[1];
+    p.B = a->batch; p.L = a->seqlen_k; p.Hk = a->num_heads_k; p.d = a->head_dim;
+    p.dbias = a->dbias; p.dbias_b = a->dbias_strides[0]; p.dbias_h = a->dbias_strides[1];
+    p.dv = a->dvalue; p.dv_b = a->dvalue_strides[0]; p.dv_r = a->dvalue_strides[1]; p.dv_h = a->dvalue_strides[2];
+    p.dw = a->dweight; p.da = a->da; p.dpb = a->dproj_bias;
+    p.n_wg = fdma::dyn_bias_bwd_workgroups((int64_t)a->batch * a->seqlen_k, &p.rows_per_wg);
+    p.part_stride = round_up((int64_t)a->num_heads_k * a->num_heads_k * a->head_dim + 2 * a->num_heads_k, 4);
+}
+
+size_t fdma_dyn_bias_bwd_workspace_bytes(const fdma_dyn_bias_args *a) {
+    if (!a || (int64_t)a->batch * a->seqlen_k <= 0) return 0;
+    fdma::DynBiasParams p;
+    fill_dyn_bias(a, p);
+    return (size_t)p.n_wg * p.part_stride * sizeof(float);
+}
+
+int fdma_dyn_bias_fwd(const fdma_dyn_bias_args *a, void *hip_stream) {
+    int rc = fdma_dyn_bias_validate(a, 0);
+    if (rc != FDMA_OK) return rc;
+    fdma::DynBiasParams p;
+    fill_dyn_bias(a, p);
+    const hipError_t e = fdma::launch_dyn_bias_fwd(p, a->dtype, static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(FDMA_ERR_LAUNCH, "bias producer launch failed: %s", hipGetErrorString(e));
+    return FDMA_OK;
+}
+
+int fdma_dyn_bias_bwd(const fdma_dyn_bias_args *a, void *hip_stream) {
+    int rc = fdma_dyn_bias_validate(a, 1);
+    if (rc != FDMA_OK) return rc;
+    fdma::DynBiasParams p;
+    fill_dyn_bias(a, p);
+    const size_t need = fdma_dyn_bias_bwd_workspace_bytes(a);
+    if (need && (!a->workspace || a->workspace_bytes < need))
+        return fail(FDMA_ERR_WORKSPACE, "bias producer backward workspace too small: need %zu bytes, got %zu", need, a->workspace_bytes);
+    p.part = static_cast<float *>(a->workspace);
+    const hipError_t e = fdma::launch_dyn_bias_bwd(p, a->dtype, static_cast<hipStream_t>(hip_stream));
+    if (e != hipSuccess) return fail(FDMA_ERR_LAUNCH, "bias producer launch failed: %s", hipGetErrorString(e));
+    return FDMA_OK;
+}
+
 }  // extern "C"

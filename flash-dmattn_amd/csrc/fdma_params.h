@@ -166,6 +166,31 @@ struct MaskParams {
 };
 hipError_t launch_make_mask(const MaskParams &p, hipStream_t stream);
 
+// Bias producer (fdma_bias.hip): bias[b, j, 0, l] = A[j] * softplus(V_flat[b, l, :] . W[j, :] + pb[j]).
+struct DynBiasParams {
+    const void *v;        // (B, L, Hk, d): strides batch / row / head in elements, d contiguous
+    const void *w;        // (Hk, Hk * d) row-major
+    const void *pb;       // (Hk) or nullptr
+    const void *a;        // (Hk)
+    void *bias;           // out (forward): element (b, j, l) at b * bias_b + j * bias_h + l
+    float *dt;            // (B * L, Hk) fp32: written by forward, read by backward
+    int64_t v_b, v_r, v_h;
+    int64_t bias_b, bias_h;
+    int32_t B, L, Hk, d;
+    // backward
+    const void *dbias;    // (b, j, l) at b * dbias_b + j * dbias_h + l
+    int64_t dbias_b, dbias_h;
+    void *dv;             // (B, L, Hk, d), strides below
+    int64_t dv_b, dv_r, dv_h;
+    void *dw, *da, *dpb;  // (Hk, Hk * d), (Hk), (Hk) or nullptr
+    float *part;          // n_wg partials of part_stride floats: dW (Hk * Hk * d), dA (Hk), dpb (Hk)
+    int64_t part_stride;
+    int32_t n_wg, rows_per_wg;
+};
+hipError_t launch_dyn_bias_fwd(const DynBiasParams &p, int dtype, hipStream_t stream);
+hipError_t launch_dyn_bias_bwd(const DynBiasParams &p, int dtype, hipStream_t stream);
+int dyn_bias_bwd_workgroups(int64_t n_rows, int *rows_per_wg);
+
 // Dynamic-LDS limit of a kernel, raised once per device (and again only for a larger request) instead of on every
 // launch: one `static DynSmemLimit` per launch site.  Later launches make no runtime call besides the launch itself.
 struct DynSmemLimit {

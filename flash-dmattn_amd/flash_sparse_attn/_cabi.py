@@ -86,6 +86,20 @@ class MaskArgs(ctypes.Structure):
     ]
 
 
+class DynBiasArgs(ctypes.Structure):
+    _fields_ = [
+        ("value", ctypes.c_void_p), ("weight", ctypes.c_void_p), ("proj_bias", ctypes.c_void_p), ("a", ctypes.c_void_p),
+        ("bias", ctypes.c_void_p), ("dt", ctypes.c_void_p),
+        ("value_strides", ctypes.c_int64 * 3), ("bias_strides", ctypes.c_int64 * 2),
+        ("batch", ctypes.c_int32), ("seqlen_k", ctypes.c_int32), ("num_heads_k", ctypes.c_int32), ("head_dim", ctypes.c_int32),
+        ("dtype", ctypes.c_int32),
+        ("dbias", ctypes.c_void_p), ("dbias_strides", ctypes.c_int64 * 2),
+        ("dvalue", ctypes.c_void_p), ("dvalue_strides", ctypes.c_int64 * 3),
+        ("dweight", ctypes.c_void_p), ("da", ctypes.c_void_p), ("dproj_bias", ctypes.c_void_p),
+        ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
+    ]
+
+
 EXPORTS = (
     "fdma_fwd", "fdma_bwd", "fdma_fwd_workspace_bytes", "fdma_bwd_workspace_bytes",
     "fdma_fwd_validate", "fdma_bwd_validate", "fdma_last_error", "fdma_abi_version",
@@ -93,6 +107,8 @@ EXPORTS = (
     "fdma_varlen_fwd", "fdma_varlen_bwd", "fdma_varlen_fwd_validate", "fdma_varlen_bwd_validate",
     "fdma_sizeof_varlen_fwd_args", "fdma_sizeof_varlen_bwd_args",
     "fdma_create_mask", "fdma_create_mask_validate", "fdma_sizeof_mask_args",
+    "fdma_dyn_bias_fwd", "fdma_dyn_bias_bwd", "fdma_dyn_bias_bwd_workspace_bytes", "fdma_dyn_bias_validate",
+    "fdma_sizeof_dyn_bias_args",
 )
 
 
@@ -145,7 +161,16 @@ def _load() -> ctypes.CDLL:
     lib.fdma_create_mask_validate.argtypes = [ctypes.POINTER(MaskArgs)]
     lib.fdma_create_mask_validate.restype = ctypes.c_int
     lib.fdma_sizeof_mask_args.restype = ctypes.c_size_t
-    sizes = ((lib.fdma_sizeof_mask_args(), MaskArgs), (lib.fdma_sizeof_fwd_args(), FwdArgs), (lib.fdma_sizeof_bwd_args(), BwdArgs),
+    lib.fdma_dyn_bias_fwd.argtypes = [ctypes.POINTER(DynBiasArgs), ctypes.c_void_p]
+    lib.fdma_dyn_bias_fwd.restype = ctypes.c_int
+    lib.fdma_dyn_bias_bwd.argtypes = [ctypes.POINTER(DynBiasArgs), ctypes.c_void_p]
+    lib.fdma_dyn_bias_bwd.restype = ctypes.c_int
+    lib.fdma_dyn_bias_bwd_workspace_bytes.argtypes = [ctypes.POINTER(DynBiasArgs)]
+    lib.fdma_dyn_bias_bwd_workspace_bytes.restype = ctypes.c_size_t
+    lib.fdma_dyn_bias_validate.argtypes = [ctypes.POINTER(DynBiasArgs), ctypes.c_int]
+    lib.fdma_dyn_bias_validate.restype = ctypes.c_int
+    lib.fdma_sizeof_dyn_bias_args.restype = ctypes.c_size_t
+    sizes = ((lib.fdma_sizeof_dyn_bias_args(), DynBiasArgs), (lib.fdma_sizeof_mask_args(), MaskArgs), (lib.fdma_sizeof_fwd_args(), FwdArgs), (lib.fdma_sizeof_bwd_args(), BwdArgs),
              (lib.fdma_sizeof_varlen_fwd_args(), VarlenFwdArgs), (lib.fdma_sizeof_varlen_bwd_args(), VarlenBwdArgs))
     if any(n != ctypes.sizeof(t) for n, t in sizes):
         raise ImportError(f"{path}: argument block size differs from the Python mirror")

@@ -43,7 +43,7 @@
 extern "C" {
 #endif
 
-#define FDMA_ABI_VERSION 2 /* 2: fdma_varlen_* and fdma_create_mask added; everything of version 1 is unchanged */
+#define FDMA_ABI_VERSION 2 /* 2: fdma_varlen_*, fdma_create_mask and fdma_dyn_bias_* added; everything of version 1 is unchanged */
 
 enum { FDMA_DTYPE_BF16 = 0, FDMA_DTYPE_FP16 = 1 };
 
@@ -180,6 +180,40 @@ typedef struct fdma_mask_args {
 int fdma_create_mask(const fdma_mask_args *args, void *hip_stream);
 int fdma_create_mask_validate(const fdma_mask_args *args);
 size_t fdma_sizeof_mask_args(void);
+
+/*
+ * Producer of the dynamic-mask bias, fused:  bias[b, j, 0, l] = a[j] * softplus(value[b, l, :, :] . weight[j, :] + proj_bias[j])
+ * -- the `A * softplus(dt_proj(V))` in front of the attention call of the reference's Doge caller
+ * (examples/modeling/modeling_doge.py:217-222; there a chain of tensor-library calls, so this entry point has no
+ * counterpart in the reference's extension) -- and its backward, which takes the attention's dbias in the bias's own
+ * (batch, num_heads_k, 1, seqlen_k) shape and returns the gradients of value, weight, a and proj_bias.
+ *   value, dvalue : (batch, seqlen_k, num_heads_k, head_dim), strides {batch, row, head} in elements
+ *   weight, dweight : (num_heads_k, num_heads_k * head_dim), contiguous;  a, da, proj_bias, dproj_bias : (num_heads_k)
+ *   bias, dbias   : (batch, num_heads_k, 1, >= seqlen_k), strides {batch, head} in elements, key dimension contiguous
+ *   dt            : (batch * seqlen_k, num_heads_k) fp32, written by forward and read by backward
+ * All tensors have the dtype given; num_heads_k <= 32, head_dim % 8 == 0, (num_heads_k * head_dim) % 16 == 0.
+ * Backward needs fdma_dyn_bias_bwd_workspace_bytes() of scratch; its sums are folded in a fixed order (bit-reproducible).
+ */
+typedef struct fdma_dyn_bias_args {
+    const void *value, *weight, *proj_bias /* may be NULL */, *a;
+    void *bias;
+    float *dt;
+    int64_t value_strides[3], bias_strides[2];
+    int32_t batch, seqlen_k, num_heads_k, head_dim, dtype;
+    /* backward only */
+    const void *dbias;
+    int64_t dbias_strides[2];
+    void *dvalue;
+    int64_t dvalue_strides[3];
+    void *dweight, *da, *dproj_bias /* NULL iff proj_bias is NULL */;
+    void *workspace;
+    size_t workspace_bytes;
+} fdma_dyn_bias_args;
+int fdma_dyn_bias_fwd(const fdma_dyn_bias_args *args, void *hip_stream);
+int fdma_dyn_bias_bwd(const fdma_dyn_bias_args *args, void *hip_stream);
+size_t fdma_dyn_bias_bwd_workspace_bytes(const fdma_dyn_bias_args *args);
+int fdma_dyn_bias_validate(const fdma_dyn_bias_args *args, int backward);
+size_t fdma_sizeof_dyn_bias_args(void);
 
 /* Message of the last error raised on the calling thread ("" if none). */
 const char *fdma_last_error(void);

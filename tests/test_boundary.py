@@ -35,6 +35,7 @@ def test_struct_mirrors_match_compiled_sizes():
     assert _cabi.lib.fdma_sizeof_varlen_fwd_args() == ctypes.sizeof(_cabi.VarlenFwdArgs)
     assert _cabi.lib.fdma_sizeof_varlen_bwd_args() == ctypes.sizeof(_cabi.VarlenBwdArgs)
     assert _cabi.lib.fdma_sizeof_mask_args() == ctypes.sizeof(_cabi.MaskArgs)
+    assert _cabi.lib.fdma_sizeof_dyn_bias_args() == ctypes.sizeof(_cabi.DynBiasArgs)
 
 
 def _valid_fwd():
@@ -297,3 +298,33 @@ def test_mask_builder_validation():
         setattr(a, field, value)
         assert _cabi.lib.fdma_create_mask_validate(a) < 0, field
         assert message in _cabi.last_error()
+
+
+def test_bias_producer_validation_and_workspace():
+    """Argument rules of fdma_dyn_bias_* (the producer behind flash_sparse_attn.utils.bias), checked without a GPU."""
+    from flash_sparse_attn import _cabi
+
+    def good():
+        a = _cabi.DynBiasArgs()
+        for name in ("value", "weight", "a", "bias", "dt", "dbias", "dvalue", "dweight", "da"):
+            setattr(a, name, 0x1000)
+        a.batch, a.seqlen_k, a.num_heads_k, a.head_dim, a.dtype = 2, 1000, 8, 128, 0
+        a.value_strides[:] = (1000 * 1024, 1024, 128)
+        a.dvalue_strides[:] = (1000 * 1024, 1024, 128)
+        a.bias_strides[:] = (8 * 1000, 1000)
+        a.dbias_strides[:] = (8 * 1000, 1000)
+        return a
+
+    assert _cabi.lib.fdma_dyn_bias_validate(good(), 0) == 0, _cabi.last_error()
+    assert _cabi.lib.fdma_dyn_bias_validate(good(), 1) == 0, _cabi.last_error()
+    # 2000 tokens -> 32 workgroups of 64 tokens, each with Hk * Hk * d + 2 * Hk fp32 partial sums
+    assert _cabi.lib.fdma_dyn_bias_bwd_workspace_bytes(good()) == 32 * (8 * 8 * 128 + 16) * 4
+    for field, value, backward, message in (("dtype", 5, 0, "fp16 or bf16"), ("num_heads_k", 33, 0, "1 to 32 kv heads"),
+                                            ("head_dim", 12, 0, "multiple of 8"), ("weight", 0, 0, "device pointers"),
+                                            ("value", 0x1008, 0, "16-byte aligned"), ("dweight", 0, 1, "device pointers"),
+                                            ("dproj_bias", 0x1000, 1, "exactly when proj_bias"),
+                                            ("dvalue", 0x1004, 1, "8-byte aligned")):
+        a = good()
+        setattr(a, field, value)
+        assert _cabi.lib.fdma_dyn_bias_validate(a, backward) < 0, field
+        assert message in _cabi.last_error(), (field, _cabi.last_error())
