@@ -5,7 +5,7 @@
 // call, and the same again backwards.  The column-summed dBias that the attention backward returns in the bias's own
 // [B, Hkv, 1, Lk] shape is consumed here directly.
 //
-// Forward: one wave owns 32 tokens.  V rows are the A operand and W rows the B operand of MFMA 32x32x16, both straight
+// Forward: a workgroup owns 32 tokens, each of its four waves a quarter of the columns.  V rows are the A operand and W rows the B operand of MFMA 32x32x16, both straight
 // from global memory (every lane reads 16 contiguous bytes of its own row per step: no LDS, no transposes); the
 // accumulator column of lane j < Hkv holds dt of 16 of the tokens, finished in place.  HBM traffic is one read of V.
 // Backward: a workgroup owns a run of tokens; d_dt = dBias * A * sigmoid(dt) goes to LDS, then a thread owns four
@@ -20,13 +20,16 @@ namespace {
 __device__ __forceinline__ float softplus_f(float x) { return x > 20.f ? x : log1pf(__expf(x)); }  // torch: beta 1, threshold 20
 __device__ __forceinline__ float sigmoid_f(float x) { return x > 20.f ? 1.f : 1.f / (1.f + __expf(-x)); }  // d softplus / dx, same threshold
 
-template <typename T>
+// SPLITK: the four waves of a workgroup share 32 tokens, a quarter of the columns each (few tokens: more waves in
+// flight); otherwise every wave owns 32 tokens of its own and reads whole rows.
+template <typename T, bool SPLITK>
 __global__ void __launch_bounds__(256) dyn_bias_fwd_kernel(const DynBiasParams p) {
     using E = Elem<T>;
+    __shared__ float s_acc[SPLITK ? 3 : 1][16][64];
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, r = lane & 31, g = lane >> 5;
     const int64_t n_rows = (int64_t)p.B * p.L;
-    const int64_t row0 = ((int64_t)blockIdx.x * 4 + wave) * 32;
-    if (row0 >= n_rows) return;
+    const int64_t row0 = SPLITK ? (int64_t)blockIdx.x * 32 : ((int64_t)blockIdx.x * 4 + wave) * 32;
+    if (!SPLITK && row0 >= n_rows) return;  // (no barrier on this path)
     const int K = p.Hk * p.d;
     int64_t row = row0 + r;
     if (row >= n_rows) row = n_rows - 1;  // clamped duplicate, never stored
@@ -41,25 +44,34 @@ __global__ void __launch_bounds__(256) dyn_bias_fwd_kernel(const DynBiasParams p
     // second half of a line is asked for a trip later, when the line may have left the caches again), and all loads
     // of a trip are issued before its first MFMA
     constexpr int KU = 8;
-    const int n_ks = K / 16;
-    for (int ks0 = 0; ks0 < n_ks; ks0 += KU) {
+    const int n_ks = K / 16, per_wave = SPLITK ? ((n_ks + 3) / 4 + KU - 1) / KU * KU : n_ks;
+    const int ks_begin = SPLITK ? wave * per_wave : 0;
+    const int ks_end = ks_begin + per_wave < n_ks ? ks_begin + per_wave : n_ks;
+    for (int ks0 = ks_begin; ks0 < ks_end; ks0 += KU) {
         u32x4_t a[KU], bw[KU];
 #pragma unroll
         for (int u = 0; u < KU; u++) {
-            const int ks = ks0 + u < n_ks ? ks0 + u : n_ks - 1;  // (a short last trip re-reads the last step and drops it)
+            const int ks = ks0 + u < ks_end ? ks0 + u : ks_end - 1;  // (a short last trip re-reads the last step and drops it)
             const int kk = ks * 16 + 8 * g, head = kk / p.d, dd = kk - head * p.d;
             a[u] = *(const u32x4_t *)(vrow + (int64_t)head * p.v_h + dd);
             bw[u] = *(const u32x4_t *)(wrow + kk);
         }
 #pragma unroll
         for (int u = 0; u < KU; u++) {
-            const uint32_t m = (ks0 + u < n_ks) ? wmask : 0u;
+            const uint32_t m = (ks0 + u < ks_end) ? wmask : 0u;
 #pragma unroll
             for (int e = 0; e < 4; e++) bw[u][e] &= m;
             acc = E::mfma(a[u], bw[u], acc);
         }
     }
-    if (r < p.Hk) {
+    if (SPLITK) {
+        if (wave > 0) {
+#pragma unroll
+            for (int i = 0; i < 16; i++) s_acc[wave - 1][i][lane] = acc[i];
+        }
+        __syncthreads();
+    }
+    if ((!SPLITK || wave == 0) && r < p.Hk) {
         const float a_j = E::lo((uint32_t)((const uint16_t *)p.a)[r]);
         const float pb_j = p.pb ? E::lo((uint32_t)((const uint16_t *)p.pb)[r]) : 0.f;
 #pragma unroll
@@ -67,7 +79,9 @@ __global__ void __launch_bounds__(256) dyn_bias_fwd_kernel(const DynBiasParams p
             const int64_t rr = row0 + 8 * (i / 4) + 4 * g + (i % 4);  // accumulator register i: this tile row, column r
             if (rr < n_rows) {
                 const int bb = (int)(rr / p.L), ll = (int)(rr % p.L);
-                const float dt = acc[i] + pb_j;
+                float dt = acc[i];
+                if (SPLITK) dt = ((dt + s_acc[0][i][lane]) + s_acc[1][i][lane]) + s_acc[2][i][lane];
+                dt += pb_j;
                 p.dt[rr * p.Hk + r] = dt;
                 ((uint16_t *)p.bias)[bb * p.bias_b + (int64_t)r * p.bias_h + ll] = (uint16_t)(E::pack2(a_j * softplus_f(dt), 0.f) & 0xffffu);
             }
@@ -205,7 +219,8 @@ __global__ void __launch_bounds__(256) dyn_bias_reduce_kernel(const DynBiasParam
     const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (e >= per) return;
     float s = 0.f;
-    for (int c = 0; c < p.n_wg; c++) s += p.part[c * p.part_stride + e];
+#pragma unroll 8
+    for (int c = 0; c < p.n_wg; c++) s += p.part[c * p.part_stride + e];  // (independent loads, one chain of additions)
     const uint16_t out = (uint16_t)(E::pack2(s, 0.f) & 0xffffu);
     if (e < (int64_t)Hk * K) ((uint16_t *)p.dw)[e] = out;
     else if (e < (int64_t)Hk * K + Hk) ((uint16_t *)p.da)[e - (int64_t)Hk * K] = out;
@@ -217,17 +232,26 @@ __global__ void __launch_bounds__(256) dyn_bias_reduce_kernel(const DynBiasParam
 hipError_t launch_dyn_bias_fwd(const DynBiasParams &p, int dtype, hipStream_t stream) {
     const int64_t n_rows = (int64_t)p.B * p.L;
     if (n_rows <= 0) return hipSuccess;
-    const dim3 grid((unsigned)((n_rows + 127) / 128));
-    if (dtype == 0) hipLaunchKernelGGL(dyn_bias_fwd_kernel<bf16_tag>, grid, dim3(256), 0, stream, p);
-    else hipLaunchKernelGGL(dyn_bias_fwd_kernel<fp16_tag>, grid, dim3(256), 0, stream, p);
+    if (n_rows < 131072) {  // fewer than 4096 token tiles: split the columns over the waves as well
+        const dim3 grid((unsigned)((n_rows + 31) / 32));
+        if (dtype == 0) hipLaunchKernelGGL((dyn_bias_fwd_kernel<bf16_tag, true>), grid, dim3(256), 0, stream, p);
+        else hipLaunchKernelGGL((dyn_bias_fwd_kernel<fp16_tag, true>), grid, dim3(256), 0, stream, p);
+    } else {
+        const dim3 grid((unsigned)((n_rows + 127) / 128));
+        if (dtype == 0) hipLaunchKernelGGL((dyn_bias_fwd_kernel<bf16_tag, false>), grid, dim3(256), 0, stream, p);
+        else hipLaunchKernelGGL((dyn_bias_fwd_kernel<fp16_tag, false>), grid, dim3(256), 0, stream, p);
+    }
     return hipGetLastError();
 }
 
 int dyn_bias_bwd_workgroups(int64_t n_rows, int *rows_per_wg) {
-    // runs of whole 64-token passes, at most 512 workgroups (the partials are Hkv * Hkv * d floats each)
-    int64_t rows = (n_rows + 511) / 512;
-    rows = (rows + 63) / 64 * 64;
-    if (rows < 64) rows = 64;
+    // runs of 32 tokens while that gives at most 512 workgroups (the partials are Hkv * Hkv * d floats each), else
+    // longer runs of whole 64-token passes
+    int64_t rows = 32;
+    if ((n_rows + 31) / 32 > 512) {
+        rows = (n_rows + 511) / 512;
+        rows = (rows + 63) / 64 * 64;
+    }
     *rows_per_wg = (int)rows;
     return (int)((n_rows + rows - 1) / rows);
 }

@@ -317,8 +317,8 @@ def test_bias_producer_validation_and_workspace():
 
     assert _cabi.lib.fdma_dyn_bias_validate(good(), 0) == 0, _cabi.last_error()
     assert _cabi.lib.fdma_dyn_bias_validate(good(), 1) == 0, _cabi.last_error()
-    # 2000 tokens -> 32 workgroups of 64 tokens, each with Hk * Hk * d + 2 * Hk fp32 partial sums
-    assert _cabi.lib.fdma_dyn_bias_bwd_workspace_bytes(good()) == 32 * (8 * 8 * 128 + 16) * 4
+    # 2000 tokens -> 63 workgroups of 32 tokens, each with Hk * Hk * d + 2 * Hk fp32 partial sums
+    assert _cabi.lib.fdma_dyn_bias_bwd_workspace_bytes(good()) == 63 * (8 * 8 * 128 + 16) * 4
     for field, value, backward, message in (("dtype", 5, 0, "fp16 or bf16"), ("num_heads_k", 33, 0, "1 to 32 kv heads"),
                                             ("head_dim", 12, 0, "multiple of 8"), ("weight", 0, 0, "device pointers"),
                                             ("value", 0x1008, 0, "16-byte aligned"), ("dweight", 0, 1, "device pointers"),
