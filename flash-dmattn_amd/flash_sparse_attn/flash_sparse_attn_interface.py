@@ -90,15 +90,8 @@ def _check_inputs(q, k, v, mask, bias) -> None:
 
 @torch.library.custom_op("flash_sparse_attn::_flash_sparse_attn_forward", mutates_args=(), device_types="cuda")
 def _flash_sparse_attn_forward(
-    q: torch.Tensor,
-    k: torch.Tensor,
-    v: torch.Tensor,
-    mask: Optional[torch.Tensor],
-    bias: Optional[torch.Tensor],
-    softmax_scale: float,
-    is_causal: bool,
-    softcap: float,
-    return_softmax: bool,
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Optional[torch.Tensor], bias: Optional[torch.Tensor],
+    softmax_scale: float, is_causal: bool, softcap: float, return_softmax: bool,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     _check_inputs(q, k, v, mask, bias)
     q, k, v = [_aligned(x, 8) for x in (q, k, v)]
@@ -126,15 +119,8 @@ def _flash_sparse_attn_forward(
 
 @torch.library.register_fake("flash_sparse_attn::_flash_sparse_attn_forward")
 def _flash_sparse_attn_forward_fake(
-    q: torch.Tensor,
-    k: torch.Tensor,
-    v: torch.Tensor,
-    mask: Optional[torch.Tensor],
-    bias: Optional[torch.Tensor],
-    softmax_scale: float,
-    is_causal: bool,
-    softcap: float,
-    return_softmax: bool,
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Optional[torch.Tensor], bias: Optional[torch.Tensor],
+    softmax_scale: float, is_causal: bool, softcap: float, return_softmax: bool,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     batch_size, seqlen_q, num_heads, _ = q.shape
     out = torch.empty_like(q, memory_format=torch.contiguous_format)
@@ -150,22 +136,10 @@ _wrapped_flash_sparse_attn_forward = _flash_sparse_attn_forward
     "flash_sparse_attn::_flash_sparse_attn_backward", mutates_args=("dq", "dk", "dv", "dbias"), device_types="cuda"
 )
 def _flash_sparse_attn_backward(
-    dout: torch.Tensor,
-    q: torch.Tensor,
-    k: torch.Tensor,
-    v: torch.Tensor,
-    mask: Optional[torch.Tensor],
-    bias: Optional[torch.Tensor],
-    out: torch.Tensor,
-    softmax_lse: torch.Tensor,
-    dq: Optional[torch.Tensor],
-    dk: Optional[torch.Tensor],
-    dv: Optional[torch.Tensor],
-    dbias: Optional[torch.Tensor],
-    softmax_scale: float,
-    is_causal: bool,
-    softcap: float,
-    deterministic: bool,
+    dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Optional[torch.Tensor], bias:
+    Optional[torch.Tensor], out: torch.Tensor, softmax_lse: torch.Tensor, dq: Optional[torch.Tensor], dk:
+    Optional[torch.Tensor], dv: Optional[torch.Tensor], dbias: Optional[torch.Tensor], softmax_scale: float,
+    is_causal: bool, softcap: float, deterministic: bool,
 ) -> torch.Tensor:
     _check_inputs(q, k, v, mask, bias)
     if out.dtype != q.dtype:
@@ -246,22 +220,10 @@ def _flash_sparse_attn_backward(
 
 @torch.library.register_fake("flash_sparse_attn::_flash_sparse_attn_backward")
 def _flash_sparse_attn_backward_fake(
-    dout: torch.Tensor,
-    q: torch.Tensor,
-    k: torch.Tensor,
-    v: torch.Tensor,
-    mask: Optional[torch.Tensor],
-    bias: Optional[torch.Tensor],
-    out: torch.Tensor,
-    softmax_lse: torch.Tensor,
-    dq: Optional[torch.Tensor],
-    dk: Optional[torch.Tensor],
-    dv: Optional[torch.Tensor],
-    dbias: Optional[torch.Tensor],
-    softmax_scale: float,
-    is_causal: bool,
-    softcap: float,
-    deterministic: bool,
+    dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Optional[torch.Tensor], bias:
+    Optional[torch.Tensor], out: torch.Tensor, softmax_lse: torch.Tensor, dq: Optional[torch.Tensor], dk:
+    Optional[torch.Tensor], dv: Optional[torch.Tensor], dbias: Optional[torch.Tensor], softmax_scale: float,
+    is_causal: bool, softcap: float, deterministic: bool,
 ) -> torch.Tensor:
     batch_size, seqlen_q, num_heads, _ = q.shape
     return torch.empty((batch_size, num_heads, round_multiple(seqlen_q, 128)), device=q.device, dtype=torch.float32)
@@ -287,17 +249,9 @@ class FlashDMAttnFunc(torch.autograd.Function):
 
     @staticmethod
     def forward(
-        ctx: torch.autograd.function.FunctionCtx,
-        q: torch.Tensor,
-        k: torch.Tensor,
-        v: torch.Tensor,
-        mask: Optional[torch.Tensor],
-        bias: Optional[torch.Tensor],
-        softmax_scale: Optional[float],
-        is_causal: Optional[bool],
-        softcap: Optional[float],
-        deterministic: Optional[bool],
-        return_softmax: Optional[bool],
+        ctx: torch.autograd.function.FunctionCtx, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask:
+        Optional[torch.Tensor], bias: Optional[torch.Tensor], softmax_scale: Optional[float], is_causal:
+        Optional[bool], softcap: Optional[float], deterministic: Optional[bool], return_softmax: Optional[bool],
         is_grad_enabled: bool = True,
     ):
         is_grad = is_grad_enabled and any(x.requires_grad for x in [q, k, v])
@@ -323,15 +277,7 @@ class FlashDMAttnFunc(torch.autograd.Function):
         bias = _pad_key_dim(bias, k.shape[1], 8)
 
         out_padded, softmax_lse, S_dmask = _wrapped_flash_sparse_attn_forward(
-            q,
-            k,
-            v,
-            mask,
-            bias,
-            softmax_scale,
-            is_causal=is_causal,
-            softcap=softcap,
-            return_softmax=return_softmax,
+            q, k, v, mask, bias, softmax_scale, is_causal=is_causal, softcap=softcap, return_softmax=return_softmax,
         )
 
         if is_grad:
@@ -365,22 +311,8 @@ class FlashDMAttnFunc(torch.autograd.Function):
             dout_padded = torch.nn.functional.pad(dout, [0, 8 - head_size_og % 8])
 
         _wrapped_flash_sparse_attn_backward(
-            dout_padded,
-            q,
-            k,
-            v,
-            mask,
-            bias,
-            out,
-            softmax_lse,
-            dq,
-            dk,
-            dv,
-            dbias,
-            ctx.softmax_scale,
-            ctx.is_causal,
-            ctx.softcap,
-            ctx.deterministic,
+            dout_padded, q, k, v, mask, bias, out, softmax_lse, dq, dk, dv, dbias, ctx.softmax_scale, ctx.is_causal,
+            ctx.softcap, ctx.deterministic,
         )
 
         # We could have padded the head dimension
@@ -399,16 +331,9 @@ class FlashDMAttnFunc(torch.autograd.Function):
 
 
 def flash_sparse_attn_func(
-    query: torch.Tensor,
-    key: torch.Tensor,
-    value: torch.Tensor,
-    attn_mask: Optional[torch.Tensor] = None,
-    attn_bias: Optional[torch.Tensor] = None,
-    softmax_scale: Optional[float] = None,
-    is_causal: Optional[bool] = None,
-    softcap: Optional[float] = None,
-    deterministic: Optional[bool] = None,
-    return_attn_probs: Optional[bool] = None,
+    query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, attn_mask: Optional[torch.Tensor] = None, attn_bias:
+    Optional[torch.Tensor] = None, softmax_scale: Optional[float] = None, is_causal: Optional[bool] = None, softcap:
+    Optional[float] = None, deterministic: Optional[bool] = None, return_attn_probs: Optional[bool] = None,
 ):
     """Dynamic-mask attention with MQA/GQA: K, V may have fewer heads than Q (the number of Q heads
     must be divisible by the number of KV heads; Q head h attends to KV head h // (H // Hkv)).
@@ -491,21 +416,10 @@ def _check_varlen_inputs(q, k, v, cu_seqlens_q, cu_seqlens_k) -> None:
 
 @torch.library.custom_op("flash_sparse_attn::_flash_sparse_attn_varlen_forward", mutates_args=(), device_types="cuda")
 def _flash_sparse_attn_varlen_forward(
-    q: torch.Tensor,
-    k: torch.Tensor,
-    v: torch.Tensor,
-    cu_seqlens_q: torch.Tensor,
-    cu_seqlens_k: torch.Tensor,
-    max_seqlen_q: int,
-    max_seqlen_k: int,
-    softmax_scale: float,
-    is_causal: bool,
-    softcap: float = 0.0,
-    return_softmax: bool = False,
-    block_table: Optional[torch.Tensor] = None,
-    leftpad_k: Optional[torch.Tensor] = None,
-    seqused_k: Optional[torch.Tensor] = None,
-    zero_tensors: bool = False,
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor,
+    max_seqlen_q: int, max_seqlen_k: int, softmax_scale: float, is_causal: bool, softcap: float = 0.0, return_softmax:
+    bool = False, block_table: Optional[torch.Tensor] = None, leftpad_k: Optional[torch.Tensor] = None, seqused_k:
+    Optional[torch.Tensor] = None, zero_tensors: bool = False,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     """Ragged-batch forward (interface.py:129-167 of the reference).  Rows of `out` / `softmax_lse` that belong to
     no sequence (beyond cu_seqlens_q[-1]) are zero-filled when `zero_tensors` is set and left unwritten otherwise."""
@@ -531,21 +445,10 @@ def _flash_sparse_attn_varlen_forward(
 
 @torch.library.register_fake("flash_sparse_attn::_flash_sparse_attn_varlen_forward")
 def _flash_sparse_attn_varlen_forward_fake(
-    q: torch.Tensor,
-    k: torch.Tensor,
-    v: torch.Tensor,
-    cu_seqlens_q: torch.Tensor,
-    cu_seqlens_k: torch.Tensor,
-    max_seqlen_q: int,
-    max_seqlen_k: int,
-    softmax_scale: float,
-    is_causal: bool,
-    softcap: float = 0.0,
-    return_softmax: bool = False,
-    block_table: Optional[torch.Tensor] = None,
-    leftpad_k: Optional[torch.Tensor] = None,
-    seqused_k: Optional[torch.Tensor] = None,
-    zero_tensors: bool = False,
+    q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor,
+    max_seqlen_q: int, max_seqlen_k: int, softmax_scale: float, is_causal: bool, softcap: float = 0.0, return_softmax:
+    bool = False, block_table: Optional[torch.Tensor] = None, leftpad_k: Optional[torch.Tensor] = None, seqused_k:
+    Optional[torch.Tensor] = None, zero_tensors: bool = False,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     total_q, num_heads, _ = q.shape
     out = torch.empty_like(q, memory_format=torch.contiguous_format)
@@ -561,24 +464,10 @@ _wrapped_flash_sparse_attn_varlen_forward = _flash_sparse_attn_varlen_forward
     "flash_sparse_attn::_flash_sparse_attn_varlen_backward", mutates_args=("dq", "dk", "dv"), device_types="cuda"
 )
 def _flash_sparse_attn_varlen_backward(
-    dout: torch.Tensor,
-    q: torch.Tensor,
-    k: torch.Tensor,
-    v: torch.Tensor,
-    out: torch.Tensor,
-    softmax_lse: torch.Tensor,
-    dq: Optional[torch.Tensor],
-    dk: Optional[torch.Tensor],
-    dv: Optional[torch.Tensor],
-    cu_seqlens_q: torch.Tensor,
-    cu_seqlens_k: torch.Tensor,
-    max_seqlen_q: int,
-    max_seqlen_k: int,
-    softmax_scale: float,
-    is_causal: bool,
-    softcap: float,
-    deterministic: bool,
-    zero_tensors: bool = False,
+    dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, softmax_lse:
+    torch.Tensor, dq: Optional[torch.Tensor], dk: Optional[torch.Tensor], dv: Optional[torch.Tensor], cu_seqlens_q:
+    torch.Tensor, cu_seqlens_k: torch.Tensor, max_seqlen_q: int, max_seqlen_k: int, softmax_scale: float, is_causal:
+    bool, softcap: float, deterministic: bool, zero_tensors: bool = False,
 ) -> torch.Tensor:
     """Ragged-batch backward (interface.py:291-339 of the reference).  Gradient rows that belong to no sequence are
     zero-filled when `zero_tensors` is set and left unwritten otherwise (flash_api.cpp:1209-1214)."""
@@ -630,24 +519,10 @@ def _flash_sparse_attn_varlen_backward(
 
 @torch.library.register_fake("flash_sparse_attn::_flash_sparse_attn_varlen_backward")
 def _flash_sparse_attn_varlen_backward_fake(
-    dout: torch.Tensor,
-    q: torch.Tensor,
-    k: torch.Tensor,
-    v: torch.Tensor,
-    out: torch.Tensor,
-    softmax_lse: torch.Tensor,
-    dq: Optional[torch.Tensor],
-    dk: Optional[torch.Tensor],
-    dv: Optional[torch.Tensor],
-    cu_seqlens_q: torch.Tensor,
-    cu_seqlens_k: torch.Tensor,
-    max_seqlen_q: int,
-    max_seqlen_k: int,
-    softmax_scale: float,
-    is_causal: bool,
-    softcap: float,
-    deterministic: bool,
-    zero_tensors: bool = False,
+    dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, softmax_lse:
+    torch.Tensor, dq: Optional[torch.Tensor], dk: Optional[torch.Tensor], dv: Optional[torch.Tensor], cu_seqlens_q:
+    torch.Tensor, cu_seqlens_k: torch.Tensor, max_seqlen_q: int, max_seqlen_k: int, softmax_scale: float, is_causal:
+    bool, softcap: float, deterministic: bool, zero_tensors: bool = False,
 ) -> torch.Tensor:
     total_q, num_heads, _ = q.shape
     return torch.empty((num_heads, total_q), device=q.device, dtype=torch.float32)
@@ -662,21 +537,10 @@ class FlashAttnVarlenFunc(torch.autograd.Function):
 
     @staticmethod
     def forward(
-        ctx,
-        q: torch.Tensor,
-        k: torch.Tensor,
-        v: torch.Tensor,
-        cu_seqlens_q: torch.Tensor,
-        cu_seqlens_k: torch.Tensor,
-        max_seqlen_q: int,
-        max_seqlen_k: int,
-        softmax_scale: Optional[float],
-        is_causal: Optional[bool],
-        softcap: Optional[float],
-        deterministic: Optional[bool],
-        return_softmax: Optional[bool],
-        block_table: Optional[torch.Tensor],
-        is_grad_enabled: bool = True,
+        ctx, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: torch.Tensor, cu_seqlens_k:
+        torch.Tensor, max_seqlen_q: int, max_seqlen_k: int, softmax_scale: Optional[float], is_causal: Optional[bool],
+        softcap: Optional[float], deterministic: Optional[bool], return_softmax: Optional[bool], block_table:
+        Optional[torch.Tensor], is_grad_enabled: bool = True,
     ):
         is_grad = is_grad_enabled and any(x.requires_grad for x in [q, k, v])
         if softmax_scale is None:
@@ -725,19 +589,10 @@ class FlashAttnVarlenFunc(torch.autograd.Function):
 
 
 def flash_sparse_attn_varlen_func(
-    query: torch.Tensor,
-    key: torch.Tensor,
-    value: torch.Tensor,
-    cu_seqlens_q: torch.Tensor,
-    cu_seqlens_k: torch.Tensor,
-    max_seqlen_q: int,
-    max_seqlen_k: int,
-    softmax_scale: Optional[float] = None,
-    is_causal: Optional[bool] = None,
-    softcap: Optional[float] = None,
-    deterministic: Optional[bool] = None,
-    return_attn_probs: Optional[bool] = None,
-    block_table: Optional[torch.Tensor] = None,
+    query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, cu_seqlens_q: torch.Tensor, cu_seqlens_k:
+    torch.Tensor, max_seqlen_q: int, max_seqlen_k: int, softmax_scale: Optional[float] = None, is_causal:
+    Optional[bool] = None, softcap: Optional[float] = None, deterministic: Optional[bool] = None, return_attn_probs:
+    Optional[bool] = None, block_table: Optional[torch.Tensor] = None,
 ):
     """Ragged-batch ("varlen") attention without mask or bias, signature and semantics of the reference's
     `flash_sparse_attn_varlen_func` (interface.py:687-760).
