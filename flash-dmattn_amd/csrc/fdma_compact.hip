@@ -199,19 +199,29 @@ __global__ void __launch_bounds__(256) compact_zero_kernel(const BwdParams p, co
 // One workgroup: prefix of 128-key units over the pairs and the split the dK/dV kernel will use.
 __global__ void __launch_bounds__(256) compact_plan_kernel(const int32_t *count, const int32_t *idx, int ld, int32_t *plan,
                                                             int pairs, int G, int Lq, int Lk, int causal) {
-    __shared__ int s_sum, s_max;
+    __shared__ int s_sum, s_max, s_n[256], s_units;
     const int tid = threadIdx.x;
-    if (tid == 0) {
-        int u = 0, n_max = 0;
-        for (int i = 0; i < pairs; i++) {
-            plan[DKDV_PLAN_HDR + i] = u;
-            const int n = (count[i] + 127) / 128;
-            u += n;
-            n_max = n > n_max ? n : n_max;
+    // units per pair and their prefix: the counts are fetched 256 at a time by all threads (one memory latency per
+    // chunk instead of one per pair), the prefix over a chunk is then taken from LDS by one thread
+    int u = 0, n_max = 0;  // (meaningful in thread 0)
+    for (int base = 0; base < pairs; base += 256) {
+        if (base + tid < pairs) s_n[tid] = (count[base + tid] + 127) / 128;
+        __syncthreads();
+        if (tid == 0) {
+            const int m = pairs - base < 256 ? pairs - base : 256;
+            for (int i = 0; i < m; i++) {
+                plan[DKDV_PLAN_HDR + base + i] = u;
+                u += s_n[i];
+                n_max = s_n[i] > n_max ? s_n[i] : n_max;
+            }
         }
+        __syncthreads();
+    }
+    if (tid == 0) {
         plan[DKDV_PLAN_HDR + pairs] = u;
         plan[0] = u;
         plan[3] = dkdv_list_len(n_max, dkdv_lists_per_pair(pairs));
+        s_units = u;
         s_sum = 0;
         s_max = 0;
     }
@@ -219,7 +229,7 @@ __global__ void __launch_bounds__(256) compact_plan_kernel(const int32_t *count,
     // query blocks per unit: their sum sizes the parts, their maximum the number of segment slots
     int sum = 0, mx = 0;
     for (int i = 0; i < pairs; i++) {
-        const int n = (count[i] + 127) / 128;
+        const int n = pairs <= 256 ? s_n[i] : (count[i] + 127) / 128;  // (up to 256 pairs the counts are still in LDS)
         for (int u = tid; u < n; u += 256) {
             const int nt = dkdv_query_blocks(Lq, Lk, causal, idx[(size_t)i * ld + u * 128]);
             sum += nt;
@@ -231,7 +241,7 @@ __global__ void __launch_bounds__(256) compact_plan_kernel(const int32_t *count,
     __syncthreads();
     if (tid == 0) {
         int Gs, Sm;
-        dkdv_split(plan[0], G, Gs, Sm);
+        dkdv_split(s_units, G, Gs, Sm);
         int Q = 1 << 30;
         if (Sm > 1) {
             const int64_t even = ((int64_t)G * s_sum + DKDV_TARGET_PARTS - 1) / DKDV_TARGET_PARTS;
