@@ -328,3 +328,33 @@ def test_bias_producer_validation_and_workspace():
         setattr(a, field, value)
         assert _cabi.lib.fdma_dyn_bias_validate(a, backward) < 0, field
         assert message in _cabi.last_error(), (field, _cabi.last_error())
+
+
+def test_missing_library_fails_loudly():
+    """Without libfdma_hip.so there is nothing to fall back to: the operator module refuses to import, the package reports
+    no backend (as the reference does without its extension), and asking for one raises."""
+    import subprocess
+    import sys
+
+    code = r'''
+import importlib, sys
+sys.path.insert(0, sys.argv[1])
+try:
+    importlib.import_module("flash_sparse_attn.flash_sparse_attn_interface")
+    print("IMPORTED")
+except ImportError as e:
+    print("ImportError:", e)
+import flash_sparse_attn as pkg
+print("CUDA_AVAILABLE", pkg.CUDA_AVAILABLE, pkg.flash_sparse_attn_func, pkg.get_available_backends())
+try:
+    pkg.flash_sparse_attn_func_auto()
+    print("RETURNED")
+except RuntimeError as e:
+    print("RuntimeError:", e)
+'''
+    env = dict(os.environ, FDMA_LIB="/nonexistent/libfdma_hip.so")
+    out = subprocess.run([sys.executable, "-c", code, os.path.join(ROOT, "flash-dmattn_amd")], env=env, capture_output=True,
+                         text=True, timeout=300).stdout
+    assert "ImportError:" in out and "no fallback" in out and "IMPORTED" not in out, out
+    assert "CUDA_AVAILABLE False None []" in out, out
+    assert "RuntimeError: No flash attention backend is available" in out and "RETURNED" not in out, out
