@@ -8,8 +8,9 @@ callers that keep their own tensor program lose nothing, callers that switch get
 and two backwards instead of the chain of library kernels, and the attention's dBias -- returned in the bias's own
 [batch, kv heads, 1, keys] shape -- is consumed directly.
 
-For fp16 / bf16 tensors on the GPU whose shapes the kernels take, the work runs in libfdma_hip.so
-(`fdma_dyn_bias_fwd` / `fdma_dyn_bias_bwd`); anything else runs the same tensor program as the reference's caller.
+For fp16 / bf16 tensors on the GPU the work runs in libfdma_hip.so (`fdma_dyn_bias_fwd` / `fdma_dyn_bias_bwd`; a shape
+the kernels were not built for raises RuntimeError); CPU and fp32 tensors run the same tensor program as the
+reference's caller.
 """
 from typing import Optional
 
@@ -26,13 +27,22 @@ def _tensor_program(value_states, weight, a, proj_bias):
 
 
 def _native_ok(value_states, weight, a, proj_bias) -> bool:
-    if not (value_states.is_cuda and value_states.dim() == 4 and value_states.dtype in (torch.bfloat16, torch.float16)):
+    """True when the kernels take the call.  16-bit tensors on the GPU are the kernels' business: a shape they were not
+    built for is an error, not a reason to fall back quietly; CPU and fp32 tensors run the caller's tensor program."""
+    if not (value_states.is_cuda and value_states.dtype in (torch.bfloat16, torch.float16)):
         return False
+    if value_states.dim() != 4:
+        raise RuntimeError("value_states must have shape (batch, key_len, num_kv_heads, head_dim)")
     b, l, hk, d = value_states.shape
     others = [weight, a] + ([proj_bias] if proj_bias is not None else [])
     if any(t.dtype != value_states.dtype or t.device != value_states.device for t in others):
-        return False
-    return hk <= 32 and d % 8 == 0 and (hk * d) % 16 == 0 and tuple(weight.shape) == (hk, hk * d) and a.numel() == hk
+        raise RuntimeError("dt_proj_weight, A and dt_proj_bias must have the dtype and device of value_states")
+    if tuple(weight.shape) != (hk, hk * d) or a.numel() != hk or (proj_bias is not None and proj_bias.numel() != hk):
+        raise RuntimeError("dt_proj_weight must be (num_kv_heads, num_kv_heads * head_dim), A and dt_proj_bias (num_kv_heads)")
+    if hk > 32 or d % 8 != 0 or (hk * d) % 16 != 0:
+        raise RuntimeError("the bias producer is built for up to 32 kv heads, head_dim % 8 == 0 and "
+                           "(num_kv_heads * head_dim) % 16 == 0")
+    return True
 
 
 class _DynamicMaskBias(torch.autograd.Function):

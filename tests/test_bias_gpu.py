@@ -88,3 +88,17 @@ def test_bias_producer_is_bit_reproducible_and_feeds_the_operator():
     q = torch.randn(B, L, H, d, device=DEV).to(torch.bfloat16)
     out = flash_sparse_attn_func(q, kv[:, :, 0], kv[:, :, 1], keep, bias, None, True)
     assert torch.isfinite(out.float()).all()
+
+
+def test_bias_producer_rejects_shapes_it_was_not_built_for():
+    v = torch.randn(1, 64, 2, 12, device=DEV).to(torch.bfloat16)   # head_dim not a multiple of 8
+    w = torch.randn(2, 24, device=DEV).to(torch.bfloat16)
+    a = torch.ones(2, device=DEV).to(torch.bfloat16)
+    with pytest.raises(RuntimeError, match="head_dim % 8"):
+        dynamic_mask_bias(v, w, a)
+    v = torch.randn(1, 64, 2, 16, device=DEV).to(torch.bfloat16)
+    with pytest.raises(RuntimeError, match="dtype and device"):
+        dynamic_mask_bias(v, torch.randn(2, 32, device=DEV), a)
+    # CPU tensors run the caller's tensor program
+    out = dynamic_mask_bias(v.cpu(), torch.randn(2, 32).to(torch.bfloat16), a.cpu())
+    assert out.shape == (1, 2, 1, 64)
