@@ -42,6 +42,21 @@ def _aligned(x: Optional[torch.Tensor], elems: int) -> Optional[torch.Tensor]:
     return x if ok else x.contiguous().clone(memory_format=torch.contiguous_format)
 
 
+def _direct_when_eager(op):
+    """Callable for one of the operators below.  On plain tensors in eager mode it runs the operator's Python
+    body directly: the dispatch of a torch.library operator costs about 20 us per call, more than a small
+    attention call takes on the device.  Under torch.compile, and for fake tensors or tensor subclasses, the
+    registered operator is called, as the reference always does (flash_sparse_attn_interface.py:126, 432)."""
+    body = op._init_fn
+
+    def call(*args, **kwargs):
+        if torch.compiler.is_compiling() or any(type(a) is not torch.Tensor for a in args[:3]):
+            return op(*args, **kwargs)
+        return body(*args, **kwargs)
+
+    return call
+
+
 def _check_inputs(q, k, v, mask, bias) -> None:
     """Device / dtype / rank / shape checks of mha_fwd (flash_api.cpp:371-438, 477-479)."""
     if q.dtype not in (torch.float16, torch.bfloat16):
@@ -107,7 +122,7 @@ def _flash_sparse_attn_forward(
         return out, softmax_lse, p
     args = _cabi.FwdArgs()
     _cabi.fill_fwd(args, q, k, v, mask, bias, out, softmax_lse, softmax_scale, is_causal, softcap)
-    with torch.cuda.device(q.device):
+    with _cabi.device_guard(q.device):
         nbytes = _cabi.lib.fdma_fwd_workspace_bytes(args)
         workspace = None
         if nbytes:
@@ -129,7 +144,7 @@ def _flash_sparse_attn_forward_fake(
     return out, softmax_lse, p
 
 
-_wrapped_flash_sparse_attn_forward = _flash_sparse_attn_forward
+_wrapped_flash_sparse_attn_forward = _direct_when_eager(_flash_sparse_attn_forward)
 
 
 @torch.library.custom_op(
@@ -195,7 +210,7 @@ def _flash_sparse_attn_backward(
     args.dbias_strides[:] = _cabi._bcast3(dbias_w) if dbias_w is not None else (0, 0, 0)
     args.softmax_d = softmax_d.data_ptr()
     args.deterministic = int(bool(deterministic))
-    with torch.cuda.device(q.device):
+    with _cabi.device_guard(q.device):
         nbytes = _cabi.lib.fdma_bwd_workspace_bytes(args)
         workspace = None
         if nbytes:
@@ -229,7 +244,7 @@ def _flash_sparse_attn_backward_fake(
     return torch.empty((batch_size, num_heads, round_multiple(seqlen_q, 128)), device=q.device, dtype=torch.float32)
 
 
-_wrapped_flash_sparse_attn_backward = _flash_sparse_attn_backward
+_wrapped_flash_sparse_attn_backward = _direct_when_eager(_flash_sparse_attn_backward)
 
 
 def _pad_key_dim(t: Optional[torch.Tensor], seqlen_k: int, elems: int) -> Optional[torch.Tensor]:
@@ -438,7 +453,7 @@ def _flash_sparse_attn_varlen_forward(
     args = _cabi.VarlenFwdArgs()
     _cabi.fill_varlen_fwd(args, q, k, v, out, softmax_lse, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
                           softmax_scale, is_causal, softcap)
-    with torch.cuda.device(q.device):
+    with _cabi.device_guard(q.device):
         _cabi.check(_cabi.lib.fdma_varlen_fwd(args, _cabi.current_stream(q.device)))
     return out, softmax_lse, p
 
@@ -457,7 +472,7 @@ def _flash_sparse_attn_varlen_forward_fake(
     return out, softmax_lse, p
 
 
-_wrapped_flash_sparse_attn_varlen_forward = _flash_sparse_attn_varlen_forward
+_wrapped_flash_sparse_attn_varlen_forward = _direct_when_eager(_flash_sparse_attn_varlen_forward)
 
 
 @torch.library.custom_op(
@@ -509,7 +524,7 @@ def _flash_sparse_attn_varlen_backward(
     args.dv_strides[:] = (dv_w.stride(0), dv_w.stride(1))
     args.softmax_d = softmax_d.data_ptr()
     args.deterministic = int(bool(deterministic))
-    with torch.cuda.device(q.device):
+    with _cabi.device_guard(q.device):
         _cabi.check(_cabi.lib.fdma_varlen_bwd(args, _cabi.current_stream(q.device)))
     for given, work in ((dq, dq_w), (dk, dk_w), (dv, dv_w)):
         if given is not None and work is not given:
@@ -528,7 +543,7 @@ def _flash_sparse_attn_varlen_backward_fake(
     return torch.empty((num_heads, total_q), device=q.device, dtype=torch.float32)
 
 
-_wrapped_flash_sparse_attn_varlen_backward = _flash_sparse_attn_varlen_backward
+_wrapped_flash_sparse_attn_varlen_backward = _direct_when_eager(_flash_sparse_attn_varlen_backward)
 
 
 class FlashAttnVarlenFunc(torch.autograd.Function):

@@ -68,7 +68,7 @@ class _DynamicMaskBias(torch.autograd.Function):
         args.bias_strides[:] = (bias_store.stride(0), bias_store.stride(1))
         args.batch, args.seqlen_k, args.num_heads_k, args.head_dim = b, l, hk, d
         args.dtype = _cabi.dtype_code(v)
-        with torch.cuda.device(v.device):
+        with _cabi.device_guard(v.device):
             _cabi.check(_cabi.lib.fdma_dyn_bias_fwd(args, _cabi.current_stream(v.device)))
         ctx.save_for_backward(v, w, av, pb if pb is not None else torch.empty(0, device=v.device), dt)
         ctx.has_pb = pb is not None
@@ -98,7 +98,7 @@ class _DynamicMaskBias(torch.autograd.Function):
         args.dvalue_strides[:] = dv.stride()[:3]
         args.dweight, args.da = dw.data_ptr(), da.data_ptr()
         args.dproj_bias = dpb.data_ptr() if dpb is not None else None
-        with torch.cuda.device(v.device):
+        with _cabi.device_guard(v.device):
             nbytes = _cabi.lib.fdma_dyn_bias_bwd_workspace_bytes(args)
             ws = torch.empty(max(nbytes, 1), dtype=torch.uint8, device=v.device)
             args.workspace, args.workspace_bytes = ws.data_ptr(), nbytes

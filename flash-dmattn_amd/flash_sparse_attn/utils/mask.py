@@ -84,7 +84,7 @@ def _native_mask(attention_bias, attention_mask, window_size, min_dtype, block_s
     a.type = 0 if kind == "topk" else 1
     a.dtype = _cabi.dtype_code(bias)
     a.min_value = float(min_dtype)
-    with torch.cuda.device(bias.device):
+    with _cabi.device_guard(bias.device):
         _cabi.check(_cabi.lib.fdma_create_mask(a, _cabi.current_stream(bias.device)))
     return out
 

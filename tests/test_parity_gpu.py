@@ -353,6 +353,10 @@ DECODE_CASES = {
     "mha_no_mask": (2, 777, 4, 4, 128, None, 1, None),
     "gqa8_shared_mask": (1, 3000, 16, 2, 128, 1, 16, 64),
     "short": (3, 40, 8, 2, 64, 2, 2, 7),
+    # 5000 keys per workgroup, all kept: the kept-key list (4096 entries) is worked off in two rounds
+    "dense_list_overflow": (8, 20000, 8, 8, 64, None, 1, None),
+    "gqa16_per_head_bias": (1, 5000, 32, 2, 128, 2, 32, 300),
+    "odd_head_dim": (2, 1500, 6, 2, 40, 2, 2, 99),
 }
 
 
@@ -379,6 +383,40 @@ def test_cfg5_full_size_decode():
     ro, rl = eager.attention_forward(qd, kd, vd, md, bd, None, False)
     assert_out_close(out, ro)
     _check_lse(lse, rl)
+
+
+def test_decode_long_splits_and_fp16():
+    """One workgroup per (batch entry, kv head) walks 40 000 keys: three mask fetches of 16 384 keys each.  fp16."""
+    B, Lk, H, Hk, D, W = 32, 40000, 16, 8, 64, 700
+    g = torch.Generator(device=DEV).manual_seed(5)
+    qd = torch.randn(B, 1, H, D, device=DEV, generator=g).to(torch.float16)
+    kd = torch.randn(B, Lk, Hk, D, device=DEV, generator=g).to(torch.float16)
+    vd = torch.randn(B, Lk, Hk, D, device=DEV, generator=g).to(torch.float16)
+    bd = torch.randn(B, Hk, 1, Lk, device=DEV, generator=g).to(torch.float16)
+    md = torch.zeros_like(bd, dtype=torch.bool).scatter_(-1, bd.float().topk(W, dim=-1).indices, True)
+    out, lse, _ = _op()(qd, kd, vd, md, bd, None, False, None, None, True)
+    ro, rl = eager.attention_forward(qd, kd, vd, md, bd, None, False)
+    assert_out_close(out, ro)
+    _check_lse(lse, rl)
+
+
+def test_decode_rows_far_apart():
+    """K and V rows 131 072 elements apart (views into wider buffers): the gather needs 64-bit offsets."""
+    B, Lk, H, Hk, D, W = 1, 3000, 8, 2, 128, 500
+    q, k, v, mask, bias = make_inputs(B, 1, Lk, H, Hk, D, (B, Hk, 1, Lk), (B, Hk, 1, Lk), W, seed=21)
+    qd, kd, vd, md, bd = _to_dev(q, k, v, mask, bias)
+    wide_k = torch.zeros(B, Lk, 131072, dtype=kd.dtype, device=DEV)
+    wide_v = torch.zeros(B, Lk, 131072, dtype=vd.dtype, device=DEV)
+    wide_k[..., : Hk * D] = kd.reshape(B, Lk, Hk * D)
+    wide_v[..., : Hk * D] = vd.reshape(B, Lk, Hk * D)
+    kw = wide_k[..., : Hk * D].view(B, Lk, Hk, D)
+    vw = wide_v[..., : Hk * D].view(B, Lk, Hk, D)
+    assert kw.stride(1) == 131072 and kw.stride(-1) == 1
+    out, lse, _ = _op()(qd, kw, vw, md, bd, None, False, None, None, True)
+    ref, ref_lse, _ = _op()(qd, kd, vd, md, bd, None, False, None, None, True)
+    assert torch.equal(out, ref) and torch.equal(lse, ref_lse)
+    ro, rl = c_oracle.forward(q, k, v, mask, bias, None, False)
+    assert_out_close(out.cpu(), ro)
 
 
 def test_direct_c_abi_call_without_the_python_operator():
