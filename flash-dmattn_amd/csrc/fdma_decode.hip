@@ -128,6 +128,8 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) decode_kernel(const FwdParams 
     // staging: this lane's row within a load instruction and its chunk
     const int srow = lane / CH, sc = lane % CH;
     const uint32_t st_off = (uint32_t)((srow * SM::S + sc * 8) * 2);
+    const bool pad_lane = sc >= nchunk;             // head dimension below D: these lanes stage zeros
+    const int scl = pad_lane ? nchunk - 1 : sc;
 
     typedef const __attribute__((address_space(1))) char *gptr_t;  // global address space survives the integer round trip
     auto uniform_ptr = [](const void *ptr) -> gptr_t {
@@ -192,22 +194,19 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) decode_kernel(const FwdParams 
             uint32_t braw = 0;
             bool bvalid = false;
             auto load_batch = [&](int t0) {
-                if (sc < nchunk) {  // rows beyond the list repeat its last row: their scores are dropped below
+                // rows beyond the list repeat its last row (their scores are dropped below); lanes beyond the head
+                // dimension fetch its last chunk and are cleared when the batch is staged
 #pragma unroll
-                    for (int j = 0; j < NI; j++) {
-                        const int t = t0 + j * RPI + srow;
-                        const uint32_t rel = s_idx[t < total ? t : total - 1];
-                        if (WIDE) {
-                            kreg[j] = *(const __attribute__((address_space(1))) u32x4_t *)(kb0 + ((int64_t)rel * p.k_r + sc * 8) * 2);
-                            vreg[j] = *(const __attribute__((address_space(1))) u32x4_t *)(vb0 + ((int64_t)rel * p.v_r + sc * 8) * 2);
-                        } else {
-                            kreg[j] = *(const __attribute__((address_space(1))) u32x4_t *)(kb0 + (rel * (uint32_t)p.k_r + sc * 8) * 2u);
-                            vreg[j] = *(const __attribute__((address_space(1))) u32x4_t *)(vb0 + (rel * (uint32_t)p.v_r + sc * 8) * 2u);
-                        }
+                for (int j = 0; j < NI; j++) {
+                    const int t = t0 + j * RPI + srow;
+                    const uint32_t rel = s_idx[t < total ? t : total - 1];
+                    if (WIDE) {
+                        kreg[j] = *(const __attribute__((address_space(1))) u32x4_t *)(kb0 + ((int64_t)rel * p.k_r + scl * 8) * 2);
+                        vreg[j] = *(const __attribute__((address_space(1))) u32x4_t *)(vb0 + ((int64_t)rel * p.v_r + scl * 8) * 2);
+                    } else {
+                        kreg[j] = *(const __attribute__((address_space(1))) u32x4_t *)(kb0 + (rel * (uint32_t)p.k_r + scl * 8) * 2u);
+                        vreg[j] = *(const __attribute__((address_space(1))) u32x4_t *)(vb0 + (rel * (uint32_t)p.v_r + scl * 8) * 2u);
                     }
-                } else {
-#pragma unroll
-                    for (int j = 0; j < NI; j++) kreg[j] = vreg[j] = u32x4_t{0, 0, 0, 0};
                 }
                 if (!PERHEAD) {  // one fused value per key: lane i < 32 fetches the bias of the batch's key i
                     bvalid = lane < DEC_TILE && t0 + lane < total;
@@ -221,8 +220,8 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) decode_kernel(const FwdParams 
                 // stage the batch (LDS operations of one wave execute in order: the reads of the previous batch are done)
 #pragma unroll
                 for (int j = 0; j < NI; j++) {
-                    *(u32x4_t *)(sK + st_off + j * RPI * SM::S * 2) = kreg[j];
-                    *(u32x4_t *)(sV + st_off + j * RPI * SM::S * 2) = vreg[j];
+                    *(u32x4_t *)(sK + st_off + j * RPI * SM::S * 2) = pad_lane ? u32x4_t{0, 0, 0, 0} : kreg[j];
+                    *(u32x4_t *)(sV + st_off + j * RPI * SM::S * 2) = pad_lane ? u32x4_t{0, 0, 0, 0} : vreg[j];
                 }
                 if (!PERHEAD && lane < DEC_TILE) sB[lane] = bvalid ? E::lo(braw) * kLog2e : -INFINITY;
                 // additive term of this lane's 16 (key, column) pairs: register 8 blk + e <-> key 16 blk + 8 g + e of the batch
