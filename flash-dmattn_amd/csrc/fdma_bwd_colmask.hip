@@ -95,23 +95,32 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
         Sm = plan[2];
         Q = plan[4];
         const int per = Gs * Sm;
-        // unit lists per XCD (see DkdvPlan); within a list all units of one split index sit side by side:
-        // neighbours in time then stream the same Q / dO tiles through that XCD's L2
-        const int P = f.B * f.Hk, k = dkdv_lists_per_pair(P);
-        const int list_len = plan[3];
-        if (list_len == 0) return;
+        int sub;
         const int x = blockIdx.x % 8, l = blockIdx.x / 8;
-        const int span = list_len * per;
-        const int ls = l / span, within = l % span;
-        if (ls >= P * k / 8) return;
-        // Consecutive workgroups of an XCD go to its shader engines in turn; unit weights fall with the unit
-        // index, so the start of the unit order is rotated with the split index -- otherwise one engine would
-        // receive the heavy unit of every group and the others would idle behind it.
-        const int sub = within / list_len, pos = (within % list_len + sub) % list_len;
-        const int vlist = x + 8 * ls, fold = vlist % k;
-        pair = vlist / k;
-        n_block = 2 * k * (pos >> 1) + ((pos & 1) ? 2 * k - 1 - fold : fold);
-        if (n_block >= plan[DKDV_PLAN_HDR + pair + 1] - plan[DKDV_PLAN_HDR + pair]) return;
+        if (per > 1) {
+            // Split units: the plan holds, per XCD, the list of the parts that exist -- (pair, unit, part of the
+            // unit), longest parts first.  Workgroup l of an XCD takes entry l; consecutive workgroups of an XCD go
+            // to its shader engines in turn, and with the existing parts side by side every engine gets its share.
+            const int cap = gridDim.x / 8;
+            const int32_t *lists = plan + plan[5];
+            if (l >= lists[x]) return;
+            const int32_t *e = lists + 8 + 2 * ((int64_t)x * cap + l);
+            pair = e[0];
+            n_block = e[1] & 0xffff;
+            sub = e[1] >> 16;
+        } else {
+            // unit lists per XCD: the units of a pair are dealt to its k lists, the lists to the XCDs
+            const int P = f.B * f.Hk, k = dkdv_lists_per_pair(P);
+            const int list_len = plan[3];
+            if (list_len == 0) return;
+            const int ls = l / list_len, pos = l % list_len;
+            if (ls >= P * k / 8) return;
+            const int vlist = x + 8 * ls, fold = vlist % k;
+            pair = vlist / k;
+            n_block = dkdv_unit_at(pos, fold, k);
+            if (n_block >= plan[DKDV_PLAN_HDR + pair + 1] - plan[DKDV_PLAN_HDR + pair]) return;
+            sub = 0;
+        }
         const int unit = plan[DKDV_PLAN_HDR + pair] + n_block;
         const int gper = G / Gs;
         g_lo = (sub / Sm) * gper;

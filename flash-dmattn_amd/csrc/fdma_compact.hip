@@ -15,6 +15,8 @@
 // All of this is O(Lk * d) traffic in front of O(Lq * count * d) MFMA work.
 #include <cstdlib>
 
+#include <atomic>
+
 #include "fdma_common.h"
 #include "fdma_params.h"
 
@@ -51,7 +53,9 @@ Layout layout_of(const FwdParams &p, bool backward) {
         int grid, slots;
         dkdv_split_bounds((int)pairs, (p.Lk + 127) / 128, p.H / p.Hk, grid, slots);
         const int dpad = p.d <= 64 ? 64 : 128;
-        l.off_plan = o;    o += align256((DKDV_PLAN_HDR + pairs + 1) * 4);
+        // header, prefix of the units over the pairs and, per XCD, the list of the parts that exist (two ints each;
+        // the kernel's grid bounds their number)
+        l.off_plan = o;    o += align256((DKDV_PLAN_HDR + pairs + 1 + 8 + 2 * (size_t)grid) * 4);
         l.off_part_kv = o; o += align256((size_t)slots * 2 * dpad * 128 * 4);
         l.off_part_db = o; o += align256((size_t)slots * (p.H / p.Hk) * 128 * 4);
     }
@@ -196,10 +200,15 @@ __global__ void __launch_bounds__(256) compact_zero_kernel(const BwdParams p, co
     }
 }
 
-// One workgroup: prefix of 128-key units over the pairs and the split the dK/dV kernel will use.
+// One workgroup: prefix of 128-key units over the pairs, the split the dK/dV kernel will use and, when units are
+// split, the per-XCD lists of the parts that exist.  `slots`: workgroups of the dK/dV kernel the device holds at a
+// time; `cap`: entries a per-XCD list has room for (that kernel's workgroups per XCD).
 __global__ void __launch_bounds__(256) compact_plan_kernel(const int32_t *count, const int32_t *idx, int ld, int32_t *plan,
-                                                            int pairs, int G, int Lq, int Lk, int causal) {
+                                                            int pairs, int G, int Lq, int Lk, int causal, int slots, int cap) {
+    constexpr int MAXU = DKDV_ENOUGH_UNITS;  // units are split only below this many (and there are no more pairs than units)
     __shared__ int s_sum, s_max, s_n[256], s_units;
+    __shared__ int s_Gs, s_Sm, s_Q, s_fit, s_q1, s_parts2, s_over2;
+    __shared__ int s_first[MAXU + 1], s_nt[MAXU], s_len[MAXU], s_nseg[MAXU], s_uoff[MAXU], s_lcount[8 * MAXU], s_cand[64][8];
     const int tid = threadIdx.x;
     // units per pair and their prefix: the counts are fetched 256 at a time by all threads (one memory latency per
     // chunk instead of one per pair), the prefix over a chunk is then taken from LDS by one thread
@@ -211,6 +220,7 @@ __global__ void __launch_bounds__(256) compact_plan_kernel(const int32_t *count,
             const int m = pairs - base < 256 ? pairs - base : 256;
             for (int i = 0; i < m; i++) {
                 plan[DKDV_PLAN_HDR + base + i] = u;
+                if (base + i < MAXU) s_first[base + i] = u;
                 u += s_n[i];
                 n_max = s_n[i] > n_max ? s_n[i] : n_max;
             }
@@ -221,39 +231,167 @@ __global__ void __launch_bounds__(256) compact_plan_kernel(const int32_t *count,
         plan[DKDV_PLAN_HDR + pairs] = u;
         plan[0] = u;
         plan[3] = dkdv_list_len(n_max, dkdv_lists_per_pair(pairs));
+        if (pairs <= MAXU) s_first[pairs] = u;
         s_units = u;
         s_sum = 0;
         s_max = 0;
     }
     __syncthreads();
+    const int U = s_units;
+    int Gs0, Sm0;
+    dkdv_split(U, G, Gs0, Sm0);
+    if (Gs0 * Sm0 <= 1 || pairs >= MAXU) {  // no split (or hardly any pair with keys): nothing else to plan
+        if (tid == 0) { plan[1] = 1; plan[2] = 1; plan[4] = 1 << 30; }
+        return;
+    }
+    // From here on U < MAXU, hence pairs < MAXU and (pairs being at most 256 then or not) every count is in reach:
+    // thread g works on unit g.  Its pair: the last one that starts at or before g.
+    auto pair_of = [&](int g) -> int {
+        int lo = 0, hi = pairs;  // s_first[lo] <= g < s_first[hi]
+        while (hi - lo > 1) {
+            const int mid = (lo + hi) >> 1;
+            if (s_first[mid] <= g) lo = mid; else hi = mid;
+        }
+        return lo;
+    };
     // query blocks per unit: their sum sizes the parts, their maximum the number of segment slots
     int sum = 0, mx = 0;
-    for (int i = 0; i < pairs; i++) {
-        const int n = pairs <= 256 ? s_n[i] : (count[i] + 127) / 128;  // (up to 256 pairs the counts are still in LDS)
-        for (int u = tid; u < n; u += 256) {
-            const int nt = dkdv_query_blocks(Lq, Lk, causal, idx[(size_t)i * ld + u * 128]);
-            sum += nt;
-            mx = nt > mx ? nt : mx;
-        }
+    for (int g = tid; g < U; g += 256) {
+        const int i = pair_of(g);
+        const int nt = dkdv_query_blocks(Lq, Lk, causal, idx[(size_t)i * ld + (g - s_first[i]) * 128]);
+        s_nt[g] = nt;
+        sum += nt;
+        mx = nt > mx ? nt : mx;
     }
     atomicAdd(&s_sum, sum);
     atomicMax(&s_max, mx);
     __syncthreads();
     if (tid == 0) {
-        int Gs, Sm;
-        dkdv_split(s_units, G, Gs, Sm);
-        int Q = 1 << 30;
-        if (Sm > 1) {
+        int Q = 1 << 30, fit = 1;
+        if (Sm0 > 1) {
             const int64_t even = ((int64_t)G * s_sum + DKDV_TARGET_PARTS - 1) / DKDV_TARGET_PARTS;
-            const int fit = (s_max + Sm - 1) / Sm;  // Sm slots must cover the longest unit
+            fit = (s_max + Sm0 - 1) / Sm0;  // Sm slots must cover the longest unit
+            if (fit < 1) fit = 1;
             Q = (int)(even > fit ? even : fit);
+        }
+        s_Gs = Gs0; s_Sm = Sm0; s_Q = Q; s_fit = fit;
+        s_q1 = 1 << 30;
+        s_parts2 = 0;
+        s_over2 = 0;
+    }
+    if (tid < 64) {
+#pragma unroll
+        for (int e = 0; e < 8; e++) s_cand[tid][e] = 0;
+    }
+    __syncthreads();
+    const int k = dkdv_lists_per_pair(pairs);
+    // Segment length.  Q above gives about DKDV_TARGET_PARTS parts, i.e. more than one round of workgroups: with
+    // parts of unequal length (many units, few segments each) the short ones fill the gaps behind the long ones, but
+    // nearly equal parts queue up in whole rounds and the last one is mostly empty.  So the smallest Q whose parts all
+    // fit the device at once is looked for as well (the number of parts falls with Q), and the two are compared by an
+    // estimate of the time of the last workgroup, in query blocks: one round ends with its longest part; several
+    // rounds take the even share plus about half a longest part (measured), and every round pays the start-up and the
+    // partial-result write of a workgroup (about 2.5 blocks).  64 candidates (the last one is Q itself), four
+    // threads each: a thread takes every fourth unit and adds the parts it finds to the candidate's eight XCD counters
+    // (the dK/dV kernel deals the units of a pair to k lists, dkdv_list_of, and the lists to the XCDs).
+    if (Sm0 > 1) {
+        const int Sm = Sm0, fit = s_fit;
+        const int cand = tid & 63, quarter = tid >> 6;
+        const int step = (s_max - fit + 61) / 62 > 0 ? (s_max - fit + 61) / 62 : 1;
+        const int Qc = cand == 63 ? s_Q : fit + cand * step;
+        const float rq = 1.0f / (float)Qc;
+        int c[8] = {0, 0, 0, 0, 0, 0, 0, 0};
+        int i = 0;
+        for (int g = quarter; g < U; g += 4) {
+            while (s_first[i + 1] <= g) i++;
+            const int x = (i * k + dkdv_list_of(g - s_first[i], k)) & 7;
+            // ceil(nt / Qc), exactly: the half keeps the float quotient off the integers
+            int ns = (int)(((float)(s_nt[g] + Qc - 1) + 0.5f) * rq);
+            ns = ns < Sm ? ns : Sm;
+#pragma unroll
+            for (int e = 0; e < 8; e++) c[e] += x == e ? ns : 0;
+        }
+#pragma unroll
+        for (int e = 0; e < 8; e++) if (c[e]) atomicAdd(&s_cand[cand][e], c[e]);
+        __syncthreads();
+        if (tid < 64) {
+            int worst = 0, parts = 0;
+#pragma unroll
+            for (int e = 0; e < 8; e++) { worst = s_cand[tid][e] > worst ? s_cand[tid][e] : worst; parts += s_cand[tid][e]; }
+            if (tid == 63) { s_parts2 = parts * Gs0; s_over2 = worst * Gs0 * 8 > slots; }  // (more than one round on some XCD)
+            else if (worst * Gs0 * 8 <= slots) atomicMin(&s_q1, Qc);
+        }
+    }
+    __syncthreads();
+    if (tid == 0) {
+        int Sm = Sm0, Q = s_Q;
+        if (Sm > 1) {
+            if (s_over2 && s_q1 < (1 << 30)) {
+                const int r = (s_parts2 + slots - 1) / slots;
+                const float rounds = (float)(r < 2 ? 2 : r);
+                const float several = (float)Gs0 * (float)s_sum / (float)slots + 0.45f * (float)Q + 2.5f * rounds;
+                const float one = (float)s_q1 + 2.5f;
+                if (one < several) Q = s_q1;
+            }
             if (Q < 1) Q = 1;
             Sm = dkdv_segments(s_max, Q, Sm);
             if (Sm < 1) Sm = 1;
         }
-        plan[1] = Gs;
+        plan[1] = Gs0;
         plan[2] = Sm;
         plan[4] = Q;
+        plan[5] = DKDV_PLAN_HDR + pairs + 1;  // where the lists begin
+        s_Q = Q; s_Sm = Sm;
+    }
+    const int n_lists = pairs * k;  // a multiple of 8, at most 8 * MAXU
+    for (int vl = tid; vl < n_lists; vl += 256) s_lcount[vl] = 0;
+    __syncthreads();
+    // The parts that exist, per XCD: list after list (an XCD holds every eighth list); inside a list the units with
+    // the longest parts first (all parts of a unit are equally long: its query blocks cut into equal segments), the
+    // parts of a unit side by side.  The kernel's workgroups start in this order: the short ones fill the gaps at the
+    // end.  Which units a list holds stays as dealt -- that balances the lists; only their order inside it is by length.
+    const int Q = s_Q, Sm = s_Sm;
+    for (int g = tid; g < U; g += 256) {
+        const int n_seg = dkdv_segments(s_nt[g], Q, Sm);
+        s_nseg[g] = n_seg;
+        s_len[g] = n_seg > 0 ? (s_nt[g] + n_seg - 1) / n_seg : 0;
+    }
+    __syncthreads();
+    for (int g = tid; g < U; g += 256) {
+        const int i = pair_of(g), first = s_first[i], n = s_first[i + 1] - first, un = g - first;
+        const int mine = s_len[g], fold = dkdv_list_of(un, k);
+        int before = 0;  // parts of the units of the same list that come first
+        for (int v = 0; v < n; v++) {
+            const bool first_v = dkdv_list_of(v, k) == fold && (s_len[first + v] > mine || (s_len[first + v] == mine && v < un));
+            before += first_v ? s_nseg[first + v] : 0;
+        }
+        s_uoff[g] = Gs0 * before;
+        atomicAdd(&s_lcount[i * k + fold], Gs0 * s_nseg[g]);
+    }
+    __syncthreads();
+    int32_t *lists = plan + DKDV_PLAN_HDR + pairs + 1;
+    if (tid < 8) {
+        int off = 0;
+        for (int vl = tid; vl < n_lists; vl += 8) {
+            const int t = s_lcount[vl];
+            s_lcount[vl] = off;  // from here on: where the list begins in its XCD's entries
+            off += t;
+        }
+        lists[tid] = off < cap ? off : cap;  // (the grid is sized for every part: off <= cap)
+    }
+    __syncthreads();
+    for (int g = tid; g < U; g += 256) {
+        const int i = pair_of(g), un = g - s_first[i], vl = i * k + dkdv_list_of(un, k), ns = s_nseg[g];
+        int o = s_lcount[vl] + s_uoff[g];
+        int32_t *e = lists + 8 + 2 * ((size_t)(vl & 7) * cap);
+        for (int gi = 0; gi < Gs0; gi++)
+            for (int sg = 0; sg < ns; sg++) {
+                if (o < cap) {
+                    e[2 * o] = i;
+                    e[2 * o + 1] = un | ((gi * Sm + sg) << 16);
+                }
+                o++;
+            }
     }
 }
 
@@ -307,6 +445,19 @@ void dkdv_split_bounds(int pairs, int n_max, int G, int &grid, int &slots) {
     slots = (int)sl;
 }
 
+// compute units of the current device (cached per device)
+static int device_cus() {
+    static std::atomic<int> cus[16];
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return 256;
+    int n = cus[dev].load(std::memory_order_relaxed);
+    if (n == 0) {
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || n <= 0) n = 256;
+        cus[dev].store(n, std::memory_order_relaxed);
+    }
+    return n;
+}
+
 hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, BwdParams *bp) {
     const Layout l = layout_of(p, bp != nullptr);
     char *w = static_cast<char *>(ws);
@@ -325,8 +476,11 @@ hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, 
     if ((e = hipGetLastError()) != hipSuccess) return e;
     if (bp) {
         int32_t *plan = (int32_t *)(w + l.off_plan);
+        int grid, slots;
+        dkdv_split_bounds(pairs, (p.Lk + 127) / 128, p.H / p.Hk, grid, slots);
+        const int plan_cap = grid / 8;  // entries per XCD list: the dK/dV kernel's workgroups per XCD
         hipLaunchKernelGGL(compact_plan_kernel, dim3(1), dim3(256), 0, stream, count, idx, l.ld, plan, pairs, p.H / p.Hk, p.Lq,
-                           p.Lk, p.causal);
+                           p.Lk, p.causal, 2 * device_cus(), plan_cap);
         if ((e = hipGetLastError()) != hipSuccess) return e;
         p.cmp.plan = plan;
         bp->dkv_part = (float *)(w + l.off_part_kv);

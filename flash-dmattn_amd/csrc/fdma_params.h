@@ -75,6 +75,15 @@ __host__ __device__ inline int dkdv_segments(int n_tot, int Q, int Sm) {
 __host__ __device__ inline int dkdv_lists_per_pair(int pairs) {
     return pairs % 8 == 0 ? 1 : (pairs % 4 == 0 ? 2 : (pairs % 2 == 0 ? 4 : 8));
 }
+// The units of a pair are dealt to its k lists in a snake (0 .. k-1, k-1 .. 0, ...): position `pos` of list `fold`
+// holds unit dkdv_unit_at(pos, fold, k); unit u sits in list dkdv_list_of(u, k).
+__host__ __device__ inline int dkdv_unit_at(int pos, int fold, int k) {
+    return 2 * k * (pos >> 1) + ((pos & 1) ? 2 * k - 1 - fold : fold);
+}
+__host__ __device__ inline int dkdv_list_of(int u, int k) {
+    const int rem = u % (2 * k);
+    return rem < k ? rem : 2 * k - 1 - rem;
+}
 __host__ __device__ inline int dkdv_list_len(int units_in_largest_pair, int k) {
     return 2 * ((units_in_largest_pair + 2 * k - 1) / (2 * k));
 }
