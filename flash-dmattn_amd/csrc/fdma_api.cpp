@@ -318,9 +318,7 @@ int fdma_bwd(const fdma_bwd_args *a, void *hip_stream) {
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     hipError_t e;
     if (a->f.seqlen_q > 0 && fdma::use_compact(p.f)) {
-        const fdma::FwdParams orig = p.f;
         e = fdma::compact_setup(p.f, static_cast<char *>(a->workspace) + dbias_accum_bytes(a), a->f.dtype, stream, &p);
-        if (e == hipSuccess) e = fdma::compact_zero_dropped(p, orig, stream);
         if (e != hipSuccess) return fail(FDMA_ERR_LAUNCH, "backward launch failed: %s", hipGetErrorString(e));
     }
     e = fdma::launch_bwd(p, a->f.dtype, stream);

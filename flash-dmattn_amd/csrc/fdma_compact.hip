@@ -122,12 +122,12 @@ __global__ void __launch_bounds__(SCAN_THREADS) compact_scan_kernel(const FwdPar
 
 // orig: the caller's tensors.  kc / vc: dense [B*Hk, Lk, d] destinations.
 template <typename T>
-__global__ void __launch_bounds__(256) compact_gather_kernel(const FwdParams p, const int32_t *idx, const int32_t *count,
-                                                              float *fb, uint16_t *kc, uint16_t *vc, int ld, int Hfb) {
+__device__ __forceinline__ void gather_block(const FwdParams &p, const int32_t *idx, const int32_t *count, float *fb,
+                                             uint16_t *kc, uint16_t *vc, int ld, int Hfb, int block_x, int pair) {
     using E = Elem<T>;
-    const int pair = blockIdx.y, b = pair / p.Hk, hk = pair % p.Hk;
+    const int b = pair / p.Hk, hk = pair % p.Hk;
     const int n = count[pair];
-    const int c0 = blockIdx.x * GATHER_KEYS;
+    const int c0 = block_x * GATHER_KEYS;
     if (c0 >= n) return;
     __shared__ int s_src[GATHER_KEYS];
     const int tid = threadIdx.x;
@@ -165,15 +165,20 @@ __global__ void __launch_bounds__(256) compact_gather_kernel(const FwdParams p, 
     }
 }
 
+template <typename T>
+__global__ void __launch_bounds__(256) compact_gather_kernel(const FwdParams p, const int32_t *idx, const int32_t *count,
+                                                              float *fb, uint16_t *kc, uint16_t *vc, int ld, int Hfb) {
+    gather_block<T>(p, idx, count, fb, kc, vc, ld, Hfb, blockIdx.x, blockIdx.y);
+}
+
 // Gradient rows (dK, dV) and columns (dBias) of dropped keys: no workgroup of the compacted backward
 // owns them, and the operator's contract is that they come back as zeros.
-__global__ void __launch_bounds__(256) compact_zero_kernel(const BwdParams p, const uint8_t *mask, int64_t m_b, int64_t m_h,
-                                                            int Hm, bool dbias_direct) {
-    const FwdParams &f = p.f;
-    const int pair = blockIdx.y, b = pair / f.Hk, hk = pair % f.Hk;
-    const int hm = Hm == 1 ? 0 : hk;
-    const uint8_t *mrow = mask + b * m_b + hm * m_h;
-    const int c0 = blockIdx.x * GATHER_KEYS;
+__device__ __forceinline__ void zero_block(const BwdParams &p, bool dbias_direct, int block_x, int pair) {
+    const FwdParams &f = p.f;  // (the caller's tensors: the mask is the original one)
+    const int b = pair / f.Hk, hk = pair % f.Hk;
+    const int hm = f.Hm == 1 ? 0 : hk;
+    const uint8_t *mrow = f.mask + b * f.m_b + hm * f.m_h;
+    const int c0 = block_x * GATHER_KEYS;
     const int tid = threadIdx.x;
     const int CH = f.d / 8;
     uint16_t *dkb = (uint16_t *)p.dk + b * p.dk_b + hk * p.dk_h;
@@ -203,8 +208,8 @@ __global__ void __launch_bounds__(256) compact_zero_kernel(const BwdParams p, co
 // One workgroup: prefix of 128-key units over the pairs, the split the dK/dV kernel will use and, when units are
 // split, the per-XCD lists of the parts that exist.  `slots`: workgroups of the dK/dV kernel the device holds at a
 // time; `cap`: entries a per-XCD list has room for (that kernel's workgroups per XCD).
-__global__ void __launch_bounds__(256) compact_plan_kernel(const int32_t *count, const int32_t *idx, int ld, int32_t *plan,
-                                                            int pairs, int G, int Lq, int Lk, int causal, int slots, int cap) {
+__device__ __forceinline__ void plan_block(const int32_t *count, const int32_t *idx, int ld, int32_t *plan, int pairs, int G,
+                                           int Lq, int Lk, int causal, int slots, int cap) {
     constexpr int MAXU = DKDV_ENOUGH_UNITS;  // units are split only below this many (and there are no more pairs than units)
     __shared__ int s_sum, s_max, s_n[256], s_units;
     __shared__ int s_Gs, s_Sm, s_Q, s_fit, s_q1, s_parts2, s_over2;
@@ -395,6 +400,24 @@ __global__ void __launch_bounds__(256) compact_plan_kernel(const int32_t *count,
     }
 }
 
+// Everything the compacted backward needs after the scan, in one launch: layer 0 of the grid gathers K / V rows,
+// layer 1 clears the gradients of dropped keys, and one workgroup of layer 2 makes the dK/dV plan.
+// The plan is a chain of dependent steps of a single workgroup (18 us); side by side with the other two it costs nothing.
+template <typename T>
+__global__ void __launch_bounds__(256) compact_bwd_prepass_kernel(const BwdParams bp, const int32_t *idx, int32_t *cnt_unused,
+                                                                   const int32_t *count, float *fb, uint16_t *kc, uint16_t *vc,
+                                                                   int ld, int Hfb, int32_t *plan, int slots, int cap) {
+    (void)cnt_unused;
+    const FwdParams &f = bp.f;
+    if (blockIdx.z == 0) {
+        gather_block<T>(f, idx, count, fb, kc, vc, ld, Hfb, blockIdx.x, blockIdx.y);
+    } else if (blockIdx.z == 1) {
+        zero_block(bp, bp.dbias != nullptr && bp.dbias_accum == nullptr, blockIdx.x, blockIdx.y);
+    } else if (blockIdx.x == 0 && blockIdx.y == 0) {
+        plan_block(count, idx, ld, plan, f.B * f.Hk, f.H / f.Hk, f.Lq, f.Lk, f.causal, slots, cap);
+    }
+}
+
 // FDMA_COMPACT: 0 = never, 2 = whenever the mask form allows it, anything else / unset = when it also pays.
 // Read on every call, so that one process can time both paths.
 int compaction_mode() {
@@ -469,18 +492,25 @@ hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, 
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     const dim3 grid((p.Lk + GATHER_KEYS - 1) / GATHER_KEYS, pairs);
-    if (dtype == 0)
-        hipLaunchKernelGGL((compact_gather_kernel<bf16_tag>), grid, dim3(256), 0, stream, p, idx, count, fb, kc, vc, l.ld, l.Hfb);
-    else
-        hipLaunchKernelGGL((compact_gather_kernel<fp16_tag>), grid, dim3(256), 0, stream, p, idx, count, fb, kc, vc, l.ld, l.Hfb);
-    if ((e = hipGetLastError()) != hipSuccess) return e;
-    if (bp) {
+    if (!bp) {
+        if (dtype == 0)
+            hipLaunchKernelGGL((compact_gather_kernel<bf16_tag>), grid, dim3(256), 0, stream, p, idx, count, fb, kc, vc, l.ld, l.Hfb);
+        else
+            hipLaunchKernelGGL((compact_gather_kernel<fp16_tag>), grid, dim3(256), 0, stream, p, idx, count, fb, kc, vc, l.ld, l.Hfb);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+    } else {
+        // (p is bp->f, still describing the caller's tensors here)
         int32_t *plan = (int32_t *)(w + l.off_plan);
-        int grid, slots;
-        dkdv_split_bounds(pairs, (p.Lk + 127) / 128, p.H / p.Hk, grid, slots);
-        const int plan_cap = grid / 8;  // entries per XCD list: the dK/dV kernel's workgroups per XCD
-        hipLaunchKernelGGL(compact_plan_kernel, dim3(1), dim3(256), 0, stream, count, idx, l.ld, plan, pairs, p.H / p.Hk, p.Lq,
-                           p.Lk, p.causal, 2 * device_cus(), plan_cap);
+        int dkdv_grid, slots;
+        dkdv_split_bounds(pairs, (p.Lk + 127) / 128, p.H / p.Hk, dkdv_grid, slots);
+        const int plan_cap = dkdv_grid / 8;  // entries per XCD list: the dK/dV kernel's workgroups per XCD
+        const dim3 grid3(grid.x, pairs, 3);
+        if (dtype == 0)
+            hipLaunchKernelGGL((compact_bwd_prepass_kernel<bf16_tag>), grid3, dim3(256), 0, stream, *bp, idx, cnt, count, fb, kc, vc,
+                               l.ld, l.Hfb, plan, 2 * device_cus(), plan_cap);
+        else
+            hipLaunchKernelGGL((compact_bwd_prepass_kernel<fp16_tag>), grid3, dim3(256), 0, stream, *bp, idx, cnt, count, fb, kc, vc,
+                               l.ld, l.Hfb, plan, 2 * device_cus(), plan_cap);
         if ((e = hipGetLastError()) != hipSuccess) return e;
         p.cmp.plan = plan;
         bp->dkv_part = (float *)(w + l.off_part_kv);
@@ -501,11 +531,5 @@ hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, 
     return hipSuccess;
 }
 
-hipError_t compact_zero_dropped(const BwdParams &p, const FwdParams &orig, hipStream_t stream) {
-    const dim3 grid((orig.Lk + GATHER_KEYS - 1) / GATHER_KEYS, orig.B * orig.Hk);
-    const bool dbias_direct = p.dbias != nullptr && p.dbias_accum == nullptr;
-    hipLaunchKernelGGL(compact_zero_kernel, grid, dim3(256), 0, stream, p, orig.mask, orig.m_b, orig.m_h, orig.Hm, dbias_direct);
-    return hipGetLastError();
-}
 
 }  // namespace fdma

@@ -236,12 +236,12 @@ hipError_t launch_bwd_dq(const BwdParams &p, int dtype, hipStream_t stream);
 
 // Column compaction: use_compact() decides from the problem alone (no device data), compact_bytes() is
 // the scratch it needs, compact_setup() launches the gather pre-pass into `ws` and rewrites p.k / p.v /
-// p.cmp; compact_zero_dropped() zero-fills the gradient rows / columns of dropped keys.
+// p.cmp; for a backward call (bp given) the same launch zero-fills the gradient rows / columns of dropped keys
+// and makes the dK/dV plan.
 bool use_compact(const FwdParams &p);
 size_t compact_bytes(const FwdParams &p, bool backward);
 // bp != nullptr: backward -- also plans the dK/dV split and sets bp->dkv_part / bp->db_part
 hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, BwdParams *bp = nullptr);
-hipError_t compact_zero_dropped(const BwdParams &p, const FwdParams &orig, hipStream_t stream);
 // host-side bounds over every possible unit count 1..U_max: workgroups to launch, partial slots to hold
 // (n_max = units of one pair at most)
 void dkdv_split_bounds(int pairs, int n_max, int G, int &grid, int &slots);
