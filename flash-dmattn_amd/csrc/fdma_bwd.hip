@@ -21,6 +21,7 @@
 // read-modify-write traffic.
 #include "fdma_common.h"
 #include "fdma_params.h"
+#include "fdma_bwd_dot.h"
 
 #include <type_traits>
 
@@ -41,28 +42,7 @@ __device__ __forceinline__ uint32_t nz_bytes_to_bits(uint32_t x) {
 // ------------------------------------------------------------------------------------------------
 template <typename T>
 __global__ void __launch_bounds__(256) bwd_dot_kernel(const BwdParams p) {
-    using E = Elem<T>;
-    const int CH = (p.f.d + 7) / 8;               // 16-byte chunks per row
-    const int lanes = CH <= 8 ? 8 : 16;           // lanes cooperating on one row (power of two)
-    const int rows_per_block = 256 / lanes;
-    const int sub = threadIdx.x % lanes;
-    const int row = blockIdx.x * rows_per_block + threadIdx.x / lanes;
-    const int h = blockIdx.y, b = blockIdx.z;
-    // a ragged batch is one run of total_q rows (its batch strides are 0 and the grid has one batch entry)
-    const int n_rows = p.f.cu_q ? p.f.total_q : p.f.Lq, n_out = p.f.cu_q ? p.f.total_q : p.Lq_rounded;
-    float acc = 0.f;
-    if (row < n_rows) {
-        const uint16_t *op = (const uint16_t *)p.f.o + b * p.f.o_b + (int64_t)row * p.f.o_r + h * p.f.o_h;
-        const uint16_t *dp = (const uint16_t *)p.dout + b * p.do_b + (int64_t)row * p.do_r + h * p.do_h;
-        for (int c = sub; c < CH; c += lanes) {
-            u32x4_t ov = *(const u32x4_t *)(op + c * 8);
-            u32x4_t dv = *(const u32x4_t *)(dp + c * 8);
-#pragma unroll
-            for (int e = 0; e < 4; e++) acc += E::lo(ov[e]) * E::lo(dv[e]) + E::hi(ov[e]) * E::hi(dv[e]);
-        }
-    }
-    for (int off = lanes / 2; off > 0; off >>= 1) acc += __shfl_xor(acc, off);
-    if (sub == 0 && row < n_out) p.softmax_d[b * p.sd_b + h * p.sd_h + row] = acc;
+    bwd_dot_block<T>(p, blockIdx.x, blockIdx.y, blockIdx.z);
 }
 
 // ------------------------------------------------------------------------------------------------
@@ -533,8 +513,8 @@ template <typename T, int D>
 hipError_t launch_bwd_t(const BwdParams &p, hipStream_t stream) {
     const FwdParams &f = p.f;
     hipError_t e;
-    // 1. D = rowsum(dO * O)
-    {
+    // 1. D = rowsum(dO * O)  (the compacted backward has done it in its pre-pass launch)
+    if (!p.dot_done) {
         const int CH = (f.d + 7) / 8, lanes = CH <= 8 ? 8 : 16, rpb = 256 / lanes;
         dim3 grid(((f.cu_q ? f.total_q : p.Lq_rounded) + rpb - 1) / rpb, f.H, f.cu_q ? 1 : f.B);
         hipLaunchKernelGGL((bwd_dot_kernel<T>), grid, dim3(256), 0, stream, p);

@@ -19,6 +19,7 @@
 
 #include "fdma_common.h"
 #include "fdma_params.h"
+#include "fdma_bwd_dot.h"
 
 namespace fdma {
 
@@ -211,9 +212,10 @@ __device__ __forceinline__ void zero_block(const BwdParams &p, bool dbias_direct
 __device__ __forceinline__ void plan_block(const int32_t *count, const int32_t *idx, int ld, int32_t *plan, int pairs, int G,
                                            int Lq, int Lk, int causal, int slots, int cap) {
     constexpr int MAXU = DKDV_ENOUGH_UNITS;  // units are split only below this many (and there are no more pairs than units)
+    constexpr int MAXL = 1024;               // ... and with at most this many unit lists (LDS: every block of the launch pays for it)
     __shared__ int s_sum, s_max, s_n[256], s_units;
     __shared__ int s_Gs, s_Sm, s_Q, s_fit, s_q1, s_parts2, s_over2;
-    __shared__ int s_first[MAXU + 1], s_nt[MAXU], s_len[MAXU], s_nseg[MAXU], s_uoff[MAXU], s_lcount[8 * MAXU], s_cand[64][8];
+    __shared__ int s_first[MAXU + 1], s_nt[MAXU], s_len[MAXU], s_nseg[MAXU], s_uoff[MAXU], s_lcount[MAXL], s_cand[64][8];
     const int tid = threadIdx.x;
     // units per pair and their prefix: the counts are fetched 256 at a time by all threads (one memory latency per
     // chunk instead of one per pair), the prefix over a chunk is then taken from LDS by one thread
@@ -245,7 +247,7 @@ __device__ __forceinline__ void plan_block(const int32_t *count, const int32_t *
     const int U = s_units;
     int Gs0, Sm0;
     dkdv_split(U, G, Gs0, Sm0);
-    if (Gs0 * Sm0 <= 1 || pairs >= MAXU) {  // no split (or hardly any pair with keys): nothing else to plan
+    if (Gs0 * Sm0 <= 1 || pairs >= MAXU || pairs * dkdv_lists_per_pair(pairs) > MAXL) {  // no split (or hardly any pair with keys): nothing else to plan
         if (tid == 0) { plan[1] = 1; plan[2] = 1; plan[4] = 1 << 30; }
         return;
     }
@@ -348,7 +350,7 @@ __device__ __forceinline__ void plan_block(const int32_t *count, const int32_t *
         plan[5] = DKDV_PLAN_HDR + pairs + 1;  // where the lists begin
         s_Q = Q; s_Sm = Sm;
     }
-    const int n_lists = pairs * k;  // a multiple of 8, at most 8 * MAXU
+    const int n_lists = pairs * k;  // a multiple of 8, at most MAXL
     for (int vl = tid; vl < n_lists; vl += 256) s_lcount[vl] = 0;
     __syncthreads();
     // The parts that exist, per XCD: list after list (an XCD holds every eighth list); inside a list the units with
@@ -401,7 +403,8 @@ __device__ __forceinline__ void plan_block(const int32_t *count, const int32_t *
 }
 
 // Everything the compacted backward needs after the scan, in one launch: layer 0 of the grid gathers K / V rows,
-// layer 1 clears the gradients of dropped keys, and one workgroup of layer 2 makes the dK/dV plan.
+// layer 1 clears the gradients of dropped keys, one workgroup of layer 2 makes the dK/dV plan, and the layers from 3
+// on compute D = rowsum(dO * O), which depends on none of the others.
 // The plan is a chain of dependent steps of a single workgroup (18 us); side by side with the other two it costs nothing.
 template <typename T>
 __global__ void __launch_bounds__(256) compact_bwd_prepass_kernel(const BwdParams bp, const int32_t *idx, int32_t *cnt_unused,
@@ -413,8 +416,14 @@ __global__ void __launch_bounds__(256) compact_bwd_prepass_kernel(const BwdParam
         gather_block<T>(f, idx, count, fb, kc, vc, ld, Hfb, blockIdx.x, blockIdx.y);
     } else if (blockIdx.z == 1) {
         zero_block(bp, bp.dbias != nullptr && bp.dbias_accum == nullptr, blockIdx.x, blockIdx.y);
-    } else if (blockIdx.x == 0 && blockIdx.y == 0) {
-        plan_block(count, idx, ld, plan, f.B * f.Hk, f.H / f.Hk, f.Lq, f.Lk, f.causal, slots, cap);
+    } else if (blockIdx.z == 2) {
+        if (blockIdx.x == 0 && blockIdx.y == 0)
+            plan_block(count, idx, ld, plan, f.B * f.Hk, f.H / f.Hk, f.Lq, f.Lk, f.causal, slots, cap);
+    } else {  // the blocks of D = rowsum(dO * O), laid out over the remaining layers
+        const int nbx = (bp.Lq_rounded + bwd_dot_rows_per_block(f.d) - 1) / bwd_dot_rows_per_block(f.d);
+        const int64_t lin = ((int64_t)(blockIdx.z - 3) * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+        if (lin >= (int64_t)nbx * f.H * f.B) return;
+        bwd_dot_block<T>(bp, (int)(lin % nbx), (int)((lin / nbx) % f.H), (int)(lin / ((int64_t)nbx * f.H)));
     }
 }
 
@@ -504,7 +513,12 @@ hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, 
         int dkdv_grid, slots;
         dkdv_split_bounds(pairs, (p.Lk + 127) / 128, p.H / p.Hk, dkdv_grid, slots);
         const int plan_cap = dkdv_grid / 8;  // entries per XCD list: the dK/dV kernel's workgroups per XCD
-        const dim3 grid3(grid.x, pairs, 3);
+        const int dot_rows = bwd_dot_rows_per_block(p.d);
+        const int64_t dot_blocks = (int64_t)((bp->Lq_rounded + dot_rows - 1) / dot_rows) * p.H * p.B;
+        const int64_t layer = (int64_t)grid.x * pairs;
+        const int64_t dot_layers = (dot_blocks + layer - 1) / layer;
+        const bool with_dot = p.cu_q == nullptr && 3 + dot_layers <= 65535;
+        const dim3 grid3(grid.x, pairs, with_dot ? (unsigned)(3 + dot_layers) : 3);
         if (dtype == 0)
             hipLaunchKernelGGL((compact_bwd_prepass_kernel<bf16_tag>), grid3, dim3(256), 0, stream, *bp, idx, cnt, count, fb, kc, vc,
                                l.ld, l.Hfb, plan, 2 * device_cus(), plan_cap);
@@ -512,6 +526,7 @@ hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, 
             hipLaunchKernelGGL((compact_bwd_prepass_kernel<fp16_tag>), grid3, dim3(256), 0, stream, *bp, idx, cnt, count, fb, kc, vc,
                                l.ld, l.Hfb, plan, 2 * device_cus(), plan_cap);
         if ((e = hipGetLastError()) != hipSuccess) return e;
+        bp->dot_done = with_dot ? 1 : 0;
         p.cmp.plan = plan;
         bp->dkv_part = (float *)(w + l.off_part_kv);
         bp->db_part = (float *)(w + l.off_part_db);

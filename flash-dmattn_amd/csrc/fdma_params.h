@@ -156,6 +156,7 @@ struct BwdParams {
     // compacted dK/dV kernel, split mode: per part [2][Dpad][128] fp32 (dK^T, dV^T) and [G][128] fp32 (dBias)
     float *dkv_part;
     float *db_part;
+    int32_t dot_done;          // softmax_d has been computed by an earlier launch of this call
 };
 
 // Keep-mask builder (fdma_mask.hip): one row of `Lk` 16-bit bias values per (batch, head, row).
