@@ -385,6 +385,34 @@ def test_cfg5_full_size_decode():
     _check_lse(lse, rl)
 
 
+SPLIT_PLAN_CASES = {
+    # name: (B, Lq, Lk, H, Hk, D, window, causal) -- few 128-key blocks after compaction, so the dK/dV kernel splits
+    # them over query heads and query segments; the (batch, kv head) pairs are dealt to 8 / 4 / 2 / 1 lists per pair
+    "three_pairs": (3, 1500, 1500, 4, 1, 64, 700, True),
+    "six_pairs_gqa2": (1, 2000, 2000, 12, 6, 128, 900, True),
+    "five_pairs_mha_noncausal": (5, 1024, 1024, 1, 1, 64, 500, False),
+    "two_pairs_gqa8": (1, 6000, 6000, 16, 2, 128, 1500, True),
+    "short_queries": (2, 700, 3000, 8, 2, 64, 1000, True),
+    "sixteen_pairs_one_block": (2, 900, 900, 16, 8, 64, 100, True),
+}
+
+
+@pytest.mark.parametrize("name", list(SPLIT_PLAN_CASES))
+def test_compacted_backward_split_plans_vs_eager_fp32(name):
+    os.environ["FDMA_COMPACT"] = "2"
+    B, Lq, Lk, H, Hk, D, W, causal = SPLIT_PLAN_CASES[name]
+    q, k, v, mask, bias = make_inputs(B, Lq, Lk, H, Hk, D, (B, Hk, 1, Lk), (B, Hk, 1, Lk), W, seed=11)
+    out, lse, (dq, dk, dv, db) = _run_fwd_bwd(q, k, v, mask, bias, causal)
+    qd, kd, vd, md, bd = _to_dev(q, k, v, mask, bias)
+    ro, rdq, rdk, rdv, rdb = eager.attention_forward_backward(qd, kd, vd, md, bd, None, causal)
+    assert_out_close(out, ro)
+    for g, r, n in ((dq, rdq, "dq"), (dk, rdk, "dk"), (dv, rdv, "dv"), (db, rdb, "dbias")):
+        assert_grad_close(g, r, n)
+    # a second call must give the same bits (fixed-order reduction of the parts)
+    out2, _, (dq2, dk2, dv2, db2) = _run_fwd_bwd(q, k, v, mask, bias, causal)
+    assert torch.equal(dk, dk2) and torch.equal(dv, dv2) and torch.equal(db, db2) and torch.equal(dq, dq2)
+
+
 def test_decode_long_splits_and_fp16():
     """One workgroup per (batch entry, kv head) walks 40 000 keys: three mask fetches of 16 384 keys each.  fp16."""
     B, Lk, H, Hk, D, W = 32, 40000, 16, 8, 64, 700
