@@ -357,6 +357,9 @@ DECODE_CASES = {
     "dense_list_overflow": (8, 20000, 8, 8, 64, None, 1, None),
     "gqa16_per_head_bias": (1, 5000, 32, 2, 128, 2, 32, 300),
     "odd_head_dim": (2, 1500, 6, 2, 40, 2, 2, 99),
+    # 40 query heads on one kv head: two workgroups per split (32 + 8 columns)
+    "mqa40_two_column_chunks": (1, 2000, 40, 1, 64, 1, 1, 300),
+    "mqa40_per_head_mask_and_bias": (1, 1200, 40, 1, 128, 40, 40, 200),
 }
 
 
