@@ -407,10 +407,9 @@ __device__ __forceinline__ void plan_block(const int32_t *count, const int32_t *
 // on compute D = rowsum(dO * O), which depends on none of the others.
 // The plan is a chain of dependent steps of a single workgroup (18 us); side by side with the other two it costs nothing.
 template <typename T>
-__global__ void __launch_bounds__(256) compact_bwd_prepass_kernel(const BwdParams bp, const int32_t *idx, int32_t *cnt_unused,
+__global__ void __launch_bounds__(256) compact_bwd_prepass_kernel(const BwdParams bp, const int32_t *idx,
                                                                    const int32_t *count, float *fb, uint16_t *kc, uint16_t *vc,
                                                                    int ld, int Hfb, int32_t *plan, int slots, int cap) {
-    (void)cnt_unused;
     const FwdParams &f = bp.f;
     if (blockIdx.z == 0) {
         gather_block<T>(f, idx, count, fb, kc, vc, ld, Hfb, blockIdx.x, blockIdx.y);
@@ -520,10 +519,10 @@ hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, 
         const bool with_dot = p.cu_q == nullptr && 3 + dot_layers <= 65535;
         const dim3 grid3(grid.x, pairs, with_dot ? (unsigned)(3 + dot_layers) : 3);
         if (dtype == 0)
-            hipLaunchKernelGGL((compact_bwd_prepass_kernel<bf16_tag>), grid3, dim3(256), 0, stream, *bp, idx, cnt, count, fb, kc, vc,
+            hipLaunchKernelGGL((compact_bwd_prepass_kernel<bf16_tag>), grid3, dim3(256), 0, stream, *bp, idx, count, fb, kc, vc,
                                l.ld, l.Hfb, plan, 2 * device_cus(), plan_cap);
         else
-            hipLaunchKernelGGL((compact_bwd_prepass_kernel<fp16_tag>), grid3, dim3(256), 0, stream, *bp, idx, cnt, count, fb, kc, vc,
+            hipLaunchKernelGGL((compact_bwd_prepass_kernel<fp16_tag>), grid3, dim3(256), 0, stream, *bp, idx, count, fb, kc, vc,
                                l.ld, l.Hfb, plan, 2 * device_cus(), plan_cap);
         if ((e = hipGetLastError()) != hipSuccess) return e;
         bp->dot_done = with_dot ? 1 : 0;

@@ -165,7 +165,7 @@ __global__ void __launch_bounds__(64 * NW, (NQ == 1 && NW == 4) ? 2 : 1) fwd_col
             sBits[w0 + 1] = (uint32_t)(ball >> 32);
         }
     }
-    __syncthreads();
+    if (!CMP) __syncthreads();  // (compacted keys have no bitmap: every tile up to n_end is active)
 
     // smallest active tile >= j, or n_end.  The bitmap word comes from LDS; readfirstlane tells the compiler that
     // the result is wave-uniform, so tile bases, loop conditions and load addresses stay in scalar registers.
