@@ -260,6 +260,17 @@ def _pad_key_dim(t: Optional[torch.Tensor], seqlen_k: int, elems: int) -> Option
     return t
 
 
+def _nothing_to_differentiate(grad_enabled: bool, *tensors: Optional[torch.Tensor]) -> bool:
+    """True for an eager call on plain tensors none of which asks for a gradient: the autograd node would record
+    nothing, and going through it costs about 10 us per call -- as much as a decode-sized kernel takes."""
+    if torch.compiler.is_compiling():
+        return False
+    for t in tensors:
+        if t is not None and (type(t) is not torch.Tensor or (grad_enabled and t.requires_grad)):
+            return False
+    return True
+
+
 class FlashDMAttnFunc(torch.autograd.Function):
 
     @staticmethod
@@ -388,19 +399,12 @@ def flash_sparse_attn_func(
         softmax_lse [optional]: (batch_size, nheads, seqlen), fp32 logsumexp of each score row
             (+inf for rows with no visible key).
     """
-    return FlashDMAttnFunc.apply(
-        query,
-        key,
-        value,
-        attn_mask,
-        attn_bias,
-        softmax_scale,
-        is_causal,
-        softcap,
-        deterministic,
-        return_attn_probs,
-        torch.is_grad_enabled(),
-    )
+    grad_enabled = torch.is_grad_enabled()
+    args = (query, key, value, attn_mask, attn_bias, softmax_scale, is_causal, softcap, deterministic, return_attn_probs,
+            grad_enabled)
+    if _nothing_to_differentiate(grad_enabled, query, key, value, attn_bias):
+        return FlashDMAttnFunc.forward(None, *args)  # (the context is only touched when gradients are wanted)
+    return FlashDMAttnFunc.apply(*args)
 
 
 def _check_varlen_inputs(q, k, v, cu_seqlens_q, cu_seqlens_k) -> None:
@@ -622,8 +626,9 @@ def flash_sparse_attn_varlen_func(
     Returns out (total_q, nheads, headdim), or (out, softmax_lse (nheads, total_q), S_dmask (empty)) when
     `return_attn_probs` is set.  Paged KV (`block_table`) and softcapping raise RuntimeError.
     """
-    return FlashAttnVarlenFunc.apply(
-        query, key, value, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k,
-        softmax_scale, is_causal, softcap, deterministic, return_attn_probs, block_table,
-        torch.is_grad_enabled(),
-    )
+    grad_enabled = torch.is_grad_enabled()
+    args = (query, key, value, cu_seqlens_q, cu_seqlens_k, max_seqlen_q, max_seqlen_k, softmax_scale, is_causal, softcap,
+            deterministic, return_attn_probs, block_table, grad_enabled)
+    if _nothing_to_differentiate(grad_enabled, query, key, value):
+        return FlashAttnVarlenFunc.forward(None, *args)
+    return FlashAttnVarlenFunc.apply(*args)
