@@ -117,7 +117,8 @@ def count_tiles(mask, Lq, Lk, causal, H, tile=64):
 def compaction_applies(mask, c):
     """Mirror of the library's rule for taking the column-compaction path (query-broadcast keep-mask with
     1 or Hkv heads, a problem large enough for the pre-pass to pay, not switched off)."""
-    mode = os.environ.get("FDMA_COMPACT", "1")[:1]
+    from flash_sparse_attn import _cabi
+    mode = {_cabi.COMPACT_NEVER: "0", _cabi.COMPACT_ALWAYS: "2"}.get(_cabi.get_compact_mode(), "1")
     form_ok = mask.shape[2] == 1 and mask.shape[1] in (1, c["Hk"]) and c["Lq"] >= 2
     pays = c["Lq"] >= 128 and c["Lk"] >= 128 and c["Lq"] * (c["H"] // c["Hk"]) * c["Lk"] >= 1 << 21
     return mode != "0" and form_ok and (mode == "2" or pays)
@@ -169,9 +170,9 @@ def time_gpu(fn, steps, warmup):
 
 
 def run_config(name, steps, warmup, device, compact=True, backward=True):
-    from flash_sparse_attn import flash_sparse_attn_func
+    from flash_sparse_attn import _cabi, flash_sparse_attn_func
 
-    os.environ["FDMA_COMPACT"] = "1" if compact else "0"  # the library reads it on every call
+    _cabi.set_compact_mode(_cabi.COMPACT_AUTO if compact else _cabi.COMPACT_NEVER)  # the compact_mode field of every call
     c = CONFIGS[name]
     q, k, v, mask, bias = make_case(c, device)
     scale = c["scale"]
@@ -344,7 +345,7 @@ def main():
     ap.add_argument("--all", action="store_true", help="also time configurations 1, 3, 4, 5")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-compact", action="store_true",
-                    help="switch the column-compaction path off (FDMA_COMPACT=0): time the tile-skipping kernels")
+                    help="switch the column-compaction path off (compact_mode = never): time the tile-skipping kernels")
     ap.add_argument("--calib-copy", action="store_true",
                     help="also run one plain 256 MiB device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--traffic-bytes", type=float, default=None,
@@ -409,7 +410,7 @@ def main():
         ts = run_config("cfg2", max(3, args.steps // 2), max(1, args.warmup // 2), device, compact=False, backward=False)
         out["tile_skip_path"] = {"ms_fwd": ts["ms_fwd"], "n_exec_tiles": ts["n_exec"], "tflops_fwd": ts["tflops_fwd"],
                                  "frac_of_peak": ts["tflops_fwd"] / PEAK_BF16_TFLOPS,
-                                 "kernel": "fdma::fwd_colmask_kernel<bf16, 128, causal> (FDMA_COMPACT=0)"}
+                                 "kernel": "fdma::fwd_colmask_kernel<bf16, 128, causal> (compact_mode = never)"}
     if args.traffic_bytes is not None:
         out["roofline"]["traffic"] = args.traffic_bytes
     if args.calib_copy:

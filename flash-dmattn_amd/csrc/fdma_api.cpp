@@ -80,6 +80,8 @@ int validate_common(const fdma_fwd_args *a, bool backward) {
     if (a->softcap != 0.f) return fail(FDMA_ERR_UNSUPPORTED, "softcap is not supported by this build");
     if (a->head_dim > 128) return fail(FDMA_ERR_UNSUPPORTED, "head dimensions above 128 are not built yet (got %d)", a->head_dim);
     if (!std::isfinite(a->softmax_scale)) return fail(FDMA_ERR_INVALID, "softmax_scale must be finite");
+    if (a->compact_mode < FDMA_COMPACT_AUTO || a->compact_mode > FDMA_COMPACT_ALWAYS)
+        return fail(FDMA_ERR_INVALID, "compact_mode must be FDMA_COMPACT_AUTO, _NEVER or _ALWAYS (got %d)", a->compact_mode);
     return FDMA_OK;
 }
 
@@ -106,6 +108,7 @@ void fill_fwd_params(const fdma_fwd_args *a, fdma::FwdParams &p) {
     p.scale = a->softmax_scale;
     p.scale_log2 = a->softmax_scale * 1.4426950408889634f;
     p.splits = 1;
+    p.compact_mode = a->compact_mode;
     p.lse_b = (int64_t)a->num_heads * a->seqlen_q;
     p.lse_h = a->seqlen_q;
 }

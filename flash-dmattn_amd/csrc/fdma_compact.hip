@@ -13,8 +13,6 @@
 //           gathered and pre-scaled into an fp32 vector;
 //   (backward) zero   rows of dK / dV and columns of dBias that belong to dropped keys.
 // All of this is O(Lk * d) traffic in front of O(Lq * count * d) MFMA work.
-#include <cstdlib>
-
 #include <atomic>
 
 #include "fdma_common.h"
@@ -426,18 +424,11 @@ __global__ void __launch_bounds__(256) compact_bwd_prepass_kernel(const BwdParam
     }
 }
 
-// FDMA_COMPACT: 0 = never, 2 = whenever the mask form allows it, anything else / unset = when it also pays.
-// Read on every call, so that one process can time both paths.
-int compaction_mode() {
-    const char *e = getenv("FDMA_COMPACT");
-    return (e && e[0] == '0') ? 0 : ((e && e[0] == '2') ? 2 : 1);
-}
-
 }  // namespace
 
 bool use_compact(const FwdParams &p) {
-    const int mode = compaction_mode();
-    if (mode == 0 || !p.mask || p.m_r != 0) return false;
+    const int mode = p.compact_mode;  // 0 = when it pays, 1 = never, 2 = whenever the mask form allows it
+    if (mode == 1 || !p.mask || p.m_r != 0) return false;
     if (p.bias && p.bi_r != 0) return false;
     if (!(p.Hm == 1 || p.Hm == p.Hk)) return false;
     if (p.Lq < 2 || p.Lk < 1 || (int64_t)p.Lk * p.d >= (int64_t)1 << 31) return false;

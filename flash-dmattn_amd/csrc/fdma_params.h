@@ -114,6 +114,7 @@ struct FwdParams {
     float *o_part;      // (splits, B, H, Lq, d) fp32
     float *lse_part;    // (splits, B, H, Lq) fp32, natural log, -inf for an empty split
     int32_t splits;
+    int32_t compact_mode;  // FDMA_COMPACT_* of the C ABI: 0 = decide from the problem, 1 = never, 2 = whenever the mask form allows
     Compact cmp;        // when cmp.on, k / v (and their strides) describe the compacted copies
 };
 

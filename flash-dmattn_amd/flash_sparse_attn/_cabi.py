@@ -30,6 +30,7 @@ class FwdArgs(ctypes.Structure):
         ("num_heads_mask", ctypes.c_int32), ("num_heads_bias", ctypes.c_int32),
         ("head_dim", ctypes.c_int32), ("dtype", ctypes.c_int32), ("is_causal", ctypes.c_int32),
         ("softmax_scale", ctypes.c_float), ("softcap", ctypes.c_float),
+        ("compact_mode", ctypes.c_int32),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
     ]
 
@@ -113,6 +114,36 @@ EXPORTS = (
 )
 
 
+# Column compaction policy handed to every attention call (fdma_fwd_args.compact_mode): 0 = the library decides
+# from the problem, 1 = never (tile skipping only), 2 = whenever the mask form allows it.  The environment variable
+# FDMA_COMPACT is read ONCE, here, as the default ("0" = never, "2" = always); set_compact_mode() changes it for
+# the process, compact_mode() for a with-block.
+COMPACT_AUTO, COMPACT_NEVER, COMPACT_ALWAYS = 0, 1, 2
+_compact_mode = {"0": COMPACT_NEVER, "2": COMPACT_ALWAYS}.get(os.environ.get("FDMA_COMPACT", "")[:1], COMPACT_AUTO)
+
+
+def get_compact_mode() -> int:
+    return _compact_mode
+
+
+def set_compact_mode(mode: int) -> int:
+    """Set the compaction policy of later calls; returns the previous one."""
+    global _compact_mode
+    if mode not in (COMPACT_AUTO, COMPACT_NEVER, COMPACT_ALWAYS):
+        raise ValueError("compact mode must be COMPACT_AUTO, COMPACT_NEVER or COMPACT_ALWAYS")
+    previous, _compact_mode = _compact_mode, mode
+    return previous
+
+
+@contextlib.contextmanager
+def compact_mode(mode: int):
+    previous = set_compact_mode(mode)
+    try:
+        yield
+    finally:
+        set_compact_mode(previous)
+
+
 def lib_path() -> str:
     return os.environ.get("FDMA_LIB", _DEFAULT_LIB)
 
@@ -145,8 +176,8 @@ def _load() -> ctypes.CDLL:
     lib.fdma_abi_version.restype = ctypes.c_int
     lib.fdma_sizeof_fwd_args.restype = ctypes.c_size_t
     lib.fdma_sizeof_bwd_args.restype = ctypes.c_size_t
-    if lib.fdma_abi_version() != 2:
-        raise ImportError(f"{path}: ABI version {lib.fdma_abi_version()} != 2")
+    if lib.fdma_abi_version() != 3:
+        raise ImportError(f"{path}: ABI version {lib.fdma_abi_version()} != 3")
     lib.fdma_varlen_fwd.argtypes = [ctypes.POINTER(VarlenFwdArgs), ctypes.c_void_p]
     lib.fdma_varlen_fwd.restype = ctypes.c_int
     lib.fdma_varlen_bwd.argtypes = [ctypes.POINTER(VarlenBwdArgs), ctypes.c_void_p]
@@ -214,7 +245,7 @@ def _bcast3(t: torch.Tensor) -> Sequence[int]:
     return tuple(0 if t.size(i) == 1 else t.stride(i) for i in range(3))
 
 
-_FWD_STRUCT = struct.Struct("@7P18q10i2fPN")
+_FWD_STRUCT = struct.Struct("@7P18q10i2fiPN")
 assert _FWD_STRUCT.size == ctypes.sizeof(FwdArgs)
 
 
@@ -234,7 +265,7 @@ def fill_fwd(a: FwdArgs, q, k, v, mask, bias, out, lse, softmax_scale, is_causal
         batch, seqlen_q, k.shape[1], num_heads, k.shape[2],
         mask.shape[1] if mask is not None else 1, bias.shape[1] if bias is not None else 1,
         head_dim, dtype_code(q), int(bool(is_causal)),
-        float(softmax_scale), float(softcap), 0, 0,
+        float(softmax_scale), float(softcap), _compact_mode, 0, 0,
     )
 
 

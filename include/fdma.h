@@ -43,7 +43,7 @@
 extern "C" {
 #endif
 
-#define FDMA_ABI_VERSION 2 /* 2: fdma_varlen_*, fdma_create_mask and fdma_dyn_bias_* added; everything of version 1 is unchanged */
+#define FDMA_ABI_VERSION 3 /* 3: fdma_fwd_args.compact_mode (the struct grew); 2: fdma_varlen_*, fdma_create_mask, fdma_dyn_bias_* */
 
 enum { FDMA_DTYPE_BF16 = 0, FDMA_DTYPE_FP16 = 1 };
 
@@ -53,6 +53,17 @@ enum {
     FDMA_ERR_UNSUPPORTED = -2, /* valid for the reference, not built here (e.g. head_dim > 128)   */
     FDMA_ERR_WORKSPACE = -3,   /* workspace missing or too small                                  */
     FDMA_ERR_LAUNCH = -4       /* the HIP runtime refused a launch                                */
+};
+
+/* Column compaction (fdma_fwd_args.compact_mode).  A keep-mask that is broadcast over the queries, with 1 or
+ * num_heads_k heads, drops whole key columns; the library can then gather the kept K / V rows into dense copies
+ * (in the workspace) and run attention over those alone, so that the work follows the number of kept keys.
+ * The result is the same function of the inputs either way.  The mode decides the workspace size, so the
+ * *_workspace_bytes call and the launch must see the same value (a mismatch is caught: FDMA_ERR_WORKSPACE). */
+enum {
+    FDMA_COMPACT_AUTO = 0,  /* compact when the mask form allows it and the problem is large enough to pay for the pre-pass */
+    FDMA_COMPACT_NEVER = 1, /* tile skipping only */
+    FDMA_COMPACT_ALWAYS = 2 /* compact whenever the mask form allows it */
 };
 
 typedef struct fdma_fwd_args {
@@ -70,7 +81,8 @@ typedef struct fdma_fwd_args {
     int32_t is_causal;
     float softmax_scale;
     float softcap; /* must be 0: softcapping is not built */
-    void *workspace;        /* split-KV partials for the decode path; may be NULL if bytes == 0 */
+    int32_t compact_mode;   /* FDMA_COMPACT_*; 0 = let the library decide */
+    void *workspace;        /* split-KV partials (decode) or the compacted K / V copies; may be NULL if bytes == 0 */
     size_t workspace_bytes; /* >= fdma_fwd_workspace_bytes(args) */
 } fdma_fwd_args;
 

@@ -6,6 +6,14 @@ CPU oracle and the GPU kernels see identical bits.
 """
 import torch
 
+def set_compact(mode) -> None:
+    """Compaction policy of the following operator calls: "0" = tile skipping only, "2" = column compaction whenever
+    the mask form allows it, None or anything else = the library's own cost rule (conftest.py resets it after
+    every test)."""
+    from flash_sparse_attn import _cabi
+    _cabi.set_compact_mode({"0": _cabi.COMPACT_NEVER, "2": _cabi.COMPACT_ALWAYS}.get(mode, _cabi.COMPACT_AUTO))
+
+
 # tolerances of the hot path (bf16): max-abs error of the output, relative error of gradients
 OUT_ATOL = 2e-2
 GRAD_RTOL = 5e-2

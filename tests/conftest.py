@@ -9,6 +9,15 @@ for p in (ROOT, os.path.join(ROOT, "flash-dmattn_amd")):
         sys.path.insert(0, p)
 
 
+@pytest.fixture(autouse=True)
+def _library_decides_compaction():
+    """Tests that pin the compaction policy (tests/_util.set_compact) do not leak it into the next test."""
+    yield
+    mod = sys.modules.get("flash_sparse_attn._cabi")
+    if mod is not None:
+        mod.set_compact_mode(mod.COMPACT_AUTO)
+
+
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu on the GPU box)")
 

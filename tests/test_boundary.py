@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(_cabi.lib_path())
     for name in declared:
         assert hasattr(lib, name), f"{name} not exported"
-    assert lib.fdma_abi_version() == 2
+    assert lib.fdma_abi_version() == 3
 
 
 def test_struct_mirrors_match_compiled_sizes():
@@ -170,9 +170,9 @@ def test_product_package_never_imports_the_oracle():
                 assert "oracle" not in text.lower(), f"{fn} mentions the oracle"
 
 
-def test_compaction_workspace_rule(monkeypatch):
+def test_compaction_workspace_rule():
     """fdma_*_workspace_bytes is pure host arithmetic: the column-compaction path asks for scratch exactly when the
-    mask is query-broadcast with 1 or Hkv heads and FDMA_COMPACT allows it (0 = never, 2 = whenever the form allows)."""
+    mask is query-broadcast with 1 or Hkv heads and the call's compact_mode allows it."""
     import torch
     from flash_sparse_attn import _cabi
 
@@ -191,13 +191,15 @@ def test_compaction_workspace_rule(monkeypatch):
     big = args(4096, 4096, 4, 2, 2, 1)
     per_query = args(4096, 4096, 4, 2, 2, 4096)
     per_qhead = args(4096, 4096, 4, 2, 4, 1)
-    monkeypatch.setenv("FDMA_COMPACT", "0")
+    assert small.compact_mode == _cabi.COMPACT_AUTO == 0   # (the default of a freshly filled block)
+    big.compact_mode = _cabi.COMPACT_NEVER
     assert _cabi.lib.fdma_fwd_workspace_bytes(big) == 0
-    monkeypatch.setenv("FDMA_COMPACT", "2")
+    for a in (small, per_query, per_qhead):
+        a.compact_mode = _cabi.COMPACT_ALWAYS
     assert _cabi.lib.fdma_fwd_workspace_bytes(small) > 0
     assert _cabi.lib.fdma_fwd_workspace_bytes(per_query) == 0
     assert _cabi.lib.fdma_fwd_workspace_bytes(per_qhead) == 0
-    monkeypatch.delenv("FDMA_COMPACT")
+    small.compact_mode = big.compact_mode = _cabi.COMPACT_AUTO
     assert _cabi.lib.fdma_fwd_workspace_bytes(small) == 0       # too small for the pre-pass to pay
     need = _cabi.lib.fdma_fwd_workspace_bytes(big)
     kv_bytes = 2 * 4096 * 2 * 64 * 2

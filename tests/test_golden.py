@@ -11,7 +11,7 @@ import pytest
 import torch
 
 from oracle import c_oracle, eager
-from _util import assert_grad_close, assert_out_close
+from _util import assert_grad_close, assert_out_close, set_compact
 
 PATH = os.path.join(os.path.dirname(os.path.abspath(__file__)), "golden", "vectors.npz")
 VEC = np.load(PATH)  # allow_pickle stays False
@@ -109,7 +109,7 @@ def _check_lse(lse, ref):
 def test_operator_matches_golden_vectors(name, compact, monkeypatch):
     from flash_sparse_attn import flash_sparse_attn_func
 
-    monkeypatch.setenv("FDMA_COMPACT", compact)  # tile skipping / column compaction where the mask form allows it
+    set_compact(compact)  # tile skipping / column compaction where the mask form allows it
     q, k, v, do, mask, bias, causal, scale = _load(name)
     dev = "cuda"
     qd, kd, vd = [t.to(dev).requires_grad_(True) for t in (q, k, v)]

@@ -15,7 +15,7 @@ import pytest
 import torch
 
 from oracle import c_oracle, eager
-from _util import assert_grad_close, assert_out_close, make_inputs, topk_keep_mask
+from _util import assert_grad_close, assert_out_close, make_inputs, set_compact, topk_keep_mask
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -32,11 +32,11 @@ def _to_dev(*ts):
 
 @pytest.fixture(autouse=True)
 def _default_compaction_mode():
-    """FDMA_COMPACT picks the path for query-broadcast masks (0 = tile skipping, 2 = column compaction whenever
-    the mask form allows it, unset = the library's own cost rule); the library reads it on every call."""
-    os.environ.pop("FDMA_COMPACT", None)
+    """set_compact picks the path for query-broadcast masks ("0" = tile skipping, "2" = column compaction whenever
+    the mask form allows it, None = the library's own cost rule); it is the compact_mode field of every call."""
+    set_compact(None)
     yield
-    os.environ.pop("FDMA_COMPACT", None)
+    set_compact(None)
 
 
 def _run_fwd_bwd(q, k, v, mask, bias, causal, scale=None, dout=None, need_grad=True):
@@ -113,7 +113,7 @@ def _eligible_for_compaction(name):
 def test_forward_backward_vs_c_oracle(name, compact):
     if compact == "2" and not _eligible_for_compaction(name):
         pytest.skip("mask form has no column-compaction path; covered by the other mode")
-    os.environ["FDMA_COMPACT"] = compact
+    set_compact(compact)
     B, Lq, Lk, H, Hk, D, bshape, mshape, W, causal = SMALL_CASES[name]
     (q, k, v, mask, bias, dout), (ro, rl), (rdq, rdk, rdv, rdb) = _small_case(name)
     out, lse, (dq, dk, dv, db) = _run_fwd_bwd(q, k, v, mask, bias, causal, dout=dout)
@@ -130,7 +130,7 @@ def test_forward_backward_vs_c_oracle(name, compact):
 
 @pytest.mark.parametrize("compact", ["0", "2"])
 def test_fp16_inputs(compact):
-    os.environ["FDMA_COMPACT"] = compact
+    set_compact(compact)
     q, k, v, mask, bias = make_inputs(1, 256, 256, 2, 1, 64, (1, 1, 1, 256), (1, 1, 1, 256), 128, seed=0, dtype=torch.float16)
     out, lse, (dq, dk, dv, db) = _run_fwd_bwd(q, k, v, mask, bias, True)
     ro, rl = c_oracle.forward(q, k, v, mask, bias, None, True)
@@ -150,7 +150,7 @@ def test_cfg1_reference_plumbing_config():
     ro, rl = c_oracle.forward(q, k, v, full, bias, 0.125, True)
     rdq, rdk, rdv, rdb = c_oracle.backward(q, k, v, torch.ones_like(ro), full, bias, 0.125, True)
     for m, compact in ((full, "1"), (colmask, "0"), (colmask, "2")):
-        os.environ["FDMA_COMPACT"] = compact
+        set_compact(compact)
         out, lse, (dq, dk, dv, db) = _run_fwd_bwd(q, k, v, m, bias, True, scale=0.125)
         assert_out_close(out.cpu(), ro)
         _check_lse(lse.cpu(), rl)
@@ -208,7 +208,7 @@ def test_column_mask_with_an_all_dropped_pair_and_late_first_key():
     """Query-broadcast mask whose (batch 0, kv head 1) row keeps nothing and whose other rows keep no key
     before column 150: that pair's outputs and gradients are exactly zero, rows that see no kept key give
     O = 0 / LSE = +inf, and everything else matches the oracle."""
-    os.environ["FDMA_COMPACT"] = "2"
+    set_compact("2")
     B, L, H, Hk, D = 2, 320, 4, 2, 64
     q, k, v, mask, bias = make_inputs(B, L, L, H, Hk, D, (B, Hk, 1, L), (B, Hk, 1, L), 60, seed=5)
     mask[..., :150] = False
@@ -243,7 +243,7 @@ def test_deterministic_rerun_is_bit_identical(form):
     if form == "per_query_mask":
         q, k, v, mask, bias = make_inputs(2, 384, 384, 4, 2, 64, (2, 2, 384, 384), (2, 2, 384, 384), 96, seed=7)
     else:  # dK / dV blocks split over several workgroups, partial sums folded in a fixed order
-        os.environ["FDMA_COMPACT"] = "2"
+        set_compact("2")
         q, k, v, mask, bias = make_inputs(2, 640, 640, 4, 2, 64, (2, 4, 1, 640), (2, 2, 1, 640), 300, seed=7)
     a = _run_fwd_bwd(q, k, v, mask, bias, True)
     b = _run_fwd_bwd(q, k, v, mask, bias, True)
@@ -287,7 +287,7 @@ def test_large_grid_256_row_workgroups_vs_eager_fp32(name, compact):
     """d = 128 problems whose grid is large enough for the forward to take its 256-row, 8-wave workgroups (split
     K / V staging roles), on the original and on the compacted key axis; ragged lengths so that the last query
     block and the last key tile are partial, both dtypes, causal with empty rows and non-causal."""
-    os.environ["FDMA_COMPACT"] = compact
+    set_compact(compact)
     B, Lq, Lk, H, Hk, D, W, causal, dtype = LARGE_GRID_CASES[name]
     q, k, v, mask, bias = make_inputs(B, Lq, Lk, H, Hk, D, (B, Hk, 1, Lk), (B, Hk, 1, Lk), W, seed=5)
     q, k, v, bias = [t.to(dtype) for t in (q, k, v, bias)]
@@ -402,7 +402,7 @@ SPLIT_PLAN_CASES = {
 
 @pytest.mark.parametrize("name", list(SPLIT_PLAN_CASES))
 def test_compacted_backward_split_plans_vs_eager_fp32(name):
-    os.environ["FDMA_COMPACT"] = "2"
+    set_compact("2")
     B, Lq, Lk, H, Hk, D, W, causal = SPLIT_PLAN_CASES[name]
     q, k, v, mask, bias = make_inputs(B, Lq, Lk, H, Hk, D, (B, Hk, 1, Lk), (B, Hk, 1, Lk), W, seed=11)
     out, lse, (dq, dk, dv, db) = _run_fwd_bwd(q, k, v, mask, bias, causal)
@@ -460,9 +460,9 @@ def test_direct_c_abi_call_without_the_python_operator():
     lse = torch.empty(1, 2, 128, dtype=torch.float32, device=DEV)
     a = _cabi.FwdArgs()
     _cabi.fill_fwd(a, qd, kd, vd, md, bd, out, lse, 0.125, True, 0.0)
-    os.environ["FDMA_COMPACT"] = "0"
+    a.compact_mode = _cabi.COMPACT_NEVER
     assert _cabi.lib.fdma_fwd_workspace_bytes(a) == 0
-    os.environ["FDMA_COMPACT"] = "2"
+    a.compact_mode = _cabi.COMPACT_ALWAYS
     need = _cabi.lib.fdma_fwd_workspace_bytes(a)
     assert need > 0
     if need:  # a caller that ignores the scratch request gets an error code and a message, not a fault
@@ -543,7 +543,7 @@ def test_graph_capture_and_replay_matches_eager(compact):
     """Forward + backward captured into a HIP graph (the library launches only kernels: no memset nodes, no host
     synchronisation, scratch comes from torch's graph-private pool) and replayed several times with eager work in
     between; every replay must reproduce the eager result bit for bit."""
-    os.environ["FDMA_COMPACT"] = compact
+    set_compact(compact)
     q, k, v, mask, bias = make_inputs(2, 512, 512, 4, 2, 64, (2, 2, 1, 512), (2, 2, 1, 512), 100, seed=3)
     qd, kd, vd, md, bd = _to_dev(q, k, v, mask, bias)
     qd, kd, vd, bd = [t.requires_grad_(True) for t in (qd, kd, vd, bd)]

@@ -10,7 +10,7 @@ import pytest
 import torch
 
 from oracle import eager
-from _util import GRAD_RTOL, OUT_ATOL, make_inputs
+from _util import GRAD_RTOL, OUT_ATOL, make_inputs, set_compact
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -46,7 +46,7 @@ def test_random_case_vs_eager_fp32(it, monkeypatch):
     from flash_sparse_attn import flash_sparse_attn_func
 
     c = _draw(it)
-    monkeypatch.setenv("FDMA_COMPACT", c["compact"])
+    set_compact(c["compact"])
     print({k: (str(v) if k == "dtype" else v) for k, v in c.items()}, flush=True)
     q, k, v, mask, bias = make_inputs(c["B"], c["Lq"], c["Lk"], c["H"], c["Hk"], c["D"], c["bias_shape"], c["mask_shape"], c["W"],
                                       seed=1000 + it, dtype=c["dtype"])
