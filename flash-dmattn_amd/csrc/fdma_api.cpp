@@ -8,6 +8,7 @@
 
 #include <hip/hip_runtime.h>
 
+#include <atomic>
 #include <cmath>
 #include <cstdarg>
 #include <cstdio>
@@ -181,6 +182,35 @@ int fill_varlen_params(const fdma_varlen_fwd_args *a, fdma::FwdParams &p) {
 
 }  // namespace
 
+// Scratch of fdma_fwd_noalloc: one array per GPU, part of the library's code object, alive until the process ends.
+// In host code the name below is only a handle for hipGetSymbolAddress -- it is not a device address; the address
+// that kernels and copies may use is looked up once per device (each GPU has its own copy at its own address).
+static __device__ __align__(256) unsigned char scratch[FDMA_NOALLOC_SCRATCH_BYTES];
+
+namespace {
+
+constexpr int kScratchDevices = 64;
+std::atomic<void *> g_scratch_ptr[kScratchDevices];
+
+// device address of `scratch` on the current device
+int scratch_of_current_device(void **out) {
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return fail(FDMA_ERR_LAUNCH, "hipGetDevice failed: %s", hipGetErrorString(e));
+    const bool cached = dev >= 0 && dev < kScratchDevices;
+    void *ptr = cached ? g_scratch_ptr[dev].load(std::memory_order_acquire) : nullptr;
+    if (!ptr) {
+        e = hipGetSymbolAddress(&ptr, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !ptr)
+            return fail(FDMA_ERR_LAUNCH, "hipGetSymbolAddress(scratch) failed on device %d: %s", dev, hipGetErrorString(e));
+        if (cached) g_scratch_ptr[dev].store(ptr, std::memory_order_release);
+    }
+    *out = ptr;
+    return FDMA_OK;
+}
+
+}  // namespace
+
 extern "C" {
 
 const char *fdma_last_error(void) { return g_err; }
@@ -239,6 +269,26 @@ int fdma_fwd(const fdma_fwd_args *a, void *hip_stream) {
     }
     if (e != hipSuccess) return fail(FDMA_ERR_LAUNCH, "forward launch failed: %s", hipGetErrorString(e));
     return FDMA_OK;
+}
+
+int fdma_fwd_noalloc(const fdma_fwd_args *a, void *hip_stream) {
+    g_err[0] = 0;
+    int rc = validate_common(a, false);
+    if (rc != FDMA_OK) return rc;
+    const size_t need = fdma_fwd_workspace_bytes(a);
+    if (need > (size_t)FDMA_NOALLOC_SCRATCH_BYTES)
+        return fail(FDMA_ERR_WORKSPACE, "fdma_fwd_noalloc: this problem needs %zu bytes of scratch, the library's static scratch holds %zu",
+                    need, (size_t)FDMA_NOALLOC_SCRATCH_BYTES);
+    fdma_fwd_args with_scratch = *a;
+    with_scratch.workspace = nullptr;
+    with_scratch.workspace_bytes = 0;
+    if (need) {
+        void *ptr = nullptr;
+        if ((rc = scratch_of_current_device(&ptr)) != FDMA_OK) return rc;
+        with_scratch.workspace = ptr;
+        with_scratch.workspace_bytes = FDMA_NOALLOC_SCRATCH_BYTES;
+    }
+    return fdma_fwd(&with_scratch, hip_stream);
 }
 
 int fdma_bwd_validate(const fdma_bwd_args *a) {

@@ -103,7 +103,7 @@ class DynBiasArgs(ctypes.Structure):
 
 
 EXPORTS = (
-    "fdma_fwd", "fdma_bwd", "fdma_fwd_workspace_bytes", "fdma_bwd_workspace_bytes",
+    "fdma_fwd", "fdma_fwd_noalloc", "fdma_bwd", "fdma_fwd_workspace_bytes", "fdma_bwd_workspace_bytes",
     "fdma_fwd_validate", "fdma_bwd_validate", "fdma_last_error", "fdma_abi_version",
     "fdma_sizeof_fwd_args", "fdma_sizeof_bwd_args",
     "fdma_varlen_fwd", "fdma_varlen_bwd", "fdma_varlen_fwd_validate", "fdma_varlen_bwd_validate",
@@ -118,6 +118,7 @@ EXPORTS = (
 # from the problem, 1 = never (tile skipping only), 2 = whenever the mask form allows it.  The environment variable
 # FDMA_COMPACT is read ONCE, here, as the default ("0" = never, "2" = always); set_compact_mode() changes it for
 # the process, compact_mode() for a with-block.
+NOALLOC_SCRATCH_BYTES = 8 << 20
 COMPACT_AUTO, COMPACT_NEVER, COMPACT_ALWAYS = 0, 1, 2
 _compact_mode = {"0": COMPACT_NEVER, "2": COMPACT_ALWAYS}.get(os.environ.get("FDMA_COMPACT", "")[:1], COMPACT_AUTO)
 
@@ -161,6 +162,8 @@ def _load() -> ctypes.CDLL:
         raise ImportError(f"cannot load {path}: {e}") from e
     lib.fdma_fwd.argtypes = [ctypes.POINTER(FwdArgs), ctypes.c_void_p]
     lib.fdma_fwd.restype = ctypes.c_int
+    lib.fdma_fwd_noalloc.argtypes = [ctypes.POINTER(FwdArgs), ctypes.c_void_p]
+    lib.fdma_fwd_noalloc.restype = ctypes.c_int
     lib.fdma_bwd.argtypes = [ctypes.POINTER(BwdArgs), ctypes.c_void_p]
     lib.fdma_bwd.restype = ctypes.c_int
     lib.fdma_fwd_validate.argtypes = [ctypes.POINTER(FwdArgs)]

@@ -43,7 +43,7 @@
 extern "C" {
 #endif
 
-#define FDMA_ABI_VERSION 3 /* 3: fdma_fwd_args.compact_mode (the struct grew); 2: fdma_varlen_*, fdma_create_mask, fdma_dyn_bias_* */
+#define FDMA_ABI_VERSION 3 /* 3: fdma_fwd_args.compact_mode (the struct grew), fdma_fwd_noalloc; 2: fdma_varlen_*, fdma_create_mask, fdma_dyn_bias_* */
 
 enum { FDMA_DTYPE_BF16 = 0, FDMA_DTYPE_FP16 = 1 };
 
@@ -110,6 +110,21 @@ int fdma_fwd(const fdma_fwd_args *args, void *hip_stream);
 /* Backward attention: dq, dk, dv, dbias, softmax_d.  Every output element is written exactly once
  * (no zero-fill needed by the caller), including masked / skipped regions of dbias. */
 int fdma_bwd(const fdma_bwd_args *args, void *hip_stream);
+
+/*
+ * fdma_fwd for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
+ * harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose mha_fwd allocates its split-KV
+ * partials with torch, flash_api.cpp:340-345).  args->workspace / workspace_bytes are ignored; the scratch of the
+ * decode path (split-KV partials) or of the compaction path lives in a static device array of
+ * FDMA_NOALLOC_SCRATCH_BYTES inside the library, which every GPU the library runs on holds until the process ends.
+ * A problem whose fdma_fwd_workspace_bytes() exceeds that returns FDMA_ERR_WORKSPACE and launches nothing.  The
+ * call makes no hipMalloc / hipFree (nor any other allocating call); results are bit-identical to fdma_fwd's.
+ * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (different streams or host
+ * threads) race on it -- serialise them.  Nothing in the array needs to start at zero; every call overwrites
+ * what it reads.
+ */
+#define FDMA_NOALLOC_SCRATCH_BYTES (8u << 20)
+int fdma_fwd_noalloc(const fdma_fwd_args *args, void *hip_stream);
 
 /* Scratch the caller must provide.  0 when none is needed.  Validate nothing but shapes. */
 size_t fdma_fwd_workspace_bytes(const fdma_fwd_args *args);

@@ -1,0 +1,79 @@
+"""fdma_fwd_noalloc -- the forward entry point that allocates nothing -- against fdma_fwd, through the C ABI.
+
+Both run the same kernels; the only difference is where the scratch lives (a static device array inside the library
+instead of a caller-provided workspace), so outputs and LSE must agree bit for bit.  Each case is called twice in a
+row, the second time on a smaller problem, so that whatever the first call left in the shared array is in place when
+the second one runs.  The outputs are also held to the oracle (the path's tolerance: max-abs error <= 2e-2).
+"""
+import pytest
+import torch
+
+from oracle import eager
+from _util import assert_out_close, make_inputs
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _call(entry, q, k, v, mask, bias, causal, mode, own_workspace):
+    from flash_sparse_attn import _cabi
+
+    B, Lq, H, D = q.shape
+    out = torch.full_like(q, float("nan"))
+    lse = torch.full((B, H, Lq), float("nan"), dtype=torch.float32, device=q.device)
+    a = _cabi.FwdArgs()
+    _cabi.fill_fwd(a, q, k, v, mask, bias, out, lse, D ** -0.5, causal, 0.0)
+    a.compact_mode = mode
+    need = _cabi.lib.fdma_fwd_workspace_bytes(a)
+    ws = None
+    if own_workspace and need:
+        ws = torch.empty(need, dtype=torch.uint8, device=q.device)
+        a.workspace, a.workspace_bytes = ws.data_ptr(), need
+    rc = getattr(_cabi.lib, entry)(a, _cabi.current_stream(q.device))
+    torch.cuda.synchronize()
+    return rc, out, lse, need
+
+
+def _case(kind, size, seed):
+    if kind == "decode":       # Lq = 1: split-KV partials in the scratch
+        B, Lk, H, Hk, D = size
+        q, k, v, mask, bias = make_inputs(B, 1, Lk, H, Hk, D, (B, Hk, 1, Lk), (B, Hk, 1, Lk), Lk // 8, seed=seed)
+        return q, k, v, mask, bias, False
+    B, L, H, Hk, D = size      # compacted forward: index lists and dense K / V copies in the scratch
+    q, k, v, mask, bias = make_inputs(B, L, L, H, Hk, D, (B, Hk, 1, L), (B, Hk, 1, L), L // 4, seed=seed)
+    return q, k, v, mask, bias, True
+
+
+@pytest.mark.parametrize("kind,sizes", [
+    ("decode", [(4, 32768, 16, 4, 128), (2, 8192, 8, 2, 128)]),
+    ("compact", [(1, 1024, 8, 2, 128), (2, 320, 4, 2, 64)]),
+])
+def test_noalloc_entry_point_matches_fdma_fwd_twice_in_a_row(kind, sizes):
+    from flash_sparse_attn import _cabi
+
+    mode = _cabi.COMPACT_ALWAYS if kind == "compact" else _cabi.COMPACT_AUTO
+    for n, size in enumerate(sizes):
+        q, k, v, mask, bias, causal = _case(kind, size, seed=100 + n)
+        qd, kd, vd, md, bd = [t.to(DEV) for t in (q, k, v, mask, bias)]
+        print(f"no-alloc case {kind} {size}", flush=True)
+        rc0, out0, lse0, need = _call("fdma_fwd", qd, kd, vd, md, bd, causal, mode, own_workspace=True)
+        assert rc0 == 0, _cabi.last_error()
+        assert 0 < need <= _cabi.NOALLOC_SCRATCH_BYTES, need   # the case does use scratch, and it fits
+        rc1, out1, lse1, _ = _call("fdma_fwd_noalloc", qd, kd, vd, md, bd, causal, mode, own_workspace=False)
+        assert rc1 == 0, _cabi.last_error()
+        assert torch.equal(out0.view(torch.int16), out1.view(torch.int16))
+        assert torch.equal(lse0.view(torch.int32), lse1.view(torch.int32))
+        ref, _ = eager.attention_forward(qd, kd, vd, md, bd, q.shape[-1] ** -0.5, causal)
+        assert_out_close(out1, ref)
+
+
+def test_noalloc_entry_point_rejects_what_does_not_fit():
+    from flash_sparse_attn import _cabi
+
+    L = 8192  # the compacted copies of K and V alone are 2 * 8192 * 2 * 128 * 2 bytes = 8 MiB
+    q, k, v, mask, bias, causal = _case("compact", (1, L, 4, 2, 128), seed=7)
+    qd, kd, vd, md, bd = [t.to(DEV) for t in (q, k, v, mask, bias)]
+    rc, out, _, need = _call("fdma_fwd_noalloc", qd, kd, vd, md, bd, causal, _cabi.COMPACT_ALWAYS, own_workspace=False)
+    assert need > _cabi.NOALLOC_SCRATCH_BYTES
+    assert rc == -3 and "static scratch" in _cabi.last_error()
+    assert torch.isnan(out.float()).all()   # nothing was launched
