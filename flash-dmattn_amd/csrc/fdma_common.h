@@ -53,6 +53,16 @@ template <> struct Elem<bf16_tag> {
     }
     static __device__ __forceinline__ float lo(uint32_t u) { return __uint_as_float(u << 16); }
     static __device__ __forceinline__ float hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
+    // acc + lo(pk) + hi(pk) in one instruction (v_dot2c_f32_bf16 with the constant (1, 1))
+    static __device__ __forceinline__ float add_pair(uint32_t pk, float acc) {
+        const bf16x2_t ones = {(__bf16)1.0f, (__bf16)1.0f};
+        return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, pk), ones, acc, false);
+    }
+    // Side-row arithmetic (see fdma_fwd_colmask.hip): an fp32 number x is handed to the MFMA as 16-bit pieces.
+    // kPieceScale: the pieces of a bias value hold x * kPieceScale and meet the constant 1 / kPieceScale (keeps the
+    // pieces inside the type's range).  kRefWeight: weight of the coarse piece of a reference point.  bf16 has the
+    // range of fp32, so both are 1.
+    static constexpr float kPieceScale = 1.f, kRefWeight = 1.f, kMaxFinite = 3.3895314e38f;
 };
 
 template <> struct Elem<fp16_tag> {
@@ -72,7 +82,43 @@ template <> struct Elem<fp16_tag> {
         f16x2_t h = __builtin_bit_cast(f16x2_t, u);
         return (float)h[1];
     }
+    static __device__ __forceinline__ float add_pair(uint32_t pk, float acc) {
+        const f16x2_t ones = {(_Float16)1.0f, (_Float16)1.0f};
+        return __builtin_amdgcn_fdot2(__builtin_bit_cast(f16x2_t, pk), ones, acc, false);
+    }
+    // fp16 ends at 65504: bias pieces hold x / 2 (|bias * log2e| < 94507), the coarse reference piece x / 64
+    static constexpr float kPieceScale = 0.5f, kRefWeight = 64.f, kMaxFinite = 65504.f;
 };
+
+// Three 16-bit pieces whose sum (in fp32) is x * kPieceScale to the last bit of x (8 or 11 significant bits each);
+// a non-finite x goes into the first piece alone.  Returned as {piece0 | piece1 << 16, piece2}.
+template <typename T> __device__ __forceinline__ u32x2_t split3(float x) {
+    using E = Elem<T>;
+    const float u = x * E::kPieceScale;
+    const uint32_t w0 = E::pack2(u, 0.f);
+    const float r1 = (__builtin_fabsf(u) <= 3.0e38f) ? u - E::lo(w0) : 0.f;
+    const uint32_t w1 = E::pack2(r1, 0.f);
+    const float r2 = r1 - E::lo(w1);
+    u32x2_t out;
+    out[0] = (w0 & 0xffffu) | (w1 << 16);
+    out[1] = E::pack2(r2, 0.f) & 0xffffu;
+    return out;
+}
+
+// Reference point of a softmax row as the MFMA sees it: minus the reference in two 16-bit pieces (a, b), worth
+// kRefWeight * a + b.  Returns the packed pair (a low, b high) and, in `enc`, the number the pair really stands for.
+template <typename T> __device__ __forceinline__ uint32_t encode_ref(float ref, float &enc) {
+    using E = Elem<T>;
+    const float lim = E::kMaxFinite;
+    float a = -ref * (1.f / E::kRefWeight);
+    a = fminf(fmaxf(a, -lim), lim);
+    const float ra = E::lo(E::pack2(a, 0.f)) * E::kRefWeight;
+    float b = -ref - ra;
+    b = fminf(fmaxf(b, -lim), lim);
+    const uint32_t w = E::pack2(a, b);
+    enc = -(E::lo(w) * E::kRefWeight + E::hi(w));
+    return w;
+}
 
 typedef __attribute__((address_space(3))) char lds_char_t;
 typedef __attribute__((address_space(3))) s16x4_t lds_s16x4_t;

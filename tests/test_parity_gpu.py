@@ -141,6 +141,55 @@ def test_fp16_inputs(compact):
         assert_grad_close(g.cpu(), r, n)
 
 
+@pytest.mark.parametrize("compact", ["0", "2"])
+@pytest.mark.parametrize("kind", ["late_bias_bf16", "late_bias_noncausal_bf16", "late_keys_fp16", "huge_scores_fp16", "first_tile_tiny_bf16"])
+def test_scores_that_leave_the_range_of_the_first_tile(kind, compact):
+    """The column-mask forward takes the reference point of every softmax row from the first key tile it visits and
+    checks later tiles against it; a workgroup in which a later score climbs out of that range (2^22 for bf16, 2^18 for
+    fp16 above the first tile's maximum) starts again on its classic path.  These inputs force that: keys, or bias
+    values, beyond the first tile that score tens of nats above it; fp16 scores too large for the 16-bit pieces that
+    carry the reference point (beyond 4e6 in the exp2 domain); and a first tile far BELOW the rest.  (Scaled-up keys
+    are tried in fp16 only: with 8-bit mantissas the rounding of the inputs alone moves such outputs by 0.1.)"""
+    set_compact(compact)
+    dtype = torch.float16 if kind.endswith("fp16") else torch.bfloat16
+    B, L, H, Hk, D = 1, 384, 4, 2, 64
+    q, k, v, mask, bias = make_inputs(B, L, L, H, Hk, D, (B, Hk, 1, L), (B, Hk, 1, L), 256, seed=41, dtype=dtype)
+    causal = kind != "late_bias_noncausal_bf16"
+    if kind.startswith("late_keys"):      # keys 200.. score 3x higher and carry +25 of bias: tens of nats above the first 64
+        k = k.clone()
+        k[:, 200:] = (k[:, 200:].float() * 3).to(dtype)
+        bias = bias.clone()
+        bias[..., 200:] += 25.0
+    elif kind.startswith("late_bias"):
+        bias = bias.clone()
+        bias[..., 130:] += 60.0
+    elif kind == "huge_scores_fp16":      # |q . k| * scale * log2(e) up to about 1e7
+        q = (q.float().sign() * 230).to(dtype)
+        k = (k.float().sign() * 230).to(dtype)
+    else:                                 # the first tile scores far below every other key
+        k = k.clone()
+        k[:, :64] = (k[:, :64].float() * 0.01).to(dtype)
+        bias = bias.clone()
+        bias[..., :64] -= 50.0
+    scale = 1.0 if kind == "huge_scores_fp16" else None
+    out, lse, (dq, dk, dv, db) = _run_fwd_bwd(q, k, v, mask, bias, causal, scale=scale)
+    ro, rl = c_oracle.forward(q, k, v, mask, bias, scale, causal)
+    if kind == "huge_scores_fp16":
+        # fp32 accumulators resolve scores of 4e6 to 0.5: keys that tie in q . k are told apart by their bias only
+        # coarsely, so the output is held to the value range and to the LSE, not to the oracle's mixture
+        assert torch.isfinite(out.float()).all() and out.float().abs().max() <= v.float().abs().max()
+    else:
+        assert_out_close(out.cpu(), ro)
+    assert torch.equal(torch.isinf(lse.cpu()), torch.isinf(rl))
+    fin = torch.isfinite(rl)
+    # (the scaled queries are rounded to 16 bits before the MFMAs: the LSE of huge scores carries that relative error)
+    assert ((lse.cpu()[fin] - rl[fin]).abs() <= 1e-2 + 3e-3 * rl[fin].abs()).all()
+    if kind != "huge_scores_fp16":  # (gradients of 1e7-sized scores overflow the 16-bit outputs; the forward is the point)
+        rdq, rdk, rdv, rdb = c_oracle.backward(q, k, v, torch.ones_like(ro), mask, bias, scale, causal)
+        for g, r, n in ((dq, rdq, "dq"), (dk, rdk, "dk"), (dv, rdv, "dv"), (db, rdb, "dbias")):
+            assert_grad_close(g.cpu(), r, n)
+
+
 def test_cfg1_reference_plumbing_config():
     """Config 1 of the benchmark: B=1, L=256, H=2, Hkv=1 (MQA), d=64, bias [B,Hkv,1,Lk], mask = top-128
     keys by bias intersected with causal (given both as a full-shape mask and as column mask +
