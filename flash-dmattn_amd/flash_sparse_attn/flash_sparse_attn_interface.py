@@ -42,13 +42,11 @@ def _aligned(x: Optional[torch.Tensor], elems: int) -> Optional[torch.Tensor]:
     return x if ok else x.contiguous().clone(memory_format=torch.contiguous_format)
 
 
-def _direct_when_eager(op):
+def _direct_when_eager(op, body):
     """Callable for one of the operators below.  On plain tensors in eager mode it runs the operator's Python
     body directly: the dispatch of a torch.library operator costs about 20 us per call, more than a small
     attention call takes on the device.  Under torch.compile, and for fake tensors or tensor subclasses, the
     registered operator is called, as the reference always does (flash_sparse_attn_interface.py:126, 432)."""
-    body = op._init_fn
-
     def call(*args, **kwargs):
         if torch.compiler.is_compiling() or any(type(a) is not torch.Tensor for a in args[:3]):
             return op(*args, **kwargs)
@@ -103,8 +101,7 @@ def _check_inputs(q, k, v, mask, bias) -> None:
             raise RuntimeError(f"Key length dimension in {name} must be seqlen_k_rounded")
 
 
-@torch.library.custom_op("flash_sparse_attn::_flash_sparse_attn_forward", mutates_args=(), device_types="cuda")
-def _flash_sparse_attn_forward(
+def _flash_sparse_attn_forward_body(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Optional[torch.Tensor], bias: Optional[torch.Tensor],
     softmax_scale: float, is_causal: bool, softcap: float, return_softmax: bool,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
@@ -132,6 +129,9 @@ def _flash_sparse_attn_forward(
     return out, softmax_lse, p
 
 
+_flash_sparse_attn_forward = torch.library.custom_op("flash_sparse_attn::_flash_sparse_attn_forward", mutates_args=(), device_types="cuda")(_flash_sparse_attn_forward_body)
+
+
 @torch.library.register_fake("flash_sparse_attn::_flash_sparse_attn_forward")
 def _flash_sparse_attn_forward_fake(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Optional[torch.Tensor], bias: Optional[torch.Tensor],
@@ -144,13 +144,10 @@ def _flash_sparse_attn_forward_fake(
     return out, softmax_lse, p
 
 
-_wrapped_flash_sparse_attn_forward = _direct_when_eager(_flash_sparse_attn_forward)
+_wrapped_flash_sparse_attn_forward = _direct_when_eager(_flash_sparse_attn_forward, _flash_sparse_attn_forward_body)
 
 
-@torch.library.custom_op(
-    "flash_sparse_attn::_flash_sparse_attn_backward", mutates_args=("dq", "dk", "dv", "dbias"), device_types="cuda"
-)
-def _flash_sparse_attn_backward(
+def _flash_sparse_attn_backward_body(
     dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Optional[torch.Tensor], bias:
     Optional[torch.Tensor], out: torch.Tensor, softmax_lse: torch.Tensor, dq: Optional[torch.Tensor], dk:
     Optional[torch.Tensor], dv: Optional[torch.Tensor], dbias: Optional[torch.Tensor], softmax_scale: float,
@@ -233,6 +230,11 @@ def _flash_sparse_attn_backward(
     return softmax_d
 
 
+_flash_sparse_attn_backward = torch.library.custom_op(
+    "flash_sparse_attn::_flash_sparse_attn_backward", mutates_args=("dq", "dk", "dv", "dbias"), device_types="cuda"
+)(_flash_sparse_attn_backward_body)
+
+
 @torch.library.register_fake("flash_sparse_attn::_flash_sparse_attn_backward")
 def _flash_sparse_attn_backward_fake(
     dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Optional[torch.Tensor], bias:
@@ -244,7 +246,7 @@ def _flash_sparse_attn_backward_fake(
     return torch.empty((batch_size, num_heads, round_multiple(seqlen_q, 128)), device=q.device, dtype=torch.float32)
 
 
-_wrapped_flash_sparse_attn_backward = _direct_when_eager(_flash_sparse_attn_backward)
+_wrapped_flash_sparse_attn_backward = _direct_when_eager(_flash_sparse_attn_backward, _flash_sparse_attn_backward_body)
 
 
 def _pad_key_dim(t: Optional[torch.Tensor], seqlen_k: int, elems: int) -> Optional[torch.Tensor]:
@@ -269,6 +271,13 @@ def _nothing_to_differentiate(grad_enabled: bool, *tensors: Optional[torch.Tenso
         if t is not None and (type(t) is not torch.Tensor or (grad_enabled and t.requires_grad)):
             return False
     return True
+
+
+class _NoGradContext:
+    """Stands in for the autograd context when FlashDMAttnFunc.forward is called directly (nothing to differentiate)."""
+
+    def save_for_backward(self, *tensors):
+        pass
 
 
 class FlashDMAttnFunc(torch.autograd.Function):
@@ -403,7 +412,7 @@ def flash_sparse_attn_func(
     args = (query, key, value, attn_mask, attn_bias, softmax_scale, is_causal, softcap, deterministic, return_attn_probs,
             grad_enabled)
     if _nothing_to_differentiate(grad_enabled, query, key, value, attn_bias):
-        return FlashDMAttnFunc.forward(None, *args)  # (the context is only touched when gradients are wanted)
+        return FlashDMAttnFunc.forward(_NoGradContext(), *args)
     return FlashDMAttnFunc.apply(*args)
 
 
@@ -433,8 +442,7 @@ def _check_varlen_inputs(q, k, v, cu_seqlens_q, cu_seqlens_k) -> None:
         raise RuntimeError("cu_seqlens_k must have shape (batch_size + 1)")
 
 
-@torch.library.custom_op("flash_sparse_attn::_flash_sparse_attn_varlen_forward", mutates_args=(), device_types="cuda")
-def _flash_sparse_attn_varlen_forward(
+def _flash_sparse_attn_varlen_forward_body(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor,
     max_seqlen_q: int, max_seqlen_k: int, softmax_scale: float, is_causal: bool, softcap: float = 0.0, return_softmax:
     bool = False, block_table: Optional[torch.Tensor] = None, leftpad_k: Optional[torch.Tensor] = None, seqused_k:
@@ -462,6 +470,9 @@ def _flash_sparse_attn_varlen_forward(
     return out, softmax_lse, p
 
 
+_flash_sparse_attn_varlen_forward = torch.library.custom_op("flash_sparse_attn::_flash_sparse_attn_varlen_forward", mutates_args=(), device_types="cuda")(_flash_sparse_attn_varlen_forward_body)
+
+
 @torch.library.register_fake("flash_sparse_attn::_flash_sparse_attn_varlen_forward")
 def _flash_sparse_attn_varlen_forward_fake(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, cu_seqlens_q: torch.Tensor, cu_seqlens_k: torch.Tensor,
@@ -476,13 +487,10 @@ def _flash_sparse_attn_varlen_forward_fake(
     return out, softmax_lse, p
 
 
-_wrapped_flash_sparse_attn_varlen_forward = _direct_when_eager(_flash_sparse_attn_varlen_forward)
+_wrapped_flash_sparse_attn_varlen_forward = _direct_when_eager(_flash_sparse_attn_varlen_forward, _flash_sparse_attn_varlen_forward_body)
 
 
-@torch.library.custom_op(
-    "flash_sparse_attn::_flash_sparse_attn_varlen_backward", mutates_args=("dq", "dk", "dv"), device_types="cuda"
-)
-def _flash_sparse_attn_varlen_backward(
+def _flash_sparse_attn_varlen_backward_body(
     dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, softmax_lse:
     torch.Tensor, dq: Optional[torch.Tensor], dk: Optional[torch.Tensor], dv: Optional[torch.Tensor], cu_seqlens_q:
     torch.Tensor, cu_seqlens_k: torch.Tensor, max_seqlen_q: int, max_seqlen_k: int, softmax_scale: float, is_causal:
@@ -536,6 +544,11 @@ def _flash_sparse_attn_varlen_backward(
     return softmax_d
 
 
+_flash_sparse_attn_varlen_backward = torch.library.custom_op(
+    "flash_sparse_attn::_flash_sparse_attn_varlen_backward", mutates_args=("dq", "dk", "dv"), device_types="cuda"
+)(_flash_sparse_attn_varlen_backward_body)
+
+
 @torch.library.register_fake("flash_sparse_attn::_flash_sparse_attn_varlen_backward")
 def _flash_sparse_attn_varlen_backward_fake(
     dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, out: torch.Tensor, softmax_lse:
@@ -547,7 +560,7 @@ def _flash_sparse_attn_varlen_backward_fake(
     return torch.empty((num_heads, total_q), device=q.device, dtype=torch.float32)
 
 
-_wrapped_flash_sparse_attn_varlen_backward = _direct_when_eager(_flash_sparse_attn_varlen_backward)
+_wrapped_flash_sparse_attn_varlen_backward = _direct_when_eager(_flash_sparse_attn_varlen_backward, _flash_sparse_attn_varlen_backward_body)
 
 
 class FlashAttnVarlenFunc(torch.autograd.Function):

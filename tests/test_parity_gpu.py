@@ -190,6 +190,31 @@ def test_scores_that_leave_the_range_of_the_first_tile(kind, compact):
             assert_grad_close(g.cpu(), r, n)
 
 
+@pytest.mark.parametrize("D", [36, 100])
+def test_head_dim_that_is_not_a_multiple_of_8(D):
+    """FlashDMAttnFunc pads q, k, v (and dout) with zero columns up to a multiple of 8 and slices the outputs and
+    gradients back (flash_sparse_attn_interface.py:415-419, 466-469, 491-493 of the reference); the default scale is
+    that of the ORIGINAL head dim."""
+    q, k, v, mask, bias = make_inputs(2, 200, 264, 4, 2, D, (2, 2, 1, 264), (2, 2, 1, 264), 96, seed=D)
+    for compact in ("0", "2"):
+        set_compact(compact)
+        out, lse, (dq, dk, dv, db) = _run_fwd_bwd(q, k, v, mask, bias, True)
+        assert out.shape == q.shape and dq.shape == q.shape and dk.shape == k.shape and dv.shape == v.shape
+        ro, rl = c_oracle.forward(q, k, v, mask, bias, None, True)
+        assert_out_close(out.cpu(), ro)
+        _check_lse(lse.cpu(), rl)
+        rdq, rdk, rdv, rdb = c_oracle.backward(q, k, v, torch.ones_like(ro), mask, bias, None, True)
+        for g, r, n in ((dq, rdq, "dq"), (dk, rdk, "dk"), (dv, rdv, "dv"), (db, rdb, "dbias")):
+            assert_grad_close(g.cpu(), r, n)
+    # without gradients (the call that skips the autograd node), per-query mask: the general kernels
+    qd, kd, vd = _to_dev(q, k, v)
+    full = mask.expand(2, 2, 200, 264).contiguous().to(DEV)
+    with torch.no_grad():
+        out2 = _op()(qd, kd, vd, full, bias.to(DEV), None, True)
+    assert out2.shape == q.shape
+    assert_out_close(out2.cpu(), ro)
+
+
 def test_cfg1_reference_plumbing_config():
     """Config 1 of the benchmark: B=1, L=256, H=2, Hkv=1 (MQA), d=64, bias [B,Hkv,1,Lk], mask = top-128
     keys by bias intersected with causal (given both as a full-shape mask and as column mask +
