@@ -126,6 +126,20 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) fwd_colmask_kernel(c
     const int shift = LkS - LqS;
     const int wrow0 = m0 + wave * 32;  // first query row of this wave
 
+    // ---- Q fragments: the loads are issued first of all (they depend on the workgroup's coordinates only), the
+    // values are looked at -- scaled -- after the set-up below, whose own memory traffic they overlap with
+    u32x4_t qf[KS];
+    {
+        const int qrow = wrow0 + r;
+        const int qc = qrow < LqS ? qrow : LqS - 1;
+        const uint16_t *qp = (const uint16_t *)p.q + b * p.q_b + (sq.q0 + qc) * p.q_r + h * p.q_h;
+#pragma unroll
+        for (int ks = 0; ks < KS; ks++) {
+            const int c = ks * 16 + g * 8;
+            qf[ks] = *(const u32x4_t *)(qp + (c < p.d ? c : 0));  // (chunks beyond d are cleared when scaled)
+        }
+    }
+
     const int hm = p.mask ? (p.Hm == p.H ? h : (p.Hm == 1 ? 0 : h / (p.H / p.Hm))) : 0;
     const int hb = p.bias ? (p.Hb == p.H ? h : (p.Hb == 1 ? 0 : h / (p.H / p.Hb))) : 0;
     const uint8_t *mrow = p.mask ? p.mask + b * p.m_b + hm * p.m_h : nullptr;
@@ -213,25 +227,6 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) fwd_colmask_kernel(c
         it_word &= it_word - 1;
         return j < n_end ? j : n_end;
     };
-
-    // ---- Q fragments
-    u32x4_t qf[KS];
-    {
-        const int qrow = wrow0 + r;
-        const int qc = qrow < LqS ? qrow : LqS - 1;
-        const uint16_t *qp = (const uint16_t *)p.q + b * p.q_b + (sq.q0 + qc) * p.q_r + h * p.q_h;
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++) {
-            const int c = ks * 16 + g * 8;
-            u32x4_t v = {0, 0, 0, 0};
-            if (qrow < LqS && c < p.d) v = *(const u32x4_t *)(qp + c);
-            // Q is scaled by softmax_scale * log2(e) once, here (the reference also rounds the scaled Q to the
-            // input type, flash_fwd_kernel.h:428-439): the MFMAs then produce exp2-domain scores directly
-#pragma unroll
-            for (int e = 0; e < 4; e++) v[e] = E::pack2(E::lo(v[e]) * p.scale_log2, E::hi(v[e]) * p.scale_log2);
-            qf[ks] = v;
-        }
-    }
 
     f32x16_t o[DB];
     float row_sum = 0.f;
@@ -551,14 +546,35 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) fwd_colmask_kernel(c
         set_tile_x(j0);
         load_regs(false);
         load_regs(true);
+        u32x4_t k1[K_IT];  // K(1) travels in registers of its own, together with K(0)
+        set_tile_k(jn1 < n_end ? jn1 : j0);
+        if (role_k) {
+#pragma unroll
+            for (int it = 0; it < K_IT; it++)
+                k1[it] = *(const __attribute__((address_space(1))) u32x4_t *)(tb_k + (last_k ? soff_l[it] : soff[it]));
+        }
         store_k(0);
         store_x(0);
-        set_tile_k(jn1 < n_end ? jn1 : j0);
         set_tile_x(jn1 < n_end ? jn1 : j0);
-        load_regs(false);
+        if (role_k) {
+#pragma unroll
+            for (int it = 0; it < K_IT; it++) sreg[it] = k1[it];
+        }
         store_k(1);
         set_tile_k(jn2 < n_end ? jn2 : j0);
         load_regs(false);
+        // Q is scaled by softmax_scale * log2(e) once, here (the reference also rounds the scaled Q to the input type,
+        // flash_fwd_kernel.h:428-439): the MFMAs then produce exp2-domain scores directly
+        {
+            const bool row_ok = wrow0 + r < LqS;
+#pragma unroll
+            for (int ks = 0; ks < KS; ks++) {
+                const bool ok = row_ok && ks * 16 + g * 8 < p.d;
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    qf[ks][e] = ok ? E::pack2(E::lo(qf[ks][e]) * p.scale_log2, E::hi(qf[ks][e]) * p.scale_log2) : 0u;
+            }
+        }
         __syncthreads();
 
         f32x16_t sA, sB;
