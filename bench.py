@@ -29,11 +29,57 @@ import torch  # noqa: E402
 
 PEAK_BF16_TFLOPS = 2500.0  # MI355X dense bf16 MFMA
 PEAK_HBM_GBS = 8000.0      # MI355X HBM3E
-# HBM bytes per launch of the forward kernel on the headline workload, from two rocprofv3 --pmc runs of
-# this script (FETCH_SIZE, WRITE_SIZE; each scaled by what the counter reads for a 256 MiB device copy,
-# see --calib-copy): compacted kernel 82 MiB read + 65 MiB written, tile-skipping kernel 141 + 65 MiB.
-# Override with --traffic-bytes after re-measuring.
-MEASURED_FWD_TRAFFIC_BYTES = {True: 147.0 * 1024 * 1024, False: 206.0 * 1024 * 1024}
+# HBM bytes per launch of the forward kernel on the headline workload come from two rocprofv3 --pmc runs of this
+# script (FETCH_SIZE, WRITE_SIZE; each scaled by what the counter reads for a 256 MiB device copy, see --calib-copy).
+# `python bench.py --summarise-pmc <fetch csv> <write csv>` turns the two counter files into TRAFFIC_FILE, which is
+# tracked; a normal run reports what that file says (null when it is missing).  --traffic-bytes overrides it.
+TRAFFIC_FILE = os.path.join(ROOT, "profiles", "fwd_colmask_cfg2_hbm_traffic.txt")
+
+
+def read_traffic(compacted):
+    """HBM bytes per launch of the forward kernel (compacted or tile-skipping variant) from TRAFFIC_FILE, or None."""
+    key = "compacted_bytes" if compacted else "tile_skip_bytes"
+    try:
+        for line in open(TRAFFIC_FILE):
+            if line.startswith(key + " ="):
+                return float(line.split("=")[1].split()[0])
+    except OSError:
+        pass
+    return None
+
+
+def summarise_pmc(fetch_csv, write_csv):
+    """Reads the counter_collection CSVs of the two --pmc passes (FETCH_SIZE, then WRITE_SIZE; both with --calib-copy)
+    and writes TRAFFIC_FILE: per forward kernel variant, read + written HBM bytes per launch, each counter scaled by
+    what it reads for the 256 MiB copy."""
+    import csv
+    import re
+
+    def per_kernel(path, counter):
+        acc = {}
+        for row in csv.DictReader(open(path)):
+            if row.get("Counter_Name") != counter:
+                continue
+            name = row["Kernel_Name"]
+            acc.setdefault(name, []).append(float(row["Counter_Value"]))
+        return {k: sum(v) / len(v) for k, v in acc.items()}
+
+    fetch, write = per_kernel(fetch_csv, "FETCH_SIZE"), per_kernel(write_csv, "WRITE_SIZE")
+    copy_kib = 256.0 * 1024
+    f_scale = copy_kib / next(v for k, v in fetch.items() if "copyBuffer" in k)
+    w_scale = copy_kib / next(v for k, v in write.items() if "copyBuffer" in k)
+    lines = ["# HBM traffic per launch of fdma::fwd_colmask_kernel on bench.py's headline workload (cfg2), written by",
+             "# `python bench.py --summarise-pmc`; FETCH_SIZE / WRITE_SIZE are KiB per dispatch, scaled by the factors below",
+             "fetch_scale = %.4f" % f_scale, "write_scale = %.4f" % w_scale]
+    for key, cmp_flag in (("compacted_bytes", "true"), ("tile_skip_bytes", "false")):
+        pat = re.compile(r"fwd_colmask_kernel<.*128.*, %s>" % cmp_flag)
+        fk = [v for k, v in fetch.items() if pat.search(k)]
+        wk = [v for k, v in write.items() if pat.search(k)]
+        if fk and wk:
+            lines.append("%s = %.0f   (read %.1f MiB + written %.1f MiB)" % (
+                key, (fk[0] * f_scale + wk[0] * w_scale) * 1024, fk[0] * f_scale / 1024, wk[0] * w_scale / 1024))
+    open(TRAFFIC_FILE, "w").write("\n".join(lines) + "\n")
+    print("\n".join(lines))
 
 CONFIGS = {
     # name: B, Lq, Lk, H, Hk, D, bias shape, window, causal, passes
@@ -307,6 +353,44 @@ def run_ragged_batch(steps, warmup, device):
             "ms_fwd_bwd": ms_fb, "tflops_fwd_bwd": 3.5 * flops / ms_fb / 1e9}
 
 
+def run_sweeps(steps, warmup, device):
+    """Runtime against the window W and against the sequence length L (the reference's claim: README.md:181-191,
+    benchmarks/forward_performance.py:661-718), for both paths of the column-mask kernels.  Shapes: H=32, Hkv=8, d=128,
+    bias [1,8,1,L], mask = top-W of the bias per row, causal.  W sweep at L=8192; L sweep at W=1024.  A least-squares
+    line ms = a + b * x is fitted to every column."""
+    def fit(xs, ys):
+        n = len(xs)
+        mx, my = sum(xs) / n, sum(ys) / n
+        sxx = sum((x - mx) ** 2 for x in xs)
+        b = sum((x - mx) * (y - my) for x, y in zip(xs, ys)) / sxx
+        a = my - b * mx
+        ss_res = sum((y - (a + b * x)) ** 2 for x, y in zip(xs, ys))
+        ss_tot = sum((y - my) ** 2 for y in ys) or 1.0
+        return {"intercept_ms": a, "slope_ms_per_1024": b * 1024, "r2": 1.0 - ss_res / ss_tot}
+
+    def sweep(points, key):
+        rows = []
+        for c in points:
+            CONFIGS["_sweep"] = c
+            row = {"L": c["Lq"], "W": c["W"]}
+            for compact, tag in ((True, "compacted"), (False, "tile_skip")):
+                r = run_config("_sweep", steps, warmup, device, compact)
+                row["ms_fwd_" + tag] = r["ms_fwd"]
+                row["ms_fwd_bwd_" + tag] = r["ms_fwd_bwd"]
+                row["n_exec_" + tag] = r["n_exec"]
+            rows.append(row)
+        del CONFIGS["_sweep"]
+        fits = {col: fit([r[key] for r in rows], [r[col] for r in rows])
+                for col in ("ms_fwd_compacted", "ms_fwd_bwd_compacted", "ms_fwd_tile_skip", "ms_fwd_bwd_tile_skip")}
+        return {"points": rows, "fit_ms_vs_" + key: fits}
+
+    def cfg(L, W):
+        return dict(B=1, Lq=L, Lk=L, H=32, Hk=8, D=128, bias=(1, 8, 1, L), W=W, causal=True, bwd=True, scale=None)
+
+    return {"w_sweep": sweep([cfg(8192, W) for W in (256, 512, 1024, 2048, 4096, 8192)], "W"),
+            "l_sweep": sweep([cfg(L, 1024) for L in (2048, 4096, 8192, 16384, 32768)], "L")}
+
+
 def cpu_baseline(device_cfg="cfg2", groups=8, chunk=2):
     """The fp32 safe-eager restatement (oracle/eager.py, a port of the reference's eager formula) timed
     on the host cores for a bounded sample of the headline workload: `groups` KV groups (each with its
@@ -350,7 +434,12 @@ def main():
                     help="also run one plain 256 MiB device copy (reference point for FETCH_SIZE / WRITE_SIZE counters)")
     ap.add_argument("--traffic-bytes", type=float, default=None,
                     help="HBM bytes per launch of the dominant kernel from rocprofv3 --pmc runs (reported as roofline.traffic)")
+    ap.add_argument("--summarise-pmc", nargs=2, metavar=("FETCH_CSV", "WRITE_CSV"),
+                    help="no GPU work: turn the counter CSVs of two rocprofv3 --pmc passes into " + os.path.relpath(TRAFFIC_FILE, ROOT))
     args = ap.parse_args()
+    if args.summarise_pmc:
+        summarise_pmc(*args.summarise_pmc)
+        return
     if args.gpus != 1:
         print("bench.py measures one GPU: the hot path has no multi-GPU part in this build; run with --gpus 1", file=sys.stderr)
         sys.exit(2)
@@ -399,7 +488,7 @@ def main():
             "peak": PEAK_BF16_TFLOPS,
             "unit": "TFLOP/s",
             "frac": main_res["tflops_fwd"] / PEAK_BF16_TFLOPS,
-            "traffic": MEASURED_FWD_TRAFFIC_BYTES[bool(main_res["compacted"])],
+            "traffic": read_traffic(bool(main_res["compacted"])),
             "kernel": kernel,
             "flops_per_launch": 4.0 * 64 * 64 * c["D"] * main_res["n_exec"],
             "duration_ms": main_res["ms_fwd"],
@@ -424,6 +513,7 @@ def main():
         out["mask_builder"] = run_mask_builder(max(3, args.steps // 2), max(1, args.warmup // 2), device)
         out["bias_producer"] = run_bias_producer(max(3, args.steps // 2), max(1, args.warmup // 2), device)
         out["ragged_batch"] = run_ragged_batch(max(3, args.steps // 4), max(1, args.warmup // 2), device)
+        out.update(run_sweeps(max(3, args.steps // 4), max(1, args.warmup // 2), device))
     if not args.no_cpu:
         out["cpu_baseline"] = cpu_baseline("cfg2", groups=8)
     print(json.dumps(out))
