@@ -209,6 +209,18 @@ int scratch_of_current_device(void **out) {
     return FDMA_OK;
 }
 
+// A stream that is being captured into a HIP graph is refused: the one capture of forward + backward through the
+// tensor library ended in a host-side crash when the capture was closed, the cause is not known, and until it is
+// the library does not record its launches into graphs.  A clear error here replaces that crash.
+int refuse_capture(void *hip_stream, const char *who) {
+    hipStreamCaptureStatus st = hipStreamCaptureStatusNone;
+    const hipError_t e = hipStreamIsCapturing(static_cast<hipStream_t>(hip_stream), &st);
+    if (e != hipSuccess) return fail(FDMA_ERR_LAUNCH, "%s: hipStreamIsCapturing failed: %s", who, hipGetErrorString(e));
+    if (st != hipStreamCaptureStatusNone)
+        return fail(FDMA_ERR_UNSUPPORTED, "%s: the stream is being captured into a HIP graph; capture of this library's launches is not supported", who);
+    return FDMA_OK;
+}
+
 }  // namespace
 
 extern "C" {
@@ -237,6 +249,7 @@ size_t fdma_fwd_workspace_bytes(const fdma_fwd_args *a) {
 }
 
 int fdma_fwd(const fdma_fwd_args *a, void *hip_stream) {
+    if (int cap = refuse_capture(hip_stream, "fdma_fwd")) return cap;
     g_err[0] = 0;
     int rc = validate_common(a, false);
     if (rc != FDMA_OK) return rc;
@@ -342,6 +355,7 @@ size_t fdma_bwd_workspace_bytes(const fdma_bwd_args *a) {
 }
 
 int fdma_bwd(const fdma_bwd_args *a, void *hip_stream) {
+    if (int cap = refuse_capture(hip_stream, "fdma_bwd")) return cap;
     int rc = fdma_bwd_validate(a);
     if (rc != FDMA_OK) return rc;
     fdma::BwdParams p;
@@ -388,6 +402,7 @@ int fdma_varlen_fwd_validate(const fdma_varlen_fwd_args *a) {
 }
 
 int fdma_varlen_fwd(const fdma_varlen_fwd_args *a, void *hip_stream) {
+    if (int cap = refuse_capture(hip_stream, "fdma_varlen_fwd")) return cap;
     g_err[0] = 0;
     int rc = validate_varlen(a, false);
     if (rc != FDMA_OK) return rc;
@@ -419,6 +434,7 @@ int fdma_varlen_bwd_validate(const fdma_varlen_bwd_args *a) {
 }
 
 int fdma_varlen_bwd(const fdma_varlen_bwd_args *a, void *hip_stream) {
+    if (int cap = refuse_capture(hip_stream, "fdma_varlen_bwd")) return cap;
     int rc = fdma_varlen_bwd_validate(a);
     if (rc != FDMA_OK) return rc;
     fdma::BwdParams p;
@@ -488,6 +504,7 @@ static uint32_t to_bits16(float x, int dtype) {
 }
 
 int fdma_create_mask(const fdma_mask_args *a, void *hip_stream) {
+    if (int cap = refuse_capture(hip_stream, "fdma_create_mask")) return cap;
     int rc = fdma_create_mask_validate(a);
     if (rc != FDMA_OK) return rc;
     fdma::MaskParams p;
@@ -554,6 +571,7 @@ size_t fdma_dyn_bias_bwd_workspace_bytes(const fdma_dyn_bias_args *a) {
 }
 
 int fdma_dyn_bias_fwd(const fdma_dyn_bias_args *a, void *hip_stream) {
+    if (int cap = refuse_capture(hip_stream, "fdma_dyn_bias_fwd")) return cap;
     int rc = fdma_dyn_bias_validate(a, 0);
     if (rc != FDMA_OK) return rc;
     fdma::DynBiasParams p;
@@ -564,6 +582,7 @@ int fdma_dyn_bias_fwd(const fdma_dyn_bias_args *a, void *hip_stream) {
 }
 
 int fdma_dyn_bias_bwd(const fdma_dyn_bias_args *a, void *hip_stream) {
+    if (int cap = refuse_capture(hip_stream, "fdma_dyn_bias_bwd")) return cap;
     int rc = fdma_dyn_bias_validate(a, 1);
     if (rc != FDMA_OK) return rc;
     fdma::DynBiasParams p;

@@ -511,6 +511,8 @@ __global__ void __launch_bounds__(NTHREADS) bwd_dkdv_reduce_kernel(const BwdPara
     const int U = plan[0], Gs = plan[1], Sm = plan[2], Q = plan[4], per = Gs * Sm;
     const int unit = blockIdx.x;
     if (per == 1 || unit >= U) return;
+    // a plan whose lists overflowed left parts uncomputed: every sum starts from NaN then
+    const float start = plan[6] != 0 ? __builtin_nanf("") : 0.f;
     int lo = 0, hi = f.B * f.Hk;
     while (hi - lo > 1) {
         const int mid = (lo + hi) >> 1;
@@ -531,7 +533,7 @@ __global__ void __launch_bounds__(NTHREADS) bwd_dkdv_reduce_kernel(const BwdPara
     for (int c = 2 * blockIdx.y + half; c == 2 * (int)blockIdx.y + half && c * 8 < f.d; c += NTHREADS / KV_BN) {
         float ak[8], av[8];
 #pragma unroll
-        for (int e = 0; e < 8; e++) { ak[e] = 0.f; av[e] = 0.f; }
+        for (int e = 0; e < 8; e++) { ak[e] = start; av[e] = start; }
         // written slots in a fixed order, two at a time so that more loads are in flight
         const int n_w = Gs * n_seg;
         for (int j = 0; j < n_w; j += 2) {
@@ -574,12 +576,12 @@ __global__ void __launch_bounds__(NTHREADS) bwd_dkdv_reduce_kernel(const BwdPara
         };
         if (f.Hb == f.H) {
             for (int gi = half; gi < G; gi += NTHREADS / KV_BN) {
-                float tot = 0.f;
+                float tot = start;
                 for (int sg = 0; sg < n_seg; sg++) tot += dbp[((int64_t)((gi / gper) * Sm + sg) * G + gi % gper) * KV_BN];
                 emit(hk * G + gi, tot);
             }
         } else if (half == 0) {
-            float tot = 0.f;
+            float tot = start;
             for (int gs = 0; gs < Gs; gs++)
                 for (int sg = 0; sg < n_seg; sg++)
                     for (int gl = 0; gl < gper; gl++) tot += dbp[((int64_t)(gs * Sm + sg) * G + gl) * KV_BN];
@@ -959,8 +961,8 @@ hipError_t launch_dq(const BwdParams &p, hipStream_t stream) {
     constexpr int BN = D > 64 ? 32 : 64;  // at d = 128 a 64-key tile would spill registers
     auto kern = p.f.cmp.on ? bwd_dq_colmask_kernel<T, D, BN, CAUSAL, true> : bwd_dq_colmask_kernel<T, D, BN, CAUSAL, false>;
     const int smem = DqcSmem<D, BN>::TOTAL;
-    static DynSmemLimit smem_limit;
-    hipError_t e = smem_limit.ensure((const void *)kern, (int)smem);
+    static DynSmemLimit smem_limit[2];  // one per instantiation: the limit is a property of the kernel
+    hipError_t e = smem_limit[p.f.cmp.on ? 1 : 0].ensure((const void *)kern, (int)smem);
     if (e != hipSuccess) return e;
     dim3 grid(xcd_grid(f.B * f.Hk, (f.Lq + Q_BM - 1) / Q_BM, f.H / f.Hk));
     hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, stream, p);

@@ -235,6 +235,7 @@ __device__ __forceinline__ void plan_block(const int32_t *count, const int32_t *
     if (tid == 0) {
         plan[DKDV_PLAN_HDR + pairs] = u;
         plan[0] = u;
+        plan[6] = 0;  // set below when a per-XCD list does not hold all of its parts
         plan[3] = dkdv_list_len(n_max, dkdv_lists_per_pair(pairs));
         if (pairs <= MAXU) s_first[pairs] = u;
         s_units = u;
@@ -383,6 +384,9 @@ __device__ __forceinline__ void plan_block(const int32_t *count, const int32_t *
             off += t;
         }
         lists[tid] = off < cap ? off : cap;  // (the grid is sized for every part: off <= cap)
+        // Should that ever not hold, parts would be missing from the sums: say so, and the reduce kernel turns the
+        // gradients of the whole call into NaN instead of handing out sums with parts left out.
+        if (off > cap) plan[6] = 1;
     }
     __syncthreads();
     for (int g = tid; g < U; g += 256) {

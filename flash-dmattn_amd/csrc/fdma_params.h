@@ -36,7 +36,8 @@ struct Compact {
 // k = 8 / gcd(pairs, 8) lists, unit u going to list snake(u mod 2k) -- low key blocks see the most queries
 // under a causal mask, and the fold gives every list the same mix of heavy and light units.
 //   plan[0] = U, plan[1] = Gs, plan[2] = Sm (segment slots per unit and head group), plan[3] = list length
-//   bound (units), plan[4] = Q, plan[8 + i] = first unit of pair i (i = 0..pairs)
+//   bound (units), plan[4] = Q, plan[5] = where the lists begin, plan[6] = 1 when a per-XCD list overflowed (the
+//   reduce kernel then writes NaN gradients), plan[8 + i] = first unit of pair i (i = 0..pairs)
 constexpr int DKDV_PLAN_HDR = 8;
 #ifndef FDMA_DKDV_TARGET
 #define FDMA_DKDV_TARGET 768

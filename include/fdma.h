@@ -27,9 +27,10 @@
  * Layouts (all strides in ELEMENTS, innermost dimension contiguous):
  *   q, out, dout, dq : (batch, seqlen_q, num_heads,   head_dim)   strides {batch, row, head}
  *   k, v, dk, dv     : (batch, seqlen_k, num_heads_k, head_dim)   strides {batch, row, head}
- *   mask  (uint8 / bool, 1 = keep) : ({batch|1}, {1|Hk|H}, {seqlen_q|1}, >= seqlen_k)
- *   bias, dbias (same dtype as q)  : ({batch|1}, {1|Hk|H}, {seqlen_q|1}, >= seqlen_k)
+ *   mask  (uint8 / bool, 1 = keep) : ({batch|1}, {1|Hk|H}, {seqlen_q|1}, >= round_up(seqlen_k, 16) READABLE)
+ *   bias, dbias (same dtype as q)  : ({batch|1}, {1|Hk|H}, {seqlen_q|1}, >= round_up(seqlen_k, 8)  READABLE)
  *                                     strides {batch, head, row}; 0 marks a broadcast dim
+ *                                     (rows are read in 16-byte vectors, see "Readable lengths" below)
  *   lse       : (batch, num_heads, seqlen_q) fp32, contiguous; +inf for rows with no visible key
  *   softmax_d : (batch, num_heads, round_up(seqlen_q,128)) fp32, contiguous
  */
@@ -50,10 +51,23 @@ enum { FDMA_DTYPE_BF16 = 0, FDMA_DTYPE_FP16 = 1 };
 enum {
     FDMA_OK = 0,
     FDMA_ERR_INVALID = -1,     /* argument validation failed (the reference raises RuntimeError) */
-    FDMA_ERR_UNSUPPORTED = -2, /* valid for the reference, not built here (e.g. head_dim > 128)   */
+    FDMA_ERR_UNSUPPORTED = -2, /* valid for the reference, not built here (e.g. head_dim > 128,
+                                  a stream under HIP graph capture)                              */
     FDMA_ERR_WORKSPACE = -3,   /* workspace missing or too small                                  */
     FDMA_ERR_LAUNCH = -4       /* the HIP runtime refused a launch                                */
 };
+
+/* HIP graph capture: NOT supported.  Every entry point that launches work first asks hipStreamIsCapturing about
+ * `hip_stream` and returns FDMA_ERR_UNSUPPORTED, launching nothing, when the stream is being captured.  (The one
+ * capture of forward + backward through the tensor library ended in a host crash when the capture was closed; its
+ * cause is not known, so the library refuses instead.)
+ *
+ * Readable lengths of mask and bias rows.  The kernels read mask rows in 16-byte and bias rows in 16-byte
+ * (8-element) vectors: each row of `mask` must be readable up to seqlen_k rounded up to 16 bytes, each row of `bias`
+ * up to seqlen_k rounded up to 8 elements, whatever lies there; this also holds for the last row of the buffer, and for a fully
+ * broadcast mask or bias of a single row.  The library cannot check it (it never sees the row length).  The reference
+ * asks for more: rows of exactly round_up(seqlen_k, 128) elements (flash_api.cpp:420, 431, 437).  Values beyond
+ * seqlen_k are never used, and dbias is only written up to seqlen_k. */
 
 /* Column compaction (fdma_fwd_args.compact_mode).  A keep-mask that is broadcast over the queries, with 1 or
  * num_heads_k heads, drops whole key columns; the library can then gather the kept K / V rows into dense copies
@@ -112,8 +126,9 @@ int fdma_fwd(const fdma_fwd_args *args, void *hip_stream);
 int fdma_bwd(const fdma_bwd_args *args, void *hip_stream);
 
 /*
- * fdma_fwd for callers that cannot allocate device memory: code under HIP graph capture, tight serving loops,
- * harnesses that forbid hipMalloc.  It has no counterpart in the reference (whose mha_fwd allocates its split-KV
+ * fdma_fwd for callers that cannot allocate device memory: tight serving loops, harnesses that forbid hipMalloc
+ * (and code under HIP graph capture, once capture is supported: today this call refuses a capturing stream like
+ * every other).  It has no counterpart in the reference (whose mha_fwd allocates its split-KV
  * partials with torch, flash_api.cpp:340-345).  args->workspace / workspace_bytes are ignored; the scratch of the
  * decode path (split-KV partials) or of the compaction path lives in a static device array of
  * FDMA_NOALLOC_SCRATCH_BYTES inside the library, which every GPU the library runs on holds until the process ends.
