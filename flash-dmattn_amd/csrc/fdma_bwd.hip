@@ -547,15 +547,16 @@ hipError_t launch_bwd_t(const BwdParams &p, hipStream_t stream) {
         else e = f.causal ? launch(bwd_dkdv_kernel<T, D, true, false>, KvSmem<D, false>::TOTAL) : launch(bwd_dkdv_kernel<T, D, false, false>, KvSmem<D, false>::TOTAL);
         if (e != hipSuccess) return e;
     }
-    if (p.dbias_accum) {
-        hipLaunchKernelGGL((dbias_convert_kernel<T>), dim3(1024), dim3(256), 0, stream, p, nb, f.Hb, nr, f.Lk);
-        if ((e = hipGetLastError()) != hipSuccess) return e;
-    }
-    // 3. dQ
+    // 3. dQ (the launch of a compacted backward also sums the dK / dV / dBias partial results of step 2)
     if (colmask) {
         if ((e = launch_bwd_dq_colmask(p, dtype_code, stream)) != hipSuccess) return e;
     } else {
         if ((e = launch_bwd_dq(p, dtype_code, stream)) != hipSuccess) return e;
+    }
+    // 4. shared dBias elements: fp32 sums to the output type
+    if (p.dbias_accum) {
+        hipLaunchKernelGGL((dbias_convert_kernel<T>), dim3(1024), dim3(256), 0, stream, p, nb, f.Hb, nr, f.Lk);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
     }
     return hipSuccess;
 }

@@ -60,7 +60,7 @@ constexpr int KV_BN = 128;  // key columns per workgroup (32 per wave)
 template <int D> struct KvcSmem {
     static constexpr int BM = D > 64 ? 32 : 64;
     static constexpr bool V_LDS = D > 64;
-    static constexpr int S = D + 8;
+    static constexpr int S = LdsTile<D>::S;
     static constexpr int Q_BYTES = BM * S * 2;
     static constexpr int STAGE = 2 * Q_BYTES + 2 * BM * 4;  // Q, dO, LSE, D
     static constexpr int OFF_V = 2 * STAGE;
@@ -73,6 +73,7 @@ template <typename T, int D, bool CAUSAL, bool CMP>
 __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const BwdParams p) {
     using E = Elem<T>;
     using SM = KvcSmem<D>;
+    using TL = LdsTile<D>;
     constexpr int BM = SM::BM;       // query rows per step
     constexpr int SUB = KV_BM / BM;  // steps per planning block
     constexpr bool V_LDS = SM::V_LDS;
@@ -151,7 +152,8 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
 
     // ---- stationary K / V fragments (B operands): lane holds K[key][16ks + 8g .. +8]
     u32x4_t kf[KS], vf[V_LDS ? 1 : KS];
-    char *sVrow = smem + SM::OFF_V + ((wave * 32 + r) * SM::S + g * 8) * 2;  // V_LDS: this lane's V row, its chunks
+    char *sVt = smem + SM::OFF_V;
+    uint32_t v_base = TL::frag_base(wave * 32 + r, g);  // V_LDS: this lane's V row, its chunks
     {
         const uint16_t *kp = (const uint16_t *)f.k + b * f.k_b + (sq.k0 + key_c) * f.k_r + hk * f.k_h;
         const uint16_t *vp = (const uint16_t *)f.v + b * f.v_b + (sq.k0 + key_c) * f.v_r + hk * f.v_h;
@@ -165,7 +167,7 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
 #pragma unroll
             for (int e = 0; e < 4; e++) kv[e] = E::pack2(E::lo(kv[e]) * f.scale_log2, E::hi(kv[e]) * f.scale_log2);
             kf[ks] = kv;
-            if (V_LDS) *(u32x4_t *)(sVrow + ks * 32) = vv;
+            if (V_LDS) *(u32x4_t *)(sVt + TL::frag_at(v_base, ks)) = vv;
             else vf[ks] = vv;
         }
     }
@@ -281,7 +283,7 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
         char *base = smem + buf * SM::STAGE;
 #pragma unroll
         for (int it = 0; it < Q_IT; it++) {
-            const int off = ((qr0 + it * RPP) * SM::S + qc * 8) * 2;
+            const uint32_t off = TL::chunk(qr0 + it * RPP, qc);
             *(u32x4_t *)(base + off) = qreg[it];
             *(u32x4_t *)(base + SM::Q_BYTES + off) = doreg[it];
         }
@@ -295,8 +297,8 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
     const int tj = lane & 15, te = tj >> 2, tc = tj & 3;
     const int tcp = (tc == 1) ? 2 : (tc == 2 ? 1 : tc);
     const int tdh = (lane >> 4) & 1;
-    const uint32_t tr_off = (uint32_t)(((8 * g + te) * SM::S + 16 * tdh + 4 * tcp) * 2);
-    const uint32_t a_off = (uint32_t)((a_row * SM::S + g * 8) * 2);
+    uint32_t tr_off = TL::tr_base(g, te, tdh, tcp);
+    uint32_t a_off = TL::frag_base(a_row, g);
 
     float colsum = 0.f;
     float cconst = 0.f;
@@ -323,6 +325,9 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
         const char *sDO = sQ + SM::Q_BYTES;
         const float *sLSE = (const float *)(sQ + 2 * SM::Q_BYTES);
         const float *sDD = sLSE + BM;
+        // The swizzled addresses are these lane constants XOR a compile-time value: recomputed where they are used
+        // (one VALU operation each); hoisted out of the loop they would cost 30 registers that the kernel does not have.
+        if (TL::SWZ) asm volatile("" : "+v"(a_off), "+v"(tr_off), "+v"(v_base));
 
         // ---- S = Q K^T and dP = dO V^T (M = query, N = key); fragment reads run a batch ahead
         f32x16_t s[MB], dp[MB];
@@ -335,7 +340,7 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
             u32x4_t a[NF];
             auto frag = [&](int fi) {
                 const int which = fi & 1, mb = (fi >> 1) % MB, ks = (fi >> 1) / MB;
-                return *(const u32x4_t *)((which ? sDO : sQ) + a_off + (32 * mb * SM::S + ks * 16) * 2);
+                return *(const u32x4_t *)((which ? sDO : sQ) + TL::frag_at(a_off, ks) + 32 * mb * TL::ROW_BYTES);
             };
 #pragma unroll
             for (int fi = 0; fi < FR; fi++) a[fi] = frag(fi);
@@ -343,7 +348,7 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
             for (int fi = 0; fi < NF; fi++) {
                 if (fi + FR < NF) a[fi + FR] = frag(fi + FR);
                 const int which = fi & 1, mb = (fi >> 1) % MB, ks = (fi >> 1) / MB;
-                if (which) dp[mb] = E::mfma(a[fi], V_LDS ? *(const u32x4_t *)(sVrow + ks * 32) : vf[V_LDS ? 0 : ks], dp[mb]);
+                if (which) dp[mb] = E::mfma(a[fi], V_LDS ? *(const u32x4_t *)(sVt + TL::frag_at(v_base, ks)) : vf[V_LDS ? 0 : ks], dp[mb]);
                 else s[mb] = E::mfma(a[fi], kf[ks], s[mb]);
             }
         }
@@ -405,9 +410,9 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
             u32x4_t a1[2], a2[2];
             auto frag = [&](int idx, int slot) {
                 const int qb = idx / DB, db = idx % DB;
-                const uint32_t off = tr_off + (uint32_t)((16 * qb * SM::S + 32 * db) * 2);
-                const u32x2_t lo = lds_read_tr16(sDO, off), hi = lds_read_tr16(sDO, off + 4 * SM::S * 2);
-                const u32x2_t lo2 = lds_read_tr16(sQ, off), hi2 = lds_read_tr16(sQ, off + 4 * SM::S * 2);
+                const uint32_t off = TL::tr_at(tr_off, qb, db, 0), off_hi = TL::tr_at(tr_off, qb, db, 1);
+                const u32x2_t lo = lds_read_tr16(sDO, off), hi = lds_read_tr16(sDO, off_hi);
+                const u32x2_t lo2 = lds_read_tr16(sQ, off), hi2 = lds_read_tr16(sQ, off_hi);
                 a1[slot] = u32x4_t{lo[0], lo[1], hi[0], hi[1]};
                 a2[slot] = u32x4_t{lo2[0], lo2[1], hi2[0], hi2[1]};
             };
@@ -501,16 +506,16 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
     }
 }
 
-// Sums the partial results of the blocks that the compacted dK/dV kernel split over several workgroups, in a
-// fixed order, and writes dK (scaled), dV and dBias to the original rows / columns of the kept keys.
+// Sums the partial results of one unit that the compacted dK/dV kernel split over several workgroups, in a fixed
+// order, and writes dK (scaled), dV and dBias to the original rows / columns of the kept keys.  `y` picks a pair of
+// 8-wide head-dim chunks (0 .. D/16 - 1), so that few units still give many work items; item y == 0 also folds the
+// unit's dBias columns.  Called by the workgroups that the dQ launch sets aside for it (see bwd_dq_colmask_kernel).
 template <typename T, int D>
-__global__ void __launch_bounds__(NTHREADS) bwd_dkdv_reduce_kernel(const BwdParams p) {
+__device__ __forceinline__ void dkdv_reduce_item(const BwdParams &p, const int unit, const int y) {
     using E = Elem<T>;
     const FwdParams &f = p.f;
     const int32_t *plan = f.cmp.plan;
-    const int U = plan[0], Gs = plan[1], Sm = plan[2], Q = plan[4], per = Gs * Sm;
-    const int unit = blockIdx.x;
-    if (per == 1 || unit >= U) return;
+    const int Gs = plan[1], Sm = plan[2], Q = plan[4], per = Gs * Sm;
     // a plan whose lists overflowed left parts uncomputed: every sum starts from NaN then
     const float start = plan[6] != 0 ? __builtin_nanf("") : 0.f;
     int lo = 0, hi = f.B * f.Hk;
@@ -529,32 +534,35 @@ __global__ void __launch_bounds__(NTHREADS) bwd_dkdv_reduce_kernel(const BwdPara
     // segments of this unit that were written (same rule as in the main kernel)
     const int n_seg = dkdv_segments(dkdv_query_blocks(f.Lq, f.Lk, f.causal, f.cmp.idx[(int64_t)pair * f.cmp.ld + n0]), Q, Sm);
     const float *base = p.dkv_part + (int64_t)unit * per * 2 * D * KV_BN + kk;
-    // blockIdx.y picks a pair of 8-wide head-dim chunks, so that few units still give many workgroups
-    for (int c = 2 * blockIdx.y + half; c == 2 * (int)blockIdx.y + half && c * 8 < f.d; c += NTHREADS / KV_BN) {
+    for (int c = 2 * y + half; c == 2 * y + half && c * 8 < f.d; c += NTHREADS / KV_BN) {
         float ak[8], av[8];
 #pragma unroll
         for (int e = 0; e < 8; e++) { ak[e] = start; av[e] = start; }
-        // written slots in a fixed order, two at a time so that more loads are in flight
+        // written slots in a fixed order, four at a time: a workgroup here sits beside the dQ workgroups and should
+        // give its place back soon, so the loads of four slots are in flight together (slots past the end repeat
+        // the last one and are not added)
         const int n_w = Gs * n_seg;
-        for (int j = 0; j < n_w; j += 2) {
-            const bool two = j + 1 < n_w;
-            const int j1 = two ? j + 1 : j;
-            const float *p0 = base + (int64_t)((j / n_seg) * Sm + j % n_seg) * 2 * D * KV_BN;
-            const float *p1 = base + (int64_t)((j1 / n_seg) * Sm + j1 % n_seg) * 2 * D * KV_BN;
-            float k0[8], v0[8], k1[8], v1[8];
+        for (int j = 0; j < n_w; j += 4) {
+            float kq[4][8], vq[4][8];
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-                k0[e] = p0[(c * 8 + e) * KV_BN];
-                v0[e] = p0[(D + c * 8 + e) * KV_BN];
-                k1[e] = p1[(c * 8 + e) * KV_BN];
-                v1[e] = p1[(D + c * 8 + e) * KV_BN];
+            for (int t = 0; t < 4; t++) {
+                const int jt = j + t < n_w ? j + t : n_w - 1;
+                const float *pt = base + (int64_t)((jt / n_seg) * Sm + jt % n_seg) * 2 * D * KV_BN;
+#pragma unroll
+                for (int e = 0; e < 8; e++) {
+                    kq[t][e] = pt[(c * 8 + e) * KV_BN];
+                    vq[t][e] = pt[(D + c * 8 + e) * KV_BN];
+                }
             }
 #pragma unroll
-            for (int e = 0; e < 8; e++) {
-                ak[e] += k0[e];
-                av[e] += v0[e];
-                if (two) { ak[e] += k1[e]; av[e] += v1[e]; }
-            }
+            for (int t = 0; t < 4; t++)
+                if (j + t < n_w) {
+#pragma unroll
+                    for (int e = 0; e < 8; e++) {
+                        ak[e] += kq[t][e];
+                        av[e] += vq[t][e];
+                    }
+                }
         }
         if (live) {
             u32x4_t wk, wv;
@@ -567,7 +575,7 @@ __global__ void __launch_bounds__(NTHREADS) bwd_dkdv_reduce_kernel(const BwdPara
             *(u32x4_t *)((uint16_t *)p.dv + b * p.dv_b + (int64_t)okey * p.dv_r + hk * p.dv_h + c * 8) = wv;
         }
     }
-    if (f.bias && live && blockIdx.y == 0) {
+    if (f.bias && live && y == 0) {
         const int gper = G / Gs;
         const float *dbp = p.db_part + (int64_t)unit * per * G * KV_BN + kk;  // [part][local head][key]
         auto emit = [&](int hb, float tot) {
@@ -590,6 +598,39 @@ __global__ void __launch_bounds__(NTHREADS) bwd_dkdv_reduce_kernel(const BwdPara
     }
 }
 
+// Workgroup `rb` of `nrb` reducing workgroups takes every nrb-th of the U units x D/16 chunk pairs.  The first item
+// goes to the workgroup in the middle: when there are fewer items than workgroups (few units, each cut into many
+// parts: long sums) they run in the middle of the launch's interleaved stretch, neither beside the heaviest dQ
+// workgroups at its start nor in its tail.
+template <typename T, int D>
+__device__ __forceinline__ void dkdv_reduce_blocks(const BwdParams &p, const int rb, const int nrb) {
+    const int32_t *plan = p.f.cmp.plan;
+    const int U = plan[0];
+    if (plan[1] * plan[2] == 1) return;  // no unit was split: the dK/dV kernel wrote the results itself
+    const int first = rb >= nrb / 2 ? rb - nrb / 2 : rb + nrb - nrb / 2;
+    for (int item = first; item < U * (D / 16); item += nrb) dkdv_reduce_item<T, D>(p, item / (D / 16), item % (D / 16));
+}
+
+// The dQ launch of a compacted backward carries the reduction of the dK/dV partials along: `red_octets` groups of 8
+// consecutive workgroups (one per XCD) do that instead of dQ work, one such group after every `period - 1` groups
+// of dQ workgroups.  The reduction only moves memory while the dQ workgroups keep the matrix units busy, so side by
+// side it costs next to nothing; as a launch of its own it took as long as its memory traffic.
+struct RedInterleave {
+    int red_octets, period, start;
+};
+inline RedInterleave red_interleave(int dq_octets, int items) {
+    RedInterleave r;
+    r.red_octets = (items < 1024 ? items : 1024) / 8;
+    if (r.red_octets < 1) r.red_octets = 1;
+    r.period = (dq_octets + r.red_octets) / r.red_octets;
+    r.period = r.period < 2 ? 2 : (r.period > 4 ? 4 : r.period);
+    if (r.red_octets > dq_octets / (r.period - 1)) r.red_octets = dq_octets / (r.period - 1);
+    if (r.red_octets < 1) r.red_octets = 1;  // (dq_octets >= 1 and period == 2 then)
+    // the interleaved stretch ends with the launch; the dQ groups in front of it are the heaviest ones
+    r.start = dq_octets - r.red_octets * (r.period - 1);
+    return r;
+}
+
 template <typename T, int D, bool CAUSAL, bool CMP>
 hipError_t launch_dkdv_c(const BwdParams &p, hipStream_t stream) {
     const FwdParams &f = p.f;
@@ -598,14 +639,11 @@ hipError_t launch_dkdv_c(const BwdParams &p, hipStream_t stream) {
     static DynSmemLimit smem_limit;
     hipError_t e = smem_limit.ensure((const void *)kern, (int)smem);
     if (e != hipSuccess) return e;
-    const int units_max = f.B * f.Hk * ((f.Lk + KV_BN - 1) / KV_BN);
     if (CMP) {
         int grid, slots;
         dkdv_split_bounds(f.B * f.Hk, (f.Lk + KV_BN - 1) / KV_BN, f.H / f.Hk, grid, slots);
         hipLaunchKernelGGL(kern, dim3(grid), dim3(NTHREADS), smem, stream, p);
-        if ((e = hipGetLastError()) != hipSuccess) return e;
-        hipLaunchKernelGGL((bwd_dkdv_reduce_kernel<T, D>), dim3(units_max, D / 16), dim3(NTHREADS), 0, stream, p);
-        return hipGetLastError();
+        return hipGetLastError();  // (the partial results are summed by workgroups of the dQ launch)
     }
     dim3 grid(xcd_grid(f.B * f.Hk, (f.Lk + KV_BN - 1) / KV_BN, 1));
     hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, stream, p);
@@ -625,7 +663,7 @@ constexpr int MAX_TILES = 16384;
 
 
 template <int D, int BN> struct DqcSmem {
-    static constexpr int S = D + 8;
+    static constexpr int S = LdsTile<D>::S;
     static constexpr int K_BYTES = BN * S * 2;
     static constexpr int OFF_K = 0;
     static constexpr int OFF_V = OFF_K + 2 * K_BYTES;
@@ -638,6 +676,7 @@ template <typename T, int D, int BN, bool CAUSAL, bool CMP>
 __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdParams p) {
     using E = Elem<T>;
     using SM = DqcSmem<D, BN>;
+    using TL = LdsTile<D>;
     constexpr int KS = D / 16;
     constexpr int DB = D / 32;
     constexpr int MB = BN / 32;
@@ -652,11 +691,31 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 31, g = lane >> 5;
     const int G = f.H / f.Hk;
     const int n_mb = (f.Lq + Q_BM - 1) / Q_BM;
-    const XcdMap wm = xcd_map(blockIdx.x, f.B * f.Hk, n_mb, G);
+    int lid = blockIdx.x;  // index among the dQ workgroups
+    if (CMP) {
+        // groups of 8 workgroups (one per XCD): every `period`-th of the first red_octets * period groups sums
+        // partial results of the dK/dV kernel instead
+        const int R = p.red_octets, period = p.red_period;
+        int o = lid >> 3;
+        const int o2 = o - p.red_start;  // the groups before red_start are all dQ groups
+        if (o2 >= 0) {
+            if (o2 < R * period) {
+                if (o2 % period == period - 1) {
+                    dkdv_reduce_blocks<T, D>(p, (o2 / period) * 8 + (lid & 7), R * 8);
+                    return;
+                }
+                o -= o2 / period;
+            } else {
+                o -= R;
+            }
+        }
+        lid = o * 8 + (lid & 7);
+    }
+    const XcdMap wm = xcd_map(lid, f.B * f.Hk, n_mb, G);
     if (!wm.valid) return;
     const int m_block = n_mb - 1 - wm.unit;  // heaviest first under causal
     const int b = wm.pair / f.Hk, hk = wm.pair % f.Hk;
-    const int h = hk * G + (blockIdx.x / 8) % G;
+    const int h = hk * G + (lid / 8) % G;
     const int m0 = m_block * Q_BM;
     const SeqInfo sq = seq_info(f, b);  // this batch entry's lengths and first rows (ragged batch: from cu_seqlens)
     const int LqS = sq.Lq, LkS = sq.Lk;
@@ -824,7 +883,7 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
         char *sV = smem + SM::OFF_V + buf * SM::K_BYTES;
 #pragma unroll
         for (int it = 0; it < K_IT; it++) {
-            const int off = ((kr0 + it * RPP) * SM::S + kc * 8) * 2;
+            const uint32_t off = TL::chunk(kr0 + it * RPP, kc);
             *(u32x4_t *)(sK + off) = kreg[it];
             *(u32x4_t *)(sV + off) = vreg[it];
         }
@@ -840,11 +899,11 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
     };
 
     const int a_row = pi_row(r);
-    const uint32_t a_off = (uint32_t)((a_row * SM::S + g * 8) * 2);
+    const uint32_t a_off = TL::frag_base(a_row, g);
     const int tj = lane & 15, te = tj >> 2, tc = tj & 3;
     const int tcp = (tc == 1) ? 2 : (tc == 2 ? 1 : tc);
     const int tdh = (lane >> 4) & 1;
-    const uint32_t tr_off = (uint32_t)(((8 * g + te) * SM::S + 16 * tdh + 4 * tcp) * 2);
+    const uint32_t tr_off = TL::tr_base(g, te, tdh, tcp);
 
     int jc = next_active(0);
     if (jc < n_end) {
@@ -882,7 +941,7 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
             u32x4_t a[NF];
             auto frag = [&](int fi) {
                 const int which = fi & 1, mb = (fi >> 1) % MB, ks = (fi >> 1) / MB;
-                return *(const u32x4_t *)((which ? sV : sK) + a_off + (32 * mb * SM::S + ks * 16) * 2);
+                return *(const u32x4_t *)((which ? sV : sK) + TL::frag_at(a_off, ks) + 32 * mb * TL::ROW_BYTES);
             };
 #pragma unroll
             for (int fi = 0; fi < FR; fi++) a[fi] = frag(fi);
@@ -925,8 +984,7 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdPa
             const u32x4_t bop = {dpk[4 * kb], dpk[4 * kb + 1], dpk[4 * kb + 2], dpk[4 * kb + 3]};
 #pragma unroll
             for (int db = 0; db < DB; db++) {
-                const uint32_t off = tr_off + (uint32_t)((16 * kb * SM::S + 32 * db) * 2);
-                const u32x2_t lo = lds_read_tr16(sK, off), hi = lds_read_tr16(sK, off + 4 * SM::S * 2);
+                const u32x2_t lo = lds_read_tr16(sK, TL::tr_at(tr_off, kb, db, 0)), hi = lds_read_tr16(sK, TL::tr_at(tr_off, kb, db, 1));
                 const u32x4_t a = {lo[0], lo[1], hi[0], hi[1]};
                 dq[db] = E::mfma(a, bop, dq[db]);
             }
@@ -964,8 +1022,18 @@ hipError_t launch_dq(const BwdParams &p, hipStream_t stream) {
     static DynSmemLimit smem_limit[2];  // one per instantiation: the limit is a property of the kernel
     hipError_t e = smem_limit[p.f.cmp.on ? 1 : 0].ensure((const void *)kern, (int)smem);
     if (e != hipSuccess) return e;
-    dim3 grid(xcd_grid(f.B * f.Hk, (f.Lq + Q_BM - 1) / Q_BM, f.H / f.Hk));
-    hipLaunchKernelGGL(kern, grid, dim3(NTHREADS), smem, stream, p);
+    const int n_dq = xcd_grid(f.B * f.Hk, (f.Lq + Q_BM - 1) / Q_BM, f.H / f.Hk);  // a multiple of 8
+    if (p.f.cmp.on) {
+        const int units_max = f.B * f.Hk * ((f.Lk + KV_BN - 1) / KV_BN);
+        const RedInterleave ri = red_interleave(n_dq / 8, units_max * (D / 16));
+        BwdParams pr = p;
+        pr.red_octets = ri.red_octets;
+        pr.red_period = ri.period;
+        pr.red_start = ri.start;
+        hipLaunchKernelGGL(kern, dim3(n_dq + 8 * ri.red_octets), dim3(NTHREADS), smem, stream, pr);
+        return hipGetLastError();
+    }
+    hipLaunchKernelGGL(kern, dim3(n_dq), dim3(NTHREADS), smem, stream, p);
     return hipGetLastError();
 }
 

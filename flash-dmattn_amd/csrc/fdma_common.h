@@ -132,6 +132,45 @@ __device__ __forceinline__ u32x2_t lds_read_tr16(const char *smem_base, uint32_t
     return __builtin_bit_cast(u32x2_t, v);
 }
 
+// Row-major LDS tile of 16-bit elements ([row][head dim]) that is read two ways: as MFMA fragments (ds_read_b128:
+// lane (r, g) takes the 16 bytes of chunk 2*ks + g of row pi_row(r)) and through transposing reads (lds_read_tr16:
+// 16 lanes take four 8-byte pieces of each of four consecutive rows), and written row by row (16 lanes per row).
+// At head dim 128 a row is exactly 256 bytes, the width of the LDS banks, and the 16-byte chunks of a row are
+// permuted by a XOR with a function of the row: chunk c of row `row` lives at chunk c ^ swz(row) with
+// swz(row) = 4*(row & 3) + ((row >> 2) & 3).  Four consecutive rows then sit in four different 64-byte quarters of
+// the banks (what the transposing reads need: measured 145 bytes/clk per CU against 60 with rows padded to 272
+// bytes) and sixteen consecutive rows in sixteen different chunks (what the fragment reads need: 230 bytes/clk, the
+// same as with padding).  Other head dims keep rows padded by 8 elements.
+// Offsets are bytes; a "base" is a lane constant, the *_at functions add the compile-time part.
+template <int D> struct LdsTile {
+    static constexpr bool SWZ = D == 128;
+    static constexpr int S = SWZ ? D : D + 8;  // row stride, elements
+    static constexpr int ROW_BYTES = S * 2;
+    static __device__ __forceinline__ uint32_t swz(int row) { return (uint32_t)(((row & 3) << 2) | ((row >> 2) & 3)); }
+    // 16-byte chunk c of a row (tile writes)
+    static __device__ __forceinline__ uint32_t chunk(int row, int c) {
+        return SWZ ? (uint32_t)row * 256u + ((((uint32_t)c) ^ swz(row)) << 4) : (uint32_t)((row * S + c * 8) * 2);
+    }
+    // fragment reads: chunk 2*ks + g of `row`; rows 32 apart share the base (add 32 * ROW_BYTES)
+    static __device__ __forceinline__ uint32_t frag_base(int row, int g) {
+        return SWZ ? (uint32_t)row * 256u + ((((uint32_t)g) ^ swz(row)) << 4) : (uint32_t)((row * S + g * 8) * 2);
+    }
+    static __device__ __forceinline__ uint32_t frag_at(uint32_t base, int ks) {
+        return SWZ ? (base ^ ((uint32_t)ks << 5)) : base + (uint32_t)ks * 32u;
+    }
+    // transposing reads: lane (g, te, tdh, tcp) supplies row 8*g + te, elements 16*tdh + 4*tcp .. +3 of a 32-element
+    // block db, in 16-row block rb; hi = 1: the same four rows further down
+    static __device__ __forceinline__ uint32_t tr_base(int g, int te, int tdh, int tcp) {
+        return SWZ ? (uint32_t)(8 * g + te) * 256u + (((uint32_t)te << 6) | ((((uint32_t)(2 * tdh + (tcp >> 1))) ^ (uint32_t)(2 * g)) << 4) |
+                                                     ((uint32_t)(tcp & 1) << 3))
+                   : (uint32_t)(((8 * g + te) * S + 16 * tdh + 4 * tcp) * 2);
+    }
+    static __device__ __forceinline__ uint32_t tr_at(uint32_t base, int rb, int db, int hi) {
+        return SWZ ? (base ^ (((uint32_t)db << 6) | ((uint32_t)hi << 4))) + (uint32_t)(hi * 4 * 256 + rb * 16 * 256)
+                   : base + (uint32_t)(((16 * rb + 4 * hi) * S + 32 * db) * 2);
+    }
+};
+
 // max / sum across the two 32-lane halves of a wave (lanes l and l ^ 32)
 __device__ __forceinline__ float xhalf_max(float x) {
     uint32_t u = __float_as_uint(x);

@@ -159,6 +159,7 @@ struct BwdParams {
     float *dkv_part;
     float *db_part;
     int32_t dot_done;          // softmax_d has been computed by an earlier launch of this call
+    int32_t red_octets, red_period, red_start;  // compacted backward: workgroups of the dQ launch that sum the dK/dV partials (set by that launch)
 };
 
 // Keep-mask builder (fdma_mask.hip): one row of `Lk` 16-bit bias values per (batch, head, row).
