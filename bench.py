@@ -56,18 +56,21 @@ def summarise_pmc(fetch_csv, write_csv):
     import re
 
     def per_kernel(path, counter):
+        """mean per dispatch of every kernel, and the largest value among the runtime's copy kernel dispatches: the
+        process makes other, small device copies too; the 256 MiB calibration copy is the largest of them"""
         acc = {}
         for row in csv.DictReader(open(path)):
             if row.get("Counter_Name") != counter:
                 continue
             name = row["Kernel_Name"]
             acc.setdefault(name, []).append(float(row["Counter_Value"]))
-        return {k: sum(v) / len(v) for k, v in acc.items()}
+        copies = [max(v) for k, v in acc.items() if "copyBuffer" in k]
+        return {k: sum(v) / len(v) for k, v in acc.items()}, max(copies)
 
-    fetch, write = per_kernel(fetch_csv, "FETCH_SIZE"), per_kernel(write_csv, "WRITE_SIZE")
+    (fetch, f_copy), (write, w_copy) = per_kernel(fetch_csv, "FETCH_SIZE"), per_kernel(write_csv, "WRITE_SIZE")
     copy_kib = 256.0 * 1024
-    f_scale = copy_kib / next(v for k, v in fetch.items() if "copyBuffer" in k)
-    w_scale = copy_kib / next(v for k, v in write.items() if "copyBuffer" in k)
+    f_scale = copy_kib / f_copy
+    w_scale = copy_kib / w_copy
     lines = ["# HBM traffic per launch of fdma::fwd_colmask_kernel on bench.py's headline workload (cfg2), written by",
              "# `python bench.py --summarise-pmc`; FETCH_SIZE / WRITE_SIZE are KiB per dispatch, scaled by the factors below",
              "fetch_scale = %.4f" % f_scale, "write_scale = %.4f" % w_scale]
