@@ -23,8 +23,9 @@
 // start from the constant 0, and what leaves the MFMAs is the finished exp2 argument.  The reference point of a
 // row is any number near its running maximum (the softmax does not depend on it); it is set by the first tile and
 // then left alone as long as no probability exceeds 2^14 -- which the sum of the probabilities shows, so the
-// common path has no maximum at all: exp2, convert to 16 bits (two per instruction), dot2 with (1, 1) for the row
-// sum: two vector instructions per score.  A half tile that fails the check (or a wave whose rows have no
+// common path has no maximum at all: exp2, convert to 16 bits (two per instruction), one addition to the row sum
+// (plain fp32 additions: a 16-bit dot product with (1, 1) would halve their number, but it runs on the matrix pipe's
+// side of the SIMD and cost 2-3 % of the kernel): 2.5 vector instructions per score.  A half tile that fails the check (or a wave whose rows have no
 // reference yet) takes the classic path: maximum, new reference, rescale of O and of the sums.
 //   Software pipeline over HALF tiles (32 keys).  One step issues the score MFMAs of half tile h+1, the P V MFMAs
 // of half tile h-1 and, between them, the softmax instructions of half tile h: the three have no dependence on one
@@ -378,7 +379,7 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) fwd_colmask_kernel(c
     // Fragment addresses of a half tile.  Scores: side rows + KS k-steps of K for the 32 keys of half `kh` of stage
     // `kbuf`; P V: the two 16-key k-steps of half `vh` of V^T stage `vbuf`, DB row blocks each.
     constexpr int NQK = KS + 1, NPV = 2 * DB, NF = NQK + NPV;
-    constexpr int FR = NQK < 8 ? NQK : 8;  // fragment reads run FR MFMAs ahead of their MFMAs
+    constexpr int FR = 4;  // fragment reads run FR MFMAs ahead of their MFMAs (8 ahead: 19 spilled registers)
     auto frag_ptr = [&](int f, int kbuf, int kh, int vbuf, int vh) -> const u32x4_t * {
         if (f == 0) return (const u32x4_t *)(smem + SM::OFF_X + kbuf * SM::X_BYTES + (32 * kh + a_row) * 32 + g * 16);
         if (f < NQK)
@@ -463,30 +464,27 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) fwd_colmask_kernel(c
     // One step of the pipeline.  MFMAs: scores of the NEXT half tile (half kh of K stage kbuf) into `snext`, and
     // O^T += V^T P^T of the PREVIOUS half tile (probabilities pprev, half vh of V^T stage vbuf).  Vector ALU, between
     // them: softmax of the CURRENT half tile `scur` (first column col0) into `pcur` -- the common path, no maximum.
-    // A step also moves one staged operand from the registers to LDS and issues its next loads: V (and, in wave 0,
-    // the side rows) BEHIND the MFMAs of the first step of a tile (STAGE), K IN FRONT of the MFMAs of the second.
-    // With split roles the two waves of a SIMD have different roles: after the barrier between the two steps one of
-    // them stages K while the other is in its MFMAs, and towards the next barrier it is the other way round.  (Half
-    // tiles on the causal diagonal are masked before the step, in code of their own: only they pay for it.)
-    auto step = [&](auto stage_c, f32x16_t &scur, f32x16_t &snext, uint32_t (&pcur)[8],
+    // A step also moves one staged operand from the registers to LDS, piece by piece between its MFMAs, and issues that
+    // operand's next loads behind them: V (and, in wave 0, the side rows) in the first step of a tile (STAGE), K in the
+    // second.  With split roles the two waves of a SIMD have different roles.  (Staging as a phase of its own, after or
+    // in front of the MFMAs, left the matrix pipe to the SIMD's other wave alone for a fifth of every tile.  Half tiles
+    // on the causal diagonal are masked before the step, in code of their own: only they pay for it.)
+    auto step = [&](auto stage_c, auto do_v_c, auto do_k_c, f32x16_t &scur, f32x16_t &snext, uint32_t (&pcur)[8],
                     const uint32_t (&pprev)[8], int kbuf, int kh, int vbuf, int vh, int j_next, int jx_next) {
         constexpr bool STAGE = decltype(stage_c)::value;
-        if (!STAGE) {  // K(t+2) into the stage whose scores were finished before the barrier, then the loads of K(j_next)
-            store_k(kbuf ^ 1);
-            set_tile_k(j_next);
-            load_regs(false);
-            __builtin_amdgcn_sched_barrier(0);
-        }
+        constexpr bool DO_V = STAGE && decltype(do_v_c)::value, DO_K = !STAGE && decltype(do_k_c)::value;
+        char *const sVt_w = smem + SM::OFF_VT + (vbuf ^ 1) * SM::VT_BYTES;  // V(t) goes to the stage the P V product has left
+        char *const sK_w = smem + SM::OFF_K + (kbuf ^ 1) * SM::K_BYTES;     // K(t+2) to the stage whose scores are finished
         // Order of issue: a wave issues in program order, so the vector instructions have to sit BETWEEN the MFMAs to run
         // under them.  The step is written slot by slot -- one MFMA, the fragment read of the MFMA FR slots later, an even
         // share of the softmax (the two exp2 of a pair of scores in one slot, their conversion to 16 bits and their
-        // addition to the row sum in the next) -- with a scheduling barrier after every slot.  The probabilities are
-        // relative to the reference the MFMAs have already subtracted; the row sum adds the ROUNDED values (numerator
-        // and denominator see the same numbers).
+        // addition to the row sum in the next, a piece of the staging) -- with a scheduling barrier after every slot.
+        // The probabilities are relative to the reference the MFMAs have already subtracted; the row sum adds the
+        // fp32 values, as the reference does (src/softmax.h: the sum is taken before the conversion to 16 bits).
         u32x4_t a[NF];
 #pragma unroll
         for (int f = 0; f < FR; f++) a[f] = *frag_ptr(f, kbuf, kh, vbuf, vh);
-        float psum = 0.f, x0[8], x1[8];
+        float psum0 = 0.f, psum1 = 0.f, x0[8], x1[8];
 #pragma unroll
         for (int f = 0; f < NF; f++) {
             if (f + FR < NF) a[f + FR] = *frag_ptr(f + FR, kbuf, kh, vbuf, vh);
@@ -507,13 +505,34 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) fwd_colmask_kernel(c
                     x1[k] = fast_exp2(scur[2 * k + 1]);
                 }
                 if (slot + 1 == f) {
-                    const uint32_t w = E::pack2(x0[k], x1[k]);
-                    psum = E::add_pair(w, psum);
-                    pcur[k] = w;
+                    pcur[k] = E::pack2(x0[k], x1[k]);
+                    psum0 += x0[k];
+                    psum1 += x1[k];
                 }
+            }
+            // staging, a piece per slot: one transposed row pair of V (two permutes, one 8-byte store) / one 16-byte
+            // chunk of K
+            if (DO_V) {
+#pragma unroll
+                for (int dd = 0; dd < 8; dd++)
+                    if (f == 1 + dd * ((NF - 1) / 8)) {
+                        const int w = dd >> 1;
+                        const uint32_t sel = (dd & 1) ? 0x07060302u : 0x05040100u;
+                        u32x2_t out;
+                        out[0] = __builtin_amdgcn_perm(sreg[VB + 1][w], sreg[VB + 0][w], sel);
+                        out[1] = __builtin_amdgcn_perm(sreg[VB + 3][w], sreg[VB + 2][w], sel);
+                        *(u32x2_t *)(sVt_w + ((vc * 8 + dd) * SM::SVT + 4 * vkg) * 2) = out;
+                    }
+            }
+            if (DO_K) {
+#pragma unroll
+                for (int it = 0; it < K_IT; it++)
+                    if (f == 1 + it * ((NF - 1) / K_IT))
+                        *(u32x4_t *)(sK_w + ((kr0 + it * K_RPP) * SM::SK + kc * 8) * 2) = sreg[it];
             }
             __builtin_amdgcn_sched_barrier(0);
         }
+        const float psum = psum0 + psum1;
         row_sum += psum;
         // (the results are pinned here: left alone, the compiler sinks the softmax below the staging code that follows,
         // away from the MFMAs it is meant to run under)
@@ -521,12 +540,16 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) fwd_colmask_kernel(c
         for (int i = 0; i < 8; i++) asm volatile("" : "+v"(pcur[i]));
         asm volatile("" : "+v"(row_sum));
         __builtin_amdgcn_sched_barrier(0);
-                if (STAGE) {   // V(t) into the stage the P V product has left, then the loads of V(j_next); side rows likewise
-            store_v(vbuf ^ 1);
+        if (STAGE) {  // the loads of V(j_next); side rows of the next tile, inputs of those of the tile after it
             store_x(kbuf ^ 1);  // (in front of the new loads: its inputs must not be waited for together with them)
-            set_tile_v(j_next);
-            load_regs(true);
+            if (DO_V) {
+                set_tile_v(j_next);
+                load_regs(true);
+            }
             set_tile_x(jx_next);
+        } else if (DO_K) {  // the loads of K(j_next)
+            set_tile_k(j_next);
+            load_regs(false);
         }
         if (__any(!(psum <= 16384.f))) *sFlag = 1u;
     };
@@ -619,22 +642,31 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) fwd_colmask_kernel(c
         const std::true_type yes;
         const std::false_type no;
         int t = 0;
-        while (true) {
-            const int kb = t & 1;
-            const int col0 = jc * BN;
-            if (CAUSAL && col0 + 32 > vis_wave) causal_mask(sA, col0);
-            __builtin_amdgcn_sched_barrier(0);
-            step(yes, sA, sB, pA, pB, kb, 1, kb ^ 1, 1, jn1 < n_end ? jn1 : jc, jn2 < n_end ? jn2 : jc);
-            __builtin_amdgcn_sched_barrier(0);
-            __syncthreads();
-            __builtin_amdgcn_sched_barrier(0);
-            if (CAUSAL && col0 + 64 > vis_wave) causal_mask(sB, col0 + 32);
-            step(no, sB, sA, pB, pA, kb ^ 1, 0, kb, 0, jn3 < n_end ? jn3 : jc, 0);
-            __builtin_amdgcn_sched_barrier(0);
-            t++;
-            jc = jn1; jn1 = jn2; jn2 = jn3;
-            if (jc >= n_end) break;
-            jn3 = next_tile();
+        // (the loop exists once per staging role, so that the staging pieces inside the steps are unconditional code)
+        auto tile_loop = [&](auto do_v_c, auto do_k_c) {
+            while (true) {
+                const int kb = t & 1;
+                const int col0 = jc * BN;
+                if (CAUSAL && col0 + 32 > vis_wave) causal_mask(sA, col0);
+                __builtin_amdgcn_sched_barrier(0);
+                step(yes, do_v_c, do_k_c, sA, sB, pA, pB, kb, 1, kb ^ 1, 1, jn1 < n_end ? jn1 : jc, jn2 < n_end ? jn2 : jc);
+                __builtin_amdgcn_sched_barrier(0);
+                __syncthreads();
+                __builtin_amdgcn_sched_barrier(0);
+                if (CAUSAL && col0 + 64 > vis_wave) causal_mask(sB, col0 + 32);
+                step(no, do_v_c, do_k_c, sB, sA, pB, pA, kb ^ 1, 0, kb, 0, jn3 < n_end ? jn3 : jc, 0);
+                __builtin_amdgcn_sched_barrier(0);
+                t++;
+                jc = jn1; jn1 = jn2; jn2 = jn3;
+                if (jc >= n_end) break;
+                jn3 = next_tile();
+            }
+        };
+        const bool do_v = __builtin_amdgcn_readfirstlane((int)(role_v && kt < V_ITEMS)) != 0;
+        if (do_v) {
+            tile_loop(yes, std::integral_constant<bool, !SPLIT>());
+        } else {
+            tile_loop(no, yes);
         }
         pv_half(pB, (t - 1) & 1, 1);  // P V of the last half: V of the last tile, second half
         __syncthreads();

@@ -1,7 +1,7 @@
 """Benchmark configurations 2, 3 and 4 at FULL size, forward and backward, through the Python operator.
 
 The C oracle and a dense eager pass cannot finish these sizes for every head, so each configuration is checked by
-  * size-independent properties of the whole result: V = 1 gives O in {0, 1}; rows of dBias of a per-query bias sum
+  * size-independent properties of the whole result: V = 1 gives O = 1 (to a rounding step) or 0; rows of dBias of a per-query bias sum
     to zero (sum_k dS = 0); gradients of dropped keys are exactly zero; every output is finite;
   * the fp32 eager restatement on ONE (batch entry, kv group): its query heads, its kv head, its bias / mask slice,
     against the same slice of the full-size result (groups do not interact);
@@ -85,7 +85,8 @@ def _ones_value_property(q, k, v, mask, bias, lse):
 
     ones = flash_sparse_attn_func(q, k, torch.ones_like(v), mask, bias, None, True)
     nonempty = torch.isfinite(lse).transpose(1, 2)[..., None].expand_as(ones)
-    assert torch.equal(ones[nonempty], torch.ones_like(ones[nonempty]))
+    # (the probabilities are rounded to 16 bits for the matrix pipe, their fp32 sum is not: one rounding step of slack)
+    assert (ones[nonempty].float() - 1.0).abs().max().item() <= 2.0 ** -7
     assert torch.equal(ones[~nonempty], torch.zeros_like(ones[~nonempty]))
 
 

@@ -404,7 +404,8 @@ def test_cfg2_full_size_forward_properties():
     out, lse, _ = f(qd, kd, vd, md, bd, None, True, None, None, True)
     ones, _, _ = f(qd, kd, torch.ones_like(vd), md, bd, None, True, None, None, True)
     nonempty = torch.isfinite(lse).transpose(1, 2)[..., None].expand_as(ones)  # (B, L, H, 1)
-    assert torch.equal(ones[nonempty], torch.ones_like(ones[nonempty]))
+    # (the probabilities are rounded to 16 bits for the matrix pipe, their fp32 sum is not: one rounding step of slack)
+    assert (ones[nonempty].float() - 1.0).abs().max().item() <= 2.0 ** -7
     assert torch.equal(ones[~nonempty], torch.zeros_like(ones[~nonempty]))
     # the shift must not itself be rounded: quantise the bias to multiples of 1/32 inside (-2, 2), so that bias and
     # bias + 2 are both exact in bf16 and the two calls see the same scores up to the constant
