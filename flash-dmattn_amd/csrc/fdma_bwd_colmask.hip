@@ -14,6 +14,8 @@
 // lane parks in LDS as a private spill so that two workgroups fit on a CU); Q / dO tiles and the row
 // statistics stream through double-buffered LDS, fetched two steps ahead of their use.  Workgroup ids
 // are remapped so that workgroups sharing an XCD's L2 share the streamed operands.
+#include <type_traits>
+
 #include "fdma_common.h"
 #include "fdma_params.h"
 
@@ -81,11 +83,18 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
     constexpr int DB = D / 32;
     constexpr int MB = BM / 32;
     constexpr int CH = D / 8, RPP = NTHREADS / CH, Q_IT = BM / RPP;
+    // DMA: the Q / dO tiles and the row statistics of a step go from global memory straight into LDS
+    // (global_load_lds: a wave writes 64 consecutive 16-byte or 4-byte pieces, so the swizzle of the tile is applied
+    // to the GLOBAL address of each lane's piece); no staging registers, no LDS stores, and the loads are issued
+    // between the MFMAs a whole step ahead of the barrier that publishes them.  Needs rows of exactly 256 bytes.
+    constexpr bool DMA = TL::SWZ;
+    static_assert(!DMA || (BM == 32 && NTHREADS == 256), "the direct loads are laid out for 32-row steps and four waves");
 
-    extern __shared__ __attribute__((aligned(16))) char smem[];
+    extern __shared__ __attribute__((aligned(256))) char smem[];
+    const uint32_t lds0 = lds_addr(smem);  // (a multiple of 256)
 
     const FwdParams &f = p.f;
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 31, g = lane >> 5;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = tid & 63, r = lane & 31, g = lane >> 5;
     const int G = f.H / f.Hk;
     // work item: a 128-key block of one (batch, kv head) pair, over query heads [g_lo, g_hi) and segment
     // `seg` of `Sm` of the query range; `slot` >= 0 when the block is shared by several workgroups
@@ -172,6 +181,8 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
         }
     }
 
+    v_base += lds0 + SM::OFF_V;  // from here on an absolute LDS address (see lds_ld128)
+
     f32x16_t dk[DB], dv[DB];
 #pragma unroll
     for (int db = 0; db < DB; db++)
@@ -244,11 +255,16 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
     uint32_t qoff[Q_IT], qoff_l[Q_IT], dooff[Q_IT], dooff_l[Q_IT];
 #pragma unroll
     for (int it = 0; it < Q_IT; it++) {
-        const int row = qr0 + it * RPP, row_c = row < row_last ? row : row_last;
-        qoff[it] = (uint32_t)(row * f.q_r + qcol) * 2;
-        qoff_l[it] = (uint32_t)(row_c * f.q_r + qcol) * 2;
-        dooff[it] = (uint32_t)(row * p.do_r + qcol) * 2;
-        dooff_l[it] = (uint32_t)(row_c * p.do_r + qcol) * 2;
+        // DMA: load n = 2 * wave + it of a tile fills LDS bytes [1024 n, 1024 n + 1024): rows 4n .. 4n+3, lane l the
+        // chunk POSITION l % 16 of row 4n + l / 16, which holds chunk position ^ swz(row) of the global row
+        const int n = 2 * wave + it;
+        const int row = DMA ? 4 * n + (lane >> 4) : qr0 + it * RPP, row_c = row < row_last ? row : row_last;
+        const int chunk = (lane & 15) ^ (int)TL::swz(row);
+        const int col = DMA ? ((chunk * 8 < f.d) ? chunk * 8 : 0) : qcol;
+        qoff[it] = (uint32_t)(row * f.q_r + col) * 2;
+        qoff_l[it] = (uint32_t)(row_c * f.q_r + col) * 2;
+        dooff[it] = (uint32_t)(row * p.do_r + col) * 2;
+        dooff_l[it] = (uint32_t)(row_c * p.do_r + col) * 2;
     }
     gptr_t ld_qbase = nullptr, ld_dobase = nullptr;  // block bases of the step being fetched (scalar registers)
     bool ld_partial = false;
@@ -293,12 +309,69 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
         }
     };
 
+    // ---- DMA staging: block bases of the step being fetched, and its pieces one by one.  Piece 0 .. 2*Q_IT-1: this
+    // wave's Q / dO loads (1 KB each); piece 2*Q_IT (wave 3 only): the row statistics, 32 LSE values and 32 D values
+    // as ONE 4-byte load (lanes 0-31 / 32-63), raw -- log2(e) is applied where the LSE is used, and rows beyond the
+    // end of the queries are clamped here and masked there.
+    typedef __attribute__((address_space(3))) void lds_void_t;
+    typedef const __attribute__((address_space(1))) void gvoid_t;
+    // The steps are walked with counters and running pointers (no division, no 64-bit products per step): inside a
+    // query head the query block index falls by one per step, at a head change everything jumps by loop constants.
+    typedef const __attribute__((address_space(1))) char *gbytes_t;
+    int dma_gi = g_lo, dma_mi = s_hi - 1;  // head and query block of the step being fetched
+    gbytes_t dma_q = nullptr, dma_do = nullptr, dma_stat = nullptr;  // its Q / dO block bases, this lane's statistic
+    char *dma_dst = nullptr;
+    const int64_t q_step = -(int64_t)BM * f.q_r * 2, do_step = -(int64_t)BM * p.do_r * 2;
+    const int64_t q_head = (int64_t)f.q_h * 2 - (int64_t)(n_m - 1) * q_step, do_head = (int64_t)p.do_h * 2 - (int64_t)(n_m - 1) * do_step;
+    const int64_t stat_head = (int64_t)(lane < 32 ? f.lse_h : p.sd_h) * 4 + (int64_t)(n_m - 1) * BM * 4;
+    if (DMA && n_steps > 0) {
+        const int h0 = hk * G + g_lo, m00 = dma_mi * BM;
+        dma_q = (gbytes_t)((const uint16_t *)f.q + b * f.q_b + h0 * f.q_h + (sq.q0 + m00) * f.q_r);
+        dma_do = (gbytes_t)((const uint16_t *)p.dout + b * p.do_b + h0 * p.do_h + (sq.q0 + m00) * p.do_r);
+        dma_stat = (gbytes_t)(lane < 32 ? f.lse + b * f.lse_b + h0 * f.lse_h + sq.q0 + m00 + (lane & 31)
+                                        : p.softmax_d + b * p.sd_b + h0 * p.sd_h + sq.q0 + m00 + (lane & 31));
+    }
+    // sets up the fetch of the step the counters stand at (into stage `buf`)
+    auto dma_begin = [&](int buf) {
+        ld_qbase = dma_q;
+        ld_dobase = dma_do;
+        ld_partial = dma_mi == m_last;
+        dma_dst = smem + buf * SM::STAGE;
+    };
+    // moves the counters to the following step; past the last step they stay (its tiles are fetched again and dropped)
+    auto dma_advance = [&](bool more) {
+        if (!more) return;
+        if (dma_mi == s_lo) {
+            dma_mi = s_hi - 1;
+            dma_gi++;
+            dma_q += q_head; dma_do += do_head; dma_stat += stat_head;
+        } else {
+            dma_mi--;
+            dma_q += q_step; dma_do += do_step; dma_stat -= BM * 4;
+        }
+    };
+    auto dma_piece = [&](int n) {
+        if (n < Q_IT) {
+            __builtin_amdgcn_global_load_lds((gvoid_t *)(ld_qbase + (ld_partial ? qoff_l[n] : qoff[n])),
+                                             (lds_void_t *)(dma_dst + (2 * wave + n) * 1024), 16, 0, 0);
+        } else if (n < 2 * Q_IT) {
+            __builtin_amdgcn_global_load_lds((gvoid_t *)(ld_dobase + (ld_partial ? dooff_l[n - Q_IT] : dooff[n - Q_IT])),
+                                             (lds_void_t *)(dma_dst + SM::Q_BYTES + (2 * wave + n - Q_IT) * 1024), 16, 0, 0);
+        } else {
+            // (every wave fetches the same 256 bytes: cheaper than a branch in the middle of the MFMAs.)  In the last,
+            // partial block the rows beyond the end of the queries read the last row's numbers (masked where used).
+            const int over = ld_partial ? (lane & 31) - row_last : 0;
+            __builtin_amdgcn_global_load_lds((gvoid_t *)(dma_stat - (over > 0 ? over * 4 : 0)), (lds_void_t *)(dma_dst + 2 * SM::Q_BYTES), 4, 0, 0);
+        }
+    };
+
     const int a_row = pi_row(r);
     const int tj = lane & 15, te = tj >> 2, tc = tj & 3;
     const int tcp = (tc == 1) ? 2 : (tc == 2 ? 1 : tc);
     const int tdh = (lane >> 4) & 1;
-    uint32_t tr_off = TL::tr_base(g, te, tdh, tcp);
-    uint32_t a_off = TL::frag_base(a_row, g);
+    uint32_t tr_off = lds0 + TL::tr_base(g, te, tdh, tcp);  // (absolute LDS addresses of stage 0's Q tile)
+    uint32_t a_off = lds0 + TL::frag_base(a_row, g);
+    const uint32_t stat_off = lds0 + 32 * g;  // this lane's eight rows of a block of sixteen row statistics
 
     float colsum = 0.f;
     float cconst = 0.f;
@@ -309,25 +382,40 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
     // one by one between the dK / dV MFMAs (all at once, from every wave at the same moment, they would queue up at the
     // CU's address unit while the matrix pipe idles).
     if (n_steps > 0) {
-        load_step(0, true);
-        store_step(0);
-        cconst = column_const_value();
-        load_step(n_steps > 1 ? 1 : 0, true);
+        if constexpr (DMA) {
+            column_const_load(hk * G + g_lo);
+            dma_begin(0);
+#pragma unroll
+            for (int n = 0; n <= 2 * Q_IT; n++) dma_piece(n);
+            dma_advance(n_steps > 1);
+            cconst = column_const_value();
+        } else {
+            load_step(0, true);
+            store_step(0);
+            cconst = column_const_value();
+            load_step(n_steps > 1 ? 1 : 0, true);
+        }
         __syncthreads();
     }
 
-    for (int step = 0; step < n_steps; step++) {
-        const int gi = g_lo + step / n_m, mi = s_hi - 1 - step % n_m;  // last query block first: see below
+    int cur_gi = g_lo, cur_mi = s_hi - 1;  // (DMA: head and query block of the current step, walked like the fetch)
+    // (one step; the LDS stage is a compile-time constant -- the loop below runs the steps in pairs -- so that every
+    // stage base folds into the offset field of the LDS instructions instead of costing an addition per access)
+    auto one_step = [&](auto buf_c, const int step) {
+        constexpr int buf = decltype(buf_c)::value;
+        const int gi = DMA ? cur_gi : g_lo + step / n_m, mi = DMA ? cur_mi : s_hi - 1 - step % n_m;  // last query block first: see below
         const int h = hk * G + gi;
         const int m0 = mi * BM;
-        const int buf = step & 1;
-        const char *sQ = smem + buf * SM::STAGE;
-        const char *sDO = sQ + SM::Q_BYTES;
-        const float *sLSE = (const float *)(sQ + 2 * SM::Q_BYTES);
-        const float *sDD = sLSE + BM;
         // The swizzled addresses are these lane constants XOR a compile-time value: recomputed where they are used
         // (one VALU operation each); hoisted out of the loop they would cost 30 registers that the kernel does not have.
         if (TL::SWZ) asm volatile("" : "+v"(a_off), "+v"(tr_off), "+v"(v_base));
+        // DMA: the next step's tiles go to the other stage (its readers finished before the last barrier), a piece
+        // every few MFMAs; the column constant is fetched again only when the next step belongs to another query head
+        const bool head_next = DMA && step + 1 < n_steps && mi == s_lo;
+        if constexpr (DMA) {
+            dma_begin(buf ^ 1);
+            if (head_next) column_const_load(h + 1);
+        }
 
         // ---- S = Q K^T and dP = dO V^T (M = query, N = key); fragment reads run a batch ahead
         f32x16_t s[MB], dp[MB];
@@ -340,7 +428,7 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
             u32x4_t a[NF];
             auto frag = [&](int fi) {
                 const int which = fi & 1, mb = (fi >> 1) % MB, ks = (fi >> 1) / MB;
-                return *(const u32x4_t *)((which ? sDO : sQ) + TL::frag_at(a_off, ks) + 32 * mb * TL::ROW_BYTES);
+                return lds_ld128(TL::frag_at(a_off, ks) + (uint32_t)(buf * SM::STAGE + which * SM::Q_BYTES + 32 * mb * TL::ROW_BYTES));
             };
 #pragma unroll
             for (int fi = 0; fi < FR; fi++) a[fi] = frag(fi);
@@ -348,46 +436,54 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
             for (int fi = 0; fi < NF; fi++) {
                 if (fi + FR < NF) a[fi + FR] = frag(fi + FR);
                 const int which = fi & 1, mb = (fi >> 1) % MB, ks = (fi >> 1) / MB;
-                if (which) dp[mb] = E::mfma(a[fi], V_LDS ? *(const u32x4_t *)(sVt + TL::frag_at(v_base, ks)) : vf[V_LDS ? 0 : ks], dp[mb]);
+                if (which) dp[mb] = E::mfma(a[fi], V_LDS ? lds_ld128(TL::frag_at(v_base, ks)) : vf[V_LDS ? 0 : ks], dp[mb]);
                 else s[mb] = E::mfma(a[fi], kf[ks], s[mb]);
+                if constexpr (DMA) {
+                    if (fi % 3 == 1 && fi / 3 <= 2 * Q_IT) dma_piece(fi / 3);
+                }
             }
         }
         // the registers (step i+1) go to the other LDS stage, whose readers finished before the last barrier
         __builtin_amdgcn_sched_barrier(0);
         float cconst_next = cconst;
-        if (step + 1 < n_steps) {
-            store_step(buf ^ 1);
-            cconst_next = column_const_value();
+        if constexpr (!DMA) {
+            if (step + 1 < n_steps) {
+                store_step(buf ^ 1);
+                cconst_next = column_const_value();
+            }
         }
         __builtin_amdgcn_sched_barrier(0);
 
         // ---- P = exp2(S - LSE*log2e), S already scaled and offset by the column constant ; dS = P * (dP - D)
         // diagonal step: some (query, key) pairs of this wave are above the causal diagonal
-        const bool diag = CAUSAL && (okey_wlast > m0 + shift);
+        // (DMA: the statistics are raw, so rows beyond the end of the queries -- clamped duplicates in the last, partial
+        // block -- are masked here as well)
+        const bool diag = (CAUSAL && (okey_wlast > m0 + shift)) || (DMA && m0 + BM > LqS);
         uint32_t ppk[MB * 8], dpk[MB * 8];
         float part = 0.f;
 #pragma unroll
         for (int mb = 0; mb < MB; mb++)
 #pragma unroll
             for (int blk = 0; blk < 2; blk++) {
-                const float *lp = sLSE + 32 * mb + 16 * blk + 8 * g;
-                const float *dpn = sDD + 32 * mb + 16 * blk + 8 * g;
-                const f32x4_t l0 = *(const f32x4_t *)lp, l1 = *(const f32x4_t *)(lp + 4);
-                const f32x4_t d0 = *(const f32x4_t *)dpn, d1 = *(const f32x4_t *)(dpn + 4);
+                const uint32_t so = buf * SM::STAGE + 2 * SM::Q_BYTES + (32 * mb + 16 * blk) * 4;  // LSE; D is BM floats on
+                const f32x4_t l0 = __builtin_bit_cast(f32x4_t, lds_ld128(stat_off + so)), l1 = __builtin_bit_cast(f32x4_t, lds_ld128(stat_off + so + 16));
+                const f32x4_t d0 = __builtin_bit_cast(f32x4_t, lds_ld128(stat_off + so + BM * 4)), d1 = __builtin_bit_cast(f32x4_t, lds_ld128(stat_off + so + BM * 4 + 16));
                 float pv[8], dsv[8];
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
                     const int ii = 8 * blk + e;
                     const float lse2 = e < 4 ? l0[e] : l1[e - 4];
                     const float dd = e < 4 ? d0[e] : d1[e - 4];
-                    pv[e] = fast_exp2(s[mb][ii] - lse2);
+                    pv[e] = fast_exp2(DMA ? __builtin_fmaf(lse2, -kLog2e, s[mb][ii]) : s[mb][ii] - lse2);
                     dsv[e] = dp[mb][ii] - dd;
                 }
                 if (diag) {
                     asm volatile("" ::: "memory");  // keep a real branch: only diagonal steps pay
-                    const int lim = okey - shift - m0 - 32 * mb - 16 * blk - 8 * g;  // rows e >= lim see this key
+                    int lim = CAUSAL ? okey - shift - m0 - 32 * mb - 16 * blk - 8 * g : 0;  // rows e >= lim see this key
+                    int lim_hi = DMA ? LqS - m0 - 32 * mb - 16 * blk - 8 * g : 8;            // rows e < lim_hi exist
+                    asm volatile("" : "+v"(lim), "+v"(lim_hi));  // (the comparisons stay inside the branch)
 #pragma unroll
-                    for (int e = 0; e < 8; e++) pv[e] = e >= lim ? pv[e] : 0.f;
+                    for (int e = 0; e < 8; e++) pv[e] = (e >= lim && e < lim_hi) ? pv[e] : 0.f;
                 }
 #pragma unroll
                 for (int e = 0; e < 8; e++) {
@@ -404,15 +500,16 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
 
         // ---- dV^T += dO^T P ; dK^T += Q^T dS   (M = d, N = key, contraction = query)
         // (after the last steps an existing tile is fetched again and dropped)
-        load_step(step + 2 < n_steps ? step + 2 : step, false);
+        if constexpr (!DMA) load_step(step + 2 < n_steps ? step + 2 : step, false);
         {   // the transposing fragment reads run one (query block, d block) pair ahead of the MFMAs that use them
             constexpr int NP = (BM / 16) * DB;
             u32x4_t a1[2], a2[2];
             auto frag = [&](int idx, int slot) {
                 const int qb = idx / DB, db = idx % DB;
                 const uint32_t off = TL::tr_at(tr_off, qb, db, 0), off_hi = TL::tr_at(tr_off, qb, db, 1);
-                const u32x2_t lo = lds_read_tr16(sDO, off), hi = lds_read_tr16(sDO, off_hi);
-                const u32x2_t lo2 = lds_read_tr16(sQ, off), hi2 = lds_read_tr16(sQ, off_hi);
+                constexpr uint32_t st = buf * SM::STAGE;
+                const u32x2_t lo = lds_ld_tr16(off + st + SM::Q_BYTES), hi = lds_ld_tr16(off_hi + st + SM::Q_BYTES);
+                const u32x2_t lo2 = lds_ld_tr16(off + st), hi2 = lds_ld_tr16(off_hi + st);
                 a1[slot] = u32x4_t{lo[0], lo[1], hi[0], hi[1]};
                 a2[slot] = u32x4_t{lo2[0], lo2[1], hi2[0], hi2[1]};
             };
@@ -425,8 +522,10 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
                 const u32x4_t sb = {dpk[4 * qb], dpk[4 * qb + 1], dpk[4 * qb + 2], dpk[4 * qb + 3]};
                 dv[db] = E::mfma(a1[idx & 1], pb, dv[db]);
                 dk[db] = E::mfma(a2[idx & 1], sb, dk[db]);
+                if constexpr (!DMA) {
 #pragma unroll
-                for (int n = idx * 2 * Q_IT / NP; n < (idx + 1) * 2 * Q_IT / NP; n++) load_item(n);
+                    for (int n = idx * 2 * Q_IT / NP; n < (idx + 1) * 2 * Q_IT / NP; n++) load_item(n);
+                }
             }
             // pin the order: reads of pair idx+1, then the two MFMAs of pair idx
             __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
@@ -439,7 +538,7 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
 
         // ---- dBias column sum: flush when the bias head changes
         if (has_bias) {
-            const bool last_m = (step % n_m) == n_m - 1;
+            const bool last_m = mi == s_lo;
             if (last_m && (slot >= 0 || f.Hb == f.H || gi == G - 1)) {
                 const float tot = xhalf_sum(colsum);
                 const int hb = f.Hb == f.H ? h : (f.Hb == 1 ? 0 : hk);
@@ -453,8 +552,18 @@ __global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const Bwd
             }
         }
 
-        cconst = cconst_next;
-        __syncthreads();
+        if constexpr (DMA) {
+            if (head_next) cconst = column_const_value();
+            dma_advance(step + 2 < n_steps);
+            if (cur_mi == s_lo) { cur_mi = s_hi - 1; cur_gi++; } else cur_mi--;
+        } else {
+            cconst = cconst_next;
+        }
+        __syncthreads();  // (also waits for this wave's direct loads: the next step's stage is complete behind it)
+    };
+    for (int step = 0; step < n_steps; step += 2) {
+        one_step(std::integral_constant<int, 0>(), step);
+        if (step + 1 < n_steps) one_step(std::integral_constant<int, 1>(), step + 1);
     }
 
     // a key block that no query can see still owns its dbias column

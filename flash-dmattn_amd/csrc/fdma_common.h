@@ -132,6 +132,19 @@ __device__ __forceinline__ u32x2_t lds_read_tr16(const char *smem_base, uint32_t
     return __builtin_bit_cast(u32x2_t, v);
 }
 
+// LDS accesses by absolute byte address.  A lane keeps its part of an address (row, chunk, swizzle) in one register
+// that already includes the start of the workgroup's dynamic LDS; what is added to it at compile time then lands
+// in the offset field of the instruction.  (XOR-ing compile-time bits below 256 into such an address equals XOR-ing
+// them into the offset alone as long as the dynamic LDS starts at a multiple of 256 bytes: declare it aligned(256).)
+__device__ __forceinline__ uint32_t lds_addr(const void *p) { return (uint32_t)(uintptr_t)(const lds_char_t *)p; }
+__device__ __forceinline__ u32x4_t lds_ld128(uint32_t addr) {
+    return *(const __attribute__((address_space(3))) u32x4_t *)(uintptr_t)addr;
+}
+__device__ __forceinline__ u32x2_t lds_ld_tr16(uint32_t addr) {
+    s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t *)(uintptr_t)addr);
+    return __builtin_bit_cast(u32x2_t, v);
+}
+
 // Row-major LDS tile of 16-bit elements ([row][head dim]) that is read two ways: as MFMA fragments (ds_read_b128:
 // lane (r, g) takes the 16 bytes of chunk 2*ks + g of row pi_row(r)) and through transposing reads (lds_read_tr16:
 // 16 lanes take four 8-byte pieces of each of four consecutive rows), and written row by row (16 lanes per row).
