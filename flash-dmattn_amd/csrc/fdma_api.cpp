@@ -53,6 +53,14 @@ int validate_common(const fdma_fwd_args *a, bool backward) {
     if (a->head_dim <= 0 || a->head_dim % 8 != 0)
         return fail(FDMA_ERR_INVALID, backward ? "head_size should be a multiple of 8"
                                                : "query, key, value, and out_ must have a head_size that is a multiple of 8");
+    if (a->kept.idx || a->kept.cnt || a->kept.count) {
+        if (!(a->kept.idx && a->kept.cnt && a->kept.count))
+            return fail(FDMA_ERR_INVALID, "kept: idx, cnt and count must be given together");
+        if (a->kept.ld < a->seqlen_k || a->kept.ld % 16 != 0)
+            return fail(FDMA_ERR_INVALID, "kept.ld must be a multiple of 16 and at least seqlen_k");
+        if ((reinterpret_cast<uintptr_t>(a->kept.cnt) | reinterpret_cast<uintptr_t>(a->kept.idx)) & 15)
+            return fail(FDMA_ERR_INVALID, "kept.idx and kept.cnt must be 16-byte aligned");
+    }
     if (a->num_heads % a->num_heads_k != 0)
         return fail(FDMA_ERR_INVALID, "Number of heads in key/value must divide number of heads in query");
     if (!a->q || ((!a->k || !a->v) && a->seqlen_k > 0)) return fail(FDMA_ERR_INVALID, "q, k, v must be device pointers");
@@ -110,6 +118,10 @@ void fill_fwd_params(const fdma_fwd_args *a, fdma::FwdParams &p) {
     p.scale_log2 = a->softmax_scale * 1.4426950408889634f;
     p.splits = 1;
     p.compact_mode = a->compact_mode;
+    if (a->mask && a->kept.idx && a->kept.cnt && a->kept.count) {  // (validate_common has checked the row stride)
+        p.kept_idx = a->kept.idx; p.kept_cnt = a->kept.cnt; p.kept_count = a->kept.count;
+        p.kept_ld = a->kept.ld;
+    }
     p.lse_b = (int64_t)a->num_heads * a->seqlen_q;
     p.lse_h = a->seqlen_q;
 }
@@ -351,7 +363,7 @@ size_t fdma_bwd_workspace_bytes(const fdma_bwd_args *a) {
     if (!a) return 0;
     fdma::FwdParams p;
     fill_fwd_params(&a->f, p);
-    return dbias_accum_bytes(a) + (fdma::use_compact(p) ? fdma::compact_bytes(p, true) : 0);
+    return dbias_accum_bytes(a) + (fdma::use_compact(p) ? fdma::compact_bytes(p, true, a->fwd_workspace != nullptr) : 0);
 }
 
 int fdma_bwd(const fdma_bwd_args *a, void *hip_stream) {
@@ -385,7 +397,11 @@ int fdma_bwd(const fdma_bwd_args *a, void *hip_stream) {
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     hipError_t e;
     if (a->f.seqlen_q > 0 && fdma::use_compact(p.f)) {
-        e = fdma::compact_setup(p.f, static_cast<char *>(a->workspace) + dbias_accum_bytes(a), a->f.dtype, stream, &p);
+        if (a->fwd_workspace && a->fwd_workspace_bytes < fdma::compact_bytes(p.f, false))
+            return fail(FDMA_ERR_WORKSPACE, "fwd_workspace too small: the forward call of this problem needs %zu bytes, got %zu",
+                        fdma::compact_bytes(p.f, false), a->fwd_workspace_bytes);
+        e = fdma::compact_setup(p.f, static_cast<char *>(a->workspace) + dbias_accum_bytes(a), a->f.dtype, stream, &p,
+                                a->fwd_workspace);
         if (e != hipSuccess) return fail(FDMA_ERR_LAUNCH, "backward launch failed: %s", hipGetErrorString(e));
     }
     e = fdma::launch_bwd(p, a->f.dtype, stream);
@@ -477,6 +493,14 @@ int fdma_create_mask_validate(const fdma_mask_args *a) {
     if (!empty && (!a->bias || !a->mask_out)) return fail(FDMA_ERR_INVALID, "bias and mask_out must be device pointers");
     if (reinterpret_cast<uintptr_t>(a->bias) & 1) return fail(FDMA_ERR_INVALID, "bias must be 2-byte aligned");
     if (std::isnan(a->min_value)) return fail(FDMA_ERR_INVALID, "min_dtype must not be NaN");
+    if (a->kept_idx || a->kept_cnt || a->kept_count) {
+        if (!(a->kept_idx && a->kept_cnt && a->kept_count))
+            return fail(FDMA_ERR_INVALID, "kept_idx, kept_cnt and kept_count must be given together");
+        if (a->kept_ld < a->seqlen_k || a->kept_ld % 16 != 0)
+            return fail(FDMA_ERR_INVALID, "kept_ld must be a multiple of 16 and at least seqlen_k");
+        if ((reinterpret_cast<uintptr_t>(a->kept_cnt) | reinterpret_cast<uintptr_t>(a->kept_idx)) & 15)
+            return fail(FDMA_ERR_INVALID, "kept_idx and kept_cnt must be 16-byte aligned");
+    }
     return FDMA_OK;
 }
 
@@ -521,6 +545,8 @@ int fdma_create_mask(const fdma_mask_args *a, void *hip_stream) {
     p.type = a->type;
     p.dtype = a->dtype;
     p.min_bits = to_bits16(a->min_value, a->dtype);
+    p.kept_idx = a->kept_idx; p.kept_cnt = a->kept_cnt; p.kept_count = a->kept_count;
+    p.kept_ld = a->kept_ld;
     const hipError_t e = fdma::launch_make_mask(p, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(FDMA_ERR_LAUNCH, "mask launch failed: %s", hipGetErrorString(e));
     return FDMA_OK;

@@ -18,14 +18,13 @@
 #include "fdma_common.h"
 #include "fdma_params.h"
 #include "fdma_bwd_dot.h"
+#include "fdma_scan.h"
 
 namespace fdma {
 
 namespace {
 
 constexpr int SCAN_THREADS = 1024;
-constexpr int SCAN_KEYS = 16;                          // mask bytes per thread per pass
-constexpr int SCAN_RANGE = SCAN_THREADS * SCAN_KEYS;   // keys per pass
 constexpr int GATHER_KEYS = 64;                        // compacted keys per gather workgroup
 
 inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
@@ -67,70 +66,37 @@ __global__ void __launch_bounds__(SCAN_THREADS) compact_scan_kernel(const FwdPar
     __shared__ int s_wave[SCAN_THREADS / 64];
     const int pair = blockIdx.x, b = pair / p.Hk, hk = pair % p.Hk;
     const int hm = p.Hm == 1 ? 0 : hk;
-    const uint8_t *mrow = p.mask + b * p.m_b + hm * p.m_h;
-    int32_t *irow = idx + (size_t)pair * ld;
-    int32_t *crow = cnt + (size_t)pair * ld;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-    int base = 0;
-    for (int c0 = 0; c0 < p.Lk; c0 += SCAN_RANGE) {
-        const int col = c0 + tid * SCAN_KEYS;
-        uint32_t bits = 0;
-        if (col < p.Lk) {
-            const u32x4_t mv = *(const u32x4_t *)(mrow + col);
-#pragma unroll
-            for (int e = 0; e < SCAN_KEYS; e++) {
-                const uint32_t byte = (mv[e >> 2] >> (8 * (e & 3))) & 0xffu;
-                if (byte && col + e < p.Lk) bits |= 1u << e;
-            }
-        }
-        const int n = __builtin_popcount(bits);
-        int incl = n;
-#pragma unroll
-        for (int off = 1; off < 64; off <<= 1) {
-            const int t = __shfl_up(incl, off);
-            if (lane >= off) incl += t;
-        }
-        if (lane == 63) s_wave[wave] = incl;
-        __syncthreads();
-        int woff = 0, total = 0;
-#pragma unroll
-        for (int w = 0; w < SCAN_THREADS / 64; w++) {
-            const int v = s_wave[w];
-            if (w < wave) woff += v;
-            total += v;
-        }
-        if (col < p.Lk) {
-            int run = base + woff + incl - n;
-            int32_t cv[SCAN_KEYS];
-#pragma unroll
-            for (int e = 0; e < SCAN_KEYS; e++) {
-                if (bits & (1u << e)) irow[run++] = col + e;
-                cv[e] = run;
-            }
-#pragma unroll
-            for (int q = 0; q < SCAN_KEYS / 4; q++) {
-                u32x4_t w = {(uint32_t)cv[4 * q], (uint32_t)cv[4 * q + 1], (uint32_t)cv[4 * q + 2], (uint32_t)cv[4 * q + 3]};
-                *(u32x4_t *)(crow + col + 4 * q) = w;  // ld is a multiple of 16: the row has room
-            }
-        }
-        base += total;
-        __syncthreads();
-    }
-    if (tid == 0) count[pair] = base;
+    scan_mask_row<SCAN_THREADS>(p.mask + b * p.m_b + hm * p.m_h, p.Lk, idx + (size_t)pair * ld, cnt + (size_t)pair * ld,
+                                count + pair, s_wave, true);
 }
 
 // orig: the caller's tensors.  kc / vc: dense [B*Hk, Lk, d] destinations.
 template <typename T>
-__device__ __forceinline__ void gather_block(const FwdParams &p, const int32_t *idx, const int32_t *count, float *fb,
+__device__ __forceinline__ void gather_block(const FwdParams &p, const int32_t *idx, int32_t *cnt, const int32_t *count, float *fb,
                                              uint16_t *kc, uint16_t *vc, int ld, int Hfb, int block_x, int pair) {
     using E = Elem<T>;
     const int b = pair / p.Hk, hk = pair % p.Hk;
-    const int n = count[pair];
+    const int tid = threadIdx.x;
     const int c0 = block_x * GATHER_KEYS;
+    // Lists handed over by the caller (one row per mask row): this block copies its 64 entries of the row into the
+    // per-pair arrays the kernels index (in place of the scan), and reads its own inputs from the source
+    const int32_t *src_idx = idx + (size_t)pair * ld;
+    int n;
+    if (p.kept_idx) {
+        const int srow = (p.m_b == 0 ? 0 : b) * p.Hm + (p.Hm == 1 ? 0 : hk);
+        src_idx = p.kept_idx + (size_t)srow * p.kept_ld;
+        n = p.kept_count[srow];
+        if (tid < GATHER_KEYS && c0 + tid < ld) {
+            ((int32_t *)idx)[(size_t)pair * ld + c0 + tid] = src_idx[c0 + tid];
+            cnt[(size_t)pair * ld + c0 + tid] = p.kept_cnt[(size_t)srow * p.kept_ld + c0 + tid];
+        }
+        if (block_x == 0 && tid == 0) ((int32_t *)count)[pair] = n;
+    } else {
+        n = count[pair];
+    }
     if (c0 >= n) return;
     __shared__ int s_src[GATHER_KEYS];
-    const int tid = threadIdx.x;
-    if (tid < GATHER_KEYS) s_src[tid] = (c0 + tid < n) ? idx[(size_t)pair * ld + c0 + tid] : -1;
+    if (tid < GATHER_KEYS) s_src[tid] = (c0 + tid < n) ? src_idx[c0 + tid] : -1;
     __syncthreads();
     const int CH = p.d / 8;
     const uint16_t *kb = (const uint16_t *)p.k + b * p.k_b + hk * p.k_h;
@@ -165,9 +131,9 @@ __device__ __forceinline__ void gather_block(const FwdParams &p, const int32_t *
 }
 
 template <typename T>
-__global__ void __launch_bounds__(256) compact_gather_kernel(const FwdParams p, const int32_t *idx, const int32_t *count,
+__global__ void __launch_bounds__(256) compact_gather_kernel(const FwdParams p, const int32_t *idx, int32_t *cnt, const int32_t *count,
                                                               float *fb, uint16_t *kc, uint16_t *vc, int ld, int Hfb) {
-    gather_block<T>(p, idx, count, fb, kc, vc, ld, Hfb, blockIdx.x, blockIdx.y);
+    gather_block<T>(p, idx, cnt, count, fb, kc, vc, ld, Hfb, blockIdx.x, blockIdx.y);
 }
 
 // Gradient rows (dK, dV) and columns (dBias) of dropped keys: no workgroup of the compacted backward
@@ -409,12 +375,13 @@ __device__ __forceinline__ void plan_block(const int32_t *count, const int32_t *
 // on compute D = rowsum(dO * O), which depends on none of the others.
 // The plan is a chain of dependent steps of a single workgroup (18 us); side by side with the other two it costs nothing.
 template <typename T>
-__global__ void __launch_bounds__(256) compact_bwd_prepass_kernel(const BwdParams bp, const int32_t *idx,
+__global__ void __launch_bounds__(256) compact_bwd_prepass_kernel(const BwdParams bp, const int32_t *idx, int32_t *cnt,
                                                                    const int32_t *count, float *fb, uint16_t *kc, uint16_t *vc,
-                                                                   int ld, int Hfb, int32_t *plan, int slots, int cap) {
+                                                                   int ld, int Hfb, int32_t *plan, int slots, int cap, int do_gather) {
     const FwdParams &f = bp.f;
     if (blockIdx.z == 0) {
-        gather_block<T>(f, idx, count, fb, kc, vc, ld, Hfb, blockIdx.x, blockIdx.y);
+        // (not when the lists and copies exist already: made by an earlier launch, or by the forward call)
+        if (do_gather) gather_block<T>(f, idx, cnt, count, fb, kc, vc, ld, Hfb, blockIdx.x, blockIdx.y);
     } else if (blockIdx.z == 1) {
         zero_block(bp, bp.dbias != nullptr && bp.dbias_accum == nullptr, blockIdx.x, blockIdx.y);
     } else if (blockIdx.z == 2) {
@@ -442,7 +409,10 @@ bool use_compact(const FwdParams &p) {
     return p.Lq >= 128 && p.Lk >= 128 && (int64_t)p.Lq * (p.H / p.Hk) * p.Lk >= (int64_t)1 << 21;
 }
 
-size_t compact_bytes(const FwdParams &p, bool backward) { return layout_of(p, backward).total; }
+size_t compact_bytes(const FwdParams &p, bool backward, bool reuse_fwd) {
+    const Layout l = layout_of(p, backward);
+    return backward && reuse_fwd ? l.total - l.off_plan : l.total;  // (with the forward's workspace: plan and partial sums only)
+}
 
 void dkdv_split_bounds(int pairs, int n_max, int G, int &grid, int &slots) {
     const int k = dkdv_lists_per_pair(pairs);
@@ -484,26 +454,36 @@ static int device_cus() {
     return n;
 }
 
-hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, BwdParams *bp) {
+hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, BwdParams *bp, const void *fwd_ws) {
     const Layout l = layout_of(p, bp != nullptr);
-    char *w = static_cast<char *>(ws);
+    // the lists and the K / V copies: in this call's workspace, or (backward) where the forward call left them
+    char *w = fwd_ws ? const_cast<char *>(static_cast<const char *>(fwd_ws)) : static_cast<char *>(ws);
+    // plan and partial sums of the backward: behind the lists, or alone in `ws` when the lists are the forward's
+    char *wb = fwd_ws ? static_cast<char *>(ws) - l.off_plan : static_cast<char *>(ws);
     int32_t *idx = (int32_t *)(w + l.off_idx), *cnt = (int32_t *)(w + l.off_cnt), *count = (int32_t *)(w + l.off_count);
     float *fb = (float *)(w + l.off_fb);
     uint16_t *kc = (uint16_t *)(w + l.off_k), *vc = (uint16_t *)(w + l.off_v);
     const int pairs = p.B * p.Hk;
-    hipLaunchKernelGGL(compact_scan_kernel, dim3(pairs), dim3(SCAN_THREADS), 0, stream, p, idx, cnt, count, l.ld);
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
-    const dim3 grid((p.Lk + GATHER_KEYS - 1) / GATHER_KEYS, pairs);
-    if (!bp) {
-        if (dtype == 0)
-            hipLaunchKernelGGL((compact_gather_kernel<bf16_tag>), grid, dim3(256), 0, stream, p, idx, count, fb, kc, vc, l.ld, l.Hfb);
-        else
-            hipLaunchKernelGGL((compact_gather_kernel<fp16_tag>), grid, dim3(256), 0, stream, p, idx, count, fb, kc, vc, l.ld, l.Hfb);
+    hipError_t e;
+    const bool have_lists = fwd_ws != nullptr || p.kept_idx != nullptr;
+    if (!have_lists) {
+        hipLaunchKernelGGL(compact_scan_kernel, dim3(pairs), dim3(SCAN_THREADS), 0, stream, p, idx, cnt, count, l.ld);
         if ((e = hipGetLastError()) != hipSuccess) return e;
-    } else {
+    }
+    const dim3 grid((p.Lk + GATHER_KEYS - 1) / GATHER_KEYS, pairs);
+    // (handed-over lists: the gather launch also copies them into the per-pair arrays, which the backward's other
+    // pre-pass layers read -- so it runs on its own in front of them)
+    const bool gather_alone = !bp || (p.kept_idx != nullptr && !fwd_ws);
+    if (gather_alone && !fwd_ws) {
+        if (dtype == 0)
+            hipLaunchKernelGGL((compact_gather_kernel<bf16_tag>), grid, dim3(256), 0, stream, p, idx, cnt, count, fb, kc, vc, l.ld, l.Hfb);
+        else
+            hipLaunchKernelGGL((compact_gather_kernel<fp16_tag>), grid, dim3(256), 0, stream, p, idx, cnt, count, fb, kc, vc, l.ld, l.Hfb);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+    }
+    if (bp) {
         // (p is bp->f, still describing the caller's tensors here)
-        int32_t *plan = (int32_t *)(w + l.off_plan);
+        int32_t *plan = (int32_t *)(wb + l.off_plan);
         int dkdv_grid, slots;
         dkdv_split_bounds(pairs, (p.Lk + 127) / 128, p.H / p.Hk, dkdv_grid, slots);
         const int plan_cap = dkdv_grid / 8;  // entries per XCD list: the dK/dV kernel's workgroups per XCD
@@ -513,17 +493,18 @@ hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, 
         const int64_t dot_layers = (dot_blocks + layer - 1) / layer;
         const bool with_dot = p.cu_q == nullptr && 3 + dot_layers <= 65535;
         const dim3 grid3(grid.x, pairs, with_dot ? (unsigned)(3 + dot_layers) : 3);
+        const int do_gather = (fwd_ws || gather_alone) ? 0 : 1;
         if (dtype == 0)
-            hipLaunchKernelGGL((compact_bwd_prepass_kernel<bf16_tag>), grid3, dim3(256), 0, stream, *bp, idx, count, fb, kc, vc,
-                               l.ld, l.Hfb, plan, 2 * device_cus(), plan_cap);
+            hipLaunchKernelGGL((compact_bwd_prepass_kernel<bf16_tag>), grid3, dim3(256), 0, stream, *bp, idx, cnt, count, fb, kc, vc,
+                               l.ld, l.Hfb, plan, 2 * device_cus(), plan_cap, do_gather);
         else
-            hipLaunchKernelGGL((compact_bwd_prepass_kernel<fp16_tag>), grid3, dim3(256), 0, stream, *bp, idx, count, fb, kc, vc,
-                               l.ld, l.Hfb, plan, 2 * device_cus(), plan_cap);
+            hipLaunchKernelGGL((compact_bwd_prepass_kernel<fp16_tag>), grid3, dim3(256), 0, stream, *bp, idx, cnt, count, fb, kc, vc,
+                               l.ld, l.Hfb, plan, 2 * device_cus(), plan_cap, do_gather);
         if ((e = hipGetLastError()) != hipSuccess) return e;
         bp->dot_done = with_dot ? 1 : 0;
         p.cmp.plan = plan;
-        bp->dkv_part = (float *)(w + l.off_part_kv);
-        bp->db_part = (float *)(w + l.off_part_db);
+        bp->dkv_part = (float *)(wb + l.off_part_kv);
+        bp->db_part = (float *)(wb + l.off_part_db);
     }
     p.k = kc;
     p.v = vc;

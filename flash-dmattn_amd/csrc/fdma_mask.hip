@@ -17,6 +17,7 @@
 // length; exactly half is dropped).
 #include "fdma_common.h"
 #include "fdma_params.h"
+#include "fdma_scan.h"
 
 namespace fdma {
 namespace {
@@ -245,6 +246,14 @@ __global__ void __launch_bounds__(NT) make_mask_kernel(const MaskParams p) {
             const uint8_t keep = (2 * votes > len) ? 1 : 0;
             for (int c = 0; c < len; c++) orow[c0 + c] = keep;
         }
+    }
+
+    // ---- optional second output: the row as an ordered list of kept columns with prefix counts, the form the
+    // compaction path of the attention kernels works on (they then need no pass of their own over the mask)
+    if (p.kept_idx) {
+        __syncthreads();  // the row's stores are visible to the whole workgroup
+        scan_mask_row<NT>(orow, Lk, p.kept_idx + (size_t)row * p.kept_ld, p.kept_cnt + (size_t)row * p.kept_ld,
+                          p.kept_count + row, (int *)wave_cnt, false);
     }
 }
 

@@ -117,6 +117,10 @@ struct FwdParams {
     int32_t splits;
     int32_t compact_mode;  // FDMA_COMPACT_* of the C ABI: 0 = decide from the problem, 1 = never, 2 = whenever the mask form allows
     Compact cmp;        // when cmp.on, k / v (and their strides) describe the compacted copies
+    // kept-column lists handed over by the caller (fdma_kept_keys of the C ABI; nullptr = scan the mask): one row per
+    // (mask batch entry, mask head)
+    const int32_t *kept_idx, *kept_cnt, *kept_count;
+    int32_t kept_ld;
 };
 
 // lengths and first rows of batch entry b
@@ -176,6 +180,8 @@ struct MaskParams {
     int32_t type;        // 0 = top-k, 1 = relu
     int32_t dtype;       // 0 = bf16, 1 = fp16
     uint32_t min_bits;   // the fill value for entries the incoming mask excludes, as bits of the bias type
+    int32_t *kept_idx, *kept_cnt, *kept_count;  // optional second output (nullptr = not wanted): see scan_mask_row
+    int32_t kept_ld;
 };
 hipError_t launch_make_mask(const MaskParams &p, hipStream_t stream);
 
@@ -243,9 +249,12 @@ hipError_t launch_bwd_dq(const BwdParams &p, int dtype, hipStream_t stream);
 // p.cmp; for a backward call (bp given) the same launch zero-fills the gradient rows / columns of dropped keys
 // and makes the dK/dV plan.
 bool use_compact(const FwdParams &p);
-size_t compact_bytes(const FwdParams &p, bool backward);
+size_t compact_bytes(const FwdParams &p, bool backward, bool reuse_fwd = false);
 // bp != nullptr: backward -- also plans the dK/dV split and sets bp->dkv_part / bp->db_part
-hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, BwdParams *bp = nullptr);
+// `fwd_ws` (backward only): the workspace a forward call of the same problem filled; its lists and copies are used
+// instead of being made again, and `ws` then holds the backward's plan and partial sums alone.
+hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, BwdParams *bp = nullptr,
+                         const void *fwd_ws = nullptr);
 // host-side bounds over every possible unit count 1..U_max: workgroups to launch, partial slots to hold
 // (n_max = units of one pair at most)
 void dkdv_split_bounds(int pairs, int n_max, int G, int &grid, int &slots);

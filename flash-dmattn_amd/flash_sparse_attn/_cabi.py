@@ -17,6 +17,11 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _DEFAULT_LIB = os.path.normpath(os.path.join(_HERE, "..", "lib", "libfdma_hip.so"))
 
 
+class KeptKeys(ctypes.Structure):
+    """fdma_kept_keys: the kept columns of a query-broadcast keep-mask as lists."""
+    _fields_ = [("idx", ctypes.c_void_p), ("cnt", ctypes.c_void_p), ("count", ctypes.c_void_p), ("ld", ctypes.c_int32)]
+
+
 class FwdArgs(ctypes.Structure):
     _fields_ = [
         ("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p),
@@ -32,6 +37,7 @@ class FwdArgs(ctypes.Structure):
         ("softmax_scale", ctypes.c_float), ("softcap", ctypes.c_float),
         ("compact_mode", ctypes.c_int32),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
+        ("kept", KeptKeys),
     ]
 
 
@@ -47,6 +53,7 @@ class BwdArgs(ctypes.Structure):
         ("softmax_d", ctypes.c_void_p),
         ("deterministic", ctypes.c_int32),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
+        ("fwd_workspace", ctypes.c_void_p), ("fwd_workspace_bytes", ctypes.c_size_t),
     ]
 
 
@@ -85,6 +92,8 @@ class MaskArgs(ctypes.Structure):
         ("batch", ctypes.c_int32), ("heads", ctypes.c_int32), ("rows", ctypes.c_int32), ("seqlen_k", ctypes.c_int32),
         ("window", ctypes.c_int32), ("block_size", ctypes.c_int32), ("type", ctypes.c_int32), ("dtype", ctypes.c_int32),
         ("min_value", ctypes.c_float),
+        ("kept_idx", ctypes.c_void_p), ("kept_cnt", ctypes.c_void_p), ("kept_count", ctypes.c_void_p),
+        ("kept_ld", ctypes.c_int32),
     ]
 
 
@@ -179,8 +188,8 @@ def _load() -> ctypes.CDLL:
     lib.fdma_abi_version.restype = ctypes.c_int
     lib.fdma_sizeof_fwd_args.restype = ctypes.c_size_t
     lib.fdma_sizeof_bwd_args.restype = ctypes.c_size_t
-    if lib.fdma_abi_version() != 3:
-        raise ImportError(f"{path}: ABI version {lib.fdma_abi_version()} != 3")
+    if lib.fdma_abi_version() != 4:
+        raise ImportError(f"{path}: ABI version {lib.fdma_abi_version()} != 4")
     lib.fdma_varlen_fwd.argtypes = [ctypes.POINTER(VarlenFwdArgs), ctypes.c_void_p]
     lib.fdma_varlen_fwd.restype = ctypes.c_int
     lib.fdma_varlen_bwd.argtypes = [ctypes.POINTER(VarlenBwdArgs), ctypes.c_void_p]
@@ -248,12 +257,13 @@ def _bcast3(t: torch.Tensor) -> Sequence[int]:
     return tuple(0 if t.size(i) == 1 else t.stride(i) for i in range(3))
 
 
-_FWD_STRUCT = struct.Struct("@7P18q10i2fiPN")
+_FWD_STRUCT = struct.Struct("@7P18q10i2fiPN3Pi4x")
 assert _FWD_STRUCT.size == ctypes.sizeof(FwdArgs)
 
 
-def fill_fwd(a: FwdArgs, q, k, v, mask, bias, out, lse, softmax_scale, is_causal, softcap) -> None:
-    """Fill the argument block in one struct.pack (ctypes field-by-field assignment costs ~10 us a call)."""
+def fill_fwd(a: FwdArgs, q, k, v, mask, bias, out, lse, softmax_scale, is_causal, softcap, kept=None) -> None:
+    """Fill the argument block in one struct.pack (ctypes field-by-field assignment costs ~10 us a call).
+    `kept`: None, or (idx, cnt, count, ld) -- the mask's kept columns as int32 tensors (fdma_kept_keys)."""
     ms = _bcast3(mask) if mask is not None else (0, 0, 0)
     bs = _bcast3(bias) if bias is not None else (0, 0, 0)
     batch, seqlen_q, num_heads, head_dim = q.shape
@@ -269,6 +279,8 @@ def fill_fwd(a: FwdArgs, q, k, v, mask, bias, out, lse, softmax_scale, is_causal
         mask.shape[1] if mask is not None else 1, bias.shape[1] if bias is not None else 1,
         head_dim, dtype_code(q), int(bool(is_causal)),
         float(softmax_scale), float(softcap), _compact_mode, 0, 0,
+        kept[0].data_ptr() if kept else 0, kept[1].data_ptr() if kept else 0, kept[2].data_ptr() if kept else 0,
+        kept[3] if kept else 0,
     )
 
 

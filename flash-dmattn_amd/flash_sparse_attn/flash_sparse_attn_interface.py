@@ -15,11 +15,13 @@ Differences that are visible only in cost, not in results:
   * dK / dV / dBias come out of the kernels at their final shapes; there are no expanded
     temporaries or host-side reductions (flash_api.cpp:970-983, 1027-1047).
 """
+import threading
 from typing import Any, Optional, Tuple
 
 import torch
 
 from . import _cabi
+from .utils.mask import kept_keys_of
 
 
 def maybe_contiguous(x: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
@@ -101,11 +103,37 @@ def _check_inputs(q, k, v, mask, bias) -> None:
             raise RuntimeError(f"Key length dimension in {name} must be seqlen_k_rounded")
 
 
+# Side inputs of the two operator bodies that are not part of the reference's operator signatures: the kept-key
+# lists of a mask made by the device mask builder, and the forward call's workspace (index lists and compacted K / V
+# copies), which the backward of the same autograd node reuses.  FlashDMAttnFunc sets them around its calls; a body
+# that is called without them (torch.compile, direct operator calls) takes the ordinary path.
+_tls = threading.local()
+
+
+class _handoff:
+    def __init__(self, **items):
+        self.items = items
+
+    def __enter__(self):
+        self.prev = getattr(_tls, "items", None)
+        _tls.items = self.items
+        return self.items
+
+    def __exit__(self, *exc):
+        _tls.items = self.prev
+
+
+def _handoff_get(name):
+    items = getattr(_tls, "items", None)
+    return items.get(name) if items else None
+
+
 def _flash_sparse_attn_forward_body(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Optional[torch.Tensor], bias: Optional[torch.Tensor],
     softmax_scale: float, is_causal: bool, softcap: float, return_softmax: bool,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     _check_inputs(q, k, v, mask, bias)
+    kept = _handoff_get("kept") or kept_keys_of(mask)
     q, k, v = [_aligned(x, 8) for x in (q, k, v)]
     mask = _aligned(mask, 16)
     bias = _aligned(bias, 8)
@@ -118,7 +146,7 @@ def _flash_sparse_attn_forward_body(
     if seqlen_q == 0:
         return out, softmax_lse, p
     args = _cabi.FwdArgs()
-    _cabi.fill_fwd(args, q, k, v, mask, bias, out, softmax_lse, softmax_scale, is_causal, softcap)
+    _cabi.fill_fwd(args, q, k, v, mask, bias, out, softmax_lse, softmax_scale, is_causal, softcap, kept)
     with _cabi.device_guard(q.device):
         nbytes = _cabi.lib.fdma_fwd_workspace_bytes(args)
         workspace = None
@@ -126,6 +154,10 @@ def _flash_sparse_attn_forward_body(
             workspace = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
             args.workspace, args.workspace_bytes = workspace.data_ptr(), nbytes
         _cabi.check(_cabi.lib.fdma_fwd(args, _cabi.current_stream(q.device)))
+    items = getattr(_tls, "items", None)
+    if items is not None and workspace is not None and seqlen_q > 1:
+        # (the compaction path's lists and copies; what identifies the problem they belong to goes with them)
+        items["fwd_ws_out"] = (workspace, _cabi.get_compact_mode(), None if bias is None else tuple(bias.shape))
     return out, softmax_lse, p
 
 
@@ -196,7 +228,10 @@ def _flash_sparse_attn_backward_body(
         dbias_final, dbias_w = dbias_w, torch.empty_like(bias)
 
     args = _cabi.BwdArgs()
-    _cabi.fill_fwd(args.f, q, k, v, mask, bias, out, softmax_lse, softmax_scale, is_causal, softcap)
+    _cabi.fill_fwd(args.f, q, k, v, mask, bias, out, softmax_lse, softmax_scale, is_causal, softcap, _handoff_get("kept"))
+    fwd_ws = _handoff_get("fwd_ws")
+    if fwd_ws is not None and fwd_ws[1] == _cabi.get_compact_mode() and fwd_ws[2] == (None if bias is None else tuple(bias.shape)):
+        args.fwd_workspace, args.fwd_workspace_bytes = fwd_ws[0].data_ptr(), fwd_ws[0].numel()
     args.dout = dout.data_ptr()
     args.dq, args.dk, args.dv = dq_w.data_ptr(), dk_w.data_ptr(), dv_w.data_ptr()
     args.dbias = dbias_w.data_ptr() if dbias_w is not None else None
@@ -308,15 +343,28 @@ class FlashDMAttnFunc(torch.autograd.Function):
             q = torch.nn.functional.pad(q, [0, 8 - head_size_og % 8])
             k = torch.nn.functional.pad(k, [0, 8 - head_size_og % 8])
             v = torch.nn.functional.pad(v, [0, 8 - head_size_og % 8])
+        # (the hand-overs are eager-mode business: a traced graph calls the operators as they are)
+        eager = not torch.compiler.is_compiling()
+        kept = kept_keys_of(mask) if eager else None  # (before the mask may be replaced by a padded copy)
         mask = _pad_key_dim(mask, k.shape[1], 16)
         bias = _pad_key_dim(bias, k.shape[1], 8)
 
-        out_padded, softmax_lse, S_dmask = _wrapped_flash_sparse_attn_forward(
-            q, k, v, mask, bias, softmax_scale, is_causal=is_causal, softcap=softcap, return_softmax=return_softmax,
-        )
+        if eager:
+            with _handoff(kept=kept) as side:
+                out_padded, softmax_lse, S_dmask = _wrapped_flash_sparse_attn_forward(
+                    q, k, v, mask, bias, softmax_scale, is_causal=is_causal, softcap=softcap, return_softmax=return_softmax,
+                )
+        else:
+            side = {}
+            out_padded, softmax_lse, S_dmask = _wrapped_flash_sparse_attn_forward(
+                q, k, v, mask, bias, softmax_scale, is_causal=is_causal, softcap=softcap, return_softmax=return_softmax,
+            )
 
         if is_grad:
             ctx.save_for_backward(q, k, v, mask, bias, out_padded, softmax_lse)
+            if eager:
+                ctx.kept = kept
+                ctx.fwd_ws = side.get("fwd_ws_out")
             ctx.softmax_scale = softmax_scale
             ctx.is_causal = is_causal
             ctx.softcap = softcap
@@ -345,10 +393,17 @@ class FlashDMAttnFunc(torch.autograd.Function):
         if head_size_og % 8 != 0:
             dout_padded = torch.nn.functional.pad(dout, [0, 8 - head_size_og % 8])
 
-        _wrapped_flash_sparse_attn_backward(
-            dout_padded, q, k, v, mask, bias, out, softmax_lse, dq, dk, dv, dbias, ctx.softmax_scale, ctx.is_causal,
-            ctx.softcap, ctx.deterministic,
-        )
+        if torch.compiler.is_compiling():
+            _wrapped_flash_sparse_attn_backward(
+                dout_padded, q, k, v, mask, bias, out, softmax_lse, dq, dk, dv, dbias, ctx.softmax_scale, ctx.is_causal,
+                ctx.softcap, ctx.deterministic,
+            )
+        else:
+            with _handoff(kept=getattr(ctx, "kept", None), fwd_ws=getattr(ctx, "fwd_ws", None)):
+                _wrapped_flash_sparse_attn_backward(
+                    dout_padded, q, k, v, mask, bias, out, softmax_lse, dq, dk, dv, dbias, ctx.softmax_scale, ctx.is_causal,
+                    ctx.softcap, ctx.deterministic,
+                )
 
         # We could have padded the head dimension
         dq = dq[..., : dout.shape[-1]]

@@ -84,9 +84,33 @@ def _native_mask(attention_bias, attention_mask, window_size, min_dtype, block_s
     a.type = 0 if kind == "topk" else 1
     a.dtype = _cabi.dtype_code(bias)
     a.min_value = float(min_dtype)
+    # A mask that is broadcast over the queries drops whole key columns, and the attention kernels work on the list of
+    # the kept ones: the kernel writes that list too, and it travels with the mask tensor (see kept_keys_of).
+    kept = None
+    if shape[2] == 1:
+        ld = (shape[3] + 15) // 16 * 16
+        rows = shape[0] * shape[1]
+        kept = (torch.empty((rows, ld), dtype=torch.int32, device=bias.device),
+                torch.empty((rows, ld), dtype=torch.int32, device=bias.device),
+                torch.empty((rows,), dtype=torch.int32, device=bias.device), ld)
+        a.kept_idx, a.kept_cnt, a.kept_count, a.kept_ld = kept[0].data_ptr(), kept[1].data_ptr(), kept[2].data_ptr(), ld
     with _cabi.device_guard(bias.device):
         _cabi.check(_cabi.lib.fdma_create_mask(a, _cabi.current_stream(bias.device)))
+    if kept is not None:
+        out._fdma_kept = kept + (out._version, out.data_ptr(), tuple(out.shape))
     return out
+
+
+def kept_keys_of(mask: Optional[torch.Tensor]):
+    """(idx, cnt, count, ld) written by the device mask builder for THIS mask tensor, or None: when the tensor did not
+    come from it, is not broadcast over the queries, or has been written to since."""
+    kept = getattr(mask, "_fdma_kept", None)
+    if kept is None:
+        return None
+    idx, cnt, count, ld, version, ptr, shape = kept
+    if mask._version != version or mask.data_ptr() != ptr or tuple(mask.shape) != shape:
+        return None
+    return idx, cnt, count, ld
 
 
 def _masked_bias(attention_bias: torch.Tensor, attention_mask: Optional[torch.Tensor], min_dtype: float):

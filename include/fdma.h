@@ -44,7 +44,8 @@
 extern "C" {
 #endif
 
-#define FDMA_ABI_VERSION 3 /* 3: fdma_fwd_args.compact_mode (the struct grew), fdma_fwd_noalloc; 2: fdma_varlen_*, fdma_create_mask, fdma_dyn_bias_* */
+#define FDMA_ABI_VERSION 4 /* 4: fdma_kept_keys (fdma_fwd_args.kept, fdma_mask_args.kept_*), fdma_bwd_args.fwd_workspace (the structs grew);
+                              3: fdma_fwd_args.compact_mode, fdma_fwd_noalloc; 2: fdma_varlen_*, fdma_create_mask, fdma_dyn_bias_* */
 
 enum { FDMA_DTYPE_BF16 = 0, FDMA_DTYPE_FP16 = 1 };
 
@@ -80,6 +81,23 @@ enum {
     FDMA_COMPACT_ALWAYS = 2 /* compact whenever the mask form allows it */
 };
 
+/* The kept key columns of a query-broadcast keep-mask as lists, the form the compaction path works on.  Optional
+ * second output of fdma_create_mask and optional input of fdma_fwd / fdma_bwd: when a caller hands the lists over,
+ * the attention call does not scan the bool mask again (the mask itself must still be passed: it decides the path and
+ * is what the non-compacting kernels read).  One row per mask row, in (batch entry, mask head) order -- batch entry 0
+ * only when the mask is broadcast over the batch:
+ *   idx   : (rows, ld) int32, the original columns of the kept keys of a row in ascending order, count[row] of them
+ *   cnt   : (rows, ld) int32, cnt[row][j] = kept keys among the columns 0 .. j (inclusive), for j < seqlen_k
+ *   count : (rows) int32
+ *   ld    : row stride in elements, a multiple of 16 and >= seqlen_k
+ * The lists must describe exactly the mask that is passed; nothing checks it.  The reference has no counterpart (its
+ * kernels take the bool mask only); the precedent for index lists is its Triton backend,
+ * flash_sparse_attn/flash_dmattn_triton.py:50-211. */
+typedef struct fdma_kept_keys {
+    const int32_t *idx, *cnt, *count; /* all NULL = not given */
+    int32_t ld;
+} fdma_kept_keys;
+
 typedef struct fdma_fwd_args {
     const void *q, *k, *v;
     const void *mask; /* NULL = no mask */
@@ -98,6 +116,7 @@ typedef struct fdma_fwd_args {
     int32_t compact_mode;   /* FDMA_COMPACT_*; 0 = let the library decide */
     void *workspace;        /* split-KV partials (decode) or the compacted K / V copies; may be NULL if bytes == 0 */
     size_t workspace_bytes; /* >= fdma_fwd_workspace_bytes(args) */
+    fdma_kept_keys kept;    /* optional: the mask's kept columns as lists (see fdma_kept_keys) */
 } fdma_fwd_args;
 
 typedef struct fdma_bwd_args {
@@ -116,6 +135,12 @@ typedef struct fdma_bwd_args {
     int32_t deterministic;
     void *workspace;
     size_t workspace_bytes; /* >= fdma_bwd_workspace_bytes(args) */
+    /* Optional: the workspace the forward call of the SAME problem (same f.* arguments, compact_mode included) left
+     * behind, untouched since.  When the compaction path runs, the backward then reuses the forward's index lists and
+     * compacted K / V copies instead of scanning and gathering again, and fdma_bwd_workspace_bytes() shrinks by their
+     * size.  NULL = the backward makes its own. */
+    const void *fwd_workspace;
+    size_t fwd_workspace_bytes; /* >= fdma_fwd_workspace_bytes(&args->f) */
 } fdma_bwd_args;
 
 /* Forward attention.  Asynchronous on `hip_stream` (a hipStream_t).  Returns FDMA_OK or < 0. */
@@ -218,6 +243,10 @@ typedef struct fdma_mask_args {
     int32_t type;
     int32_t dtype;
     float min_value;
+    /* optional second output: the kept columns of every mask row as lists (fdma_kept_keys), one row per bias row in
+     * (batch, head, row) order; all NULL = not wanted */
+    int32_t *kept_idx, *kept_cnt, *kept_count;
+    int32_t kept_ld; /* multiple of 16, >= seqlen_k */
 } fdma_mask_args;
 int fdma_create_mask(const fdma_mask_args *args, void *hip_stream);
 int fdma_create_mask_validate(const fdma_mask_args *args);

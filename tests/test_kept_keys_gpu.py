@@ -1,0 +1,135 @@
+"""GPU tests (`-m gpu`) of the two hand-overs around the column-compaction path:
+
+  * the device keep-mask builder writes, next to the bool mask, the kept columns of every query-broadcast row as an
+    ordered list with prefix counts (`fdma_kept_keys`), and the attention calls take the lists instead of scanning
+    the mask again;
+  * the backward of an autograd node reuses the workspace of its forward call (index lists, compacted K / V copies)
+    instead of scanning and gathering a second time (`fdma_bwd_args.fwd_workspace`).
+Neither changes what is computed: every comparison here is bit for bit against the same call without the hand-over.
+"""
+import pytest
+import torch
+
+from _util import set_compact
+from flash_sparse_attn import flash_sparse_attn_func
+from flash_sparse_attn import flash_sparse_attn_interface as iface
+from flash_sparse_attn.utils import mask as M
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda"
+
+
+def _inputs(B, Lq, Lk, H, Hk, D, Hm, seed, dtype=torch.bfloat16):
+    g = torch.Generator().manual_seed(seed)
+    q = torch.randn(B, Lq, H, D, generator=g).to(dtype).to(DEV)
+    k = torch.randn(B, Lk, Hk, D, generator=g).to(dtype).to(DEV)
+    v = torch.randn(B, Lk, Hk, D, generator=g).to(dtype).to(DEV)
+    bias = torch.randn(B, Hm, 1, Lk, generator=g).to(dtype).to(DEV)
+    return q, k, v, bias
+
+
+@pytest.mark.parametrize("shape,window,block", [((2, 3, 1, 1000), 100, None), ((1, 8, 1, 8192), 2048, None),
+                                                ((2, 2, 1, 777), 300, 64), ((3, 1, 1, 50), 50, None),
+                                                ((1, 2, 1, 40000), 1000, None)])
+def test_mask_builder_writes_the_kept_columns_as_lists(shape, window, block):
+    bias = torch.randn(shape, generator=torch.Generator().manual_seed(shape[-1])).to(torch.bfloat16).to(DEV)
+    mask = M.topk_mask(bias, None, window, torch.finfo(torch.bfloat16).min, block_size=block)
+    kept = M.kept_keys_of(mask)
+    assert kept is not None
+    idx, cnt, count, ld = kept
+    torch.cuda.synchronize()
+    rows = mask.reshape(-1, shape[-1])
+    assert ld % 16 == 0 and ld >= shape[-1] and idx.shape == cnt.shape == (rows.shape[0], ld)
+    assert torch.equal(count.long(), rows.sum(-1))
+    assert torch.equal(cnt[:, :shape[-1]].long(), rows.long().cumsum(-1))
+    for r in range(rows.shape[0]):
+        n = int(count[r])
+        assert torch.equal(idx[r, :n].long(), rows[r].nonzero().flatten())
+    # a mask that has been written to since no longer carries its lists
+    mask[..., 0] = True
+    assert M.kept_keys_of(mask) is None
+    # a per-query mask has none to begin with
+    per_query = M.topk_mask(bias.expand(-1, -1, 4, -1), None, window, torch.finfo(torch.bfloat16).min)
+    assert M.kept_keys_of(per_query) is None
+
+
+def _run(q, k, v, mask, bias, causal=True):
+    qg, kg, vg, bg = [t.detach().clone().requires_grad_(True) for t in (q, k, v, bias)]
+    out, lse, _ = flash_sparse_attn_func(qg, kg, vg, mask, bg, None, causal, None, None, True)
+    out.backward(torch.ones_like(out))
+    torch.cuda.synchronize()
+    return [out.detach(), lse.detach(), qg.grad, kg.grad, vg.grad, bg.grad]
+
+
+CASES = [
+    # B, Lq, Lk, H, Hk, D, mask heads, window
+    (1, 512, 512, 8, 2, 128, 2, 128),
+    (2, 300, 777, 4, 2, 64, 2, 200),     # key length that is no multiple of 16: the mask is padded on the way in
+    (2, 256, 640, 4, 4, 128, 1, 96),     # one mask head for all kv heads
+    (1, 1024, 1024, 8, 2, 128, 2, 1024), # everything kept
+    (1, 384, 384, 2, 1, 32, 1, 1),       # a single kept key per row
+]
+
+
+@pytest.mark.parametrize("case", range(len(CASES)))
+@pytest.mark.parametrize("mode", ["2", "auto"])
+def test_attention_with_handed_over_lists_is_bit_identical(case, mode):
+    B, Lq, Lk, H, Hk, D, Hm, W = CASES[case]
+    q, k, v, bias = _inputs(B, Lq, Lk, H, Hk, D, Hm, seed=case)
+    set_compact(mode)
+    try:
+        mask = M.topk_mask(bias, None, W, torch.finfo(bias.dtype).min)
+        assert M.kept_keys_of(mask) is not None
+        with_lists = _run(q, k, v, mask, bias)
+        plain = mask.clone()  # same values, no lists: the attention call scans it
+        assert M.kept_keys_of(plain) is None
+        scanned = _run(q, k, v, plain, bias)
+    finally:
+        set_compact("auto")
+    for a, b in zip(with_lists, scanned):
+        assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("case", range(len(CASES)))
+def test_backward_on_the_forward_workspace_is_bit_identical(case):
+    B, Lq, Lk, H, Hk, D, Hm, W = CASES[case]
+    q, k, v, bias = _inputs(B, Lq, Lk, H, Hk, D, Hm, seed=10 + case)
+    mask = M.topk_mask(bias, None, W, torch.finfo(bias.dtype).min).clone()
+    set_compact("2")
+    try:
+        reused = _run(q, k, v, mask, bias)
+        # the same operator calls by hand, outside an autograd node: the backward then has no forward workspace
+        mpad, bpad = iface._pad_key_dim(mask, Lk, 16), iface._pad_key_dim(bias, Lk, 8)
+        out, lse, _ = iface._wrapped_flash_sparse_attn_forward(q, k, v, mpad, bpad, D ** -0.5, True, 0.0, False)
+        dq, dk, dv, dbp = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), torch.empty_like(bpad)
+        iface._wrapped_flash_sparse_attn_backward(torch.ones_like(out), q, k, v, mpad, bpad, out, lse, dq, dk, dv, dbp,
+                                                  D ** -0.5, True, 0.0, False)
+        torch.cuda.synchronize()
+    finally:
+        set_compact("auto")
+    for a, b in zip(reused, [out, lse, dq, dk, dv, dbp[..., :Lk]]):
+        assert torch.equal(a, b)
+
+
+def test_deterministic_backward_with_shared_bias_does_not_take_the_forward_workspace():
+    """deterministic=True expands a batch-broadcast bias for the backward: another problem than the forward's, whose
+    workspace must then be left alone (results against the plain operator on the expanded bias)."""
+    B, Lq, Lk, H, Hk, D = 2, 256, 512, 4, 2, 64
+    q, k, v, _ = _inputs(B, Lq, Lk, H, Hk, D, Hk, seed=5)
+    bias = torch.randn(1, Hk, 1, Lk, generator=torch.Generator().manual_seed(6)).to(torch.bfloat16).to(DEV)
+    mask = M.topk_mask(bias, None, 128, torch.finfo(bias.dtype).min)
+    set_compact("2")
+    try:
+        qg, kg, vg, bg = [t.detach().clone().requires_grad_(True) for t in (q, k, v, bias)]
+        out = flash_sparse_attn_func(qg, kg, vg, mask, bg, None, True, None, True)
+        out.backward(torch.ones_like(out))
+        q2, k2, v2 = [t.detach().clone().requires_grad_(True) for t in (q, k, v)]
+        b2 = bias.expand(B, -1, -1, -1).contiguous().requires_grad_(True)
+        out2 = flash_sparse_attn_func(q2, k2, v2, mask.expand(B, -1, -1, -1).contiguous(), b2, None, True, None, True)
+        out2.backward(torch.ones_like(out2))
+        torch.cuda.synchronize()
+    finally:
+        set_compact("auto")
+    assert torch.equal(out, out2) and torch.equal(qg.grad, q2.grad) and torch.equal(kg.grad, k2.grad)
+    ref_db = b2.grad.float().sum(0, keepdim=True)
+    assert (bg.grad.float() - ref_db).abs().max().item() <= 2e-2 * ref_db.abs().max().item()
