@@ -87,7 +87,11 @@ int validate_common(const fdma_fwd_args *a, bool backward) {
     if (a->q_strides[1] >= kMaxRowStride || a->k_strides[1] >= kMaxRowStride || a->v_strides[1] >= kMaxRowStride)
         return fail(FDMA_ERR_UNSUPPORTED, "q, k, v row strides of 2^24 elements or more are not supported");
     if (a->softcap != 0.f) return fail(FDMA_ERR_UNSUPPORTED, "softcap is not supported by this build");
-    if (a->head_dim > 128) return fail(FDMA_ERR_UNSUPPORTED, "head dimensions above 128 are not built yet (got %d)", a->head_dim);
+    // head dims 129 .. 256 run in the column-mask kernels only: mask and bias absent or broadcast over the queries
+    if (a->head_dim > 128 && a->seqlen_q > 1 &&
+        ((a->mask && a->mask_strides[2] != 0) || (a->bias && a->bias_strides[2] != 0)))
+        return fail(FDMA_ERR_UNSUPPORTED, "head dimensions above 128 are built for masks and biases that are broadcast over the "
+                                          "queries (row stride 0) or absent; got head_dim %d with a per-query mask or bias", a->head_dim);
     if (!std::isfinite(a->softmax_scale)) return fail(FDMA_ERR_INVALID, "softmax_scale must be finite");
     if (a->compact_mode < FDMA_COMPACT_AUTO || a->compact_mode > FDMA_COMPACT_ALWAYS)
         return fail(FDMA_ERR_INVALID, "compact_mode must be FDMA_COMPACT_AUTO, _NEVER or _ALWAYS (got %d)", a->compact_mode);
@@ -105,8 +109,8 @@ void fill_fwd_params(const fdma_fwd_args *a, fdma::FwdParams &p) {
     p.k_b = a->k_strides[0]; p.k_r = a->k_strides[1]; p.k_h = a->k_strides[2];
     p.v_b = a->v_strides[0]; p.v_r = a->v_strides[1]; p.v_h = a->v_strides[2];
     p.o_b = a->o_strides[0]; p.o_r = a->o_strides[1]; p.o_h = a->o_strides[2];
-    if (a->mask) { p.m_b = a->mask_strides[0]; p.m_h = a->mask_strides[1]; p.m_r = a->mask_strides[2]; }
-    if (a->bias) { p.bi_b = a->bias_strides[0]; p.bi_h = a->bias_strides[1]; p.bi_r = a->bias_strides[2]; }
+    if (a->mask) { p.m_b = a->mask_strides[0]; p.m_h = a->mask_strides[1]; p.m_r = a->seqlen_q == 1 ? 0 : a->mask_strides[2]; }
+    if (a->bias) { p.bi_b = a->bias_strides[0]; p.bi_h = a->bias_strides[1]; p.bi_r = a->seqlen_q == 1 ? 0 : a->bias_strides[2]; }
     p.B = a->batch; p.Lq = a->seqlen_q; p.Lk = a->seqlen_k;
     p.H = a->num_heads; p.Hk = a->num_heads_k;
     p.Hm = a->mask ? a->num_heads_mask : 1;
@@ -157,7 +161,6 @@ int validate_varlen(const fdma_varlen_fwd_args *a, bool backward) {
     if (a->q_strides[0] >= kMaxRowStride || a->k_strides[0] >= kMaxRowStride || a->v_strides[0] >= kMaxRowStride)
         return fail(FDMA_ERR_UNSUPPORTED, "q, k, v row strides of 2^24 elements or more are not supported");
     if (a->softcap != 0.f) return fail(FDMA_ERR_UNSUPPORTED, "softcap is not supported by this build");
-    if (a->head_dim > 128) return fail(FDMA_ERR_UNSUPPORTED, "head dimensions above 128 are not built yet (got %d)", a->head_dim);
     if (!std::isfinite(a->softmax_scale)) return fail(FDMA_ERR_INVALID, "softmax_scale must be finite");
     return FDMA_OK;
 }
@@ -249,7 +252,7 @@ int fdma_fwd_validate(const fdma_fwd_args *a) {
 
 size_t fdma_fwd_workspace_bytes(const fdma_fwd_args *a) {
     if (!a) return 0;
-    if (!fdma::use_decode_path(a->seqlen_q, a->num_heads, a->num_heads_k)) {
+    if (!fdma::use_decode_path(a->seqlen_q, a->num_heads, a->num_heads_k) || a->head_dim > 128) {  // (the split-KV kernel is built up to head dim 128)
         fdma::FwdParams p;
         fill_fwd_params(a, p);
         return fdma::use_compact(p) ? fdma::compact_bytes(p, false) : 0;
@@ -270,7 +273,7 @@ int fdma_fwd(const fdma_fwd_args *a, void *hip_stream) {
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     hipError_t e;
     if (a->seqlen_q == 0) return FDMA_OK;
-    if (fdma::use_decode_path(a->seqlen_q, a->num_heads, a->num_heads_k) && a->seqlen_k > 0) {
+    if (fdma::use_decode_path(a->seqlen_q, a->num_heads, a->num_heads_k) && a->head_dim <= 128 && a->seqlen_k > 0) {
         p.splits = fdma::decode_num_splits(a->batch, a->num_heads_k, a->seqlen_k);
         if (p.splits > 1) {
             const size_t need = fdma_fwd_workspace_bytes(a);

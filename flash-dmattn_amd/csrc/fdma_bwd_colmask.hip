@@ -72,7 +72,7 @@ template <int D> struct KvcSmem {
 // CMP: the key axis is the compacted list of kept columns (fdma_compact.hip); a lane still owns one key,
 // reads it from the dense copies, and writes its gradients to the key's original row / column.
 template <typename T, int D, bool CAUSAL, bool CMP>
-__global__ void __launch_bounds__(NTHREADS, 2) bwd_dkdv_colmask_kernel(const BwdParams p) {
+__global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dkdv_colmask_kernel(const BwdParams p) {
     using E = Elem<T>;
     using SM = KvcSmem<D>;
     using TL = LdsTile<D>;
@@ -782,7 +782,7 @@ template <int D, int BN> struct DqcSmem {
 };
 
 template <typename T, int D, int BN, bool CAUSAL, bool CMP>
-__global__ void __launch_bounds__(NTHREADS, 2) bwd_dq_colmask_kernel(const BwdParams p) {
+__global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_kernel(const BwdParams p) {
     using E = Elem<T>;
     using SM = DqcSmem<D, BN>;
     using TL = LdsTile<D>;
@@ -1155,25 +1155,32 @@ bool bwd_colmask_applicable(const BwdParams &p) {
 }
 
 hipError_t launch_bwd_dkdv_colmask(const BwdParams &p, int dtype, hipStream_t stream) {
-    const bool d64 = p.f.d <= 64, c = p.f.causal != 0;
+    // head dims up to 64 / 128 / 256 (a head dim in between runs in the next larger instantiation)
+    const int dc = p.f.d <= 64 ? 0 : (p.f.d <= 128 ? 1 : 2);
+    const bool c = p.f.causal != 0;
     if (dtype == 0) {
-        if (d64) return c ? launch_dkdv<bf16_tag, 64, true>(p, stream) : launch_dkdv<bf16_tag, 64, false>(p, stream);
-        return c ? launch_dkdv<bf16_tag, 128, true>(p, stream) : launch_dkdv<bf16_tag, 128, false>(p, stream);
+        if (dc == 0) return c ? launch_dkdv<bf16_tag, 64, true>(p, stream) : launch_dkdv<bf16_tag, 64, false>(p, stream);
+        if (dc == 1) return c ? launch_dkdv<bf16_tag, 128, true>(p, stream) : launch_dkdv<bf16_tag, 128, false>(p, stream);
+        return c ? launch_dkdv<bf16_tag, 256, true>(p, stream) : launch_dkdv<bf16_tag, 256, false>(p, stream);
     }
-    if (d64) return c ? launch_dkdv<fp16_tag, 64, true>(p, stream) : launch_dkdv<fp16_tag, 64, false>(p, stream);
-    return c ? launch_dkdv<fp16_tag, 128, true>(p, stream) : launch_dkdv<fp16_tag, 128, false>(p, stream);
+    if (dc == 0) return c ? launch_dkdv<fp16_tag, 64, true>(p, stream) : launch_dkdv<fp16_tag, 64, false>(p, stream);
+    if (dc == 1) return c ? launch_dkdv<fp16_tag, 128, true>(p, stream) : launch_dkdv<fp16_tag, 128, false>(p, stream);
+    return c ? launch_dkdv<fp16_tag, 256, true>(p, stream) : launch_dkdv<fp16_tag, 256, false>(p, stream);
 }
 
 }  // namespace fdma
 
 namespace fdma {
 hipError_t launch_bwd_dq_colmask(const BwdParams &p, int dtype, hipStream_t stream) {
-    const bool d64 = p.f.d <= 64, c = p.f.causal != 0;
+    const int dc = p.f.d <= 64 ? 0 : (p.f.d <= 128 ? 1 : 2);
+    const bool c = p.f.causal != 0;
     if (dtype == 0) {
-        if (d64) return c ? launch_dq<bf16_tag, 64, true>(p, stream) : launch_dq<bf16_tag, 64, false>(p, stream);
-        return c ? launch_dq<bf16_tag, 128, true>(p, stream) : launch_dq<bf16_tag, 128, false>(p, stream);
+        if (dc == 0) return c ? launch_dq<bf16_tag, 64, true>(p, stream) : launch_dq<bf16_tag, 64, false>(p, stream);
+        if (dc == 1) return c ? launch_dq<bf16_tag, 128, true>(p, stream) : launch_dq<bf16_tag, 128, false>(p, stream);
+        return c ? launch_dq<bf16_tag, 256, true>(p, stream) : launch_dq<bf16_tag, 256, false>(p, stream);
     }
-    if (d64) return c ? launch_dq<fp16_tag, 64, true>(p, stream) : launch_dq<fp16_tag, 64, false>(p, stream);
-    return c ? launch_dq<fp16_tag, 128, true>(p, stream) : launch_dq<fp16_tag, 128, false>(p, stream);
+    if (dc == 0) return c ? launch_dq<fp16_tag, 64, true>(p, stream) : launch_dq<fp16_tag, 64, false>(p, stream);
+    if (dc == 1) return c ? launch_dq<fp16_tag, 128, true>(p, stream) : launch_dq<fp16_tag, 128, false>(p, stream);
+    return c ? launch_dq<fp16_tag, 256, true>(p, stream) : launch_dq<fp16_tag, 256, false>(p, stream);
 }
 }  // namespace fdma

@@ -50,7 +50,7 @@ Layout layout_of(const FwdParams &p, bool backward) {
     if (backward) {
         int grid, slots;
         dkdv_split_bounds((int)pairs, (p.Lk + 127) / 128, p.H / p.Hk, grid, slots);
-        const int dpad = p.d <= 64 ? 64 : 128;
+        const int dpad = p.d <= 64 ? 64 : (p.d <= 128 ? 128 : 256);
         // header, prefix of the units over the pairs and, per XCD, the list of the parts that exist (two ints each;
         // the kernel's grid bounds their number)
         l.off_plan = o;    o += align256((DKDV_PLAN_HDR + pairs + 1 + 8 + 2 * (size_t)grid) * 4);

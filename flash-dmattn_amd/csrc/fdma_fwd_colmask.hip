@@ -67,7 +67,7 @@ template <int D, int BN> struct CmSmem {
 // `count` columns, all kept; the fused bias vector comes pre-gathered, and the causal limit of a query row
 // is the number of kept columns at or below its diagonal instead of the column index itself.
 template <typename T, int D, int BN, bool CAUSAL, int NW, bool CMP>
-__global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) fwd_colmask_kernel(const FwdParams p) {
+__global__ void __launch_bounds__(64 * NW, (NW == 4 && D <= 128) ? 2 : 1) fwd_colmask_kernel(const FwdParams p) {
     constexpr int NTHREADS = 64 * NW;
     constexpr int STHREADS = 256;             // threads staging one operand
     constexpr bool SPLIT = NW == 8;           // 8 waves: the first four stage V, the last four K and the side rows
@@ -83,8 +83,10 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) fwd_colmask_kernel(c
     constexpr int K_RPP = STHREADS / CH;      // K rows staged per pass
     constexpr int K_IT = BN / K_RPP;          // passes (registers) per K tile
     constexpr int V_ITEMS = KQ * CH;          // (key quad, d chunk) items of a V tile
-    constexpr int NL = SPLIT ? 4 : K_IT + 4;  // 16-byte loads per thread and tile
+    constexpr int V_IT = (V_ITEMS + STHREADS - 1) / STHREADS;  // items per staging thread (two at head dims above 128)
+    constexpr int NL = SPLIT ? 4 : K_IT + 4 * V_IT;  // 16-byte loads per thread and tile
     constexpr int VB = SPLIT ? 0 : K_IT;      // first V staging register
+    static_assert(!SPLIT || V_IT == 1, "the role split assumes one V item per thread");
     static_assert(!SPLIT || K_IT == 4, "the role split assumes four loads per thread for either operand");
 
     extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -248,14 +250,16 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) fwd_colmask_kernel(c
     const int kc = kt % CH, kr0 = kt / CH;
     const int vkg = kt % KQ, vc = (kt / KQ) % CH;  // V: key quad and d chunk of this thread
     const uint32_t k_r2 = (uint32_t)(p.k_r * 2), v_r2 = (uint32_t)(p.v_r * 2);  // bytes per row
-    const uint32_t kcolb = (kc * 8 < p.d ? kc * 16 : 0), vcolb = (vc * 8 < p.d ? vc * 16 : 0);
+    const uint32_t kcolb = (kc * 8 < p.d ? kc * 16 : 0);
+    auto vchunk = [&](int j) -> int { return vc + j * (STHREADS / KQ); };  // d chunk of this thread's j-th V item
     const int j_last = Lk > 0 ? (Lk - 1) / BN : 0, last_row = Lk > 0 ? (Lk - 1) % BN : 0;
     uint32_t soff[NL], soff_l[NL];  // byte offsets of this thread's loads inside a full / the last tile
 #pragma unroll
     for (int n = 0; n < NL; n++) {
         const bool is_v = SPLIT ? role_v : n >= K_IT;
-        const int item = SPLIT ? n : (n >= K_IT ? n - K_IT : n);
-        const int row = is_v ? 4 * vkg + item : kr0 + item * K_RPP;
+        const int item = SPLIT ? n : (n >= K_IT ? n - K_IT : n);  // V: four loads (keys of the quad) per item
+        const int row = is_v ? 4 * vkg + (item & 3) : kr0 + item * K_RPP;
+        const uint32_t vcolb = (vchunk(item >> 2) * 8 < p.d ? vchunk(item >> 2) * 16 : 0);
         const uint32_t r2 = is_v ? v_r2 : k_r2, colb = is_v ? vcolb : kcolb;
         soff[n] = (uint32_t)row * r2 + colb;
         soff_l[n] = (uint32_t)(row < last_row ? row : last_row) * r2 + colb;
@@ -343,13 +347,13 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) fwd_colmask_kernel(c
         if (role_v && kt < V_ITEMS) {  // transpose 4 keys x 8 d in registers, write V^T[d][key quad]
             char *sVt = smem + SM::OFF_VT + vbuf * SM::VT_BYTES;
 #pragma unroll
-            for (int dd = 0; dd < 8; dd++) {
-                const int w = dd >> 1;
+            for (int dj = 0; dj < 8 * V_IT; dj++) {
+                const int j = dj >> 3, dd = dj & 7, w = dd >> 1;
                 const uint32_t sel = (dd & 1) ? 0x07060302u : 0x05040100u;
                 u32x2_t out;
-                out[0] = __builtin_amdgcn_perm(sreg[VB + 1][w], sreg[VB + 0][w], sel);
-                out[1] = __builtin_amdgcn_perm(sreg[VB + 3][w], sreg[VB + 2][w], sel);
-                *(u32x2_t *)(sVt + ((vc * 8 + dd) * SM::SVT + 4 * vkg) * 2) = out;
+                out[0] = __builtin_amdgcn_perm(sreg[VB + 4 * j + 1][w], sreg[VB + 4 * j + 0][w], sel);
+                out[1] = __builtin_amdgcn_perm(sreg[VB + 4 * j + 3][w], sreg[VB + 4 * j + 2][w], sel);
+                *(u32x2_t *)(sVt + ((vchunk(j) * 8 + dd) * SM::SVT + 4 * vkg) * 2) = out;
             }
         }
     };
@@ -514,14 +518,14 @@ __global__ void __launch_bounds__(64 * NW, NW == 4 ? 2 : 1) fwd_colmask_kernel(c
             // chunk of K
             if (DO_V) {
 #pragma unroll
-                for (int dd = 0; dd < 8; dd++)
-                    if (f == 1 + dd * ((NF - 1) / 8)) {
-                        const int w = dd >> 1;
+                for (int dj = 0; dj < 8 * V_IT; dj++)
+                    if (f == 1 + dj * ((NF - 1) / (8 * V_IT))) {
+                        const int j = dj >> 3, dd = dj & 7, w = dd >> 1;
                         const uint32_t sel = (dd & 1) ? 0x07060302u : 0x05040100u;
                         u32x2_t out;
-                        out[0] = __builtin_amdgcn_perm(sreg[VB + 1][w], sreg[VB + 0][w], sel);
-                        out[1] = __builtin_amdgcn_perm(sreg[VB + 3][w], sreg[VB + 2][w], sel);
-                        *(u32x2_t *)(sVt_w + ((vc * 8 + dd) * SM::SVT + 4 * vkg) * 2) = out;
+                        out[0] = __builtin_amdgcn_perm(sreg[VB + 4 * j + 1][w], sreg[VB + 4 * j + 0][w], sel);
+                        out[1] = __builtin_amdgcn_perm(sreg[VB + 4 * j + 3][w], sreg[VB + 4 * j + 2][w], sel);
+                        *(u32x2_t *)(sVt_w + ((vchunk(j) * 8 + dd) * SM::SVT + 4 * vkg) * 2) = out;
                     }
             }
             if (DO_K) {
@@ -779,9 +783,9 @@ bool fwd_colmask_applicable(const FwdParams &p) {
 }
 
 hipError_t launch_fwd_colmask(const FwdParams &p, int dtype, hipStream_t stream) {
-    const bool d64 = p.d <= 64;
-    if (dtype == 0) return d64 ? launch_d<bf16_tag, 64>(p, stream) : launch_d<bf16_tag, 128>(p, stream);
-    return d64 ? launch_d<fp16_tag, 64>(p, stream) : launch_d<fp16_tag, 128>(p, stream);
+    // head dims up to 64 / 128 / 256 (a head dim in between runs in the next larger instantiation)
+    if (dtype == 0) return p.d <= 64 ? launch_d<bf16_tag, 64>(p, stream) : p.d <= 128 ? launch_d<bf16_tag, 128>(p, stream) : launch_d<bf16_tag, 256>(p, stream);
+    return p.d <= 64 ? launch_d<fp16_tag, 64>(p, stream) : p.d <= 128 ? launch_d<fp16_tag, 128>(p, stream) : launch_d<fp16_tag, 256>(p, stream);
 }
 
 }  // namespace fdma

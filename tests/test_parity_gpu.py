@@ -88,6 +88,13 @@ SMALL_CASES = {
     "compact_batch_broadcast_bias": (2, 256, 256, 4, 2, 64, (1, 2, 1, 256), (2, 2, 1, 256), 64, True),
     "compact_head_dim_96_dense_mask": (1, 200, 200, 2, 1, 96, (1, 1, 1, 200), (1, 1, 1, 200), 200, True),
     "colmask_per_query_head_gqa": (1, 256, 256, 4, 2, 64, (1, 4, 1, 256), (1, 4, 1, 256), 64, True),
+    # head dims above 128 (the column-mask kernels at 256; 192 runs in the same instantiation)
+    "head_dim_256_gqa_topk": (1, 300, 300, 4, 2, 256, (1, 2, 1, 300), (1, 2, 1, 300), 100, True),
+    "head_dim_192_gqa_topk": (2, 200, 264, 4, 2, 192, (2, 4, 1, 264), (2, 1, 1, 264), 64, True),
+    "head_dim_256_plain_noncausal": (1, 256, 320, 2, 2, 256, None, None, None, False),
+    "head_dim_192_lq_lt_lk_mask_only": (1, 100, 333, 2, 1, 192, None, (1, 1, 1, 333), 120, True),
+    "head_dim_256_lq_gt_lk_empty_rows": (1, 333, 100, 2, 2, 256, (1, 2, 1, 100), (1, 2, 1, 100), 50, True),
+    "head_dim_136_bias_only": (1, 130, 130, 2, 2, 136, (1, 1, 1, 130), None, None, True),
 }
 
 
@@ -435,6 +442,9 @@ DECODE_CASES = {
     # 40 query heads on one kv head: two workgroups per split (32 + 8 columns)
     "mqa40_two_column_chunks": (1, 2000, 40, 1, 64, 1, 1, 300),
     "mqa40_per_head_mask_and_bias": (1, 1200, 40, 1, 128, 40, 40, 200),
+    # head dims above 128: a single query row goes through the column-mask forward (no split-KV kernel there)
+    "gqa4_head_dim_256": (2, 1000, 8, 2, 256, 2, 2, 128),
+    "mha_head_dim_192_no_mask": (1, 300, 2, 2, 192, None, 1, None),
 }
 
 

@@ -94,6 +94,8 @@ VARLEN_CASES = {
     "lq_gt_lk_rows_without_keys_fp16": ([200, 64, 130], [50, 64, 1], 2, 2, 128, torch.float16),
     "single_sequence_head_dim_96": ([333], [333], 2, 1, 96, torch.bfloat16),
     "empty_entries": ([64, 0, 130, 0], [64, 0, 200, 0], 2, 2, 64, torch.bfloat16),
+    "ragged_gqa_head_dim_256": ([100, 1, 257, 64], [100, 1, 257, 64], 4, 2, 256, torch.bfloat16),
+    "cross_lengths_head_dim_192_fp16": ([37, 200, 5], [300, 64, 77], 2, 1, 192, torch.float16),
 }
 
 
