@@ -420,6 +420,30 @@ class FlashDMAttnFunc(torch.autograd.Function):
         return dq, dk, dv, None, dbias, None, None, None, None, None, None
 
 
+def _column_causal_form(mask, bias, query, key, is_causal):
+    """A keep-mask that arrives with one row per query but is really a column mask under the causal rule -- every row
+    equals the last row cut off at the row's causal limit -- can run through the column-mask kernels (tile skipping,
+    column compaction) instead of the kernels that stream a mask tile per score tile.  Finding that out takes a pass
+    over the whole mask and a host synchronisation, so it is done only under the compaction policy "always"
+    (`_cabi.set_compact_mode(COMPACT_ALWAYS)` / `FDMA_COMPACT=2`).  Returns (mask, is_causal) to call the operator with:
+    the last row and True when the mask has that form, the arguments unchanged otherwise."""
+    if (mask is None or _cabi.get_compact_mode() != _cabi.COMPACT_ALWAYS or torch.compiler.is_compiling()
+            or type(mask) is not torch.Tensor or mask.dim() != 4 or mask.dtype != torch.bool):
+        return mask, is_causal
+    Lq, Lk = query.size(1), key.size(1)
+    if (mask.size(2) != Lq or Lq < 2 or mask.size(3) < Lk or mask.size(1) not in (1, key.size(2))
+            or (bias is not None and bias.size(2) != 1)):
+        return mask, is_causal
+    m = mask[..., :Lk]
+    rows = torch.arange(Lq, device=mask.device)[:, None]
+    cols = torch.arange(Lk, device=mask.device)[None, :]
+    causal = cols <= rows + (Lk - Lq)  # bottom-right aligned
+    col = m[:, :, -1:, :]              # the last row may see every key
+    if not torch.equal(m & causal if is_causal else m, col & causal):
+        return mask, is_causal
+    return col.contiguous(), True
+
+
 def flash_sparse_attn_func(
     query: torch.Tensor, key: torch.Tensor, value: torch.Tensor, attn_mask: Optional[torch.Tensor] = None, attn_bias:
     Optional[torch.Tensor] = None, softmax_scale: Optional[float] = None, is_causal: Optional[bool] = None, softcap:
@@ -464,6 +488,7 @@ def flash_sparse_attn_func(
             (+inf for rows with no visible key).
     """
     grad_enabled = torch.is_grad_enabled()
+    attn_mask, is_causal = _column_causal_form(attn_mask, attn_bias, query, key, is_causal)
     args = (query, key, value, attn_mask, attn_bias, softmax_scale, is_causal, softcap, deterministic, return_attn_probs,
             grad_enabled)
     if _nothing_to_differentiate(grad_enabled, query, key, value, attn_bias):

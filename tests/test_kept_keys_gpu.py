@@ -133,3 +133,44 @@ def test_deterministic_backward_with_shared_bias_does_not_take_the_forward_works
     assert torch.equal(out, out2) and torch.equal(qg.grad, q2.grad) and torch.equal(kg.grad, k2.grad)
     ref_db = b2.grad.float().sum(0, keepdim=True)
     assert (bg.grad.float() - ref_db).abs().max().item() <= 2e-2 * ref_db.abs().max().item()
+
+
+def test_per_query_mask_of_column_causal_form_takes_the_column_mask_kernels():
+    """Under the compaction policy "always" a [B, Hk, Lq, Lk] mask whose rows are one column mask cut off at the causal
+    limit is recognised and runs like that column mask with is_causal=True (bit for bit); a mask that differs from the
+    form in a single element is not, and goes through the per-query kernels.  Both against the C oracle."""
+    from _util import assert_grad_close, assert_out_close, make_inputs
+    from oracle import c_oracle
+
+    B, Lq, Lk, H, Hk, D, W = 2, 200, 264, 4, 2, 64, 80
+    q, k, v, colmask, bias = make_inputs(B, Lq, Lk, H, Hk, D, (B, Hk, 1, Lk), (B, Hk, 1, Lk), W, seed=3)
+    causal = torch.arange(Lk)[None, :] <= torch.arange(Lq)[:, None] + (Lk - Lq)
+    full = colmask & causal                       # (B, Hk, Lq, Lk)
+    broken = full.clone()
+    broken[1, 0, 50, 3] = ~broken[1, 0, 50, 3]   # one element off the form
+    dout = torch.randn(B, Lq, H, D, generator=torch.Generator().manual_seed(4)).to(torch.bfloat16)
+
+    def run(mask, is_causal):
+        qg, kg, vg, bg = [t.to(DEV).requires_grad_(True) for t in (q, k, v, bias)]
+        out, lse, _ = flash_sparse_attn_func(qg, kg, vg, mask.to(DEV), bg, None, is_causal, None, None, True)
+        out.backward(dout.to(DEV))
+        torch.cuda.synchronize()
+        return [out.detach(), lse.detach(), qg.grad, kg.grad, vg.grad, bg.grad]
+
+    set_compact("2")
+    try:
+        as_columns = run(colmask, True)
+        recognised = run(full, False)            # (the mask carries the causal rule itself)
+        recognised_c = run(full, True)
+        fallback = run(broken, False)
+    finally:
+        set_compact("auto")
+    for a, b, c in zip(as_columns, recognised, recognised_c):
+        assert torch.equal(a, b) and torch.equal(a, c)
+    for got, mask in ((recognised, full), (fallback, broken)):
+        ro, rl = c_oracle.forward(q, k, v, mask, bias, None, False)
+        rdq, rdk, rdv, rdb = c_oracle.backward(q, k, v, dout, mask, bias, None, False)
+        assert_out_close(got[0].cpu(), ro)
+        for g, r, name in ((got[2], rdq, "dq"), (got[3], rdk, "dk"), (got[4], rdv, "dv"), (got[5], rdb, "dbias")):
+            assert_grad_close(g.cpu(), r, name)
+    assert not torch.equal(recognised[0], fallback[0])
