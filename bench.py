@@ -273,6 +273,28 @@ def run_config(name, steps, warmup, device, compact=True, backward=True, zero_in
     return res
 
 
+def run_mfma_probe():
+    """What rate of bf16 MFMA 32x32x16 the device sustains on its own (flash-dmattn_amd/csrc/fdma_probe.hip, built
+    next to the library): 256 workgroups of 8 waves issuing nothing but MFMAs from registers, the same with one LDS
+    fragment read per MFMA, and with the forward kernel's vector work per MFMA on top -- on constant and on random
+    operands.  The published peak assumes 2.4 GHz; real operands make the device run slower, so `roofline.frac`
+    (always against the published peak) is to be read next to these.  Returns None when the probe is not built."""
+    import ctypes
+
+    path = os.path.join(ROOT, "flash-dmattn_amd", "lib", "libfdma_probe.so")
+    if not os.path.exists(path):
+        return None
+    lib = ctypes.CDLL(path)
+    lib.fdma_probe_mfma_tflops.restype = ctypes.c_double
+    lib.fdma_probe_mfma_tflops.argtypes = [ctypes.c_int, ctypes.c_int]
+    names = ("registers_only", "lds_fragment_per_mfma", "lds_fragment_and_softmax_valu_per_mfma")
+    out = {"unit": "TFLOP/s", "note": "bf16 MFMA 32x32x16 alone, 256 workgroups x 8 waves; the softmax mix is 2 exp2 + 1 "
+                                      "conversion + 2 additions per MFMA"}
+    for mode, name in enumerate(names):
+        out[name] = {"constant_operands": lib.fdma_probe_mfma_tflops(mode, 0), "random_operands": lib.fdma_probe_mfma_tflops(mode, 1)}
+    return out
+
+
 def run_mask_builder(steps, warmup, device):
     """Keep-mask construction in front of the operator (not part of `value`): flash_sparse_attn.utils.mask.topk_mask
     through the device kernel, next to the reference's tensor program (masked_fill / topk / zeros / scatter,
@@ -433,6 +455,7 @@ def main():
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--all", action="store_true", help="also time configurations 1, 3, 4, 5")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-probe", action="store_true", help="skip the matrix-pipe probe (MFMA rate on constant / random operands)")
     ap.add_argument("--no-compact", action="store_true",
                     help="switch the column-compaction path off (compact_mode = never): time the tile-skipping kernels")
     ap.add_argument("--calib-copy", action="store_true",
@@ -512,6 +535,10 @@ def main():
                         zero_inputs=True)
         out["tile_skip_path"]["zero_operands"] = {"ms_fwd": tz["ms_fwd"], "tflops_fwd": tz["tflops_fwd"],
                                                   "frac_of_peak": tz["tflops_fwd"] / PEAK_BF16_TFLOPS}
+    if not args.no_probe:
+        probe = run_mfma_probe()
+        if probe is not None:
+            out["mfma_probe"] = probe
     if args.traffic_bytes is not None:
         out["roofline"]["traffic"] = args.traffic_bytes
     if args.calib_copy:
