@@ -87,11 +87,6 @@ int validate_common(const fdma_fwd_args *a, bool backward) {
     if (a->q_strides[1] >= kMaxRowStride || a->k_strides[1] >= kMaxRowStride || a->v_strides[1] >= kMaxRowStride)
         return fail(FDMA_ERR_UNSUPPORTED, "q, k, v row strides of 2^24 elements or more are not supported");
     if (a->softcap != 0.f) return fail(FDMA_ERR_UNSUPPORTED, "softcap is not supported by this build");
-    // head dims 129 .. 256 run in the column-mask kernels only: mask and bias absent or broadcast over the queries
-    if (a->head_dim > 128 && a->seqlen_q > 1 &&
-        ((a->mask && a->mask_strides[2] != 0) || (a->bias && a->bias_strides[2] != 0)))
-        return fail(FDMA_ERR_UNSUPPORTED, "head dimensions above 128 are built for masks and biases that are broadcast over the "
-                                          "queries (row stride 0) or absent; got head_dim %d with a per-query mask or bias", a->head_dim);
     if (!std::isfinite(a->softmax_scale)) return fail(FDMA_ERR_INVALID, "softmax_scale must be finite");
     if (a->compact_mode < FDMA_COMPACT_AUTO || a->compact_mode > FDMA_COMPACT_ALWAYS)
         return fail(FDMA_ERR_INVALID, "compact_mode must be FDMA_COMPACT_AUTO, _NEVER or _ALWAYS (got %d)", a->compact_mode);

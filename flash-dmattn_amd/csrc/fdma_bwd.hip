@@ -57,10 +57,13 @@ __global__ void __launch_bounds__(256) bwd_dot_kernel(const BwdParams p) {
 // query heads of the group in registers first and leaves through a tile of its own.  Otherwise every lane
 // writes its dS over the fused-bias elements it has just read (same rows, its own column), which saves the
 // extra tile and 64 registers: at d <= 64 two workgroups then fit on a CU and cover each other's phases.
-constexpr int KV_BM = 64;   // query rows per step
 constexpr int KV_BN = 128;  // key columns per workgroup (32 per wave)
 
+// query rows per step: 64, or 32 at head dims above 128 (LDS and registers)
+template <int D> struct KvRows { static constexpr int value = D > 128 ? 32 : 64; };
+
 template <int D, bool GSUM> struct KvSmem {
+    static constexpr int KV_BM = KvRows<D>::value;
     static constexpr int S = D + 8;          // Q / dO row stride (elements)
     static constexpr int SB = KV_BN + 8;     // fused-bias / dS tile row stride (elements)
     static constexpr int Q_BYTES = KV_BM * S * 2;
@@ -78,6 +81,8 @@ template <typename T, int D, bool CAUSAL, bool GSUM>
 __global__ void __launch_bounds__(NTHREADS, (D <= 64 && !GSUM) ? 2 : 1) bwd_dkdv_kernel(const BwdParams p) {
     using E = Elem<T>;
     using SM = KvSmem<D, GSUM>;
+    constexpr int KV_BM = KvRows<D>::value;  // (query rows per step)
+    constexpr int FB_IT = KV_BM / 16;        // passes of 16 rows over the fused-bias tile
     constexpr int KS = D / 16;
     constexpr int DB = D / 32;
     constexpr int MB = KV_BM / 32;
@@ -155,8 +160,8 @@ __global__ void __launch_bounds__(NTHREADS, (D <= 64 && !GSUM) ? 2 : 1) bwd_dkdv
     const int qc = tid % CH, qr0 = tid / CH;
     const int qcol = (qc * 8 < f.d) ? qc * 8 : 0;
     const int bc = tid & 15, br0 = tid >> 4;  // fused-bias tile: 8-key chunk and first row of this thread
-    u32x4_t qreg[Q_IT], doreg[Q_IT], braw[4];
-    u32x2_t mraw[4];
+    u32x4_t qreg[Q_IT], doreg[Q_IT], braw[FB_IT];
+    u32x2_t mraw[FB_IT];
     float lreg = INFINITY, dreg = 0.f;
     bool stat_ok = false;
     // Every load of a step is unconditional and raw (clamped rows / keys; an absent mask or bias is read from K, any
@@ -196,7 +201,7 @@ __global__ void __launch_bounds__(NTHREADS, (D <= 64 && !GSUM) ? 2 : 1) bwd_dkdv
         const int64_t moff = f.mask ? b * f.m_b + hm * f.m_h + kk_c : 0;
         const int64_t boff = has_bias ? b * f.bi_b + hb * f.bi_h + kk_c : 0;
 #pragma unroll
-        for (int it = 0; it < 4; it++) {
+        for (int it = 0; it < FB_IT; it++) {
             int qq = m0 + br0 + 16 * it;
             qq = qq < f.Lq ? qq : f.Lq - 1;
             braw[it] = *(const u32x4_t *)(bias_ld + boff + (has_bias ? (int64_t)qq * f.bi_r : 0));
@@ -219,7 +224,7 @@ __global__ void __launch_bounds__(NTHREADS, (D <= 64 && !GSUM) ? 2 : 1) bwd_dkdv
         char *fb = base + 2 * SM::Q_BYTES + 2 * KV_BM * 4;
         const int kk = n0 + 8 * bc;
 #pragma unroll
-        for (int it = 0; it < 4; it++) {
+        for (int it = 0; it < FB_IT; it++) {
             u32x4_t bv = has_bias ? braw[it] : u32x4_t{0, 0, 0, 0};
             u32x2_t mv = f.mask ? mraw[it] : u32x2_t{0x01010101u, 0x01010101u};
             uint64_t keepm = kk < f.Lk ? ~0ull : 0ull;
@@ -444,7 +449,7 @@ __global__ void __launch_bounds__(NTHREADS, (D <= 64 && !GSUM) ? 2 : 1) bwd_dkdv
             uint16_t *dbp = (uint16_t *)p.dbias + b * p.db_b + hb * p.db_h;
             const int kk = n0 + 8 * bc;
 #pragma unroll
-            for (int it = 0; it < 4; it++) {
+            for (int it = 0; it < FB_IT; it++) {
                 const int ql = br0 + 16 * it, qq = m0 + ql;
                 if (qq < f.Lq && kk < f.Lk)
                     *(u32x4_t *)(dbp + (int64_t)qq * p.db_r + kk) = *(const u32x4_t *)(sDS + ql * SM::SB + 8 * bc);
@@ -565,9 +570,10 @@ hipError_t launch_bwd_t(const BwdParams &p, hipStream_t stream) {
 
 hipError_t launch_bwd(const BwdParams &p, int dtype, hipStream_t stream) {
     if (p.f.B <= 0 || p.f.Lq <= 0) return hipSuccess;
-    const bool d64 = p.f.d <= 64;
-    if (dtype == 0) return d64 ? launch_bwd_t<bf16_tag, 64>(p, stream) : launch_bwd_t<bf16_tag, 128>(p, stream);
-    return d64 ? launch_bwd_t<fp16_tag, 64>(p, stream) : launch_bwd_t<fp16_tag, 128>(p, stream);
+    // head dims up to 64 / 128 / 256 (a head dim in between runs in the next larger instantiation)
+    const int d = p.f.d;
+    if (dtype == 0) return d <= 64 ? launch_bwd_t<bf16_tag, 64>(p, stream) : d <= 128 ? launch_bwd_t<bf16_tag, 128>(p, stream) : launch_bwd_t<bf16_tag, 256>(p, stream);
+    return d <= 64 ? launch_bwd_t<fp16_tag, 64>(p, stream) : d <= 128 ? launch_bwd_t<fp16_tag, 128>(p, stream) : launch_bwd_t<fp16_tag, 256>(p, stream);
 }
 
 }  // namespace fdma

@@ -37,7 +37,7 @@ template <> struct NegInf2<fp16_tag> { static constexpr uint32_t value = 0xFC00F
 
 template <typename T, int D, bool CAUSAL, int NW>
 __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) bwd_dq_kernel(const BwdParams p) {
-    constexpr int NTHREADS = 64 * NW, BM = 32 * NW, BN = NW == 8 ? 32 : 64;
+    constexpr int NTHREADS = 64 * NW, BM = 32 * NW, BN = (NW == 8 || D > 128) ? 32 : 64;
     constexpr int FCH = BN / 8;             // 8-key chunks per mask / bias row of a tile
     constexpr int F_RPP = NTHREADS / FCH;   // mask / bias rows staged per pass
     using E = Elem<T>;
@@ -332,7 +332,7 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) bwd_dq_
 
 template <typename T, int D, bool CAUSAL, int NW>
 hipError_t launch_dq_n(const BwdParams &p, hipStream_t stream) {
-    constexpr int BM = 32 * NW, NTHREADS = 64 * NW, BN = NW == 8 ? 32 : 64;
+    constexpr int BM = 32 * NW, NTHREADS = 64 * NW, BN = (NW == 8 || D > 128) ? 32 : 64;
     auto kern = bwd_dq_kernel<T, D, CAUSAL, NW>;
     const int smem = DqSmem<D, BM, BN>::TOTAL;
     static DynSmemLimit smem_limit;
@@ -345,7 +345,7 @@ hipError_t launch_dq_n(const BwdParams &p, hipStream_t stream) {
 
 template <typename T, int D, bool CAUSAL>
 hipError_t launch_dq_c(const BwdParams &p, hipStream_t stream) {
-    if constexpr (D > 64) {
+    if constexpr (D > 64 && D <= 128) {
         // 256-row workgroups while the grid still covers the chip about twice
         if ((int64_t)p.f.B * p.f.H * ((p.f.Lq + 255) / 256) >= 512) return launch_dq_n<T, D, CAUSAL, 8>(p, stream);
     }
@@ -355,13 +355,17 @@ hipError_t launch_dq_c(const BwdParams &p, hipStream_t stream) {
 }  // namespace
 
 hipError_t launch_bwd_dq(const BwdParams &p, int dtype, hipStream_t stream) {
-    const bool d64 = p.f.d <= 64, c = p.f.causal != 0;
+    // head dims up to 64 / 128 / 256 (a head dim in between runs in the next larger instantiation)
+    const int dc = p.f.d <= 64 ? 0 : (p.f.d <= 128 ? 1 : 2);
+    const bool c = p.f.causal != 0;
     if (dtype == 0) {
-        if (d64) return c ? launch_dq_c<bf16_tag, 64, true>(p, stream) : launch_dq_c<bf16_tag, 64, false>(p, stream);
-        return c ? launch_dq_c<bf16_tag, 128, true>(p, stream) : launch_dq_c<bf16_tag, 128, false>(p, stream);
+        if (dc == 0) return c ? launch_dq_c<bf16_tag, 64, true>(p, stream) : launch_dq_c<bf16_tag, 64, false>(p, stream);
+        if (dc == 1) return c ? launch_dq_c<bf16_tag, 128, true>(p, stream) : launch_dq_c<bf16_tag, 128, false>(p, stream);
+        return c ? launch_dq_c<bf16_tag, 256, true>(p, stream) : launch_dq_c<bf16_tag, 256, false>(p, stream);
     }
-    if (d64) return c ? launch_dq_c<fp16_tag, 64, true>(p, stream) : launch_dq_c<fp16_tag, 64, false>(p, stream);
-    return c ? launch_dq_c<fp16_tag, 128, true>(p, stream) : launch_dq_c<fp16_tag, 128, false>(p, stream);
+    if (dc == 0) return c ? launch_dq_c<fp16_tag, 64, true>(p, stream) : launch_dq_c<fp16_tag, 64, false>(p, stream);
+    if (dc == 1) return c ? launch_dq_c<fp16_tag, 128, true>(p, stream) : launch_dq_c<fp16_tag, 128, false>(p, stream);
+    return c ? launch_dq_c<fp16_tag, 256, true>(p, stream) : launch_dq_c<fp16_tag, 256, false>(p, stream);
 }
 
 }  // namespace fdma

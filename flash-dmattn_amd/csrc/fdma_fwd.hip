@@ -31,9 +31,11 @@ namespace {
 // Workgroups have 4 waves (128 query rows; two per CU at d <= 64) or, at d = 128 on grids that stay large enough,
 // 8 waves (256 rows): at d = 128 only one workgroup fits on a CU, and with a single wave per SIMD nothing hides the
 // in-order issue of that wave -- a second wave per SIMD does.
-constexpr int BN = 64;
+constexpr int BN_DEFAULT = 64;  // keys per tile (32 at head dims above 128: LDS)
 
-template <int D, int BM> struct FwdSmem {
+template <int D, int BN, int NT> struct KQ_OK { static constexpr bool value = (BN / 4) * (D / 8) <= NT; };
+
+template <int D, int BM, int BN> struct FwdSmem {
     static constexpr int SK = D + 8;     // K tile row stride (elements): conflict-free 16-byte row reads
     static constexpr int SVT = BN + 8;   // V^T tile row stride
     static constexpr int SF = BN + 8;    // fused mask+bias tile row stride
@@ -48,12 +50,14 @@ template <typename T> struct NegInf2;
 template <> struct NegInf2<bf16_tag> { static constexpr uint32_t value = 0xFF80FF80u; };
 template <> struct NegInf2<fp16_tag> { static constexpr uint32_t value = 0xFC00FC00u; };
 
-template <typename T, int D, bool CAUSAL, int NW>
+template <typename T, int D, bool CAUSAL, int NW, int BN>
 __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) fwd_kernel(const FwdParams p) {
     constexpr int NTHREADS = 64 * NW, BM = 32 * NW;
-    constexpr int F_RPP = NTHREADS / 8;     // mask / bias rows staged per pass (8 threads cover the 64 keys of a row)
+    constexpr int FCH = BN / 8;             // 8-key chunks per mask / bias row of a tile
+    constexpr int F_RPP = NTHREADS / FCH;   // mask / bias rows staged per pass (FCH threads cover the keys of a row)
     using E = Elem<T>;
-    using SM = FwdSmem<D, BM>;
+    using SM = FwdSmem<D, BM, BN>;
+    static_assert(KQ_OK<D, BN, 64 * NW>::value, "a V tile is one (key quad, d chunk) item per thread at most");
     constexpr int KS = D / 16;  // contraction steps of Q K^T
     constexpr int DB = D / 32;  // 32-wide blocks of the head dimension
     constexpr int MB = BN / 32, KB = BN / 16, KQ = BN / 4;
@@ -122,7 +126,7 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) fwd_ker
     const int kc = tid % CH, kr0 = tid / CH;             // K: d chunk, first row
     const int vkg = tid % KQ, vc = (tid / KQ) % CH;      // V: key quad, d chunk
     const bool k_dvalid = kc * 8 < p.d, v_dvalid = vc * 8 < p.d;
-    const int fc = tid & 7, fr0 = tid >> 3;              // mask / bias: 8-key chunk, first row (rows fr0 + F_RPP it)
+    const int fc = tid % FCH, fr0 = tid / FCH;           // mask / bias: 8-key chunk, first row (rows fr0 + F_RPP it)
     u32x4_t kreg[K_IT], vreg[4], breg[F_IT];
     u32x2_t mreg[F_IT], mnext[F_IT];
 
@@ -386,9 +390,9 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) fwd_ker
 
 template <typename T, int D, bool CAUSAL, int NW>
 hipError_t launch_fwd_c(const FwdParams &p, hipStream_t stream) {
-    constexpr int BM = 32 * NW, NTHREADS = 64 * NW;
-    auto kern = fwd_kernel<T, D, CAUSAL, NW>;
-    const int smem = FwdSmem<D, BM>::TOTAL;
+    constexpr int BM = 32 * NW, NTHREADS = 64 * NW, BN = D > 128 ? 32 : BN_DEFAULT;
+    auto kern = fwd_kernel<T, D, CAUSAL, NW, BN>;
+    const int smem = FwdSmem<D, BM, BN>::TOTAL;
     static DynSmemLimit smem_limit;
     hipError_t e = smem_limit.ensure((const void *)kern, (int)smem);
     if (e != hipSuccess) return e;
@@ -399,7 +403,7 @@ hipError_t launch_fwd_c(const FwdParams &p, hipStream_t stream) {
 
 template <typename T, int D>
 hipError_t launch_fwd_t(const FwdParams &p, hipStream_t stream) {
-    if constexpr (D > 64) {
+    if constexpr (D > 64 && D <= 128) {
         // 256-row workgroups while the grid still covers the chip about twice
         if ((int64_t)p.B * p.H * ((p.Lq + 255) / 256) >= 512)
             return p.causal ? launch_fwd_c<T, D, true, 8>(p, stream) : launch_fwd_c<T, D, false, 8>(p, stream);
@@ -412,9 +416,9 @@ hipError_t launch_fwd_t(const FwdParams &p, hipStream_t stream) {
 hipError_t launch_fwd(const FwdParams &p, int dtype, hipStream_t stream) {
     if (p.Lq <= 0 || p.B <= 0) return hipSuccess;
     if (fwd_colmask_applicable(p)) return launch_fwd_colmask(p, dtype, stream);
-    const bool d64 = p.d <= 64;
-    if (dtype == 0) return d64 ? launch_fwd_t<bf16_tag, 64>(p, stream) : launch_fwd_t<bf16_tag, 128>(p, stream);
-    return d64 ? launch_fwd_t<fp16_tag, 64>(p, stream) : launch_fwd_t<fp16_tag, 128>(p, stream);
+    // head dims up to 64 / 128 / 256 (a head dim in between runs in the next larger instantiation)
+    if (dtype == 0) return p.d <= 64 ? launch_fwd_t<bf16_tag, 64>(p, stream) : p.d <= 128 ? launch_fwd_t<bf16_tag, 128>(p, stream) : launch_fwd_t<bf16_tag, 256>(p, stream);
+    return p.d <= 64 ? launch_fwd_t<fp16_tag, 64>(p, stream) : p.d <= 128 ? launch_fwd_t<fp16_tag, 128>(p, stream) : launch_fwd_t<fp16_tag, 256>(p, stream);
 }
 
 }  // namespace fdma

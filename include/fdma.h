@@ -52,8 +52,8 @@ enum { FDMA_DTYPE_BF16 = 0, FDMA_DTYPE_FP16 = 1 };
 enum {
     FDMA_OK = 0,
     FDMA_ERR_INVALID = -1,     /* argument validation failed (the reference raises RuntimeError) */
-    FDMA_ERR_UNSUPPORTED = -2, /* valid for the reference, not built here (e.g. head_dim > 128,
-                                  a stream under HIP graph capture)                              */
+    FDMA_ERR_UNSUPPORTED = -2, /* valid for the reference, not built here (softcap, row strides of 2^24
+                                  elements or more, a stream under HIP graph capture)            */
     FDMA_ERR_WORKSPACE = -3,   /* workspace missing or too small                                  */
     FDMA_ERR_LAUNCH = -4       /* the HIP runtime refused a launch                                */
 };

@@ -73,8 +73,6 @@ def test_validation_accepts_a_good_call_and_needs_no_gpu():
         (lambda a: (setattr(a, "bias", 0x2000), setattr(a, "num_heads_bias", 5)), "Number of heads in bias must be 1, h_k or h"),
         (lambda a: setattr(a, "q", 0x1004), "16-byte aligned"),
         (lambda a: setattr(a, "softcap", 30.0), "softcap"),
-        (lambda a: (setattr(a, "head_dim", 192), setattr(a, "mask", 0x2000), a.mask_strides.__setitem__(2, 256)),
-         "head dimensions above 128 are built for masks and biases that are broadcast over the queries"),
         (lambda a: a.k_strides.__setitem__(1, 1 << 24), "row strides of 2^24 elements or more"),
     ],
 )

@@ -95,6 +95,11 @@ SMALL_CASES = {
     "head_dim_192_lq_lt_lk_mask_only": (1, 100, 333, 2, 1, 192, None, (1, 1, 1, 333), 120, True),
     "head_dim_256_lq_gt_lk_empty_rows": (1, 333, 100, 2, 2, 256, (1, 2, 1, 100), (1, 2, 1, 100), 50, True),
     "head_dim_136_bias_only": (1, 130, 130, 2, 2, 136, (1, 1, 1, 130), None, None, True),
+    # ... and with per-query masks / biases (the general kernels at 256, 32-key tiles / 32-row steps)
+    "head_dim_256_full_mask_full_bias": (2, 200, 264, 4, 2, 256, (2, 4, 200, 264), (2, 4, 200, 264), 64, True),
+    "head_dim_192_full_bias_kv_heads": (1, 200, 264, 4, 2, 192, (1, 2, 200, 264), (1, 1, 200, 264), 64, True),
+    "head_dim_256_full_bias_batch_broadcast": (2, 100, 160, 2, 2, 256, (1, 2, 100, 160), (2, 1, 100, 160), 40, False),
+    "head_dim_192_row_bias_full_mask_lq_lt_lk": (1, 100, 333, 2, 2, 192, (1, 2, 1, 333), (1, 1, 100, 333), 100, True),
 }
 
 

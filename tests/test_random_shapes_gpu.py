@@ -1,6 +1,6 @@
 """Seeded random-shape sweep of the operator against the fp32 eager restatement (run with `-m gpu`): ragged lengths from 1
 to 900, every mask / bias form the operator takes (absent, per key column with 1 / Hkv / H heads, per query), causal
-and not, bf16 and fp16, GQA ratios 1 / 2 / 4, head dims 32 to 128, larger score scales (they exercise the lazy rescale
+and not, bf16 and fp16, GQA ratios 1 / 2 / 4, head dims 32 to 128 (and, in a second block of cases, 136 to 256), larger score scales (they exercise the lazy rescale
 of the running maximum), both paths for query-broadcast masks (tile skipping, column compaction) and a few grids large
 enough for the 8-wave kernels.  The shapes are drawn from a fixed seed, so a failure names a reproducible case."""
 import os
@@ -15,14 +15,17 @@ from _util import GRAD_RTOL, OUT_ATOL, make_inputs, set_compact
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
 N_CASES = 48
+N_WIDE = 16  # further cases, numbered from N_CASES on, with head dims above 128
 
 
 def _draw(it):
     rng = random.Random(7000 + it)
     D = rng.choice([32, 64, 96, 128, 128, 128])
+    if it >= N_CASES:
+        D = rng.choice([136, 160, 192, 256, 256])
     Hk = rng.choice([1, 2, 4])
     H = Hk * rng.choice([1, 2, 4])
-    big = it % 8 == 7
+    big = it % 8 == 7 and it < N_CASES
     B = rng.choice([1, 2, 3])
     Lq, Lk = rng.randint(1, 700), rng.randint(1, 900)
     form = rng.choice(["col", "col", "col_h", "full", "none", "bias_only", "mask_only"])
@@ -41,7 +44,7 @@ def _draw(it):
                 compact=rng.choice(["0", "1", "2"]))
 
 
-@pytest.mark.parametrize("it", range(N_CASES))
+@pytest.mark.parametrize("it", range(N_CASES + N_WIDE))
 def test_random_case_vs_eager_fp32(it, monkeypatch):
     from flash_sparse_attn import flash_sparse_attn_func
 
