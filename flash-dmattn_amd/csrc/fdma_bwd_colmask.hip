@@ -461,62 +461,67 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dkdv_colmask_k
         const bool diag = (CAUSAL && (okey_wlast > m0 + shift)) || (DMA && m0 + BM > LqS);
         uint32_t ppk[MB * 8], dpk[MB * 8];
         float part = 0.f;
+        // softmax and dS of one block of 16 query rows (8 per lane) in three pieces, so that the MFMAs of the rows whose
+        // probabilities are finished can be issued between the pieces of the next block: A = statistics, exp2, dP - D;
+        // M = masking (diagonal steps only: rows above the causal diagonal or beyond the end of the queries give
+        // P = 0); B = dS, column sum, conversion to 16 bits
+        float pv[8], dsv[8];
+        auto soft_a = [&](auto mb_c, auto blk_c) {
+            constexpr int mb = decltype(mb_c)::value, blk = decltype(blk_c)::value;
+            const uint32_t so = buf * SM::STAGE + 2 * SM::Q_BYTES + (32 * mb + 16 * blk) * 4;  // LSE; D is BM floats on
+            const f32x4_t l0 = __builtin_bit_cast(f32x4_t, lds_ld128(stat_off + so)), l1 = __builtin_bit_cast(f32x4_t, lds_ld128(stat_off + so + 16));
+            const f32x4_t d0 = __builtin_bit_cast(f32x4_t, lds_ld128(stat_off + so + BM * 4)), d1 = __builtin_bit_cast(f32x4_t, lds_ld128(stat_off + so + BM * 4 + 16));
 #pragma unroll
-        for (int mb = 0; mb < MB; mb++)
-#pragma unroll
-            for (int blk = 0; blk < 2; blk++) {
-                const uint32_t so = buf * SM::STAGE + 2 * SM::Q_BYTES + (32 * mb + 16 * blk) * 4;  // LSE; D is BM floats on
-                const f32x4_t l0 = __builtin_bit_cast(f32x4_t, lds_ld128(stat_off + so)), l1 = __builtin_bit_cast(f32x4_t, lds_ld128(stat_off + so + 16));
-                const f32x4_t d0 = __builtin_bit_cast(f32x4_t, lds_ld128(stat_off + so + BM * 4)), d1 = __builtin_bit_cast(f32x4_t, lds_ld128(stat_off + so + BM * 4 + 16));
-                float pv[8], dsv[8];
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    const int ii = 8 * blk + e;
-                    const float lse2 = e < 4 ? l0[e] : l1[e - 4];
-                    const float dd = e < 4 ? d0[e] : d1[e - 4];
-                    pv[e] = fast_exp2(DMA ? __builtin_fmaf(lse2, -kLog2e, s[mb][ii]) : s[mb][ii] - lse2);
-                    dsv[e] = dp[mb][ii] - dd;
-                }
-                if (diag) {
-                    asm volatile("" ::: "memory");  // keep a real branch: only diagonal steps pay
-                    int lim = CAUSAL ? okey - shift - m0 - 32 * mb - 16 * blk - 8 * g : 0;  // rows e >= lim see this key
-                    int lim_hi = DMA ? LqS - m0 - 32 * mb - 16 * blk - 8 * g : 8;            // rows e < lim_hi exist
-                    asm volatile("" : "+v"(lim), "+v"(lim_hi));  // (the comparisons stay inside the branch)
-#pragma unroll
-                    for (int e = 0; e < 8; e++) pv[e] = (e >= lim && e < lim_hi) ? pv[e] : 0.f;
-                }
-#pragma unroll
-                for (int e = 0; e < 8; e++) {
-                    dsv[e] *= pv[e];
-                    part += dsv[e];
-                }
-#pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    ppk[mb * 8 + blk * 4 + e] = E::pack2(pv[2 * e], pv[2 * e + 1]);
-                    dpk[mb * 8 + blk * 4 + e] = E::pack2(dsv[2 * e], dsv[2 * e + 1]);
-                }
+            for (int e = 0; e < 8; e++) {
+                const int ii = 8 * blk + e;
+                const float lse2 = e < 4 ? l0[e] : l1[e - 4];
+                const float dd = e < 4 ? d0[e] : d1[e - 4];
+                pv[e] = fast_exp2(DMA ? __builtin_fmaf(lse2, -kLog2e, s[mb][ii]) : s[mb][ii] - lse2);
+                dsv[e] = dp[mb][ii] - dd;
             }
-        colsum += part;
-
-        // ---- dV^T += dO^T P ; dK^T += Q^T dS   (M = d, N = key, contraction = query)
-        // (after the last steps an existing tile is fetched again and dropped)
-        if constexpr (!DMA) load_step(step + 2 < n_steps ? step + 2 : step, false);
-        {   // the transposing fragment reads run one (query block, d block) pair ahead of the MFMAs that use them
-            constexpr int NP = (BM / 16) * DB;
-            u32x4_t a1[2], a2[2];
-            auto frag = [&](int idx, int slot) {
-                const int qb = idx / DB, db = idx % DB;
-                const uint32_t off = TL::tr_at(tr_off, qb, db, 0), off_hi = TL::tr_at(tr_off, qb, db, 1);
-                constexpr uint32_t st = buf * SM::STAGE;
-                const u32x2_t lo = lds_ld_tr16(off + st + SM::Q_BYTES), hi = lds_ld_tr16(off_hi + st + SM::Q_BYTES);
-                const u32x2_t lo2 = lds_ld_tr16(off + st), hi2 = lds_ld_tr16(off_hi + st);
-                a1[slot] = u32x4_t{lo[0], lo[1], hi[0], hi[1]};
-                a2[slot] = u32x4_t{lo2[0], lo2[1], hi2[0], hi2[1]};
-            };
-            frag(0, 0);
+        };
+        auto soft_m = [&](auto mb_c, auto blk_c) {
+            constexpr int mb = decltype(mb_c)::value, blk = decltype(blk_c)::value;
+            if (diag) {
+                asm volatile("" ::: "memory");  // keep a real branch: only diagonal steps pay
+                int lim = CAUSAL ? okey - shift - m0 - 32 * mb - 16 * blk - 8 * g : 0;  // rows e >= lim see this key
+                int lim_hi = DMA ? LqS - m0 - 32 * mb - 16 * blk - 8 * g : 8;            // rows e < lim_hi exist
+                asm volatile("" : "+v"(lim), "+v"(lim_hi));  // (the comparisons stay inside the branch)
 #pragma unroll
-            for (int idx = 0; idx < NP; idx++) {
-                if (idx + 1 < NP) frag(idx + 1, (idx + 1) & 1);
+                for (int e = 0; e < 8; e++) pv[e] = (e >= lim && e < lim_hi) ? pv[e] : 0.f;
+            }
+        };
+        auto soft_b = [&](auto mb_c, auto blk_c) {
+            constexpr int mb = decltype(mb_c)::value, blk = decltype(blk_c)::value;
+#pragma unroll
+            for (int e = 0; e < 8; e++) {
+                dsv[e] *= pv[e];
+                part += dsv[e];
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                ppk[mb * 8 + blk * 4 + e] = E::pack2(pv[2 * e], pv[2 * e + 1]);
+                dpk[mb * 8 + blk * 4 + e] = E::pack2(dsv[2 * e], dsv[2 * e + 1]);
+            }
+        };
+        // ---- dV^T += dO^T P ; dK^T += Q^T dS   (M = d, N = key, contraction = query), pairs [idx0, idx1) of (16-row
+        // block, d block); the transposing fragment reads run one pair ahead of the MFMAs that use them
+        constexpr int NP = (BM / 16) * DB;
+        u32x4_t a1[2], a2[2];
+        auto tr_frag = [&](int idx, int slot) {
+            const int qb = idx / DB, db = idx % DB;
+            const uint32_t off = TL::tr_at(tr_off, qb, db, 0), off_hi = TL::tr_at(tr_off, qb, db, 1);
+            constexpr uint32_t st = buf * SM::STAGE;
+            const u32x2_t lo = lds_ld_tr16(off + st + SM::Q_BYTES), hi = lds_ld_tr16(off_hi + st + SM::Q_BYTES);
+            const u32x2_t lo2 = lds_ld_tr16(off + st), hi2 = lds_ld_tr16(off_hi + st);
+            a1[slot] = u32x4_t{lo[0], lo[1], hi[0], hi[1]};
+            a2[slot] = u32x4_t{lo2[0], lo2[1], hi2[0], hi2[1]};
+        };
+        auto gemm2 = [&](auto idx0_c, auto idx1_c) {
+            constexpr int idx0 = decltype(idx0_c)::value, idx1 = decltype(idx1_c)::value;
+#pragma unroll
+            for (int idx = idx0; idx < idx1; idx++) {
+                if (idx + 1 < NP) tr_frag(idx + 1, (idx + 1) & 1);
                 const int qb = idx / DB, db = idx % DB;
                 const u32x4_t pb = {ppk[4 * qb], ppk[4 * qb + 1], ppk[4 * qb + 2], ppk[4 * qb + 3]};
                 const u32x4_t sb = {dpk[4 * qb], dpk[4 * qb + 1], dpk[4 * qb + 2], dpk[4 * qb + 3]};
@@ -527,6 +532,30 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dkdv_colmask_k
                     for (int n = idx * 2 * Q_IT / NP; n < (idx + 1) * 2 * Q_IT / NP; n++) load_item(n);
                 }
             }
+        };
+        using I0 = std::integral_constant<int, 0>;
+        using I1 = std::integral_constant<int, 1>;
+        // (after the last steps an existing tile is fetched again and dropped)
+        if constexpr (!DMA) load_step(step + 2 < n_steps ? step + 2 : step, false);
+        if constexpr (MB == 1) {
+            // the MFMAs of the first 16 rows need the probabilities of those rows only: the softmax of the other 16
+            // rows is issued between them
+            soft_a(I0(), I0()); soft_m(I0(), I0()); soft_b(I0(), I0());
+            tr_frag(0, 0);
+            gemm2(I0(), std::integral_constant<int, DB / 2>());
+            soft_a(I0(), I1());
+            soft_m(I0(), I1());
+            gemm2(std::integral_constant<int, DB / 2>(), std::integral_constant<int, DB>());
+            soft_b(I0(), I1());
+            gemm2(std::integral_constant<int, DB>(), std::integral_constant<int, NP>());
+        } else {
+            static_assert(MB <= 2, "steps of 32 or 64 query rows");
+            soft_a(I0(), I0()); soft_m(I0(), I0()); soft_b(I0(), I0());
+            soft_a(I0(), I1()); soft_m(I0(), I1()); soft_b(I0(), I1());
+            soft_a(I1(), I0()); soft_m(I1(), I0()); soft_b(I1(), I0());
+            soft_a(I1(), I1()); soft_m(I1(), I1()); soft_b(I1(), I1());
+            tr_frag(0, 0);
+            gemm2(I0(), std::integral_constant<int, NP>());
             // pin the order: reads of pair idx+1, then the two MFMAs of pair idx
             __builtin_amdgcn_sched_group_barrier(0x100, 4, 0);
 #pragma unroll
@@ -535,6 +564,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dkdv_colmask_k
                 __builtin_amdgcn_sched_group_barrier(0x008, 2, 0);
             }
         }
+        colsum += part;
 
         // ---- dBias column sum: flush when the bias head changes
         if (has_bias) {
