@@ -1059,27 +1059,35 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
         const char *sV = smem + SM::OFF_V + (i & 1) * SM::K_BYTES;
         const float *bs = sBias + (i % 3) * BN + 8 * g;
 
-        // ---- S^T = K Q^T, dP^T = V dO^T
+        // ---- S^T = K Q^T, dP^T = V dO^T, dS^T = P^T * (dP^T - D), dQ^T += K^T dS^T.  A wave issues in program
+        // order, so the vector work has to sit BETWEEN the MFMAs to run under them; the tile is written slot by slot --
+        // one MFMA, the fragment read of the MFMA FR slots later, a share of the vector work, a piece of the next tile's
+        // loads -- with a scheduling barrier after every slot:
+        //   slots of S (all k-steps), then slots of dP with the exp2 of the finished scores between them, then the dQ
+        //   slots of one 16-key block with the dS arithmetic of the next block between them.
+        // The score accumulators start from the fused bias vector minus the row's log-sum-exp and the dP accumulators
+        // from minus D, so that the MFMAs deliver the exp2 argument and dP - D themselves.
         f32x16_t s[MB], dp[MB];
 #pragma unroll
         for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-            for (int blk = 0; blk < 2; blk++) {  // the score accumulators start from the fused bias vector
+            for (int blk = 0; blk < 2; blk++) {
                 const f32x4_t b0 = *(const f32x4_t *)(bs + 32 * mb + 16 * blk);
                 const f32x4_t b1 = *(const f32x4_t *)(bs + 32 * mb + 16 * blk + 4);
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
-                    s[mb][8 * blk + e] = b0[e];
-                    s[mb][8 * blk + 4 + e] = b1[e];
-                    dp[mb][8 * blk + e] = 0.f;
-                    dp[mb][8 * blk + 4 + e] = 0.f;
+                    s[mb][8 * blk + e] = b0[e] - lse2;
+                    s[mb][8 * blk + 4 + e] = b1[e] - lse2;
+                    dp[mb][8 * blk + e] = -dd;
+                    dp[mb][8 * blk + 4 + e] = -dd;
                 }
             }
+        float pv[16 * MB];
         {
-            constexpr int NF = 2 * MB * KS, FR = 8;
+            constexpr int NH = MB * KS, NF = 2 * NH, FR = 4;
             u32x4_t a[NF];
-            auto frag = [&](int fi) {
-                const int which = fi & 1, mb = (fi >> 1) % MB, ks = (fi >> 1) / MB;
+            auto frag = [&](int fi) {  // S slots first (K tile), then dP slots (V tile); k-step major, row block minor
+                const int which = fi / NH, mb = (fi % NH) % MB, ks = (fi % NH) / MB;
                 return *(const u32x4_t *)((which ? sV : sK) + TL::frag_at(a_off, ks) + 32 * mb * TL::ROW_BYTES);
             };
 #pragma unroll
@@ -1087,45 +1095,64 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
 #pragma unroll
             for (int fi = 0; fi < NF; fi++) {
                 if (fi + FR < NF) a[fi + FR] = frag(fi + FR);
-                const int which = fi & 1, mb = (fi >> 1) % MB, ks = (fi >> 1) / MB;
+                const int which = fi / NH, mb = (fi % NH) % MB, ks = (fi % NH) / MB;
                 if (which) dp[mb] = E::mfma(a[fi], dof[ks], dp[mb]);
                 else s[mb] = E::mfma(a[fi], qf[ks], s[mb]);
 #pragma unroll
                 for (int n = fi * 2 * K_IT / NF; n < (fi + 1) * 2 * K_IT / NF; n++) load_item(n);
+                if (which) {
+#pragma unroll
+                    for (int e = 0; e < 16 * MB; e++)
+                        if (e * NH / (16 * MB) == fi - NH) pv[e] = fast_exp2(s[e / 16][e % 16]);
+                }
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
-        // ---- dS^T = P^T * (dP^T - D)
         const bool diag = CAUSAL && (n0 + BN > vis_wave);
-        uint32_t dpk[8 * MB];
+        if (diag) {
 #pragma unroll
-        for (int mb = 0; mb < MB; mb++)
+            for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-            for (int blk = 0; blk < 2; blk++) {
-                float pv[8];
-#pragma unroll
-                for (int e = 0; e < 8; e++) pv[e] = fast_exp2(s[mb][8 * blk + e] - lse2);
-                if (diag) {
-                    asm volatile("" ::: "memory");
+                for (int blk = 0; blk < 2; blk++) {
                     const int lim = vis_lane - 1 - n0 - 32 * mb - 16 * blk - 8 * g;  // local columns e <= lim are visible
 #pragma unroll
-                    for (int e = 0; e < 8; e++) pv[e] = e <= lim ? pv[e] : 0.f;
+                    for (int e = 0; e < 8; e++) pv[16 * mb + 8 * blk + e] = e <= lim ? pv[16 * mb + 8 * blk + e] : 0.f;
                 }
+        }
+        __builtin_amdgcn_sched_barrier(0);
+        uint32_t dpk[8 * MB];
+        auto ds_piece = [&](int kb, int e) {  // two elements of 16-key block kb: dS = P * (dP - D), rounded to 16 bits
+            const int mb = kb >> 1, blk = kb & 1;
+            const float d0 = pv[16 * mb + 8 * blk + 2 * e] * dp[mb][8 * blk + 2 * e];
+            const float d1 = pv[16 * mb + 8 * blk + 2 * e + 1] * dp[mb][8 * blk + 2 * e + 1];
+            dpk[4 * kb + e] = E::pack2(d0, d1);
+        };
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    const float d0 = pv[2 * e] * (dp[mb][8 * blk + 2 * e] - dd);
-                    const float d1 = pv[2 * e + 1] * (dp[mb][8 * blk + 2 * e + 1] - dd);
-                    dpk[8 * mb + 4 * blk + e] = E::pack2(d0, d1);
+        for (int e = 0; e < 4; e++) ds_piece(0, e);
+        {
+            // K^T through transposing LDS reads of the row-major K tile, two reads per MFMA, FR2 MFMAs ahead
+            constexpr int NG = KB * DB, FR2 = 2;
+            u32x2_t tl[NG], th[NG];
+            auto tr_read = [&](int gi) {
+                const int kb = gi / DB, db = gi % DB;
+                tl[gi] = lds_read_tr16(sK, TL::tr_at(tr_off, kb, db, 0));
+                th[gi] = lds_read_tr16(sK, TL::tr_at(tr_off, kb, db, 1));
+            };
+#pragma unroll
+            for (int gi = 0; gi < FR2; gi++) tr_read(gi);
+#pragma unroll
+            for (int gi = 0; gi < NG; gi++) {
+                if (gi + FR2 < NG) tr_read(gi + FR2);
+                const int kb = gi / DB, db = gi % DB;
+                const u32x4_t bop = {dpk[4 * kb], dpk[4 * kb + 1], dpk[4 * kb + 2], dpk[4 * kb + 3]};
+                const u32x4_t av = {tl[gi][0], tl[gi][1], th[gi][0], th[gi][1]};
+                dq[db] = E::mfma(av, bop, dq[db]);
+                if (kb + 1 < KB) {  // the next block's dS, spread over this block's slots
+#pragma unroll
+                    for (int e = 0; e < 4; e++)
+                        if (e * DB / 4 == db) ds_piece(kb + 1, e);
                 }
-            }
-        // ---- dQ^T += K^T dS^T  (K^T through transposing LDS reads of the row-major K tile)
-#pragma unroll
-        for (int kb = 0; kb < KB; kb++) {
-            const u32x4_t bop = {dpk[4 * kb], dpk[4 * kb + 1], dpk[4 * kb + 2], dpk[4 * kb + 3]};
-#pragma unroll
-            for (int db = 0; db < DB; db++) {
-                const u32x2_t lo = lds_read_tr16(sK, TL::tr_at(tr_off, kb, db, 0)), hi = lds_read_tr16(sK, TL::tr_at(tr_off, kb, db, 1));
-                const u32x4_t a = {lo[0], lo[1], hi[0], hi[1]};
-                dq[db] = E::mfma(a, bop, dq[db]);
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
         if (jn < n_end) store_tile((i + 1) & 1, (i + 1) % 3);
