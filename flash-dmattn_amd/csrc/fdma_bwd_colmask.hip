@@ -1053,7 +1053,6 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
     int i = 0;
     while (jc < n_end) {
         const int jn = next_active(jc + 1);
-        set_tile(jn < n_end ? jn : jc);  // (after the last tile the current one is fetched again and dropped)
         const int n0 = jc * BN;
         const char *sK = smem + SM::OFF_K + (i & 1) * SM::K_BYTES;
         const char *sV = smem + SM::OFF_V + (i & 1) * SM::K_BYTES;
@@ -1082,6 +1081,10 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
                     dp[mb][8 * blk + 4 + e] = -dd;
                 }
             }
+        // the next tile's bases and side inputs (after the last tile the current one is fetched again and dropped); behind
+        // the accumulator set-up: the load of the bias / mask column must not be waited for with the LDS reads above
+        __builtin_amdgcn_sched_barrier(0);
+        set_tile(jn < n_end ? jn : jc);
         float pv[16 * MB];
         {
             constexpr int NH = MB * KS, NF = 2 * NH, FR = 4;
@@ -1110,6 +1113,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
         }
         const bool diag = CAUSAL && (n0 + BN > vis_wave);
         if (diag) {
+            asm volatile("" ::: "memory");  // (keeps this a branch: as selects, every tile would pay for the diagonal ones)
 #pragma unroll
             for (int mb = 0; mb < MB; mb++)
 #pragma unroll
@@ -1127,10 +1131,9 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
             const float d1 = pv[16 * mb + 8 * blk + 2 * e + 1] * dp[mb][8 * blk + 2 * e + 1];
             dpk[4 * kb + e] = E::pack2(d0, d1);
         };
-#pragma unroll
-        for (int e = 0; e < 4; e++) ds_piece(0, e);
         {
-            // K^T through transposing LDS reads of the row-major K tile, two reads per MFMA, FR2 MFMAs ahead
+            // K^T through transposing LDS reads of the row-major K tile, two reads per MFMA, FR2 MFMAs ahead (the first
+            // ones in front of the first block's dS arithmetic)
             constexpr int NG = KB * DB, FR2 = 2;
             u32x2_t tl[NG], th[NG];
             auto tr_read = [&](int gi) {
@@ -1140,6 +1143,9 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
             };
 #pragma unroll
             for (int gi = 0; gi < FR2; gi++) tr_read(gi);
+            __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+            for (int e = 0; e < 4; e++) ds_piece(0, e);
 #pragma unroll
             for (int gi = 0; gi < NG; gi++) {
                 if (gi + FR2 < NG) tr_read(gi + FR2);
