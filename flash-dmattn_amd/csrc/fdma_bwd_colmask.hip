@@ -1087,7 +1087,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
         set_tile(jn < n_end ? jn : jc);
         float pv[16 * MB];
         {
-            constexpr int NH = MB * KS, NF = 2 * NH, FR = 4;
+            constexpr int NH = MB * KS, NF = 2 * NH, FR = 3;
             u32x4_t a[NF];
             auto frag = [&](int fi) {  // S slots first (K tile), then dP slots (V tile); k-step major, row block minor
                 const int which = fi / NH, mb = (fi % NH) % MB, ks = (fi % NH) / MB;
