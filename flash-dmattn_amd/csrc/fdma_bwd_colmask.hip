@@ -804,10 +804,11 @@ constexpr int MAX_TILES = 16384;
 template <int D, int BN> struct DqcSmem {
     static constexpr int S = LdsTile<D>::S;
     static constexpr int K_BYTES = BN * S * 2;
+    static constexpr int NST = LdsTile<D>::SWZ ? 3 : 2;  // K / V stages: three where the tiles are fetched two ahead
     static constexpr int OFF_K = 0;
-    static constexpr int OFF_V = OFF_K + 2 * K_BYTES;
-    static constexpr int OFF_BIAS = OFF_V + 2 * K_BYTES;
-    static constexpr int OFF_BITS = OFF_BIAS + 3 * BN * 4;
+    static constexpr int OFF_V = OFF_K + NST * K_BYTES;
+    static constexpr int OFF_BIAS = OFF_V + NST * K_BYTES;
+    static constexpr int OFF_BITS = OFF_BIAS + 3 * 256;  // three bias columns (a direct load fills 256 bytes)
     static constexpr int TOTAL = OFF_BITS + MAX_TILES / 8;
 };
 
@@ -821,13 +822,26 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
     constexpr int MB = BN / 32;
     constexpr int KB = BN / 16;
     constexpr int CH = D / 8, RPP = NTHREADS / CH, K_IT = BN / RPP;
+    // DMA (compacted keys, rows of exactly 256 bytes): the K / V tiles and the fused bias column go from global memory
+    // straight into LDS (global_load_lds: a wave writes 64 consecutive 16-byte or 4-byte pieces, so the swizzle of the
+    // tile is applied to the GLOBAL address of each lane's piece), TWO tiles ahead, into a third stage: no staging
+    // registers, no LDS stores, and a tile has a whole tile time more to arrive.  (Through registers, loaded between the
+    // MFMAs of the tile whose end stores them, the stores waited for the loads: without the loads the kernel was 12 %
+    // shorter.)  The instruction is written in assembly: issued through the compiler's builtin, every later LDS read
+    // waited for ALL direct loads in flight -- the compiler cannot tell which stage they fill -- and the loads of
+    // the tile after the next one would be waited for at once.  The waits are placed by hand (publish()).
+    constexpr bool DMA = TL::SWZ && CMP;
+    constexpr int NST = SM::NST;
+    static_assert(!DMA || (RPP == 16 && NTHREADS == 256), "the direct loads are laid out for 16 chunks per row and four waves");
 
-    extern __shared__ __attribute__((aligned(16))) char smem[];
-    float *sBias = (float *)(smem + SM::OFF_BIAS);
+    // (LDS is read and written by absolute address in the tile loop: an access through a pointer into `smem` makes the
+    // compiler wait for every direct load in flight first)
+    extern __shared__ __attribute__((aligned(256))) char smem[];
+    const uint32_t lds0 = lds_addr(smem);  // (a multiple of 256)
     uint32_t *sBits = (uint32_t *)(smem + SM::OFF_BITS);
 
     const FwdParams &f = p.f;
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, r = lane & 31, g = lane >> 5;
+    const int tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = tid & 63, r = lane & 31, g = lane >> 5;
     const int G = f.H / f.Hk;
     const int n_mb = (f.Lq + Q_BM - 1) / Q_BM;
     int lid = blockIdx.x;  // index among the dQ workgroups
@@ -923,7 +937,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
     auto next_active = [&](int j) -> int {  // wave-uniform: keeps tile bases and loop conditions scalar
         if (CMP) return j < n_end ? j : n_end;
         while (j < n_end) {
-            const uint32_t w = __builtin_amdgcn_readfirstlane(sBits[j >> 5]) >> (j & 31);
+            const uint32_t w = __builtin_amdgcn_readfirstlane(lds_ld32(lds0 + SM::OFF_BITS + 4 * (j >> 5))) >> (j & 31);
             if (w) {
                 j += __builtin_ctz(w);
                 return j < n_end ? j : n_end;
@@ -964,8 +978,11 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
 
     // ---- staging: rows beyond Lk are clamped (their fused bias is -inf), head-dim chunks beyond d re-read chunk 0
     const int kc = tid % CH, kr0 = tid / CH;
-    const int kcol = (kc * 8 < f.d) ? kc * 8 : 0;
-    u32x4_t kreg[K_IT], vreg[K_IT];
+    // (DMA: the lane fills chunk POSITION kc of its row, which holds chunk kc ^ swz(row) of the global row; rows 16
+    // apart have the same swizzle)
+    const int kc_g = DMA ? (kc ^ (int)TL::swz(kr0)) : kc;
+    const int kcol = (kc_g * 8 < f.d) ? kc_g * 8 : 0;
+    u32x4_t kreg[DMA ? 1 : K_IT], vreg[DMA ? 1 : K_IT];
     // Byte offsets of this thread's loads inside a tile are loop invariants -- one set for full tiles, one for the
     // (only) partial tile at the end of the keys -- so a load is one instruction with a scalar tile base, and the
     // loads of the next tile can be issued one by one between the MFMAs of the current one.  The bias / mask of the
@@ -992,11 +1009,21 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
     uint32_t braw = 0, mraw = 0;
     const uint8_t *mrow_ld = mrow ? mrow : (const uint8_t *)kbase;
     const uint16_t *brow_ld = brow ? brow : kbase;
-    auto set_tile = [&](int j) {
+    gptr_t tb_b = nullptr;  // DMA: the fused bias row, and this lane's offset in it for the tile being fetched
+    uint32_t boff = 0;
+    // bases of the tile whose K / V are fetched next; the bias / mask column of tile jb
+    auto set_tile = [&](int j, int jb) {
         tb_k = uniform_ptr(kbase + (int64_t)j * BN * f.k_r);
         tb_v = uniform_ptr(vbase + (int64_t)j * BN * f.v_r);
         t_last = j == j_last;
-        if (tid < BN) {
+        if constexpr (DMA) {
+            // columns beyond the end of the kept keys read the last one (masked where the column is used)
+            tb_b = uniform_ptr(fbrow);
+            const int col = j * BN + (lane & 31);
+            boff = (uint32_t)(col < Lk ? col : Lk - 1) * 4u;
+        }
+        if (!DMA && tid < BN) {
+            j = jb;
             const int col = j * BN + tid;
             bcol_ok = col < Lk;
             const int cc = bcol_ok ? col : 0;
@@ -1008,55 +1035,96 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
             }
         }
     };
-    auto load_item = [&](int n) {  // 0 .. K_IT-1: K rows, K_IT .. 2*K_IT-1: V rows
-        if (n < K_IT) kreg[n] = *(const __attribute__((address_space(1))) u32x4_t *)(tb_k + (t_last ? koff_l[n] : koff[n]));
-        else vreg[n - K_IT] = *(const __attribute__((address_space(1))) u32x4_t *)(tb_v + (t_last ? voff_l[n - K_IT] : voff[n - K_IT]));
+    // one direct load: 64 lanes x 16 (or 4) bytes from `base` (wave-uniform) + this lane's offset to LDS address `dst`
+    // (wave-uniform) onwards, lane after lane
+    auto dma16 = [](gptr_t base, uint32_t off, uint32_t dst) {
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(off), "s"(base), "s"(dst));
     };
-    auto load_tile = [&](int j) {
-        set_tile(j);
-#pragma unroll
-        for (int n = 0; n < 2 * K_IT; n++) load_item(n);
+    auto dma4 = [](gptr_t base, uint32_t off, uint32_t dst) {
+        asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dword %0, %1" : : "v"(off), "s"(base), "s"(dst));
     };
-    auto store_tile = [&](int buf, int slot) {
-        char *sK = smem + SM::OFF_K + buf * SM::K_BYTES;
-        char *sV = smem + SM::OFF_V + buf * SM::K_BYTES;
-#pragma unroll
-        for (int it = 0; it < K_IT; it++) {
-            const uint32_t off = TL::chunk(kr0 + it * RPP, kc);
-            *(u32x4_t *)(sK + off) = kreg[it];
-            *(u32x4_t *)(sV + off) = vreg[it];
+    constexpr int N_DMA = 2 * K_IT + 1;  // direct loads of a wave per tile
+    int dma_stage = 0;                   // stage the tile being fetched goes to (DMA)
+    auto load_item = [&](int n) {  // 0 .. K_IT-1: K rows, K_IT .. 2*K_IT-1: V rows, 2*K_IT: the bias column (DMA)
+        if constexpr (DMA) {
+            // this wave's piece `it` of a tile: LDS bytes [1024 (wave + 4 it), + 1024), rows 4 wave + 16 it .. + 3
+            const uint32_t st0 = lds0 + (uint32_t)(dma_stage * SM::K_BYTES);
+            if (n < K_IT) dma16(tb_k, t_last ? koff_l[n] : koff[n], __builtin_amdgcn_readfirstlane(st0 + SM::OFF_K + (wave + 4 * n) * 1024));
+            else if (n < 2 * K_IT)
+                dma16(tb_v, t_last ? voff_l[n - K_IT] : voff[n - K_IT], __builtin_amdgcn_readfirstlane(st0 + SM::OFF_V + (wave + 4 * (n - K_IT)) * 1024));
+            else  // (every wave fetches the same 256 bytes -- lanes 32-63 repeat lanes 0-31 -- : no branch between the MFMAs)
+                dma4(tb_b, boff, __builtin_amdgcn_readfirstlane(lds0 + SM::OFF_BIAS + dma_stage * 256));
+        } else {
+            if (n < K_IT) kreg[n] = *(const __attribute__((address_space(1))) u32x4_t *)(tb_k + (t_last ? koff_l[n] : koff[n]));
+            else if (n < 2 * K_IT) vreg[n - K_IT] = *(const __attribute__((address_space(1))) u32x4_t *)(tb_v + (t_last ? voff_l[n - K_IT] : voff[n - K_IT]));
         }
-        if (tid < BN) {
+    };
+    auto load_tile = [&](int j, int jb) {
+        set_tile(j, jb);
+#pragma unroll
+        for (int n = 0; n < (DMA ? N_DMA : 2 * K_IT); n++) load_item(n);
+    };
+    // registers -> LDS stage `buf` (not with DMA), and the fused bias column of that tile into slot `slot`
+    auto store_tile = [&](int buf, int slot) {
+        if constexpr (!DMA) {
+            char *sK = smem + SM::OFF_K + buf * SM::K_BYTES;
+            char *sV = smem + SM::OFF_V + buf * SM::K_BYTES;
+#pragma unroll
+            for (int it = 0; it < K_IT; it++) {
+                const uint32_t off = TL::chunk(kr0 + it * RPP, kc);
+                *(u32x4_t *)(sK + off) = kreg[it];
+                *(u32x4_t *)(sV + off) = vreg[it];
+            }
+        }
+        if (!DMA && tid < BN) {
             float v = -INFINITY;
             if (CMP) {
                 if (bcol_ok) v = __uint_as_float(braw);
             } else if (bcol_ok && (!mrow || mraw)) {
                 v = brow ? E::lo(braw) * kLog2e : 0.f;
             }
-            sBias[slot * BN + tid] = v;
+            lds_st32(lds0 + SM::OFF_BIAS + 4 * (slot * BN + tid), __float_as_uint(v));
         }
     };
 
     const int a_row = pi_row(r);
-    const uint32_t a_off = TL::frag_base(a_row, g);
+    const uint32_t a_off = lds0 + SM::OFF_K + TL::frag_base(a_row, g);  // (absolute, stage 0 of K)
     const int tj = lane & 15, te = tj >> 2, tc = tj & 3;
     const int tcp = (tc == 1) ? 2 : (tc == 2 ? 1 : tc);
     const int tdh = (lane >> 4) & 1;
-    const uint32_t tr_off = TL::tr_base(g, te, tdh, tcp);
+    const uint32_t tr_off = lds0 + SM::OFF_K + TL::tr_base(g, te, tdh, tcp);
 
-    int jc = next_active(0);
+    // A wave waits for its own pieces of the next tile, then the barrier publishes everybody's (DMA: by hand -- the
+    // N_DMA loads of the tile after that, issued later, stay in flight; vmcnt in bits 3:0, lgkmcnt 0, expcnt not
+    // waited for)
+    auto publish = [&]() {
+        if constexpr (DMA) {
+            __builtin_amdgcn_s_waitcnt(0x0070 | N_DMA);
+            __builtin_amdgcn_s_barrier();
+        } else {
+            __syncthreads();
+        }
+    };
+    int jc = next_active(0), jn = n_end, jnn = n_end;
     if (jc < n_end) {
-        load_tile(jc);
+        jn = next_active(jc + 1);
+        load_tile(jc, jc);
         store_tile(0, 0);
-        __syncthreads();
+        if constexpr (DMA) {  // the second tile is on its way before the first is looked at
+            jnn = next_active(jn + 1);
+            dma_stage = 1;
+            load_tile(jn < n_end ? jn : jc, jc);
+        }
+        publish();
     }
     int i = 0;
     while (jc < n_end) {
-        const int jn = next_active(jc + 1);
+        if constexpr (!DMA) jn = next_active(jc + 1);
         const int n0 = jc * BN;
-        const char *sK = smem + SM::OFF_K + (i & 1) * SM::K_BYTES;
-        const char *sV = smem + SM::OFF_V + (i & 1) * SM::K_BYTES;
-        const float *bs = sBias + (i % 3) * BN + 8 * g;
+        const int st = DMA ? i % 3 : (i & 1);
+        const uint32_t st_off = (uint32_t)(st * SM::K_BYTES);  // (a multiple of 256: the swizzles stay XORs)
+        const uint32_t a_cur = a_off + st_off, tr_cur = tr_off + st_off;
+        const uint32_t bs = lds0 + SM::OFF_BIAS + (DMA ? (i % 3) * 256 + 32 * g : 4 * ((i % 3) * BN + 8 * g));
 
         // ---- S^T = K Q^T, dP^T = V dO^T, dS^T = P^T * (dP^T - D), dQ^T += K^T dS^T.  A wave issues in program
         // order, so the vector work has to sit BETWEEN the MFMAs to run under them; the tile is written slot by slot --
@@ -1071,8 +1139,8 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
         for (int mb = 0; mb < MB; mb++)
 #pragma unroll
             for (int blk = 0; blk < 2; blk++) {
-                const f32x4_t b0 = *(const f32x4_t *)(bs + 32 * mb + 16 * blk);
-                const f32x4_t b1 = *(const f32x4_t *)(bs + 32 * mb + 16 * blk + 4);
+                const f32x4_t b0 = __builtin_bit_cast(f32x4_t, lds_ld128(bs + 4 * (32 * mb + 16 * blk)));
+                const f32x4_t b1 = __builtin_bit_cast(f32x4_t, lds_ld128(bs + 4 * (32 * mb + 16 * blk + 4)));
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     s[mb][8 * blk + e] = b0[e] - lse2;
@@ -1080,18 +1148,28 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
                     dp[mb][8 * blk + e] = -dd;
                     dp[mb][8 * blk + 4 + e] = -dd;
                 }
+                if (DMA && jc == j_last) {  // (the bias column came as it is in memory: columns beyond the kept keys)
+                    const int lim = Lk - n0 - 32 * mb - 16 * blk - 8 * g;  // local columns e < lim exist
+#pragma unroll
+                    for (int e = 0; e < 8; e++) s[mb][8 * blk + e] = e < lim ? s[mb][8 * blk + e] : -INFINITY;
+                }
             }
         // the next tile's bases and side inputs (after the last tile the current one is fetched again and dropped); behind
         // the accumulator set-up: the load of the bias / mask column must not be waited for with the LDS reads above
         __builtin_amdgcn_sched_barrier(0);
-        set_tile(jn < n_end ? jn : jc);
+        if constexpr (DMA) {  // K / V of the tile after the next one into the stage the last tile has left
+            dma_stage = (i + 2) % 3;
+            set_tile(jnn < n_end ? jnn : jc, jn < n_end ? jn : jc);
+        } else {
+            set_tile(jn < n_end ? jn : jc, jn < n_end ? jn : jc);
+        }
         float pv[16 * MB];
         {
             constexpr int NH = MB * KS, NF = 2 * NH, FR = 3;
             u32x4_t a[NF];
             auto frag = [&](int fi) {  // S slots first (K tile), then dP slots (V tile); k-step major, row block minor
                 const int which = fi / NH, mb = (fi % NH) % MB, ks = (fi % NH) / MB;
-                return *(const u32x4_t *)((which ? sV : sK) + TL::frag_at(a_off, ks) + 32 * mb * TL::ROW_BYTES);
+                return lds_ld128(TL::frag_at(a_cur, ks) + (uint32_t)(which * (SM::OFF_V - SM::OFF_K) + 32 * mb * TL::ROW_BYTES));
             };
 #pragma unroll
             for (int fi = 0; fi < FR; fi++) a[fi] = frag(fi);
@@ -1101,8 +1179,9 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
                 const int which = fi / NH, mb = (fi % NH) % MB, ks = (fi % NH) / MB;
                 if (which) dp[mb] = E::mfma(a[fi], dof[ks], dp[mb]);
                 else s[mb] = E::mfma(a[fi], qf[ks], s[mb]);
+                constexpr int NLD = DMA ? N_DMA : 2 * K_IT;
 #pragma unroll
-                for (int n = fi * 2 * K_IT / NF; n < (fi + 1) * 2 * K_IT / NF; n++) load_item(n);
+                for (int n = fi * NLD / NF; n < (fi + 1) * NLD / NF; n++) load_item(n);
                 if (which) {
 #pragma unroll
                     for (int e = 0; e < 16 * MB; e++)
@@ -1138,8 +1217,8 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
             u32x2_t tl[NG], th[NG];
             auto tr_read = [&](int gi) {
                 const int kb = gi / DB, db = gi % DB;
-                tl[gi] = lds_read_tr16(sK, TL::tr_at(tr_off, kb, db, 0));
-                th[gi] = lds_read_tr16(sK, TL::tr_at(tr_off, kb, db, 1));
+                tl[gi] = lds_ld_tr16(TL::tr_at(tr_cur, kb, db, 0));
+                th[gi] = lds_ld_tr16(TL::tr_at(tr_cur, kb, db, 1));
             };
 #pragma unroll
             for (int gi = 0; gi < FR2; gi++) tr_read(gi);
@@ -1162,11 +1241,18 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
             }
         }
         if (jn < n_end) store_tile((i + 1) & 1, (i + 1) % 3);
-        __syncthreads();
+        publish();
         i++;
         jc = jn;
+        if constexpr (DMA) {
+            jn = jnn;
+            jnn = next_active(jn + 1);
+        }
     }
 
+    // (direct loads still in flight -- tiles fetched past the last one -- must not land in LDS that belongs to the next
+    // workgroup by then)
+    if constexpr (DMA) __builtin_amdgcn_s_waitcnt(0x0070);
     if (qrow < LqS) {
         uint16_t *dqp = (uint16_t *)p.dq + b * p.dq_b + (sq.q0 + qrow) * p.dq_r + h * p.dq_h;
 #pragma unroll

@@ -144,6 +144,8 @@ __device__ __forceinline__ u32x2_t lds_ld_tr16(uint32_t addr) {
     s16x4_t v = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4_t *)(uintptr_t)addr);
     return __builtin_bit_cast(u32x2_t, v);
 }
+__device__ __forceinline__ uint32_t lds_ld32(uint32_t addr) { return *(const __attribute__((address_space(3))) uint32_t *)(uintptr_t)addr; }
+__device__ __forceinline__ void lds_st32(uint32_t addr, uint32_t v) { *(__attribute__((address_space(3))) uint32_t *)(uintptr_t)addr = v; }
 
 // Row-major LDS tile of 16-bit elements ([row][head dim]) that is read two ways: as MFMA fragments (ds_read_b128:
 // lane (r, g) takes the 16 bytes of chunk 2*ks + g of row pi_row(r)) and through transposing reads (lds_read_tr16:
