@@ -350,18 +350,34 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dkdv_colmask_k
             dma_q += q_step; dma_do += do_step; dma_stat -= BM * 4;
         }
     };
+    // The direct loads are written in assembly and waited for by hand (publish() below): issued through the
+    // compiler's builtin, every LDS read behind one of them waited for all LDS operations in flight -- the compiler
+    // cannot tell which stage a direct load fills -- and the fragment reads could not run ahead of their MFMAs.
     auto dma_piece = [&](int n) {
+        const uint32_t dst = lds_addr(dma_dst);
         if (n < Q_IT) {
-            __builtin_amdgcn_global_load_lds((gvoid_t *)(ld_qbase + (ld_partial ? qoff_l[n] : qoff[n])),
-                                             (lds_void_t *)(dma_dst + (2 * wave + n) * 1024), 16, 0, 0);
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                         : : "v"(ld_partial ? qoff_l[n] : qoff[n]), "s"(ld_qbase), "s"(__builtin_amdgcn_readfirstlane(dst + (2 * wave + n) * 1024)));
         } else if (n < 2 * Q_IT) {
-            __builtin_amdgcn_global_load_lds((gvoid_t *)(ld_dobase + (ld_partial ? dooff_l[n - Q_IT] : dooff[n - Q_IT])),
-                                             (lds_void_t *)(dma_dst + SM::Q_BYTES + (2 * wave + n - Q_IT) * 1024), 16, 0, 0);
+            asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1"
+                         : : "v"(ld_partial ? dooff_l[n - Q_IT] : dooff[n - Q_IT]), "s"(ld_dobase),
+                             "s"(__builtin_amdgcn_readfirstlane(dst + SM::Q_BYTES + (2 * wave + n - Q_IT) * 1024)));
         } else {
             // (every wave fetches the same 256 bytes: cheaper than a branch in the middle of the MFMAs.)  In the last,
             // partial block the rows beyond the end of the queries read the last row's numbers (masked where used).
             const int over = ld_partial ? (lane & 31) - row_last : 0;
-            __builtin_amdgcn_global_load_lds((gvoid_t *)(dma_stat - (over > 0 ? over * 4 : 0)), (lds_void_t *)(dma_dst + 2 * SM::Q_BYTES), 4, 0, 0);
+            gbytes_t sp = dma_stat - (over > 0 ? over * 4 : 0);
+            asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dword %0, off"
+                         : : "v"(sp), "s"(__builtin_amdgcn_readfirstlane(dst + 2 * SM::Q_BYTES)));
+        }
+    };
+    // end of a step: a wave waits for its own direct loads (and LDS stores), then the barrier publishes everybody's
+    auto publish = [&]() {
+        if constexpr (DMA) {
+            __builtin_amdgcn_s_waitcnt(0x0070);  // vmcnt(0) lgkmcnt(0); expcnt not waited for
+            __builtin_amdgcn_s_barrier();
+        } else {
+            __syncthreads();
         }
     };
 
@@ -395,7 +411,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dkdv_colmask_k
             cconst = column_const_value();
             load_step(n_steps > 1 ? 1 : 0, true);
         }
-        __syncthreads();
+        publish();
     }
 
     int cur_gi = g_lo, cur_mi = s_hi - 1;  // (DMA: head and query block of the current step, walked like the fetch)
@@ -589,7 +605,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dkdv_colmask_k
         } else {
             cconst = cconst_next;
         }
-        __syncthreads();  // (also waits for this wave's direct loads: the next step's stage is complete behind it)
+        publish();
     };
     for (int step = 0; step < n_steps; step += 2) {
         one_step(std::integral_constant<int, 0>(), step);
