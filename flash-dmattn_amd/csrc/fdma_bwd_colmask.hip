@@ -440,23 +440,35 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dkdv_colmask_k
 #pragma unroll
             for (int i = 0; i < 16; i++) { s[mb][i] = cconst; dp[mb][i] = 0.f; }
         {
-            constexpr int NF = 2 * MB * KS, FR = D > 64 ? 4 : 8;  // fragment f: (ks, mb, which) with which = 0: Q, 1: dO
+            constexpr int NF = 2 * MB * KS, FR = D > 64 ? 3 : 8;  // fragment f: (ks, mb, which) with which = 0: Q, 1: dO
             u32x4_t a[NF];
             auto frag = [&](int fi) {
                 const int which = fi & 1, mb = (fi >> 1) % MB, ks = (fi >> 1) / MB;
                 return lds_ld128(TL::frag_at(a_off, ks) + (uint32_t)(buf * SM::STAGE + which * SM::Q_BYTES + 32 * mb * TL::ROW_BYTES));
             };
+            // (V parked in LDS: its fragment of a k-step is read one k-step ahead as well -- read where it is used, every
+            // dP MFMA waited for its own read; a scheduling barrier per MFMA keeps the reads ahead)
+            constexpr int FRV = 1;
+            u32x4_t vl[V_LDS ? KS : 1];
+            if constexpr (V_LDS) {
+#pragma unroll
+                for (int ks = 0; ks < FRV; ks++) vl[ks] = lds_ld128(TL::frag_at(v_base, ks));
+            }
 #pragma unroll
             for (int fi = 0; fi < FR; fi++) a[fi] = frag(fi);
 #pragma unroll
             for (int fi = 0; fi < NF; fi++) {
                 if (fi + FR < NF) a[fi + FR] = frag(fi + FR);
                 const int which = fi & 1, mb = (fi >> 1) % MB, ks = (fi >> 1) / MB;
-                if (which) dp[mb] = E::mfma(a[fi], V_LDS ? lds_ld128(TL::frag_at(v_base, ks)) : vf[V_LDS ? 0 : ks], dp[mb]);
+                if constexpr (V_LDS) {
+                    if (which && mb == 0 && ks + FRV < KS) vl[ks + FRV] = lds_ld128(TL::frag_at(v_base, ks + FRV));
+                }
+                if (which) dp[mb] = E::mfma(a[fi], V_LDS ? vl[V_LDS ? ks : 0] : vf[V_LDS ? 0 : ks], dp[mb]);
                 else s[mb] = E::mfma(a[fi], kf[ks], s[mb]);
                 if constexpr (DMA) {
                     if (fi % 3 == 1 && fi / 3 <= 2 * Q_IT) dma_piece(fi / 3);
                 }
+                __builtin_amdgcn_sched_barrier(0);
             }
         }
         // the registers (step i+1) go to the other LDS stage, whose readers finished before the last barrier
