@@ -506,6 +506,24 @@ def test_compacted_backward_split_plans_vs_eager_fp32(name):
     assert torch.equal(dk, dk2) and torch.equal(dv, dv2) and torch.equal(db, db2) and torch.equal(dq, dq2)
 
 
+# Numbers of kept keys around the 32-key tiles of the compacted dQ kernel at head dim 128 (one, two, three, four tiles,
+# full and partial last tiles): its tiles are fetched two ahead through three LDS stages, and the first iterations
+# and the tiles fetched past the last one are what a short key list exercises.
+@pytest.mark.parametrize("W", [1, 2, 31, 32, 33, 63, 64, 65, 96, 97, 129])
+@pytest.mark.parametrize("causal", [False, True])
+def test_compacted_backward_with_few_kept_keys_d128_vs_eager_fp32(W, causal):
+    set_compact("2")
+    B, Lq, Lk, H, Hk, D = 2, 200, 300, 4, 2, 128
+    q, k, v, mask, bias = make_inputs(B, Lq, Lk, H, Hk, D, (B, Hk, 1, Lk), (B, Hk, 1, Lk), W, seed=100 + W)
+    assert int(mask[0, 0, 0].sum()) == W
+    out, lse, (dq, dk, dv, db) = _run_fwd_bwd(q, k, v, mask, bias, causal)
+    qd, kd, vd, md, bd = _to_dev(q, k, v, mask, bias)
+    ro, rdq, rdk, rdv, rdb = eager.attention_forward_backward(qd, kd, vd, md, bd, None, causal)
+    assert_out_close(out, ro)
+    for g, r, n in ((dq, rdq, "dq"), (dk, rdk, "dk"), (dv, rdv, "dv"), (db, rdb, "dbias")):
+        assert_grad_close(g, r, n)
+
+
 def test_decode_long_splits_and_fp16():
     """One workgroup per (batch entry, kv head) walks 40 000 keys: three mask fetches of 16 384 keys each.  fp16."""
     B, Lk, H, Hk, D, W = 32, 40000, 16, 8, 64, 700
