@@ -353,6 +353,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dkdv_colmask_k
     // The direct loads are written in assembly and waited for by hand (publish() below): issued through the
     // compiler's builtin, every LDS read behind one of them waited for all LDS operations in flight -- the compiler
     // cannot tell which stage a direct load fills -- and the fragment reads could not run ahead of their MFMAs.
+    // (m0 carries the LDS address of a direct load; it is a reserved register that nothing else in this kernel uses.)
     auto dma_piece = [&](int n) {
         const uint32_t dst = lds_addr(dma_dst);
         if (n < Q_IT) {
@@ -1064,7 +1065,8 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
         }
     };
     // one direct load: 64 lanes x 16 (or 4) bytes from `base` (wave-uniform) + this lane's offset to LDS address `dst`
-    // (wave-uniform) onwards, lane after lane
+    // (wave-uniform) onwards, lane after lane.  (m0 carries the LDS address; it is a reserved register that nothing
+    // else in this kernel uses, and it is written immediately in front of every use.)
     auto dma16 = [](gptr_t base, uint32_t off, uint32_t dst) {
         asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" : : "v"(off), "s"(base), "s"(dst));
     };
