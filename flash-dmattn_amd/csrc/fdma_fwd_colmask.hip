@@ -485,6 +485,7 @@ __global__ void __launch_bounds__(64 * NW, (NW == 4 && D <= 128) ? 2 : 1) fwd_co
         // addition to the row sum in the next, a piece of the staging) -- with a scheduling barrier after every slot.
         // The probabilities are relative to the reference the MFMAs have already subtracted; the row sum adds the
         // fp32 values, as the reference does (src/softmax.h: the sum is taken before the conversion to 16 bits).
+        if (DO_K) set_tile_k(j_next);  // base of the tile whose pieces are requested between the MFMAs below
         u32x4_t a[NF];
 #pragma unroll
         for (int f = 0; f < FR; f++) a[f] = *frag_ptr(f, kbuf, kh, vbuf, vh);
@@ -529,10 +530,14 @@ __global__ void __launch_bounds__(64 * NW, (NW == 4 && D <= 128) ? 2 : 1) fwd_co
                     }
             }
             if (DO_K) {
+                // (a register goes back to fetching -- the same piece of K(j_next) -- as soon as it is stored: a whole
+                // tile then lies between every load and its store; all four loads behind the last MFMA had half a tile)
 #pragma unroll
                 for (int it = 0; it < K_IT; it++)
-                    if (f == 1 + it * ((NF - 1) / K_IT))
+                    if (f == 1 + it * ((NF - 1) / K_IT)) {
                         *(u32x4_t *)(sK_w + ((kr0 + it * K_RPP) * SM::SK + kc * 8) * 2) = sreg[it];
+                        sreg[it] = *(const __attribute__((address_space(1))) u32x4_t *)(tb_k + (last_k ? soff_l[it] : soff[it]));
+                    }
             }
             __builtin_amdgcn_sched_barrier(0);
         }
@@ -551,9 +556,6 @@ __global__ void __launch_bounds__(64 * NW, (NW == 4 && D <= 128) ? 2 : 1) fwd_co
                 load_regs(true);
             }
             set_tile_x(jx_next);
-        } else if (DO_K) {  // the loads of K(j_next)
-            set_tile_k(j_next);
-            load_regs(false);
         }
         if (__any(!(psum <= 16384.f))) *sFlag = 1u;
     };
