@@ -319,6 +319,26 @@ def run_mask_builder(steps, warmup, device):
     return res
 
 
+def run_kept_list_handoff(steps, warmup, device):
+    """cfg2 forward with a keep-mask that comes from the package's mask builder -- which hands the attention kernels the
+    kept columns as index lists with prefix counts, so that the compaction pre-pass has nothing to scan -- next to the
+    same mask as a plain bool tensor (not part of `value`)."""
+    from flash_sparse_attn import flash_sparse_attn_func
+    from flash_sparse_attn.utils import mask as M
+
+    c = CONFIGS["cfg2"]
+    q, k, v, _, bias = make_case(c, device)
+    lowest = torch.finfo(torch.bfloat16).min
+    with torch.no_grad():
+        m_lists = M.topk_mask(bias, None, c["W"], lowest)
+        m_plain = m_lists.clone()
+        has_lists = M.kept_keys_of(m_lists) is not None
+        ms_lists = time_gpu(lambda: flash_sparse_attn_func(q, k, v, m_lists, bias, c["scale"], c["causal"]), steps, warmup)
+        ms_plain = time_gpu(lambda: flash_sparse_attn_func(q, k, v, m_plain, bias, c["scale"], c["causal"]), steps, warmup)
+    return {"workload": "cfg2 forward, mask from topk_mask", "lists_handed_over": bool(has_lists),
+            "ms_fwd_with_lists": ms_lists, "ms_fwd_bool_mask_only": ms_plain}
+
+
 def run_bias_producer(steps, warmup, device):
     """The bias producer in front of the operator (not part of `value`): flash_sparse_attn.utils.bias.dynamic_mask_bias
     (one kernel forwards, two backwards) next to the tensor program of the reference's Doge caller
@@ -551,6 +571,7 @@ def main():
                                 for n in ("cfg1", "cfg3", "cfg4", "cfg5")]
         out["mask_builder"] = run_mask_builder(max(3, args.steps // 2), max(1, args.warmup // 2), device)
         out["bias_producer"] = run_bias_producer(max(3, args.steps // 2), max(1, args.warmup // 2), device)
+        out["kept_list_handoff"] = run_kept_list_handoff(args.steps, args.warmup, device)
         out["ragged_batch"] = run_ragged_batch(max(3, args.steps // 4), max(1, args.warmup // 2), device)
         out.update(run_sweeps(max(3, args.steps // 4), max(1, args.warmup // 2), device))
     if not args.no_cpu:
