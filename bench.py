@@ -339,6 +339,37 @@ def run_kept_list_handoff(steps, warmup, device):
             "ms_fwd_with_lists": ms_lists, "ms_fwd_bool_mask_only": ms_plain}
 
 
+def run_mask_bits_handoff(steps, warmup, device):
+    """cfg3 (a bias and a mask per query row) with a keep-mask that comes from the package's mask builder -- which also
+    hands the per-query attention kernels the mask packed to one bit per key -- next to the same mask as a plain bool
+    tensor (not part of `value`)."""
+    from flash_sparse_attn import flash_sparse_attn_func
+    from flash_sparse_attn.utils import mask as M
+
+    c = CONFIGS["cfg3"]
+    q, k, v, _, bias = make_case(c, device)
+    lowest = torch.finfo(torch.bfloat16).min
+    with torch.no_grad():
+        m_bits = M.topk_mask(bias, None, c["W"], lowest)
+        m_plain = m_bits.clone()
+    has_bits = M.mask_bits_of(m_bits) is not None
+    scale = c["scale"] if c["scale"] is not None else c["D"] ** -0.5
+    res = {"workload": "cfg3, mask from topk_mask", "bits_handed_over": bool(has_bits)}
+    for name, m in (("with_bits", m_bits), ("bool_mask_only", m_plain)):
+        with torch.no_grad():
+            res["ms_fwd_" + name] = time_gpu(lambda: flash_sparse_attn_func(q, k, v, m, bias, scale, c["causal"]), steps, warmup)
+        qg, kg, vg, bg = [t.detach().clone().requires_grad_(True) for t in (q, k, v, bias)]
+        dout = torch.ones_like(q)
+
+        def step():
+            for t in (qg, kg, vg, bg):
+                t.grad = None  # (no accumulation pass over the 1 GiB bias gradient inside the timed region)
+            flash_sparse_attn_func(qg, kg, vg, m, bg, scale, c["causal"]).backward(dout)
+
+        res["ms_fwd_bwd_" + name] = time_gpu(step, steps, warmup)
+    return res
+
+
 def run_bias_producer(steps, warmup, device):
     """The bias producer in front of the operator (not part of `value`): flash_sparse_attn.utils.bias.dynamic_mask_bias
     (one kernel forwards, two backwards) next to the tensor program of the reference's Doge caller
@@ -572,6 +603,7 @@ def main():
         out["mask_builder"] = run_mask_builder(max(3, args.steps // 2), max(1, args.warmup // 2), device)
         out["bias_producer"] = run_bias_producer(max(3, args.steps // 2), max(1, args.warmup // 2), device)
         out["kept_list_handoff"] = run_kept_list_handoff(args.steps, args.warmup, device)
+        out["mask_bits_handoff"] = run_mask_bits_handoff(max(3, args.steps // 2), max(1, args.warmup // 2), device)
         out["ragged_batch"] = run_ragged_batch(max(3, args.steps // 4), max(1, args.warmup // 2), device)
         out.update(run_sweeps(max(3, args.steps // 4), max(1, args.warmup // 2), device))
     if not args.no_cpu:

@@ -53,6 +53,18 @@ int validate_common(const fdma_fwd_args *a, bool backward) {
     if (a->head_dim <= 0 || a->head_dim % 8 != 0)
         return fail(FDMA_ERR_INVALID, backward ? "head_size should be a multiple of 8"
                                                : "query, key, value, and out_ must have a head_size that is a multiple of 8");
+    if (a->mask_bits.bits) {
+        if (!a->mask) return fail(FDMA_ERR_INVALID, "mask_bits without a mask");
+        // (broadcast exactly where the mask is: a zero stride of one and not of the other would describe two masks)
+        for (int i = 0; i < 3; i++)
+            if ((a->mask_bits.strides[i] == 0) != (a->mask_strides[i] == 0))
+                return fail(FDMA_ERR_INVALID, "mask_bits must be broadcast over the same dimensions as the mask");
+        if (a->seqlen_q > 1 && a->mask_bits.strides[2] != 0 && a->mask_bits.strides[2] < ((a->seqlen_k + 7) / 8 + 7) / 8 * 8)
+            return fail(FDMA_ERR_INVALID, "mask_bits rows must hold ceil(seqlen_k / 8) bytes rounded up to 8");
+        if ((reinterpret_cast<uintptr_t>(a->mask_bits.bits) | (uintptr_t)a->mask_bits.strides[0] | (uintptr_t)a->mask_bits.strides[1] |
+             (uintptr_t)a->mask_bits.strides[2]) & 7)
+            return fail(FDMA_ERR_INVALID, "mask_bits and its strides must be multiples of 8 bytes");
+    }
     if (a->kept.idx || a->kept.cnt || a->kept.count) {
         if (!(a->kept.idx && a->kept.cnt && a->kept.count))
             return fail(FDMA_ERR_INVALID, "kept: idx, cnt and count must be given together");
@@ -120,6 +132,11 @@ void fill_fwd_params(const fdma_fwd_args *a, fdma::FwdParams &p) {
     if (a->mask && a->kept.idx && a->kept.cnt && a->kept.count) {  // (validate_common has checked the row stride)
         p.kept_idx = a->kept.idx; p.kept_cnt = a->kept.cnt; p.kept_count = a->kept.count;
         p.kept_ld = a->kept.ld;
+    }
+    if (a->mask && a->mask_bits.bits) {
+        p.mbits = a->mask_bits.bits;
+        p.mb_b = a->mask_bits.strides[0]; p.mb_h = a->mask_bits.strides[1];
+        p.mb_r = a->seqlen_q == 1 ? 0 : a->mask_bits.strides[2];
     }
     p.lse_b = (int64_t)a->num_heads * a->seqlen_q;
     p.lse_h = a->seqlen_q;
@@ -491,6 +508,10 @@ int fdma_create_mask_validate(const fdma_mask_args *a) {
     if (!empty && (!a->bias || !a->mask_out)) return fail(FDMA_ERR_INVALID, "bias and mask_out must be device pointers");
     if (reinterpret_cast<uintptr_t>(a->bias) & 1) return fail(FDMA_ERR_INVALID, "bias must be 2-byte aligned");
     if (std::isnan(a->min_value)) return fail(FDMA_ERR_INVALID, "min_dtype must not be NaN");
+    if (a->bits && (a->bits_row_bytes % 8 != 0 || a->bits_row_bytes < ((a->seqlen_k + 7) / 8 + 7) / 8 * 8))
+        return fail(FDMA_ERR_INVALID, "bits_row_bytes must be a multiple of 8 and at least ceil(seqlen_k / 8) rounded up to 8");
+    if (a->bits && (reinterpret_cast<uintptr_t>(a->bits) & 7))
+        return fail(FDMA_ERR_INVALID, "bits must be 8-byte aligned");
     if (a->kept_idx || a->kept_cnt || a->kept_count) {
         if (!(a->kept_idx && a->kept_cnt && a->kept_count))
             return fail(FDMA_ERR_INVALID, "kept_idx, kept_cnt and kept_count must be given together");
@@ -545,6 +566,7 @@ int fdma_create_mask(const fdma_mask_args *a, void *hip_stream) {
     p.min_bits = to_bits16(a->min_value, a->dtype);
     p.kept_idx = a->kept_idx; p.kept_cnt = a->kept_cnt; p.kept_count = a->kept_count;
     p.kept_ld = a->kept_ld;
+    p.bits = a->bits; p.bits_row_bytes = a->bits_row_bytes;
     const hipError_t e = fdma::launch_make_mask(p, static_cast<hipStream_t>(hip_stream));
     if (e != hipSuccess) return fail(FDMA_ERR_LAUNCH, "mask launch failed: %s", hipGetErrorString(e));
     return FDMA_OK;

@@ -205,7 +205,11 @@ __global__ void __launch_bounds__(NTHREADS, (D <= 64 && !GSUM) ? 2 : 1) bwd_dkdv
             int qq = m0 + br0 + 16 * it;
             qq = qq < f.Lq ? qq : f.Lq - 1;
             braw[it] = *(const u32x4_t *)(bias_ld + boff + (has_bias ? (int64_t)qq * f.bi_r : 0));
-            mraw[it] = *(const u32x2_t *)(mask_ld + moff + (f.mask ? (int64_t)qq * f.m_r : 0));
+            // (one 8-byte load either way, from an address chosen without a branch: mask bytes of the chunk, or --
+            // a mask packed to bits -- the aligned piece of the bit row that holds the chunk's byte)
+            const uint8_t *src = (f.mask && f.mbits) ? f.mbits + b * f.mb_b + hm * f.mb_h + (int64_t)qq * f.mb_r + ((kk_c >> 3) & ~7)
+                                                     : mask_ld + moff + (f.mask ? (int64_t)qq * f.m_r : 0);
+            mraw[it] = *(const u32x2_t *)src;
         }
     };
     auto store_step = [&](int buf) {
@@ -226,7 +230,8 @@ __global__ void __launch_bounds__(NTHREADS, (D <= 64 && !GSUM) ? 2 : 1) bwd_dkdv
 #pragma unroll
         for (int it = 0; it < FB_IT; it++) {
             u32x4_t bv = has_bias ? braw[it] : u32x4_t{0, 0, 0, 0};
-            u32x2_t mv = f.mask ? mraw[it] : u32x2_t{0x01010101u, 0x01010101u};
+            u32x2_t mv = f.mask ? (f.mbits ? mask_bits_to_bytes(mask_bits_byte(mraw[it], kk < f.Lk ? kk : 0)) : mraw[it])
+                                : u32x2_t{0x01010101u, 0x01010101u};
             uint64_t keepm = kk < f.Lk ? ~0ull : 0ull;
             if (kk + 8 > f.Lk && kk < f.Lk) keepm = (1ull << (8 * (f.Lk - kk))) - 1ull;  // chunk straddles the end of the keys
             mv[0] &= (uint32_t)keepm;

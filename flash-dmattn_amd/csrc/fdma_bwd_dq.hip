@@ -117,6 +117,8 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) bwd_dq_
     u32x4_t kreg[K_IT], vreg[K_IT], breg[F_IT];
     u32x2_t mreg[F_IT], mnext[F_IT];
 
+    // (a mask that comes packed to bits: one byte per 8-key chunk instead of eight, expanded where it is looked at)
+    const uint8_t *mbits = (mbase && f.mbits) ? f.mbits + b * f.mb_b + hm * f.mb_h : nullptr;
     auto load_mask = [&](int j, u32x2_t (&dst)[F_IT]) {
         if (!mbase) return;
         int kk = j * BN + 8 * fc;
@@ -125,7 +127,10 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) bwd_dq_
         for (int it = 0; it < F_IT; it++) {
             int row = m0 + fr0 + F_RPP * it;
             row = row < f.Lq ? row : f.Lq - 1;
-            dst[it] = *(const u32x2_t *)(mbase + (int64_t)row * f.m_r + kk);
+            // (one 8-byte load either way, from an address chosen without a branch: mask bytes of the chunk, or the
+            // aligned piece of the bit row that holds the chunk's byte)
+            const uint8_t *src = mbits ? mbits + (int64_t)row * f.mb_r + ((kk >> 3) & ~7) : mbase + (int64_t)row * f.m_r + kk;
+            dst[it] = *(const u32x2_t *)src;
         }
     };
     auto finish_mask = [&](int j, u32x2_t (&dst)[F_IT]) -> bool {
@@ -134,7 +139,7 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) bwd_dq_
 #pragma unroll
         for (int it = 0; it < F_IT; it++) {
             const int row = m0 + fr0 + F_RPP * it;
-            u32x2_t mv = mbase ? dst[it] : u32x2_t{0x01010101u, 0x01010101u};
+            u32x2_t mv = mbase ? (mbits ? mask_bits_to_bytes(mask_bits_byte(dst[it], kk)) : dst[it]) : u32x2_t{0x01010101u, 0x01010101u};
             const bool ok = row < f.Lq && kk < f.Lk && !(CAUSAL && kk > row + shift);
             uint64_t keepm = ok ? ~0ull : 0ull;
             if (kk + 8 > f.Lk && kk < f.Lk) keepm = (1ull << (8 * (f.Lk - kk))) - 1ull;

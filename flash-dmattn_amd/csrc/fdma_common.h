@@ -147,6 +147,22 @@ __device__ __forceinline__ u32x2_t lds_ld_tr16(uint32_t addr) {
 __device__ __forceinline__ uint32_t lds_ld32(uint32_t addr) { return *(const __attribute__((address_space(3))) uint32_t *)(uintptr_t)addr; }
 __device__ __forceinline__ void lds_st32(uint32_t addr, uint32_t v) { *(__attribute__((address_space(3))) uint32_t *)(uintptr_t)addr = v; }
 
+// Eight mask bits (key j in bit j, lowest first) to the eight 0 / 1 bytes of the bool mask's form.  (Bits i of a
+// nibble times 0x00204081 land on positions 8 i, among others that the mask removes; no two products share a bit.)
+__device__ __forceinline__ u32x2_t mask_bits_to_bytes(uint32_t b) {
+    u32x2_t r;
+    r[0] = ((b & 0xfu) * 0x00204081u) & 0x01010101u;
+    r[1] = (((b >> 4) & 0xfu) * 0x00204081u) & 0x01010101u;
+    return r;
+}
+
+// The byte with the bits of keys kk .. kk+7 (kk a multiple of 8) out of the aligned 8-byte piece of a bit row that
+// holds it -- the kernels fetch bits in the same 8-byte loads as mask bytes, so that one instruction serves both forms.
+__device__ __forceinline__ uint32_t mask_bits_byte(u32x2_t piece, int kk) {
+    const int sh = ((kk >> 3) & 7) * 8;
+    return ((sh & 32) ? piece[1] >> (sh & 31) : piece[0] >> sh) & 0xffu;
+}
+
 // Row-major LDS tile of 16-bit elements ([row][head dim]) that is read two ways: as MFMA fragments (ds_read_b128:
 // lane (r, g) takes the 16 bytes of chunk 2*ks + g of row pi_row(r)) and through transposing reads (lds_read_tr16:
 // 16 lanes take four 8-byte pieces of each of four consecutive rows), and written row by row (16 lanes per row).

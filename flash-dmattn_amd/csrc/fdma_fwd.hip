@@ -135,6 +135,8 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) fwd_ker
     // words are ANDed with a validity pattern when they are consumed, rows of K / V beyond Lk and head-dim chunks
     // beyond d are finite duplicates that meet a -inf score or a zero Q fragment.
     const int kcol = k_dvalid ? kc * 8 : 0, vcol = v_dvalid ? vc * 8 : 0;
+    // (a mask that comes packed to bits: one byte per 8-key chunk instead of eight, expanded where it is looked at)
+    const uint8_t *mbits = (mbase && p.mbits) ? p.mbits + b * p.mb_b + hm * p.mb_h : nullptr;
     auto load_mask = [&](int j, u32x2_t (&dst)[F_IT]) {
         if (!mbase) return;
         int kk = j * BN + 8 * fc;
@@ -143,7 +145,10 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) fwd_ker
         for (int it = 0; it < F_IT; it++) {
             int row = m0 + fr0 + F_RPP * it;
             row = row < p.Lq ? row : p.Lq - 1;
-            dst[it] = *(const u32x2_t *)(mbase + (int64_t)row * p.m_r + kk);
+            // (one 8-byte load either way, from an address chosen without a branch: mask bytes of the chunk, or the
+            // aligned piece of the bit row that holds the chunk's byte)
+            const uint8_t *src = mbits ? mbits + (int64_t)row * p.mb_r + ((kk >> 3) & ~7) : mbase + (int64_t)row * p.m_r + kk;
+            dst[it] = *(const u32x2_t *)src;
         }
     };
     // validity of the chunks (rows < Lq, keys < Lk, not entirely above the causal diagonal) applied to the loaded
@@ -154,7 +159,7 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) fwd_ker
 #pragma unroll
         for (int it = 0; it < F_IT; it++) {
             const int row = m0 + fr0 + F_RPP * it;
-            u32x2_t mv = mbase ? dst[it] : u32x2_t{0x01010101u, 0x01010101u};
+            u32x2_t mv = mbase ? (mbits ? mask_bits_to_bytes(mask_bits_byte(dst[it], kk)) : dst[it]) : u32x2_t{0x01010101u, 0x01010101u};
             const bool ok = row < p.Lq && kk < p.Lk && !(CAUSAL && kk > row + shift);
             uint64_t keepm = ok ? ~0ull : 0ull;
             if (kk + 8 > p.Lk && kk < p.Lk) keepm = (1ull << (8 * (p.Lk - kk))) - 1ull;  // chunk straddles the end of the keys

@@ -255,6 +255,34 @@ __global__ void __launch_bounds__(NT) make_mask_kernel(const MaskParams p) {
         scan_mask_row<NT>(orow, Lk, p.kept_idx + (size_t)row * p.kept_ld, p.kept_cnt + (size_t)row * p.kept_ld,
                           p.kept_count + row, (int *)wave_cnt, false);
     }
+
+    // ---- optional third output: the row packed to one bit per key (key j in bit j % 8 of byte j / 8), the form in
+    // which the per-query attention kernels take a mask at an eighth of its traffic.  A thread packs 32 keys into
+    // one word; the row it reads was written by this workgroup a moment ago.
+    if (p.bits) {
+        __syncthreads();  // the row's stores are visible to the whole workgroup
+        uint8_t *bits_row = p.bits + (size_t)row * p.bits_row_bytes;
+        const int n_bytes = (Lk + 7) / 8;
+        for (int w = tid; w * 4 < n_bytes; w += NT) {
+            uint32_t word = 0;
+            const int c0 = w * 32;
+            if (vec_o && c0 + 32 <= Lk) {
+#pragma unroll
+                for (int q8 = 0; q8 < 4; q8++) {
+                    const uint64_t m8 = *(const uint64_t *)(orow + c0 + 8 * q8);  // eight 0 / 1 bytes
+                    // (bit 8 i of m8 to bit i: the product gathers them in its top byte)
+                    word |= (uint32_t)(((m8 & 0x0101010101010101ull) * 0x0102040810204080ull) >> 56) << (8 * q8);
+                }
+            } else {
+                for (int c = 0; c < 32 && c0 + c < Lk; c++) word |= (orow[c0 + c] ? 1u : 0u) << c;
+            }
+            if (w * 4 + 4 <= n_bytes) {
+                *(uint32_t *)(bits_row + w * 4) = word;  // (rows are 4-byte aligned: bits_row_bytes is a multiple of 4)
+            } else {
+                for (int k = 0; w * 4 + k < n_bytes; k++) bits_row[w * 4 + k] = (uint8_t)(word >> (8 * k));
+            }
+        }
+    }
 }
 
 }  // namespace

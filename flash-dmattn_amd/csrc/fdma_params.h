@@ -121,6 +121,10 @@ struct FwdParams {
     // (mask batch entry, mask head)
     const int32_t *kept_idx, *kept_cnt, *kept_count;
     int32_t kept_ld;
+    // the mask packed to one bit per key (fdma_mask_bits of the C ABI; nullptr = read the bool mask): strides in bytes,
+    // broadcast like the mask
+    const uint8_t *mbits;
+    int64_t mb_b, mb_h, mb_r;
 };
 
 // lengths and first rows of batch entry b
@@ -182,6 +186,8 @@ struct MaskParams {
     uint32_t min_bits;   // the fill value for entries the incoming mask excludes, as bits of the bias type
     int32_t *kept_idx, *kept_cnt, *kept_count;  // optional second output (nullptr = not wanted): see scan_mask_row
     int32_t kept_ld;
+    uint8_t *bits;           // optional third output (nullptr = not wanted): the mask packed to one bit per key
+    int64_t bits_row_bytes;
 };
 hipError_t launch_make_mask(const MaskParams &p, hipStream_t stream);
 

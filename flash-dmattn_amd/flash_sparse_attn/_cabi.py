@@ -22,6 +22,11 @@ class KeptKeys(ctypes.Structure):
     _fields_ = [("idx", ctypes.c_void_p), ("cnt", ctypes.c_void_p), ("count", ctypes.c_void_p), ("ld", ctypes.c_int32)]
 
 
+class MaskBits(ctypes.Structure):
+    """fdma_mask_bits: a per-query keep-mask packed to one bit per key (strides in bytes: batch, head, row)."""
+    _fields_ = [("bits", ctypes.c_void_p), ("strides", ctypes.c_int64 * 3)]
+
+
 class FwdArgs(ctypes.Structure):
     _fields_ = [
         ("q", ctypes.c_void_p), ("k", ctypes.c_void_p), ("v", ctypes.c_void_p),
@@ -38,6 +43,7 @@ class FwdArgs(ctypes.Structure):
         ("compact_mode", ctypes.c_int32),
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
         ("kept", KeptKeys),
+        ("mask_bits", MaskBits),
     ]
 
 
@@ -94,6 +100,7 @@ class MaskArgs(ctypes.Structure):
         ("min_value", ctypes.c_float),
         ("kept_idx", ctypes.c_void_p), ("kept_cnt", ctypes.c_void_p), ("kept_count", ctypes.c_void_p),
         ("kept_ld", ctypes.c_int32),
+        ("bits", ctypes.c_void_p), ("bits_row_bytes", ctypes.c_int64),
     ]
 
 
@@ -188,8 +195,8 @@ def _load() -> ctypes.CDLL:
     lib.fdma_abi_version.restype = ctypes.c_int
     lib.fdma_sizeof_fwd_args.restype = ctypes.c_size_t
     lib.fdma_sizeof_bwd_args.restype = ctypes.c_size_t
-    if lib.fdma_abi_version() != 4:
-        raise ImportError(f"{path}: ABI version {lib.fdma_abi_version()} != 4")
+    if lib.fdma_abi_version() != 5:
+        raise ImportError(f"{path}: ABI version {lib.fdma_abi_version()} != 5")
     lib.fdma_varlen_fwd.argtypes = [ctypes.POINTER(VarlenFwdArgs), ctypes.c_void_p]
     lib.fdma_varlen_fwd.restype = ctypes.c_int
     lib.fdma_varlen_bwd.argtypes = [ctypes.POINTER(VarlenBwdArgs), ctypes.c_void_p]
@@ -257,13 +264,16 @@ def _bcast3(t: torch.Tensor) -> Sequence[int]:
     return tuple(0 if t.size(i) == 1 else t.stride(i) for i in range(3))
 
 
-_FWD_STRUCT = struct.Struct("@7P18q10i2fiPN3Pi4x")
+_FWD_STRUCT = struct.Struct("@7P18q10i2fiPN3Pi4xP3q")
 assert _FWD_STRUCT.size == ctypes.sizeof(FwdArgs)
 
 
-def fill_fwd(a: FwdArgs, q, k, v, mask, bias, out, lse, softmax_scale, is_causal, softcap, kept=None) -> None:
+def fill_fwd(a: FwdArgs, q, k, v, mask, bias, out, lse, softmax_scale, is_causal, softcap, kept=None, bits=None) -> None:
     """Fill the argument block in one struct.pack (ctypes field-by-field assignment costs ~10 us a call).
-    `kept`: None, or (idx, cnt, count, ld) -- the mask's kept columns as int32 tensors (fdma_kept_keys)."""
+    `kept`: None, or (idx, cnt, count, ld) -- the mask's kept columns as int32 tensors (fdma_kept_keys).
+    `bits`: None, or the mask packed to one bit per key, a uint8 tensor of the mask's shape but for the last
+    dimension (fdma_mask_bits)."""
+    bt = _bcast3(bits) if bits is not None else (0, 0, 0)
     ms = _bcast3(mask) if mask is not None else (0, 0, 0)
     bs = _bcast3(bias) if bias is not None else (0, 0, 0)
     batch, seqlen_q, num_heads, head_dim = q.shape
@@ -281,6 +291,7 @@ def fill_fwd(a: FwdArgs, q, k, v, mask, bias, out, lse, softmax_scale, is_causal
         float(softmax_scale), float(softcap), _compact_mode, 0, 0,
         kept[0].data_ptr() if kept else 0, kept[1].data_ptr() if kept else 0, kept[2].data_ptr() if kept else 0,
         kept[3] if kept else 0,
+        bits.data_ptr() if bits is not None else 0, bt[0], bt[1], bt[2],
     )
 
 

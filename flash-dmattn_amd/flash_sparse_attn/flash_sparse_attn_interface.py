@@ -21,7 +21,7 @@ from typing import Any, Optional, Tuple
 import torch
 
 from . import _cabi
-from .utils.mask import kept_keys_of
+from .utils.mask import kept_keys_of, mask_bits_of
 
 
 def maybe_contiguous(x: Optional[torch.Tensor]) -> Optional[torch.Tensor]:
@@ -104,7 +104,8 @@ def _check_inputs(q, k, v, mask, bias) -> None:
 
 
 # Side inputs of the two operator bodies that are not part of the reference's operator signatures: the kept-key
-# lists of a mask made by the device mask builder, and the forward call's workspace (index lists and compacted K / V
+# lists (query-broadcast mask) or the bit-packed form (per-query mask) of a mask made by the device mask builder, and
+# the forward call's workspace (index lists and compacted K / V
 # copies), which the backward of the same autograd node reuses.  FlashDMAttnFunc sets them around its calls; a body
 # that is called without them (torch.compile, direct operator calls) takes the ordinary path.
 _tls = threading.local()
@@ -134,6 +135,9 @@ def _flash_sparse_attn_forward_body(
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     _check_inputs(q, k, v, mask, bias)
     kept = _handoff_get("kept") or kept_keys_of(mask)
+    bits = _handoff_get("bits")
+    if bits is None:
+        bits = mask_bits_of(mask)
     q, k, v = [_aligned(x, 8) for x in (q, k, v)]
     mask = _aligned(mask, 16)
     bias = _aligned(bias, 8)
@@ -146,7 +150,7 @@ def _flash_sparse_attn_forward_body(
     if seqlen_q == 0:
         return out, softmax_lse, p
     args = _cabi.FwdArgs()
-    _cabi.fill_fwd(args, q, k, v, mask, bias, out, softmax_lse, softmax_scale, is_causal, softcap, kept)
+    _cabi.fill_fwd(args, q, k, v, mask, bias, out, softmax_lse, softmax_scale, is_causal, softcap, kept, bits)
     with _cabi.device_guard(q.device):
         nbytes = _cabi.lib.fdma_fwd_workspace_bytes(args)
         workspace = None
@@ -228,7 +232,8 @@ def _flash_sparse_attn_backward_body(
         dbias_final, dbias_w = dbias_w, torch.empty_like(bias)
 
     args = _cabi.BwdArgs()
-    _cabi.fill_fwd(args.f, q, k, v, mask, bias, out, softmax_lse, softmax_scale, is_causal, softcap, _handoff_get("kept"))
+    _cabi.fill_fwd(args.f, q, k, v, mask, bias, out, softmax_lse, softmax_scale, is_causal, softcap, _handoff_get("kept"),
+                   _handoff_get("bits"))
     fwd_ws = _handoff_get("fwd_ws")
     if fwd_ws is not None and fwd_ws[1] == _cabi.get_compact_mode() and fwd_ws[2] == (None if bias is None else tuple(bias.shape)):
         args.fwd_workspace, args.fwd_workspace_bytes = fwd_ws[0].data_ptr(), fwd_ws[0].numel()
@@ -346,11 +351,12 @@ class FlashDMAttnFunc(torch.autograd.Function):
         # (the hand-overs are eager-mode business: a traced graph calls the operators as they are)
         eager = not torch.compiler.is_compiling()
         kept = kept_keys_of(mask) if eager else None  # (before the mask may be replaced by a padded copy)
+        bits = mask_bits_of(mask) if eager else None
         mask = _pad_key_dim(mask, k.shape[1], 16)
         bias = _pad_key_dim(bias, k.shape[1], 8)
 
         if eager:
-            with _handoff(kept=kept) as side:
+            with _handoff(kept=kept, bits=bits) as side:
                 out_padded, softmax_lse, S_dmask = _wrapped_flash_sparse_attn_forward(
                     q, k, v, mask, bias, softmax_scale, is_causal=is_causal, softcap=softcap, return_softmax=return_softmax,
                 )
@@ -364,6 +370,7 @@ class FlashDMAttnFunc(torch.autograd.Function):
             ctx.save_for_backward(q, k, v, mask, bias, out_padded, softmax_lse)
             if eager:
                 ctx.kept = kept
+                ctx.bits = bits
                 ctx.fwd_ws = side.get("fwd_ws_out")
             ctx.softmax_scale = softmax_scale
             ctx.is_causal = is_causal
@@ -399,7 +406,7 @@ class FlashDMAttnFunc(torch.autograd.Function):
                 ctx.softcap, ctx.deterministic,
             )
         else:
-            with _handoff(kept=getattr(ctx, "kept", None), fwd_ws=getattr(ctx, "fwd_ws", None)):
+            with _handoff(kept=getattr(ctx, "kept", None), bits=getattr(ctx, "bits", None), fwd_ws=getattr(ctx, "fwd_ws", None)):
                 _wrapped_flash_sparse_attn_backward(
                     dout_padded, q, k, v, mask, bias, out, softmax_lse, dq, dk, dv, dbias, ctx.softmax_scale, ctx.is_causal,
                     ctx.softcap, ctx.deterministic,

@@ -94,10 +94,20 @@ def _native_mask(attention_bias, attention_mask, window_size, min_dtype, block_s
                 torch.empty((rows, ld), dtype=torch.int32, device=bias.device),
                 torch.empty((rows,), dtype=torch.int32, device=bias.device), ld)
         a.kept_idx, a.kept_cnt, a.kept_count, a.kept_ld = kept[0].data_ptr(), kept[1].data_ptr(), kept[2].data_ptr(), ld
+    # A mask that varies per query row is what the per-query attention kernels spend most of their memory traffic on
+    # (a byte per score): the kernel also writes it packed to one bit per key, and the attention calls read that
+    # instead (see mask_bits_of).
+    bits = None
+    if shape[2] > 1:
+        row_bytes = ((shape[3] + 7) // 8 + 15) // 16 * 16
+        bits = torch.empty(shape[:3] + (row_bytes,), dtype=torch.uint8, device=bias.device)
+        a.bits, a.bits_row_bytes = bits.data_ptr(), row_bytes
     with _cabi.device_guard(bias.device):
         _cabi.check(_cabi.lib.fdma_create_mask(a, _cabi.current_stream(bias.device)))
     if kept is not None:
         out._fdma_kept = kept + (out._version, out.data_ptr(), tuple(out.shape))
+    if bits is not None:
+        out._fdma_bits = (bits, out._version, out.data_ptr(), tuple(out.shape))
     return out
 
 
@@ -111,6 +121,19 @@ def kept_keys_of(mask: Optional[torch.Tensor]):
     if mask._version != version or mask.data_ptr() != ptr or tuple(mask.shape) != shape:
         return None
     return idx, cnt, count, ld
+
+
+def mask_bits_of(mask: Optional[torch.Tensor]):
+    """The uint8 tensor of bits (shape of the mask but for the last dimension; key j of a row in bit j % 8 of byte
+    j // 8) written by the device mask builder for THIS mask tensor, or None: when the tensor did not come from it,
+    is broadcast over the queries, or has been written to since."""
+    rec = getattr(mask, "_fdma_bits", None)
+    if rec is None:
+        return None
+    bits, version, ptr, shape = rec
+    if mask._version != version or mask.data_ptr() != ptr or tuple(mask.shape) != shape:
+        return None
+    return bits
 
 
 def _masked_bias(attention_bias: torch.Tensor, attention_mask: Optional[torch.Tensor], min_dtype: float):

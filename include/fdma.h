@@ -44,7 +44,7 @@
 extern "C" {
 #endif
 
-#define FDMA_ABI_VERSION 4 /* 4: fdma_kept_keys (fdma_fwd_args.kept, fdma_mask_args.kept_*), fdma_bwd_args.fwd_workspace (the structs grew);
+#define FDMA_ABI_VERSION 5 /* 5: fdma_mask_bits (fdma_fwd_args.mask_bits, fdma_mask_args.bits); 4: fdma_kept_keys (fdma_fwd_args.kept, fdma_mask_args.kept_*), fdma_bwd_args.fwd_workspace (the structs grew);
                               3: fdma_fwd_args.compact_mode, fdma_fwd_noalloc; 2: fdma_varlen_*, fdma_create_mask, fdma_dyn_bias_* */
 
 enum { FDMA_DTYPE_BF16 = 0, FDMA_DTYPE_FP16 = 1 };
@@ -98,6 +98,20 @@ typedef struct fdma_kept_keys {
     int32_t ld;
 } fdma_kept_keys;
 
+/* A keep-mask that varies per query row, packed to one bit per key: the form in which the per-query kernels can
+ * take it at an eighth of the bool mask's memory traffic (these kernels are bound by the mask and bias streams).
+ * Optional second output of fdma_create_mask and optional input of fdma_fwd / fdma_bwd; the bool mask itself must
+ * still be passed (it decides the path, and kernels that do not read bits read it).  Byte j / 8 of a row holds key j
+ * in bit j % 8 (least significant bit first); bits beyond seqlen_k are not looked at.  The kernels read a row in
+ * aligned 8-byte pieces: `bits` and every stride are multiples of 8, and a row is readable up to ceil(seqlen_k / 8)
+ * rounded up to 8 bytes, whatever lies there.  Strides in BYTES, in the order of mask_strides (batch, head, row),
+ * 0 = broadcast exactly where the mask is.  The bits must describe exactly the mask that is passed; nothing checks it.  The reference has no
+ * counterpart (its kernels take the bool mask only). */
+typedef struct fdma_mask_bits {
+    const uint8_t *bits; /* NULL = not given */
+    int64_t strides[3];
+} fdma_mask_bits;
+
 typedef struct fdma_fwd_args {
     const void *q, *k, *v;
     const void *mask; /* NULL = no mask */
@@ -117,6 +131,7 @@ typedef struct fdma_fwd_args {
     void *workspace;        /* split-KV partials (decode) or the compacted K / V copies; may be NULL if bytes == 0 */
     size_t workspace_bytes; /* >= fdma_fwd_workspace_bytes(args) */
     fdma_kept_keys kept;    /* optional: the mask's kept columns as lists (see fdma_kept_keys) */
+    fdma_mask_bits mask_bits; /* optional: a per-query mask packed to bits (see fdma_mask_bits) */
 } fdma_fwd_args;
 
 typedef struct fdma_bwd_args {
@@ -247,6 +262,12 @@ typedef struct fdma_mask_args {
      * (batch, head, row) order; all NULL = not wanted */
     int32_t *kept_idx, *kept_cnt, *kept_count;
     int32_t kept_ld; /* multiple of 16, >= seqlen_k */
+    /* optional third output: the mask packed to bits (fdma_mask_bits), one row of bits_row_bytes bytes per bias row in
+     * (batch, head, row) order; NULL = not wanted.  bits and bits_row_bytes: multiples of 8, bits_row_bytes >=
+     * ceil(seqlen_k / 8) rounded up to 8; the bytes of a row up to ceil(seqlen_k / 8) are written, bits beyond
+     * seqlen_k as zeros */
+    uint8_t *bits;
+    int64_t bits_row_bytes;
 } fdma_mask_args;
 int fdma_create_mask(const fdma_mask_args *args, void *hip_stream);
 int fdma_create_mask_validate(const fdma_mask_args *args);

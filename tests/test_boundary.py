@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(_cabi.lib_path())
     for name in declared:
         assert hasattr(lib, name), f"{name} not exported"
-    assert lib.fdma_abi_version() == 4
+    assert lib.fdma_abi_version() == 5
 
 
 def test_struct_mirrors_match_compiled_sizes():
@@ -86,6 +86,33 @@ def test_validation_errors(mutate, needle):
     assert needle in _cabi.last_error(), _cabi.last_error()
     with pytest.raises(RuntimeError, match=re.escape(needle)):
         _cabi.check(rc)
+
+
+def _with_per_query_mask(a):
+    a.mask = 0x2000
+    a.num_heads_mask = 2
+    a.mask_strides[:] = (2 * 128 * 256, 128 * 256, 256)
+    a.mask_bits.bits = 0x4000
+    a.mask_bits.strides[:] = (2 * 128 * 32, 128 * 32, 32)
+    return a
+
+
+def test_mask_bits_validation():
+    from flash_sparse_attn import _cabi
+
+    a = _with_per_query_mask(_valid_fwd())
+    assert _cabi.lib.fdma_fwd_validate(a) == 0, _cabi.last_error()
+    for mutate, needle in (
+        (lambda x: setattr(x, "mask", 0), "mask_bits without a mask"),
+        (lambda x: x.mask_bits.strides.__setitem__(0, 0), "broadcast over the same dimensions"),
+        (lambda x: x.mask_bits.strides.__setitem__(2, 24), "rounded up to 8"),
+        (lambda x: setattr(x.mask_bits, "bits", 0x4004), "multiples of 8 bytes"),
+        (lambda x: x.mask_bits.strides.__setitem__(1, 128 * 32 + 4), "multiples of 8 bytes"),
+    ):
+        a = _with_per_query_mask(_valid_fwd())
+        mutate(a)
+        assert _cabi.lib.fdma_fwd_validate(a) < 0
+        assert needle in _cabi.last_error(), _cabi.last_error()
 
 
 def test_backward_validation():
@@ -299,6 +326,15 @@ def test_mask_builder_validation():
         setattr(a, field, value)
         assert _cabi.lib.fdma_create_mask_validate(a) < 0, field
         assert message in _cabi.last_error()
+    # the optional bit-packed output: 8-byte aligned rows of at least ceil(seqlen_k / 8) bytes rounded up to 8
+    a = good()
+    a.bits, a.bits_row_bytes = 0x3000, 64
+    assert _cabi.lib.fdma_create_mask_validate(a) == 0, _cabi.last_error()
+    for bits, row_bytes, message in ((0x3000, 60, "multiple of 8"), (0x3000, 56, "multiple of 8"), (0x3004, 64, "8-byte aligned")):
+        a = good()
+        a.bits, a.bits_row_bytes = bits, row_bytes
+        assert _cabi.lib.fdma_create_mask_validate(a) < 0
+        assert message in _cabi.last_error(), _cabi.last_error()
 
 
 def test_bias_producer_validation_and_workspace():
