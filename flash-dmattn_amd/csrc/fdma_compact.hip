@@ -136,6 +136,92 @@ __global__ void __launch_bounds__(256) compact_gather_kernel(const FwdParams p, 
     gather_block<T>(p, idx, cnt, count, fb, kc, vc, ld, Hfb, blockIdx.x, blockIdx.y);
 }
 
+// Scan and gather of the forward in one launch: a workgroup owns SEG_KEYS consecutive ORIGINAL columns of a pair.  It
+// counts the kept columns in front of its segment itself (at most Lk mask bytes, which all workgroups of the pair read
+// and the L2 serves), numbers its own, writes its part of `idx` and `cnt` and copies its kept K / V rows and bias values
+// to their compacted places.  One launch less in front of the attention kernel than scan + gather.
+constexpr int SEG_KEYS = 256;
+
+template <typename T>
+__global__ void __launch_bounds__(256) compact_scan_gather_kernel(const FwdParams p, int32_t *idx, int32_t *cnt, int32_t *count,
+                                                                   float *fb, uint16_t *kc, uint16_t *vc, int ld, int Hfb) {
+    using E = Elem<T>;
+    __shared__ int s_wave[4], s_src[SEG_KEYS];
+    const int pair = blockIdx.y, b = pair / p.Hk, hk = pair % p.Hk;
+    const int hm = p.Hm == 1 ? 0 : hk;
+    const uint8_t *mrow = p.mask + b * p.m_b + hm * p.m_h;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int s0 = blockIdx.x * SEG_KEYS;
+    // kept columns in front of the segment (s0 is a multiple of 16; mask rows are readable in 16-byte pieces)
+    int before = 0;
+    for (int c = tid * 16; c < s0; c += 256 * 16) {
+        const u32x4_t mv = *(const u32x4_t *)(mrow + c);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            // a byte is non-zero <=> bit 7 of ((x & 0x7f) + 0x7f) | x is set
+            const uint32_t x = mv[e];
+            before += __builtin_popcount((((x & 0x7f7f7f7fu) + 0x7f7f7f7fu) | x) & 0x80808080u);
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) before += __shfl_xor(before, off);
+    if (lane == 0) s_wave[wave] = before;
+    __syncthreads();
+    const int base = s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3];
+    __syncthreads();
+    // this segment: one column per thread
+    const int col = s0 + tid;
+    const bool kept = col < p.Lk && mrow[col] != 0;
+    const uint64_t vote = __ballot(kept);
+    const int excl_w = __builtin_popcountll(vote & ((1ull << lane) - 1ull));
+    if (lane == 0) s_wave[wave] = __builtin_popcountll(vote);
+    __syncthreads();
+    int woff = 0, n_seg = 0;
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+        const int v = s_wave[w];
+        if (w < wave) woff += v;
+        n_seg += v;
+    }
+    const int excl = woff + excl_w;  // kept columns of the segment in front of this one
+    int32_t *irow = idx + (size_t)pair * ld, *crow = cnt + (size_t)pair * ld;
+    if (kept) {
+        irow[base + excl] = col;
+        s_src[excl] = col;
+    }
+    if (col < ld) crow[col] = base + excl + (kept ? 1 : 0);  // (columns from Lk to ld repeat the total)
+    if (s0 + SEG_KEYS >= ld && tid == 0) count[pair] = base + n_seg;
+    __syncthreads();
+    if (n_seg == 0) return;
+    const int CH = p.d / 8;
+    const uint16_t *kb = (const uint16_t *)p.k + b * p.k_b + hk * p.k_h;
+    const uint16_t *vb = (const uint16_t *)p.v + b * p.v_b + hk * p.v_h;
+    uint16_t *kd = kc + ((size_t)pair * p.Lk + base) * p.d;
+    uint16_t *vd = vc + ((size_t)pair * p.Lk + base) * p.d;
+    for (int it = tid; it < n_seg * CH; it += 256) {
+        const int rr = it / CH, ch = it - rr * CH;
+        const int src = s_src[rr];
+        const u32x4_t kv = *(const u32x4_t *)(kb + (int64_t)src * p.k_r + ch * 8);
+        const u32x4_t vv = *(const u32x4_t *)(vb + (int64_t)src * p.v_r + ch * 8);
+        *(u32x4_t *)(kd + (size_t)rr * p.d + ch * 8) = kv;
+        *(u32x4_t *)(vd + (size_t)rr * p.d + ch * 8) = vv;
+    }
+    // fused bias of the compacted keys, one vector per bias class of this kv head
+    const int G = p.H / p.Hk;
+    const int nfb = Hfb == p.H ? G : 1;
+    for (int it = tid; it < n_seg * nfb; it += 256) {
+        const int gi = it / n_seg, rr = it - gi * n_seg;
+        const int src = s_src[rr];
+        const int hfb = Hfb == p.H ? hk * G + gi : hk;
+        float v = 0.f;
+        if (p.bias) {
+            const int hb = p.Hb == p.H ? hfb : (p.Hb == 1 ? 0 : hk);
+            v = E::lo((uint32_t)((const uint16_t *)p.bias)[b * p.bi_b + hb * p.bi_h + src]) * kLog2e;
+        }
+        fb[((size_t)b * Hfb + hfb) * ld + base + rr] = v;
+    }
+}
+
 // Gradient rows (dK, dV) and columns (dBias) of dropped keys: no workgroup of the compacted backward
 // owns them, and the operator's contract is that they come back as zeros.
 __device__ __forceinline__ void zero_block(const BwdParams &p, bool dbias_direct, int block_x, int pair) {
@@ -466,7 +552,15 @@ hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, 
     const int pairs = p.B * p.Hk;
     hipError_t e;
     const bool have_lists = fwd_ws != nullptr || p.kept_idx != nullptr;
-    if (!have_lists) {
+    const bool fused_scan = !have_lists && !bp;  // forward without lists: scan and gather in one launch
+    if (fused_scan) {
+        const dim3 sgrid((l.ld + SEG_KEYS - 1) / SEG_KEYS, pairs);
+        if (dtype == 0)
+            hipLaunchKernelGGL((compact_scan_gather_kernel<bf16_tag>), sgrid, dim3(256), 0, stream, p, idx, cnt, count, fb, kc, vc, l.ld, l.Hfb);
+        else
+            hipLaunchKernelGGL((compact_scan_gather_kernel<fp16_tag>), sgrid, dim3(256), 0, stream, p, idx, cnt, count, fb, kc, vc, l.ld, l.Hfb);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+    } else if (!have_lists) {
         hipLaunchKernelGGL(compact_scan_kernel, dim3(pairs), dim3(SCAN_THREADS), 0, stream, p, idx, cnt, count, l.ld);
         if ((e = hipGetLastError()) != hipSuccess) return e;
     }
@@ -474,7 +568,7 @@ hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, 
     // (handed-over lists: the gather launch also copies them into the per-pair arrays, which the backward's other
     // pre-pass layers read -- so it runs on its own in front of them)
     const bool gather_alone = !bp || (p.kept_idx != nullptr && !fwd_ws);
-    if (gather_alone && !fwd_ws) {
+    if (gather_alone && !fwd_ws && !fused_scan) {
         if (dtype == 0)
             hipLaunchKernelGGL((compact_gather_kernel<bf16_tag>), grid, dim3(256), 0, stream, p, idx, cnt, count, fb, kc, vc, l.ld, l.Hfb);
         else

@@ -90,6 +90,54 @@ def test_attention_with_handed_over_lists_is_bit_identical(case, mode):
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("Lk", [1, 15, 16, 17, 255, 256, 257, 511, 512, 513, 1000, 1281])
+@pytest.mark.parametrize("pattern", ["random", "all", "last_only", "first_segments_empty", "every_256th"])
+def test_forward_scan_and_gather_in_one_launch_at_segment_boundaries(Lk, pattern):
+    """The forward numbers and gathers the kept columns in one launch, 256 original columns per workgroup: key lengths
+    and masks around those boundaries, forward and backward against the same call on the tile-skipping kernels (other
+    order of summation: tolerances), and the backward on the forward's workspace against the backward that scans and
+    gathers for itself (bit for bit)."""
+    B, Lq, H, Hk, D = 2, 130, 4, 2, 64
+    q, k, v, bias = _inputs(B, Lq, Lk, H, Hk, D, Hk, seed=Lk)
+    g = torch.Generator().manual_seed(1000 + Lk)
+    if pattern == "random":
+        mask = torch.rand(B, Hk, 1, Lk, generator=g) < 0.3
+        mask[..., 0] = True
+    elif pattern == "all":
+        mask = torch.ones(B, Hk, 1, Lk, dtype=torch.bool)
+    elif pattern == "last_only":
+        mask = torch.zeros(B, Hk, 1, Lk, dtype=torch.bool)
+        mask[..., Lk - 1] = True
+    elif pattern == "first_segments_empty":
+        mask = torch.rand(B, Hk, 1, Lk, generator=g) < 0.5
+        mask[..., :min(Lk - 1, 512)] = False
+        mask[..., Lk - 1] = True
+    else:
+        mask = torch.zeros(B, Hk, 1, Lk, dtype=torch.bool)
+        mask[..., ::256] = True
+    mask = mask.to(DEV)
+    try:
+        set_compact("2")
+        got = _run(q, k, v, mask, bias, causal=False)
+        mpad, bpad = iface._pad_key_dim(mask, Lk, 16), iface._pad_key_dim(bias, Lk, 8)
+        out, lse, _ = iface._wrapped_flash_sparse_attn_forward(q, k, v, mpad, bpad, D ** -0.5, False, 0.0, False)
+        dq, dk, dv, dbp = torch.empty_like(q), torch.empty_like(k), torch.empty_like(v), torch.empty_like(bpad)
+        iface._wrapped_flash_sparse_attn_backward(torch.ones_like(out), q, k, v, mpad, bpad, out, lse, dq, dk, dv, dbp,
+                                                  D ** -0.5, False, 0.0, False)
+        torch.cuda.synchronize()
+        set_compact("0")
+        ref = _run(q, k, v, mask, bias, causal=False)
+    finally:
+        set_compact("auto")
+    for a, b in zip(got, [out, lse, dq, dk, dv, dbp[..., :Lk]]):
+        assert torch.equal(a, b)
+    assert (got[0].float() - ref[0].float()).abs().max().item() <= 2e-2
+    assert (got[1] - ref[1]).abs().max().item() <= 1e-3
+    for a, b, name in zip(got[2:], ref[2:], ("dq", "dk", "dv", "dbias")):
+        err = (a.float() - b.float()).abs().max().item()
+        assert err <= 5e-2 * max(1.0, b.float().abs().max().item()), (name, err)
+
+
 @pytest.mark.parametrize("case", range(len(CASES)))
 def test_backward_on_the_forward_workspace_is_bit_identical(case):
     B, Lq, Lk, H, Hk, D, Hm, W = CASES[case]
