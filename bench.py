@@ -531,8 +531,8 @@ def main():
     main_res = run_config("cfg2", args.steps, args.warmup, device, compact)
     c = CONFIGS["cfg2"]
     if main_res["compacted"]:
-        kernel = ("fdma::fwd_colmask_kernel<bf16, 128, causal, compacted>, with its pre-pass (compact_scan_kernel, "
-                  "compact_gather_kernel) in the same call: the duration is that of the whole forward call")
+        kernel = ("fdma::fwd_colmask_kernel<bf16, 128, causal, compacted>, with its pre-pass (compact_scan_gather_kernel) "
+                  "in the same call: the duration is that of the whole forward call")
         flops_model = ("4*64*64*d per executed 64x64 tile on the compacted key axis (kept columns packed to the front per "
                        "(batch, kv head)); a 64-row query block executes ceil(visible kept columns / 64) tiles")
     else:
