@@ -439,7 +439,12 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dkdv_colmask_k
 #pragma unroll
         for (int mb = 0; mb < MB; mb++)
 #pragma unroll
-            for (int i = 0; i < 16; i++) { s[mb][i] = cconst; dp[mb][i] = 0.f; }
+            for (int i = 0; i < 16; i++) {
+                // (one move per accumulator register, written out: as a plain splat the compiler builds the vector in
+                // other registers first and copies it over, 31 instructions for 16)
+                asm volatile("v_mov_b32 %0, %1" : "=v"(s[mb][i]) : "v"(cconst));
+                dp[mb][i] = 0.f;
+            }
         {
             constexpr int NF = 2 * MB * KS, FR = D > 64 ? 3 : 8;  // fragment f: (ks, mb, which) with which = 0: Q, 1: dO
             u32x4_t a[NF];
