@@ -1153,6 +1153,8 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
         publish();
     }
     int i = 0;
+    constexpr bool S_EARLY = DMA && MB == 1;
+    f32x16_t s[MB];
     while (jc < n_end) {
         if constexpr (!DMA) jn = next_active(jc + 1);
         const int n0 = jc * BN;
@@ -1169,20 +1171,26 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
         //   slots of one 16-key block with the dS arithmetic of the next block between them.
         // The score accumulators start from the fused bias vector minus the row's log-sum-exp and the dP accumulators
         // from minus D, so that the MFMAs deliver the exp2 argument and dP - D themselves.
-        f32x16_t s[MB], dp[MB];
+        // (direct loads: every wave fetches the whole bias column of a tile itself, two tiles ahead, so a wave can read
+        // the next tile's column as soon as its own load has landed; the score accumulators of the NEXT tile are set up
+        // between the last dQ MFMAs of this one -- `s` is free from the last exp2 on -- instead of in front of the first
+        // MFMA, where nothing covers the LDS reads and the 16 subtractions)
+        f32x16_t dp[MB];
 #pragma unroll
         for (int mb = 0; mb < MB; mb++)
 #pragma unroll
             for (int blk = 0; blk < 2; blk++) {
-                const f32x4_t b0 = __builtin_bit_cast(f32x4_t, lds_ld128(bs + 4 * (32 * mb + 16 * blk)));
-                const f32x4_t b1 = __builtin_bit_cast(f32x4_t, lds_ld128(bs + 4 * (32 * mb + 16 * blk + 4)));
+                if (!S_EARLY || i == 0) {
+                    const f32x4_t b0 = __builtin_bit_cast(f32x4_t, lds_ld128(bs + 4 * (32 * mb + 16 * blk)));
+                    const f32x4_t b1 = __builtin_bit_cast(f32x4_t, lds_ld128(bs + 4 * (32 * mb + 16 * blk + 4)));
 #pragma unroll
-                for (int e = 0; e < 4; e++) {
-                    s[mb][8 * blk + e] = b0[e] - lse2;
-                    s[mb][8 * blk + 4 + e] = b1[e] - lse2;
-                    dp[mb][8 * blk + e] = -dd;
-                    dp[mb][8 * blk + 4 + e] = -dd;
+                    for (int e = 0; e < 4; e++) {
+                        s[mb][8 * blk + e] = b0[e] - lse2;
+                        s[mb][8 * blk + 4 + e] = b1[e] - lse2;
+                    }
                 }
+#pragma unroll
+                for (int e = 0; e < 8; e++) dp[mb][8 * blk + e] = -dd;
                 if (DMA && jc == j_last) {  // (the bias column came as it is in memory: columns beyond the kept keys)
                     const int lim = Lk - n0 - 32 * mb - 16 * blk - 8 * g;  // local columns e < lim exist
 #pragma unroll
@@ -1250,6 +1258,7 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
             // ones in front of the first block's dS arithmetic)
             constexpr int NG = KB * DB, FR2 = 2;
             u32x2_t tl[NG], th[NG];
+            f32x4_t nb[4];  // (S_EARLY: the next tile's bias column, 16 keys of this lane's half)
             auto tr_read = [&](int gi) {
                 const int kb = gi / DB, db = gi % DB;
                 tl[gi] = lds_ld_tr16(TL::tr_at(tr_cur, kb, db, 0));
@@ -1271,6 +1280,19 @@ __global__ void __launch_bounds__(NTHREADS, D <= 128 ? 2 : 1) bwd_dq_colmask_ker
 #pragma unroll
                     for (int e = 0; e < 4; e++)
                         if (e * DB / 4 == db) ds_piece(kb + 1, e);
+                }
+                if constexpr (S_EARLY) {
+                    // the next tile's bias column (slot (i + 1) % 3, complete since the last barrier): read in the slots
+                    // of the first key block, used in those of the last
+                    const uint32_t bs_n = lds0 + SM::OFF_BIAS + (uint32_t)(((i + 1) % 3) * 256 + 32 * g);
+                    // (this wave's own copy of that column was fetched a tile ago, in front of the N_DMA loads of the
+                    // tile after it: wait for it alone -- vmcnt N_DMA, no wait for LDS reads or exports)
+                    if (kb == 0 && db == 0) __builtin_amdgcn_s_waitcnt(0x0F70 | N_DMA);
+                    if (kb == 0 && db < 4) nb[db] = __builtin_bit_cast(f32x4_t, lds_ld128(bs_n + 16 * (db & 1) + 64 * (db >> 1)));
+                    if (kb == KB - 1 && db < 4) {
+#pragma unroll
+                        for (int e = 0; e < 4; e++) s[0][4 * db + e] = nb[db][e] - lse2;
+                    }
                 }
                 __builtin_amdgcn_sched_barrier(0);
             }
