@@ -552,7 +552,9 @@ hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, 
     const int pairs = p.B * p.Hk;
     hipError_t e;
     const bool have_lists = fwd_ws != nullptr || p.kept_idx != nullptr;
-    const bool fused_scan = !have_lists && !bp;  // forward without lists: scan and gather in one launch
+    // forward without lists: scan and gather in one launch -- up to 65536 keys: every workgroup of that launch counts the
+    // mask bytes in front of its segment, Lk / 2 of them on average, which grows with the square of Lk per pair
+    const bool fused_scan = !have_lists && !bp && p.Lk <= (1 << 16);
     if (fused_scan) {
         const dim3 sgrid((l.ld + SEG_KEYS - 1) / SEG_KEYS, pairs);
         if (dtype == 0)

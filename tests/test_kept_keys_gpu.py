@@ -138,6 +138,28 @@ def test_forward_scan_and_gather_in_one_launch_at_segment_boundaries(Lk, pattern
         assert err <= 5e-2 * max(1.0, b.float().abs().max().item()), (name, err)
 
 
+@pytest.mark.parametrize("Lk", [65536, 65537, 70000])
+def test_long_key_axes_take_the_two_launch_pre_pass_above_65536_keys(Lk):
+    """Up to 65536 keys the forward numbers and gathers in one launch, above that in two (the one-launch form recounts
+    the mask in front of every 256-key segment): the same results on both sides of the limit, against tile skipping."""
+    B, Lq, H, Hk, D = 1, 160, 2, 1, 64
+    q, k, v, bias = _inputs(B, Lq, Lk, H, Hk, D, Hk, seed=7)
+    mask = (torch.rand(B, Hk, 1, Lk, generator=torch.Generator().manual_seed(Lk)) < 0.02).to(DEV)
+    mask[..., Lk - 1] = True
+    try:
+        set_compact("2")
+        got = _run(q, k, v, mask, bias, causal=True)
+        set_compact("0")
+        ref = _run(q, k, v, mask, bias, causal=True)
+    finally:
+        set_compact("auto")
+    assert (got[0].float() - ref[0].float()).abs().max().item() <= 2e-2
+    assert (got[1] - ref[1]).abs().max().item() <= 1e-3
+    for a, b, name in zip(got[2:], ref[2:], ("dq", "dk", "dv", "dbias")):
+        err = (a.float() - b.float()).abs().max().item()
+        assert err <= 5e-2 * max(1.0, b.float().abs().max().item()), (name, err)
+
+
 @pytest.mark.parametrize("case", range(len(CASES)))
 def test_backward_on_the_forward_workspace_is_bit_identical(case):
     B, Lq, Lk, H, Hk, D, Hm, W = CASES[case]
