@@ -489,6 +489,7 @@ bool use_compact(const FwdParams &p) {
     if (p.bias && p.bi_r != 0) return false;
     if (!(p.Hm == 1 || p.Hm == p.Hk)) return false;
     if (p.Lq < 2 || p.Lk < 1 || (int64_t)p.Lk * p.d >= (int64_t)1 << 31) return false;
+    if ((int64_t)p.B * p.Hk > 65535) return false;  // (the pre-pass launches carry the pair in the grid's y dimension)
     if (mode == 2) return true;
     // the pre-pass costs about one copy of K and V plus three small launches; it pays once the attention
     // itself is a few million (query, key) pairs per kv head

@@ -160,6 +160,24 @@ def test_long_key_axes_take_the_two_launch_pre_pass_above_65536_keys(Lk):
         assert err <= 5e-2 * max(1.0, b.float().abs().max().item()), (name, err)
 
 
+def test_more_pairs_than_a_grid_dimension_holds_fall_back_to_tile_skipping():
+    """65536 (batch, kv head) pairs: the pre-pass launches could not carry the pair in the grid's y dimension, so the
+    call takes the tile-skipping kernels even when compaction is asked for -- same bits as with compaction off."""
+    B, Lq, Lk, H, Hk, D = 65536, 2, 16, 1, 1, 32
+    q, k, v, bias = _inputs(B, Lq, Lk, H, Hk, D, Hk, seed=3)
+    mask = (torch.rand(B, Hk, 1, Lk, generator=torch.Generator().manual_seed(3)) < 0.5).to(DEV)
+    mask[..., 0] = True
+    try:
+        set_compact("2")
+        got = _run(q, k, v, mask, bias, causal=True)
+        set_compact("0")
+        ref = _run(q, k, v, mask, bias, causal=True)
+    finally:
+        set_compact("auto")
+    for a, b in zip(got, ref):
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("case", range(len(CASES)))
 def test_backward_on_the_forward_workspace_is_bit_identical(case):
     B, Lq, Lk, H, Hk, D, Hm, W = CASES[case]
