@@ -586,6 +586,13 @@ def main():
                         zero_inputs=True)
         out["tile_skip_path"]["zero_operands"] = {"ms_fwd": tz["ms_fwd"], "tflops_fwd": tz["tflops_fwd"],
                                                   "frac_of_peak": tz["tflops_fwd"] / PEAK_BF16_TFLOPS}
+        # ... and the default path (forward and forward + backward) on all-zero operands
+        cz = run_config("cfg2", max(3, args.steps // 2), max(1, args.warmup // 2), device, compact=True, backward=True,
+                        zero_inputs=True)
+        out["zero_operands"] = {"ms_fwd": cz["ms_fwd"], "tflops_fwd": cz["tflops_fwd"],
+                                "frac_of_peak": cz["tflops_fwd"] / PEAK_BF16_TFLOPS, "ms_fwd_bwd": cz.get("ms_fwd_bwd"),
+                                "note": "same mask, tiles and instruction stream as the headline figures, all-zero Q / K / V / "
+                                        "bias: what the schedule sustains when the device does not lower its clock"}
     if not args.no_probe:
         probe = run_mfma_probe()
         if probe is not None:
