@@ -11,6 +11,8 @@
 //           counts `cnt` (what a causal query row needs: how many kept columns are <= its limit), total;
 //   gather  wide grid: K / V rows of the kept columns copied into dense [B, Hk, count, d] buffers, bias
 //           gathered and pre-scaled into an fp32 vector;
+//   (forward, up to 65536 keys) scan and gather in ONE launch: a workgroup per 256 original columns counts the kept
+//           columns in front of its segment itself;
 //   (backward) zero   rows of dK / dV and columns of dBias that belong to dropped keys.
 // All of this is O(Lk * d) traffic in front of O(Lq * count * d) MFMA work.
 #include <atomic>
@@ -491,7 +493,7 @@ bool use_compact(const FwdParams &p) {
     if (p.Lq < 2 || p.Lk < 1 || (int64_t)p.Lk * p.d >= (int64_t)1 << 31) return false;
     if ((int64_t)p.B * p.Hk > 65535) return false;  // (the pre-pass launches carry the pair in the grid's y dimension)
     if (mode == 2) return true;
-    // the pre-pass costs about one copy of K and V plus three small launches; it pays once the attention
+    // the pre-pass costs about one copy of K and V plus a small launch or two; it pays once the attention
     // itself is a few million (query, key) pairs per kv head
     return p.Lq >= 128 && p.Lk >= 128 && (int64_t)p.Lq * (p.H / p.Hk) * p.Lk >= (int64_t)1 << 21;
 }
