@@ -87,10 +87,14 @@ __device__ __forceinline__ void gather_block(const FwdParams &p, const int32_t *
     if (p.kept_idx) {
         const int srow = (p.m_b == 0 ? 0 : b) * p.Hm + (p.Hm == 1 ? 0 : hk);
         src_idx = p.kept_idx + (size_t)srow * p.kept_ld;
+        // (lists are device data the host cannot check: a list made for a longer key axis than this call's must not
+        // take reads or gradient writes past the tensors, so counts and columns are held inside [0, Lk))
         n = p.kept_count[srow];
+        n = n < p.Lk ? n : p.Lk;
         if (tid < GATHER_KEYS && c0 + tid < ld) {
-            ((int32_t *)idx)[(size_t)pair * ld + c0 + tid] = src_idx[c0 + tid];
-            cnt[(size_t)pair * ld + c0 + tid] = p.kept_cnt[(size_t)srow * p.kept_ld + c0 + tid];
+            const int32_t col = src_idx[c0 + tid], have = p.kept_cnt[(size_t)srow * p.kept_ld + c0 + tid];
+            ((int32_t *)idx)[(size_t)pair * ld + c0 + tid] = col < p.Lk ? col : p.Lk - 1;
+            cnt[(size_t)pair * ld + c0 + tid] = have < n ? have : n;
         }
         if (block_x == 0 && tid == 0) ((int32_t *)count)[pair] = n;
     } else {
@@ -98,7 +102,10 @@ __device__ __forceinline__ void gather_block(const FwdParams &p, const int32_t *
     }
     if (c0 >= n) return;
     __shared__ int s_src[GATHER_KEYS];
-    if (tid < GATHER_KEYS) s_src[tid] = (c0 + tid < n) ? src_idx[c0 + tid] : -1;
+    if (tid < GATHER_KEYS) {
+        const int32_t col = (c0 + tid < n) ? src_idx[c0 + tid] : -1;
+        s_src[tid] = col < p.Lk ? col : p.Lk - 1;
+    }
     __syncthreads();
     const int CH = p.d / 8;
     const uint16_t *kb = (const uint16_t *)p.k + b * p.k_b + hk * p.k_h;

@@ -44,15 +44,38 @@ def _aligned(x: Optional[torch.Tensor], elems: int) -> Optional[torch.Tensor]:
     return x if ok else x.contiguous().clone(memory_format=torch.contiguous_format)
 
 
+_len_dispatch_stack = getattr(torch._C, "_len_torch_dispatch_stack", None)
+_len_function_stack = getattr(torch._C, "_len_torch_function_stack", None)
+_is_functorch_wrapped = getattr(getattr(torch._C, "_functorch", None), "is_functorch_wrapped_tensor", None)
+
+
+def _plain_eager(*tensors) -> bool:
+    """True when nothing but the device would see a call on these tensors: eager mode, no TorchDispatchMode /
+    TorchFunctionMode active (FLOP counters, profilers, fake-tensor tracing install such modes and must see the
+    registered operators), and every tensor an ordinary torch.Tensor that no functorch transform (torch.func.grad /
+    vmap / jvp) has wrapped.  Where torch lacks one of the probes the answer is False: the dispatcher is always right."""
+    if torch.compiler.is_compiling():
+        return False
+    if _len_dispatch_stack is None or _len_function_stack is None or _is_functorch_wrapped is None:
+        return False
+    if _len_dispatch_stack() > 0 or _len_function_stack() > 0:
+        return False
+    for t in tensors:
+        if t is not None and (type(t) is not torch.Tensor or _is_functorch_wrapped(t)):
+            return False
+    return True
+
+
 def _direct_when_eager(op, body):
     """Callable for one of the operators below.  On plain tensors in eager mode it runs the operator's Python
     body directly: the dispatch of a torch.library operator costs about 20 us per call, more than a small
-    attention call takes on the device.  Under torch.compile, and for fake tensors or tensor subclasses, the
-    registered operator is called, as the reference always does (flash_sparse_attn_interface.py:126, 432)."""
+    attention call takes on the device.  Under torch.compile, under an active dispatch / function mode, and for
+    fake tensors, tensor subclasses or functorch-wrapped tensors the registered operator is called, as the reference
+    always does (flash_sparse_attn_interface.py:126, 432)."""
     def call(*args, **kwargs):
-        if torch.compiler.is_compiling() or any(type(a) is not torch.Tensor for a in args[:3]):
-            return op(*args, **kwargs)
-        return body(*args, **kwargs)
+        if _plain_eager(*[a for a in args[:5] if a is None or isinstance(a, torch.Tensor)]):
+            return body(*args, **kwargs)
+        return op(*args, **kwargs)
 
     return call
 
@@ -124,6 +147,16 @@ class _handoff:
         _tls.items = self.prev
 
 
+def _lists_for(lists, mask, k, exact):
+    """The mask builder's second output (kept-key lists, or bit rows) for `mask`, if it describes the key axis of this
+    call: the lists number the kept columns of the WHOLE mask row, so a mask that is wider than K (already padded) or
+    has a key dimension of 1 (expanded later) is scanned by the kernels instead.  Bit rows may be wider than K."""
+    if lists is None or mask is None:
+        return None
+    width, seqlen_k = mask.shape[-1], k.shape[1]
+    return lists if (width == seqlen_k or (not exact and width > seqlen_k)) else None
+
+
 def _handoff_get(name):
     items = getattr(_tls, "items", None)
     return items.get(name) if items else None
@@ -134,10 +167,10 @@ def _flash_sparse_attn_forward_body(
     softmax_scale: float, is_causal: bool, softcap: float, return_softmax: bool,
 ) -> Tuple[torch.Tensor, torch.Tensor, torch.Tensor]:
     _check_inputs(q, k, v, mask, bias)
-    kept = _handoff_get("kept") or kept_keys_of(mask)
+    kept = _handoff_get("kept") or _lists_for(kept_keys_of(mask), mask, k, exact=True)
     bits = _handoff_get("bits")
     if bits is None:
-        bits = mask_bits_of(mask)
+        bits = _lists_for(mask_bits_of(mask), mask, k, exact=False)
     q, k, v = [_aligned(x, 8) for x in (q, k, v)]
     mask = _aligned(mask, 16)
     bias = _aligned(bias, 8)
@@ -305,10 +338,10 @@ def _pad_key_dim(t: Optional[torch.Tensor], seqlen_k: int, elems: int) -> Option
 def _nothing_to_differentiate(grad_enabled: bool, *tensors: Optional[torch.Tensor]) -> bool:
     """True for an eager call on plain tensors none of which asks for a gradient: the autograd node would record
     nothing, and going through it costs about 10 us per call -- as much as a decode-sized kernel takes."""
-    if torch.compiler.is_compiling():
+    if not _plain_eager(*tensors):
         return False
     for t in tensors:
-        if t is not None and (type(t) is not torch.Tensor or (grad_enabled and t.requires_grad)):
+        if t is not None and grad_enabled and t.requires_grad:
             return False
     return True
 
@@ -350,8 +383,9 @@ class FlashDMAttnFunc(torch.autograd.Function):
             v = torch.nn.functional.pad(v, [0, 8 - head_size_og % 8])
         # (the hand-overs are eager-mode business: a traced graph calls the operators as they are)
         eager = not torch.compiler.is_compiling()
-        kept = kept_keys_of(mask) if eager else None  # (before the mask may be replaced by a padded copy)
-        bits = mask_bits_of(mask) if eager else None
+        # (taken before the mask may be replaced by a padded copy; only for a mask over exactly the keys of this call)
+        kept = _lists_for(kept_keys_of(mask), mask, k, exact=True) if eager else None
+        bits = _lists_for(mask_bits_of(mask), mask, k, exact=False) if eager else None
         mask = _pad_key_dim(mask, k.shape[1], 16)
         bias = _pad_key_dim(bias, k.shape[1], 8)
 

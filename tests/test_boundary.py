@@ -188,6 +188,59 @@ def test_cpu_tensors_are_rejected_loudly():
         flash_sparse_attn_func(q, q, q)
 
 
+def test_dispatch_modes_and_functorch_see_the_registered_operators():
+    """In plain eager mode the operator bodies run directly (the dispatcher costs more than a small kernel), but a
+    TorchDispatchMode / TorchFunctionMode (FLOP counters, profilers) and functorch transforms must get the registered
+    operators, as with the reference (flash_sparse_attn_interface.py:73, 126, 432)."""
+    from torch.overrides import TorchFunctionMode
+    from torch.utils._python_dispatch import TorchDispatchMode
+
+    from flash_sparse_attn import flash_sparse_attn_func, flash_sparse_attn_varlen_func
+    from flash_sparse_attn import flash_sparse_attn_interface as itf
+
+    seen = []
+
+    class Recorder(TorchDispatchMode):
+        def __torch_dispatch__(self, func, types, args=(), kwargs=None):
+            seen.append(str(func))
+            if "_flash_sparse_attn_forward" in str(func):  # (stands in for the device: shapes of the fake kernel)
+                q = args[0]
+                return (torch.empty_like(q), torch.empty(q.shape[0], q.shape[2], q.shape[1]), torch.empty(0, dtype=q.dtype))
+            if "_flash_sparse_attn_varlen_forward" in str(func):
+                q = args[0]
+                return (torch.empty_like(q), torch.empty(q.shape[1], q.shape[0]), torch.empty(0, dtype=q.dtype))
+            return func(*args, **(kwargs or {}))
+
+    q = torch.randn(1, 8, 2, 64, dtype=torch.bfloat16)
+    assert itf._plain_eager(q, q, q)
+    with Recorder():
+        assert not itf._plain_eager(q, q, q)
+        out = flash_sparse_attn_func(q, q, q)
+        assert out.shape == q.shape
+        cu = torch.tensor([0, 8], dtype=torch.int32)
+        flash_sparse_attn_varlen_func(q[0], q[0], q[0], cu, cu, 8, 8)
+    assert any("flash_sparse_attn._flash_sparse_attn_forward" in f for f in seen)
+    assert any("flash_sparse_attn._flash_sparse_attn_varlen_forward" in f for f in seen)
+
+    class Passive(TorchFunctionMode):
+        def __torch_function__(self, func, types, args=(), kwargs=None):
+            return func(*args, **(kwargs or {}))
+
+    with Passive():
+        assert not itf._plain_eager(q)
+
+    wrapped = []
+
+    def probe(x):
+        wrapped.append(itf._plain_eager(x))
+        return x.float().sum()
+
+    torch.func.grad(probe)(torch.randn(4))
+    assert wrapped == [False]
+    assert not itf._nothing_to_differentiate(True, q.requires_grad_(True))
+    assert itf._nothing_to_differentiate(False, q)
+
+
 def test_product_package_never_imports_the_oracle():
     pkg = os.path.join(ROOT, "flash-dmattn_amd")
     for dirpath, _, files in os.walk(pkg):

@@ -262,3 +262,61 @@ def test_per_query_mask_of_column_causal_form_takes_the_column_mask_kernels():
         for g, r, name in ((got[2], rdq, "dq"), (got[3], rdk, "dk"), (got[4], rdv, "dv"), (got[5], rdb, "dbias")):
             assert_grad_close(g.cpu(), r, name)
     assert not torch.equal(recognised[0], fallback[0])
+
+
+@pytest.mark.parametrize("mode", ["2", "auto"])
+def test_builder_mask_wider_than_the_keys_is_scanned_not_trusted(mode):
+    """A mask from the device builder whose key length is the keys' rounded up to 128 (a caller that pads mask and bias
+    first): its lists number the columns of the WIDE row, kept columns beyond the keys included, so the attention call
+    must not take them.  Results equal those of the same values as a plain tensor (bit for bit) and the C oracle on the
+    first Lk columns."""
+    from _util import assert_grad_close, assert_out_close
+    from oracle import c_oracle
+
+    B, Lq, Lk, H, Hk, D, W = 2, 200, 300, 4, 2, 64, 120
+    Lw = 384
+    q, k, v, _ = _inputs(B, Lq, Lk, H, Hk, D, Hk, seed=21)
+    bias = torch.randn(B, Hk, 1, Lw, generator=torch.Generator().manual_seed(22)).to(torch.bfloat16).to(DEV)
+    set_compact(mode)
+    try:
+        mask = M.topk_mask(bias, None, W, torch.finfo(bias.dtype).min)
+        assert M.kept_keys_of(mask) is not None and mask.shape[-1] == Lw
+        assert int(mask[..., Lk:].sum()) > 0  # (kept columns beyond the keys exist: the lists would point past K)
+        with_lists = _run(q, k, v, mask, bias[..., :Lk])
+        scanned = _run(q, k, v, mask.clone(), bias[..., :Lk])
+    finally:
+        set_compact("auto")
+    for a, b in zip(with_lists, scanned):
+        assert torch.equal(a, b)
+    qc, kc, vc, mc, bc = [t.cpu() for t in (q, k, v, mask[..., :Lk], bias[..., :Lk])]
+    ro, _ = c_oracle.forward(qc, kc, vc, mc, bc, None, True)
+    rdq, rdk, rdv, rdb = c_oracle.backward(qc, kc, vc, torch.ones_like(ro), mc, bc, None, True)
+    assert_out_close(with_lists[0].cpu(), ro)
+    for g, r, name in ((with_lists[2], rdq, "dq"), (with_lists[3], rdk, "dk"), (with_lists[4], rdv, "dv")):
+        assert_grad_close(g.cpu(), r, name)
+    assert_grad_close(with_lists[5].cpu(), rdb, "dbias")
+
+
+@pytest.mark.parametrize("mode", ["2", "auto"])
+def test_builder_mask_with_key_dim_one_is_expanded_not_trusted(mode):
+    """A builder-made mask with a key dimension of 1 (one keep decision for every key) carries lists for a row of one
+    column; the operator expands the mask over the keys and must scan it instead."""
+    B, Lq, Lk, H, Hk, D = 1, 128, 256, 4, 2, 64
+    q, k, v, _ = _inputs(B, Lq, Lk, H, Hk, D, Hk, seed=23)
+    bias1 = torch.randn(B, Hk, 1, 1, generator=torch.Generator().manual_seed(24)).to(torch.bfloat16).to(DEV)
+    set_compact(mode)
+    try:
+        mask = M.topk_mask(bias1, None, 1, torch.finfo(bias1.dtype).min)
+        assert mask.shape[-1] == 1 and bool(mask.all())
+        qg, kg, vg = [t.detach().clone().requires_grad_(True) for t in (q, k, v)]
+        out = flash_sparse_attn_func(qg, kg, vg, mask, None, None, True)
+        out.backward(torch.ones_like(out))
+        q2, k2, v2 = [t.detach().clone().requires_grad_(True) for t in (q, k, v)]
+        out2 = flash_sparse_attn_func(q2, k2, v2, None, None, None, True)
+        out2.backward(torch.ones_like(out2))
+        torch.cuda.synchronize()
+    finally:
+        set_compact("auto")
+    assert (out.float() - out2.float()).abs().max().item() <= 2e-2
+    for a, b in ((qg.grad, q2.grad), (kg.grad, k2.grad), (vg.grad, v2.grad)):
+        assert (a.float() - b.float()).abs().max().item() <= 5e-2 * b.float().abs().max().item()
