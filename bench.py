@@ -1,15 +1,17 @@
 #!/usr/bin/env python3
 """Benchmark of the dynamic-mask attention hot path on one MI355X.
 
-    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all] [--no-cpu]
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--all] [--legs a,b,...] [--no-cpu]
 
 A "step" is one forward pass of `flash_sparse_attn_func` over one synthetic batch of the headline
 configuration: B=1, Lq=Lk=8192, H=32, Hkv=8 (GQA 4:1), d=128, bf16, bias [B,Hkv,1,Lk] ~ N(0,1),
 keep-mask = per-row top-2048 keys by bias intersected with causal, scale 1/sqrt(128).
 Prints ONE JSON line.  `value` is the forward's effective TFLOP/s counting only executed tiles on
 the canonical 64x64 tile grid (a tile is executed iff it holds at least one mask-and-causal-visible
-element); forward+backward, the other configurations, the roofline of the dominant kernel and a CPU
-baseline on the host cores ride along in the same line.
+element); forward+backward, the other benchmark configurations (`configs`: cfg3 and the decode shape cfg5
+against HBM, cfg4 against the matrix pipe, each with its own roofline block), the forward's runtime against the
+window W (`w_sweep_fwd`, with the fitted line), the roofline of the dominant kernel and a CPU baseline on the host
+cores ride along in the same line.
 
 Inputs are resident in HBM before the timed region starts; timing uses HIP events on the stream the
 kernels are launched on (torch's current stream).
@@ -233,7 +235,7 @@ def run_config(name, steps, warmup, device, compact=True, backward=True, zero_in
     res["ms_fwd"] = ms_fwd
     if c["Lq"] > 1:
         n_exec, n_causal, nnz = count_tiles(mask, c["Lq"], c["Lk"], c["causal"], c["H"])
-        res.update(n_exec=n_exec, tile_occupancy=n_exec / max(1, n_causal), nnz=nnz)
+        res.update(n_exec=n_exec, n_causal_tiles=n_causal, tile_occupancy=n_exec / max(1, n_causal), nnz=nnz)
         res["compacted"] = compaction_applies(mask, c)
         if res["compacted"]:
             # the kernels run on the compacted key axis: their executed tiles are counted there; the tile
@@ -263,9 +265,9 @@ def run_config(name, steps, warmup, device, compact=True, backward=True, zero_in
         dout = torch.ones_like(q)  # upstream gradient, resident like the other inputs
 
         def step():
+            qg.grad = kg.grad = vg.grad = bg.grad = None  # (first: no accumulation pass over a gradient left from the step before)
             out = flash_sparse_attn_func(qg, kg, vg, mask, bg, scale, c["causal"])
             out.backward(dout)
-            qg.grad = kg.grad = vg.grad = bg.grad = None
 
         ms_fb = time_gpu(step, max(2, steps // 2), max(1, warmup // 2))
         res["ms_fwd_bwd"] = ms_fb
@@ -293,6 +295,107 @@ def run_mfma_probe():
     for mode, name in enumerate(names):
         out[name] = {"constant_operands": lib.fdma_probe_mfma_tflops(mode, 0), "random_operands": lib.fdma_probe_mfma_tflops(mode, 1)}
     return out
+
+
+def config_roofline(name, r):
+    """Roofline block of one of the secondary configurations (the headline's is built in main()): the bound that
+    SURVEY-style accounting assigns to the configuration, the algorithmic work per call and what the measured call
+    time makes of it.  Durations are whole operator calls (all launches of the call), timed with events on the
+    launch stream."""
+    c = CONFIGS[name]
+    if c["Lq"] == 1:  # decode: HBM, touched K / V rows + side inputs
+        blk = {"bound": "hbm", "unit": "GB/s", "peak": PEAK_HBM_GBS, "bytes_per_call": r["touched_bytes"],
+               "bytes_model": "2 (K, V) * kept rows * d * 2 B + mask bytes + bias + q / out; kept rows counted from the mask",
+               "achieved": r["hbm_gbs"], "frac": r["hbm_gbs"] / PEAK_HBM_GBS, "duration_ms": r["ms_fwd"],
+               "kernel": "fdma::decode_kernel (+ combine), whole operator call"}
+        if "ms_fwd_c_abi" in r:
+            gbs = r["touched_bytes"] / r["ms_fwd_c_abi"] / 1e6
+            blk["c_abi_call"] = {"duration_ms": r["ms_fwd_c_abi"], "achieved": gbs, "frac": gbs / PEAK_HBM_GBS}
+        return blk
+    if r["mask_form"].endswith("Lq,Lk] bool + is_causal"):  # per-query mask and bias: HBM
+        B, H, Lq, Lk, D = c["B"], c["H"], c["Lq"], c["Lk"], c["D"]
+        n_causal = r["n_causal_tiles"]
+        q_bytes, kv_bytes, lse_bytes = 2.0 * B * Lq * H * D, 2.0 * B * Lk * c["Hk"] * D, 4.0 * B * H * Lq
+        tiles = n_causal * 64 * 64 * 1.0 + r["n_exec"] * 64 * 64 * 2.0  # mask of every causal tile, bias of every executed one
+        fwd = tiles + 2 * q_bytes + 2 * kv_bytes + lse_bytes            # q, out, k, v
+        # backward, algorithmic minimum: the tiles once more, every dBias element written once (zeros included),
+        # q / out / dout read and dq written, k / v read and dk / dv written
+        bwd = tiles + 2.0 * B * H * Lq * Lk + 4 * q_bytes + 4 * kv_bytes + lse_bytes
+        blk = {"bound": "hbm", "unit": "GB/s", "peak": PEAK_HBM_GBS, "bytes_per_call": fwd,
+               "bytes_model": "forward: mask bytes of every causal 64x64 tile + bias of every executed tile + q, k, v, out, lse; "
+                              "forward + backward adds the same tiles once more, the full dBias write, dout and the gradients "
+                              "(the two backward kernels each read the tiles: the measured traffic is higher)",
+               "achieved": fwd / r["ms_fwd"] / 1e6, "frac": fwd / r["ms_fwd"] / 1e6 / PEAK_HBM_GBS, "duration_ms": r["ms_fwd"],
+               "kernel": "fdma::fwd_kernel (per-query mask / bias), whole operator call"}
+        if "ms_fwd_bwd" in r:
+            tot = fwd + bwd
+            blk["fwd_bwd"] = {"bytes_per_call": tot, "duration_ms": r["ms_fwd_bwd"], "achieved": tot / r["ms_fwd_bwd"] / 1e6,
+                              "frac": tot / r["ms_fwd_bwd"] / 1e6 / PEAK_HBM_GBS,
+                              "kernels": "fwd_kernel, bwd_dot_kernel, bwd_dkdv_kernel, bwd_dq_kernel"}
+        return blk
+    flops = 4.0 * 64 * 64 * c["D"] * r["n_exec"]
+    blk = {"bound": "mfma", "unit": "TFLOP/s", "peak": PEAK_BF16_TFLOPS, "flops_per_call": flops,
+           "flops_model": "4*64*64*d per executed 64x64 tile (compacted key axis when column_compaction), 14*... forward + backward",
+           "column_compaction": bool(r.get("compacted")), "n_exec_tiles": r["n_exec"],
+           "achieved": r["tflops_fwd"], "frac": r["tflops_fwd"] / PEAK_BF16_TFLOPS, "duration_ms": r["ms_fwd"],
+           "kernel": "fdma::fwd_colmask_kernel with its pre-pass, whole operator call"}
+    if "ms_fwd_bwd" in r:
+        blk["fwd_bwd"] = {"flops_per_call": 3.5 * flops, "duration_ms": r["ms_fwd_bwd"], "achieved": r["tflops_fwd_bwd"],
+                          "frac": r["tflops_fwd_bwd"] / PEAK_BF16_TFLOPS}
+    return blk
+
+
+def time_decode_c_abi(name, steps, warmup, device):
+    """The decode configuration through the C ABI alone: one prepared argument block, fdma_fwd called back to back on
+    torch's current stream (what a serving loop written against include/fdma.h pays per call)."""
+    from flash_sparse_attn import _cabi
+
+    c = CONFIGS[name]
+    q, k, v, mask, bias = make_case(c, device)
+    out = torch.empty_like(q)
+    lse = torch.empty((c["B"], c["H"], c["Lq"]), dtype=torch.float32, device=device)
+    args = _cabi.FwdArgs()
+    _cabi.fill_fwd(args, q, k, v, mask, bias, out, lse, c["D"] ** -0.5, c["causal"], 0.0, None, None)
+    nbytes = _cabi.lib.fdma_fwd_workspace_bytes(args)
+    ws = torch.empty(max(1, nbytes), dtype=torch.uint8, device=device)
+    if nbytes:
+        args.workspace, args.workspace_bytes = ws.data_ptr(), nbytes
+    stream = _cabi.current_stream(device)
+
+    def call():
+        _cabi.check(_cabi.lib.fdma_fwd(args, stream))
+
+    return time_gpu(call, steps, warmup)
+
+
+def run_w_sweep_fwd(steps, warmup, device):
+    """Forward time against the window W at L = 8192 (H=32, Hkv=8, d=128, bias [1,8,1,L], mask = top-W of the bias,
+    causal), default path and tile skipping alone, with a least-squares line ms = a + b * W per path (the reference's
+    claim: runtime grows linearly with the window, README.md:181-191, benchmarks/forward_performance.py:661-718)."""
+    rows = []
+    for W in (256, 512, 1024, 2048, 4096, 8192):
+        CONFIGS["_sweep"] = dict(B=1, Lq=8192, Lk=8192, H=32, Hk=8, D=128, bias=(1, 8, 1, 8192), W=W, causal=True, bwd=False, scale=None)
+        row = {"W": W}
+        for compact, tag in ((True, "default"), (False, "tile_skip")):
+            r = run_config("_sweep", steps, warmup, device, compact, backward=False)
+            row["ms_fwd_" + tag] = r["ms_fwd"]
+            row["n_exec_" + tag] = r["n_exec"]
+            row["tflops_fwd_" + tag] = r["tflops_fwd"]
+        rows.append(row)
+    del CONFIGS["_sweep"]
+    fits = {col: _fit_line([r["W"] for r in rows], [r[col] for r in rows]) for col in ("ms_fwd_default", "ms_fwd_tile_skip")}
+    return {"L": 8192, "points": rows, "fit_ms_vs_W": fits}
+
+
+def _fit_line(xs, ys):
+    n = len(xs)
+    mx, my = sum(xs) / n, sum(ys) / n
+    sxx = sum((x - mx) ** 2 for x in xs)
+    b = sum((x - mx) * (y - my) for x, y in zip(xs, ys)) / sxx
+    a = my - b * mx
+    ss_res = sum((y - (a + b * x)) ** 2 for x, y in zip(xs, ys))
+    ss_tot = sum((y - my) ** 2 for y in ys) or 1.0
+    return {"intercept_ms": a, "slope_ms_per_1024": b * 1024, "r2": 1.0 - ss_res / ss_tot}
 
 
 def run_mask_builder(steps, warmup, device):
@@ -436,15 +539,7 @@ def run_sweeps(steps, warmup, device):
     benchmarks/forward_performance.py:661-718), for both paths of the column-mask kernels.  Shapes: H=32, Hkv=8, d=128,
     bias [1,8,1,L], mask = top-W of the bias per row, causal.  W sweep at L=8192; L sweep at W=1024.  A least-squares
     line ms = a + b * x is fitted to every column."""
-    def fit(xs, ys):
-        n = len(xs)
-        mx, my = sum(xs) / n, sum(ys) / n
-        sxx = sum((x - mx) ** 2 for x in xs)
-        b = sum((x - mx) * (y - my) for x, y in zip(xs, ys)) / sxx
-        a = my - b * mx
-        ss_res = sum((y - (a + b * x)) ** 2 for x, y in zip(xs, ys))
-        ss_tot = sum((y - my) ** 2 for y in ys) or 1.0
-        return {"intercept_ms": a, "slope_ms_per_1024": b * 1024, "r2": 1.0 - ss_res / ss_tot}
+    fit = _fit_line
 
     def sweep(points, key):
         rows = []
@@ -499,14 +594,22 @@ def cpu_baseline(device_cfg="cfg2", groups=8, chunk=2):
             "ms_scaled_to_full": dt * 1e3 * c["Hk"] / groups}
 
 
+DEFAULT_LEGS = ("cfg2", "tile_skip", "zero", "probe", "cfg3", "cfg4", "cfg5", "w_sweep", "cpu")
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--all", action="store_true", help="also time configurations 1, 3, 4, 5")
+    ap.add_argument("--all", action="store_true",
+                    help="also: cfg1, mask builder, bias producer, hand-overs, ragged batch, forward + backward sweeps over W and L")
+    ap.add_argument("--legs", default=None,
+                    help="comma-separated subset of the default legs to run (" + ", ".join(DEFAULT_LEGS) + "); a profile of one "
+                         "leg then holds one workload per kernel.  cfg2 (the headline) always runs")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-probe", action="store_true", help="skip the matrix-pipe probe (MFMA rate on constant / random operands)")
+    ap.add_argument("--no-backward", action="store_true", help="forward legs only")
     ap.add_argument("--no-compact", action="store_true",
                     help="switch the column-compaction path off (compact_mode = never): time the tile-skipping kernels")
     ap.add_argument("--calib-copy", action="store_true",
@@ -525,10 +628,21 @@ def main():
     if not torch.cuda.is_available():
         print("bench.py needs an MI355X", file=sys.stderr)
         sys.exit(1)
+    legs = set(DEFAULT_LEGS if args.legs is None else [x for x in args.legs.split(",") if x])
+    unknown = legs - set(DEFAULT_LEGS)
+    if unknown:
+        print("unknown legs: " + ", ".join(sorted(unknown)), file=sys.stderr)
+        sys.exit(2)
+    if args.no_cpu:
+        legs.discard("cpu")
+    if args.no_probe:
+        legs.discard("probe")
     device = torch.device("cuda:0")
     torch.cuda.set_device(device)
     compact = not args.no_compact
-    main_res = run_config("cfg2", args.steps, args.warmup, device, compact)
+    bwd = not args.no_backward
+    half = (max(3, args.steps // 2), max(1, args.warmup // 2))
+    main_res = run_config("cfg2", args.steps, args.warmup, device, compact, backward=bwd)
     c = CONFIGS["cfg2"]
     if main_res["compacted"]:
         kernel = ("fdma::fwd_colmask_kernel<bf16, 128, causal, compacted>, with its pre-pass (compact_scan_gather_kernel) "
@@ -573,27 +687,28 @@ def main():
             "duration_ms": main_res["ms_fwd"],
         },
     }
-    if compact:
+    if main_res.get("ms_fwd_bwd"):
+        out["roofline"]["fwd_bwd"] = {"flops_per_call": 14.0 * 64 * 64 * c["D"] * main_res["n_exec"], "duration_ms": main_res["ms_fwd_bwd"],
+                                      "achieved": main_res["tflops_fwd_bwd"], "frac": main_res["tflops_fwd_bwd"] / PEAK_BF16_TFLOPS}
+    if compact and "tile_skip" in legs:
         # the same workload through the tile-skipping kernel alone (one kernel per call, no pre-pass)
-        ts = run_config("cfg2", max(3, args.steps // 2), max(1, args.warmup // 2), device, compact=False, backward=False)
+        ts = run_config("cfg2", *half, device, compact=False, backward=False)
         out["tile_skip_path"] = {"ms_fwd": ts["ms_fwd"], "n_exec_tiles": ts["n_exec"], "tflops_fwd": ts["tflops_fwd"],
                                  "frac_of_peak": ts["tflops_fwd"] / PEAK_BF16_TFLOPS,
                                  "kernel": "fdma::fwd_colmask_kernel<bf16, 128, causal> (compact_mode = never)"}
-        # The same launch on all-zero Q / K / V / bias: identical mask, tiles and instruction stream.  The device lowers
+    if compact and "zero" in legs:
+        # The same launches on all-zero Q / K / V / bias: identical mask, tiles and instruction stream.  The device lowers
         # its clocks under the switching activity of real operands (a register-fed MFMA loop reaches 2.4 PFLOP/s on
-        # constant operands and 1.9 on random ones), so this is what the kernel's schedule sustains when it does not.
-        tz = run_config("cfg2", max(3, args.steps // 2), max(1, args.warmup // 2), device, compact=False, backward=False,
-                        zero_inputs=True)
-        out["tile_skip_path"]["zero_operands"] = {"ms_fwd": tz["ms_fwd"], "tflops_fwd": tz["tflops_fwd"],
-                                                  "frac_of_peak": tz["tflops_fwd"] / PEAK_BF16_TFLOPS}
-        # ... and the default path (forward and forward + backward) on all-zero operands
-        cz = run_config("cfg2", max(3, args.steps // 2), max(1, args.warmup // 2), device, compact=True, backward=True,
-                        zero_inputs=True)
+        # constant operands and 1.9 on random ones), so this is what the kernels' schedule sustains when it does not.
+        tz = run_config("cfg2", *half, device, compact=False, backward=False, zero_inputs=True)
+        out.setdefault("tile_skip_path", {})["zero_operands"] = {"ms_fwd": tz["ms_fwd"], "tflops_fwd": tz["tflops_fwd"],
+                                                                 "frac_of_peak": tz["tflops_fwd"] / PEAK_BF16_TFLOPS}
+        cz = run_config("cfg2", *half, device, compact=True, backward=bwd, zero_inputs=True)
         out["zero_operands"] = {"ms_fwd": cz["ms_fwd"], "tflops_fwd": cz["tflops_fwd"],
                                 "frac_of_peak": cz["tflops_fwd"] / PEAK_BF16_TFLOPS, "ms_fwd_bwd": cz.get("ms_fwd_bwd"),
                                 "note": "same mask, tiles and instruction stream as the headline figures, all-zero Q / K / V / "
                                         "bias: what the schedule sustains when the device does not lower its clock"}
-    if not args.no_probe:
+    if "probe" in legs:
         probe = run_mfma_probe()
         if probe is not None:
             out["mfma_probe"] = probe
@@ -604,16 +719,35 @@ def main():
         dst = torch.empty_like(src)
         dst.copy_(src)
         torch.cuda.synchronize()
+    # The other benchmark configurations, each against the roofline that bounds it: cfg3 (a bias and a mask per query
+    # row, with its dBias) and cfg5 (decode) against HBM, cfg4 (long sequence, narrow window) against the matrix pipe.
+    quarter = (max(3, args.steps // 4), max(1, args.warmup // 2))
+    configs = {}
+    for name in ("cfg3", "cfg4", "cfg5"):
+        if name not in legs:
+            continue
+        r = run_config(name, *quarter, device, compact, backward=bwd)
+        if name == "cfg5":
+            r["ms_fwd_c_abi"] = time_decode_c_abi(name, args.steps, args.warmup, device)
+        c2 = CONFIGS[name]
+        r["workload"] = "%s: B=%d Lq=%d Lk=%d H=%d Hkv=%d d=%d bias%s top-%d%s" % (
+            name, c2["B"], c2["Lq"], c2["Lk"], c2["H"], c2["Hk"], c2["D"], list(c2["bias"]), c2["W"], " ∩ causal" if c2["causal"] else "")
+        r["roofline"] = config_roofline(name, r)
+        configs[name] = r
+        torch.cuda.empty_cache()
+    if configs:
+        out["configs"] = configs
+    if "w_sweep" in legs:
+        out["w_sweep_fwd"] = run_w_sweep_fwd(*quarter, device)
     if args.all:
-        out["other_configs"] = [run_config(n, max(3, args.steps // 4), max(1, args.warmup // 2), device, compact)
-                                for n in ("cfg1", "cfg3", "cfg4", "cfg5")]
-        out["mask_builder"] = run_mask_builder(max(3, args.steps // 2), max(1, args.warmup // 2), device)
-        out["bias_producer"] = run_bias_producer(max(3, args.steps // 2), max(1, args.warmup // 2), device)
+        out["cfg1"] = run_config("cfg1", *quarter, device, compact)
+        out["mask_builder"] = run_mask_builder(*half, device)
+        out["bias_producer"] = run_bias_producer(*half, device)
         out["kept_list_handoff"] = run_kept_list_handoff(args.steps, args.warmup, device)
-        out["mask_bits_handoff"] = run_mask_bits_handoff(max(3, args.steps // 2), max(1, args.warmup // 2), device)
-        out["ragged_batch"] = run_ragged_batch(max(3, args.steps // 4), max(1, args.warmup // 2), device)
-        out.update(run_sweeps(max(3, args.steps // 4), max(1, args.warmup // 2), device))
-    if not args.no_cpu:
+        out["mask_bits_handoff"] = run_mask_bits_handoff(*half, device)
+        out["ragged_batch"] = run_ragged_batch(*quarter, device)
+        out.update(run_sweeps(*quarter, device))
+    if "cpu" in legs:
         out["cpu_baseline"] = cpu_baseline("cfg2", groups=8)
     print(json.dumps(out))
 
