@@ -307,7 +307,7 @@ def config_roofline(name, r):
         blk = {"bound": "hbm", "unit": "GB/s", "peak": PEAK_HBM_GBS, "bytes_per_call": r["touched_bytes"],
                "bytes_model": "2 (K, V) * kept rows * d * 2 B + mask bytes + bias + q / out; kept rows counted from the mask",
                "achieved": r["hbm_gbs"], "frac": r["hbm_gbs"] / PEAK_HBM_GBS, "duration_ms": r["ms_fwd"],
-               "kernel": "fdma::decode_kernel (+ combine), whole operator call"}
+               "kernel": "fdma::decode_kernel (the last workgroup of a (batch entry, kv head) merges the splits), whole operator call"}
         if "ms_fwd_c_abi" in r:
             gbs = r["touched_bytes"] / r["ms_fwd_c_abi"] / 1e6
             blk["c_abi_call"] = {"duration_ms": r["ms_fwd_c_abi"], "achieved": gbs, "frac": gbs / PEAK_HBM_GBS}
@@ -360,6 +360,10 @@ def time_decode_c_abi(name, steps, warmup, device):
     ws = torch.empty(max(1, nbytes), dtype=torch.uint8, device=device)
     if nbytes:
         args.workspace, args.workspace_bytes = ws.data_ptr(), nbytes
+    cbytes = _cabi.lib.fdma_fwd_counter_bytes(args)  # arrival counters: the splits are merged by the decode launch itself
+    counters = torch.zeros(max(1, cbytes // 4), dtype=torch.int32, device=device)
+    if cbytes:
+        args.counters, args.counters_bytes = counters.data_ptr(), cbytes
     stream = _cabi.current_stream(device)
 
     def call():
@@ -726,9 +730,11 @@ def main():
     for name in ("cfg3", "cfg4", "cfg5"):
         if name not in legs:
             continue
-        r = run_config(name, *quarter, device, compact, backward=bwd)
-        if name == "cfg5":
-            r["ms_fwd_c_abi"] = time_decode_c_abi(name, args.steps, args.warmup, device)
+        if name == "cfg5":  # (a call of some 20 us: many steps, or the two events' own resolution shows)
+            r = run_config(name, 10 * args.steps, 2 * args.warmup, device, compact, backward=False)
+            r["ms_fwd_c_abi"] = time_decode_c_abi(name, 10 * args.steps, 2 * args.warmup, device)
+        else:
+            r = run_config(name, *quarter, device, compact, backward=bwd)
         c2 = CONFIGS[name]
         r["workload"] = "%s: B=%d Lq=%d Lk=%d H=%d Hkv=%d d=%d bias%s top-%d%s" % (
             name, c2["B"], c2["Lq"], c2["Lk"], c2["H"], c2["Hk"], c2["D"], list(c2["bias"]), c2["W"], " ∩ causal" if c2["causal"] else "")

@@ -262,9 +262,14 @@ int fdma_fwd_validate(const fdma_fwd_args *a) {
     return validate_common(a, false);
 }
 
+size_t fdma_fwd_counter_bytes(const fdma_fwd_args *a) {
+    if (!a || a->seqlen_k <= 0 || a->num_heads_k <= 0 || !fdma::use_decode_path(a->seqlen_q, a->num_heads, a->num_heads_k)) return 0;
+    return (size_t)round_up(fdma::decode_num_counters(a->batch, a->num_heads, a->num_heads_k, a->seqlen_k) * 4, 256);
+}
+
 size_t fdma_fwd_workspace_bytes(const fdma_fwd_args *a) {
     if (!a) return 0;
-    if (!fdma::use_decode_path(a->seqlen_q, a->num_heads, a->num_heads_k) || a->head_dim > 128) {  // (the split-KV kernel is built up to head dim 128)
+    if (!fdma::use_decode_path(a->seqlen_q, a->num_heads, a->num_heads_k)) {
         fdma::FwdParams p;
         fill_fwd_params(a, p);
         return fdma::use_compact(p) ? fdma::compact_bytes(p, false) : 0;
@@ -285,7 +290,7 @@ int fdma_fwd(const fdma_fwd_args *a, void *hip_stream) {
     hipStream_t stream = static_cast<hipStream_t>(hip_stream);
     hipError_t e;
     if (a->seqlen_q == 0) return FDMA_OK;
-    if (fdma::use_decode_path(a->seqlen_q, a->num_heads, a->num_heads_k) && a->head_dim <= 128 && a->seqlen_k > 0) {
+    if (fdma::use_decode_path(a->seqlen_q, a->num_heads, a->num_heads_k) && a->seqlen_k > 0) {
         p.splits = fdma::decode_num_splits(a->batch, a->num_heads_k, a->seqlen_k);
         if (p.splits > 1) {
             const size_t need = fdma_fwd_workspace_bytes(a);
@@ -294,6 +299,13 @@ int fdma_fwd(const fdma_fwd_args *a, void *hip_stream) {
             const size_t rows = (size_t)p.splits * a->batch * a->num_heads * a->seqlen_q;
             p.o_part = static_cast<float *>(a->workspace);
             p.lse_part = p.o_part + rows * a->head_dim;
+            if (a->counters) {
+                const size_t cneed = fdma_fwd_counter_bytes(a);
+                if (a->counters_bytes < cneed)
+                    return fail(FDMA_ERR_WORKSPACE, "decode arrival counters too small: need %zu bytes, got %zu", cneed, a->counters_bytes);
+                if (reinterpret_cast<uintptr_t>(a->counters) & 3) return fail(FDMA_ERR_INVALID, "counters must be 4-byte aligned");
+                p.dec_counter = a->counters;
+            }
         }
         e = fdma::launch_fwd_decode(p, a->dtype, stream);
     } else {
@@ -316,17 +328,26 @@ int fdma_fwd_noalloc(const fdma_fwd_args *a, void *hip_stream) {
     int rc = validate_common(a, false);
     if (rc != FDMA_OK) return rc;
     const size_t need = fdma_fwd_workspace_bytes(a);
-    if (need > (size_t)FDMA_NOALLOC_SCRATCH_BYTES)
+    constexpr size_t kUsable = (size_t)FDMA_NOALLOC_SCRATCH_BYTES - FDMA_NOALLOC_COUNTER_BYTES;
+    if (need > kUsable)
         return fail(FDMA_ERR_WORKSPACE, "fdma_fwd_noalloc: this problem needs %zu bytes of scratch, the library's static scratch holds %zu",
-                    need, (size_t)FDMA_NOALLOC_SCRATCH_BYTES);
+                    need, kUsable);
     fdma_fwd_args with_scratch = *a;
     with_scratch.workspace = nullptr;
     with_scratch.workspace_bytes = 0;
+    with_scratch.counters = nullptr;
+    with_scratch.counters_bytes = 0;
     if (need) {
         void *ptr = nullptr;
         if ((rc = scratch_of_current_device(&ptr)) != FDMA_OK) return rc;
         with_scratch.workspace = ptr;
-        with_scratch.workspace_bytes = FDMA_NOALLOC_SCRATCH_BYTES;
+        with_scratch.workspace_bytes = kUsable;
+        // the array's tail: zero since the library was loaded, put back to zero by every decode call that used it
+        // (more counters than fit there: the merge stays a launch of its own)
+        if (fdma_fwd_counter_bytes(a) <= (size_t)FDMA_NOALLOC_COUNTER_BYTES) {
+            with_scratch.counters = reinterpret_cast<int32_t *>(static_cast<unsigned char *>(ptr) + kUsable);
+            with_scratch.counters_bytes = FDMA_NOALLOC_COUNTER_BYTES;
+        }
     }
     return fdma_fwd(&with_scratch, hip_stream);
 }

@@ -1,4 +1,6 @@
-// Single-token decode (seqlen_q == 1) for gfx950: split-KV partial attention + LSE-weighted combine.
+// Single-token decode (seqlen_q == 1) for gfx950: split-KV partial attention + LSE-weighted combine -- in ONE launch
+// when the caller provides arrival counters (the last workgroup of a (batch entry, head chunk) to finish merges the
+// splits), otherwise as a second launch.
 //
 // Replaces the reference's decode route: the `seqlenq_ngroups_swapped` reshaping of mha_fwd
 // (csrc/flash_sparse_attn/flash_api.cpp:443-475, 541-551), num_splits_heuristic (:275-349),
@@ -61,8 +63,76 @@ __device__ __forceinline__ uint32_t nz_bytes_to_bits(uint32_t x) {
 
 // PERHEAD: mask or bias differ between the query heads of a group, so a lane fetches the mask byte and the
 // bias of its own (key, head) pairs; otherwise one fused value per key serves all columns.
+// out[b,h,:] = sum_s exp(lse_s - lse) * o_s ;  lse = logsumexp_s lse_s  (empty everywhere: 0 / +inf) for one (b, h) row,
+// by ONE wave: lane s (and s + 64) fetches lse_s, the weights are made once and left in the wave's own piece of LDS
+// (`s_w`, room for 128 floats), then lane e sums its head-dim elements over the splits with the loads of eight splits
+// in flight: two dependent trips to memory per row, whatever the number of splits.  COHERENT: the partials were written
+// by other workgroups of the SAME launch (possibly on another XCD, behind another L2): they are fetched with
+// device-scope loads.  Both users of this function sum in the same order, so their results agree bit for bit.
+template <bool COHERENT> __device__ __forceinline__ float part_load(const float *ptr) {
+    if (COHERENT) return __uint_as_float(__hip_atomic_load((const uint32_t *)ptr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT));
+    return *ptr;
+}
+
+__device__ __forceinline__ void part_store(float *ptr, float v) {
+    __hip_atomic_store((uint32_t *)ptr, __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+template <typename T, bool COHERENT>
+__device__ __forceinline__ void combine_row(const FwdParams &p, int64_t row, int lane, float *s_w) {
+    using E = Elem<T>;
+    const int64_t rows = (int64_t)p.B * p.H;
+    const float lv0 = lane < p.splits ? part_load<COHERENT>(p.lse_part + (int64_t)lane * rows + row) : -INFINITY;
+    const float lv1 = lane + 64 < p.splits ? part_load<COHERENT>(p.lse_part + (int64_t)(lane + 64) * rows + row) : -INFINITY;
+    // the partial outputs of the first eight splits for this lane's first two elements are requested right behind
+    // the LSEs (they do not depend on them): one trip to memory instead of two for up to eight splits
+    const int64_t step = rows * p.d;
+    const float *op_row = p.o_part + row * p.d;
+    const int n0 = p.splits < 8 ? p.splits : 8;
+    float v0[8], v1[8];
+#pragma unroll
+    for (int u = 0; u < 8; u++) {
+        v0[u] = (u < n0 && lane < p.d) ? part_load<COHERENT>(op_row + lane + (int64_t)u * step) : 0.f;
+        v1[u] = (u < n0 && lane + 64 < p.d) ? part_load<COHERENT>(op_row + lane + 64 + (int64_t)u * step) : 0.f;
+    }
+    float mx = fmaxf(lv0, lv1);
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
+    const float w0 = mx == -INFINITY ? 0.f : __expf(lv0 - mx), w1 = mx == -INFINITY ? 0.f : __expf(lv1 - mx);  // exp(-inf) = 0 for empty splits
+    float sum = w0 + w1;
+#pragma unroll
+    for (int off = 32; off >= 1; off >>= 1) sum += __shfl_xor(sum, off);
+    s_w[lane] = w0;
+    s_w[lane + 64] = w1;
+    __builtin_amdgcn_wave_barrier();  // (the LDS operations of one wave execute in order: the weights are readable below)
+    const float inv = sum > 0.f ? 1.f / sum : 0.f;
+    const int b = (int)(row / p.H), h = (int)(row % p.H);
+    for (int e = lane, n = 0; e < p.d; e += 64, n++) {
+        const float *op = op_row + e;
+        float acc = 0.f;
+        int s = 0;
+        if (n < 2) {  // (the splits in ascending order, as everywhere: sums do not depend on how they were fetched)
+#pragma unroll
+            for (int u = 0; u < 8; u++)
+                if (u < n0) acc = fmaf(s_w[u], n == 0 ? v0[u] : v1[u], acc);
+            s = n0;
+        }
+        for (; s + 8 <= p.splits; s += 8) {
+            float v[8];
+#pragma unroll
+            for (int u = 0; u < 8; u++) v[u] = part_load<COHERENT>(op + (int64_t)(s + u) * step);
+#pragma unroll
+            for (int u = 0; u < 8; u++) acc = fmaf(s_w[s + u], v[u], acc);
+        }
+        for (; s < p.splits; s++) acc = fmaf(s_w[s], part_load<COHERENT>(op + (int64_t)s * step), acc);
+        ((uint16_t *)p.o)[b * p.o_b + h * p.o_h + e] = (uint16_t)(E::pack2(acc * inv, 0.f) & 0xffffu);
+    }
+    if (lane == 0) p.lse[row] = mx == -INFINITY ? INFINITY : mx + __logf(sum);
+    __builtin_amdgcn_wave_barrier();  // (s_w is rewritten for the wave's next row)
+}
+
 template <typename T, int D, bool PERHEAD, bool WIDE>
-__global__ void __launch_bounds__(DEC_THREADS, 2) decode_kernel(const FwdParams p, int keys_per_split) {
+__global__ void __launch_bounds__(DEC_THREADS, D <= 128 ? 2 : 1) decode_kernel(const FwdParams p, int keys_per_split) {
     using E = Elem<T>;
     using SM = DecSmem<D>;
     constexpr int CH = D / 8;         // 16-byte chunks per row
@@ -357,64 +427,53 @@ __global__ void __launch_bounds__(DEC_THREADS, 2) decode_kernel(const FwdParams 
         const int hh = hk * G + g0 + col;
         const float inv = lt > 0.f ? 1.f / lt : 0.f;
         if (p.splits > 1) {
+            // (device-scope stores: written through to where every XCD sees them, so that the merging workgroup of
+            // this launch -- or the merge launch -- reads them whichever L2 it sits behind)
             const int64_t row = ((int64_t)split * p.B + b) * p.H + hh;
-            p.o_part[row * p.d + e] = ot * inv;
-            if (e == 0) p.lse_part[row] = lt > 0.f ? (mx + __builtin_amdgcn_logf(lt)) * kLn2 : -INFINITY;
+            part_store(p.o_part + row * p.d + e, ot * inv);
+            if (e == 0) part_store(p.lse_part + row, lt > 0.f ? (mx + __builtin_amdgcn_logf(lt)) * kLn2 : -INFINITY);
         } else {
             uint16_t *op = (uint16_t *)p.o + b * p.o_b + hh * p.o_h;
             op[e] = (uint16_t)(E::pack2(ot * inv, 0.f) & 0xffffu);
             if (e == 0) p.lse[(int64_t)b * p.H + hh] = lt > 0.f ? (mx + __builtin_amdgcn_logf(lt)) * kLn2 : INFINITY;
         }
     }
+    // ---- phase 4 (arrival counters given): the workgroup that finishes last among the splits of its (batch entry,
+    // head chunk) merges their partial results, so the call is one launch.  The partials above are device-scope
+    // stores; every wave waits until its own have been acknowledged, the barrier collects the waves, and one thread
+    // then counts the workgroup in with a device-scope atomic (no cache write-back or invalidate is involved: a fence
+    // would walk the whole L2 in every workgroup, which made this launch four times longer than the two it replaces).
+    // The counter starts at zero, and the last arrival puts it back to zero for the next call.  Nothing waits for
+    // another workgroup: one that is not last just ends.
+    if (p.splits > 1 && p.dec_counter) {
+        __shared__ int s_last;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) {
+            int32_t *cnt = p.dec_counter + ((int64_t)b * gridDim.y + blockIdx.y);
+            const int old = __hip_atomic_fetch_add(cnt, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            const int last = old == p.splits - 1;
+            if (last) __hip_atomic_store(cnt, 0, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+            s_last = last;
+        }
+        __syncthreads();
+        if (s_last) {
+            for (int col = wave; col < ncol; col += 4)
+                combine_row<T, true>(p, (int64_t)b * p.H + hk * G + g0 + col, lane, (float *)(smem + wave * 512));
+        }
+    }
 }
 
-// out[b,h,:] = sum_s exp(lse_s - lse) * o_s ;  lse = logsumexp_s lse_s  (empty everywhere: 0 / +inf).
-// One workgroup per (b, h) row.  Thread s < splits fetches lse_s, the weights are made once per row and left in LDS,
-// then thread e sums its head-dim element over the splits with the loads of eight splits in flight: two dependent
-// trips to memory per row, whatever the number of splits.
-constexpr int CMB_THREADS = 128;  // >= the largest number of splits (decode_num_splits)
+// The merge as a launch of its own (no arrival counters given): one wave per (b, h) row, four rows per workgroup.
+constexpr int CMB_THREADS = 256;
+constexpr int CMB_MAX_SPLITS = 128;  // >= the largest number of splits (decode_num_splits): a lane holds two of them
 
 template <typename T>
 __global__ void __launch_bounds__(CMB_THREADS) decode_combine_kernel(const FwdParams p) {
-    using E = Elem<T>;
-    __shared__ float s_w[CMB_THREADS];
-    __shared__ float s_red[4];
-    const int64_t rows = (int64_t)p.B * p.H;
-    const int64_t row = blockIdx.x;
-    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const float lv = tid < p.splits ? p.lse_part[(int64_t)tid * rows + row] : -INFINITY;
-    float mx = lv;
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) mx = fmaxf(mx, __shfl_xor(mx, off));
-    if (lane == 0) s_red[wave] = mx;
-    __syncthreads();
-    mx = fmaxf(s_red[0], s_red[1]);
-    const float w = mx == -INFINITY ? 0.f : __expf(lv - mx);  // exp(-inf) = 0 for empty splits
-    float sum = w;
-#pragma unroll
-    for (int off = 32; off >= 1; off >>= 1) sum += __shfl_xor(sum, off);
-    if (lane == 0) s_red[2 + wave] = sum;
-    s_w[tid] = w;
-    __syncthreads();
-    sum = s_red[2] + s_red[3];
-    const float inv = sum > 0.f ? 1.f / sum : 0.f;
-    const int b = (int)(row / p.H), h = (int)(row % p.H);
-    for (int e = tid; e < p.d; e += CMB_THREADS) {
-        const float *op = p.o_part + row * p.d + e;
-        const int64_t step = rows * p.d;
-        float acc = 0.f;
-        int s = 0;
-        for (; s + 8 <= p.splits; s += 8) {
-            float v[8];
-#pragma unroll
-            for (int u = 0; u < 8; u++) v[u] = op[(int64_t)(s + u) * step];
-#pragma unroll
-            for (int u = 0; u < 8; u++) acc = fmaf(s_w[s + u], v[u], acc);
-        }
-        for (; s < p.splits; s++) acc = fmaf(s_w[s], op[(int64_t)s * step], acc);
-        ((uint16_t *)p.o)[b * p.o_b + h * p.o_h + e] = (uint16_t)(E::pack2(acc * inv, 0.f) & 0xffffu);
-    }
-    if (tid == 0) p.lse[row] = mx == -INFINITY ? INFINITY : mx + __logf(sum);
+    __shared__ float s_w[CMB_THREADS / 64][CMB_MAX_SPLITS];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int64_t row = (int64_t)blockIdx.x * (CMB_THREADS / 64) + wave;
+    if (row < (int64_t)p.B * p.H) combine_row<T, false>(p, row, lane, s_w[wave]);
 }
 
 template <typename T, int D, bool PERHEAD, bool WIDE>
@@ -445,11 +504,12 @@ hipError_t launch_decode_t(const FwdParams &p, hipStream_t stream) {
     const bool perhead = G > 1 && ((p.mask && p.Hm == p.H) || (p.bias && p.Hb == p.H));
     hipError_t e;
     if (p.d <= 64) e = perhead ? launch_decode_d<T, 64, true>(p, keys_per_split, stream) : launch_decode_d<T, 64, false>(p, keys_per_split, stream);
-    else e = perhead ? launch_decode_d<T, 128, true>(p, keys_per_split, stream) : launch_decode_d<T, 128, false>(p, keys_per_split, stream);
+    else if (p.d <= 128) e = perhead ? launch_decode_d<T, 128, true>(p, keys_per_split, stream) : launch_decode_d<T, 128, false>(p, keys_per_split, stream);
+    else e = perhead ? launch_decode_d<T, 256, true>(p, keys_per_split, stream) : launch_decode_d<T, 256, false>(p, keys_per_split, stream);
     if (e != hipSuccess) return e;
-    if (p.splits > 1) {
+    if (p.splits > 1 && !p.dec_counter) {  // (with arrival counters the decode launch has merged its splits itself)
         const int64_t rows = (int64_t)p.B * p.H;
-        hipLaunchKernelGGL((decode_combine_kernel<T>), dim3((unsigned)rows), dim3(CMB_THREADS), 0, stream, p);
+        hipLaunchKernelGGL((decode_combine_kernel<T>), dim3((unsigned)((rows + CMB_THREADS / 64 - 1) / (CMB_THREADS / 64))), dim3(CMB_THREADS), 0, stream, p);
         e = hipGetLastError();
     }
     return e;
@@ -472,7 +532,7 @@ int decode_num_splits(int B, int Hk, int Lk) {
     if ((int64_t)splits * 8192 > Lk) splits = (256 + pairs - 1) / pairs;
     const int max_by_len = (Lk + 255) / 256;
     if (splits > max_by_len) splits = max_by_len;
-    if (splits > 128) splits = 128;
+    if (splits > CMB_MAX_SPLITS) splits = CMB_MAX_SPLITS;
     if (splits < 1) splits = 1;
     // shrink so that no split is empty after rounding keys_per_split up to a multiple of 256
     while (splits > 1) {
@@ -481,6 +541,12 @@ int decode_num_splits(int B, int Hk, int Lk) {
         splits--;
     }
     return splits;
+}
+
+int64_t decode_num_counters(int B, int H, int Hk, int Lk) {
+    if (B <= 0 || Hk <= 0 || decode_num_splits(B, Hk, Lk) <= 1) return 0;
+    const int G = H / Hk;
+    return (int64_t)B * Hk * ((G + DEC_COLS - 1) / DEC_COLS);
 }
 
 hipError_t launch_fwd_decode(const FwdParams &p, int dtype, hipStream_t stream) {

@@ -115,6 +115,9 @@ struct FwdParams {
     float *o_part;      // (splits, B, H, Lq, d) fp32
     float *lse_part;    // (splits, B, H, Lq) fp32, natural log, -inf for an empty split
     int32_t splits;
+    // split-KV decode in one launch: one arrival counter per (batch entry, workgroup row of the grid), zero on entry and
+    // left zero (fdma_fwd_args.counters of the C ABI); nullptr = the merge is a launch of its own
+    int32_t *dec_counter;
     int32_t compact_mode;  // FDMA_COMPACT_* of the C ABI: 0 = decide from the problem, 1 = never, 2 = whenever the mask form allows
     Compact cmp;        // when cmp.on, k / v (and their strides) describe the compacted copies
     // kept-column lists handed over by the caller (fdma_kept_keys of the C ABI; nullptr = scan the mask): one row per
@@ -267,6 +270,8 @@ void dkdv_split_bounds(int pairs, int n_max, int G, int &grid, int &slots);
 
 // number of KV splits the decode path uses for this shape (1 = no workspace needed)
 int decode_num_splits(int B, int Hk, int Lk);
+// arrival counters the one-launch decode needs for this shape (0 without splits)
+int64_t decode_num_counters(int B, int H, int Hk, int Lk);
 bool use_decode_path(int Lq, int H, int Hk);
 
 }  // namespace fdma

@@ -44,6 +44,7 @@ class FwdArgs(ctypes.Structure):
         ("workspace", ctypes.c_void_p), ("workspace_bytes", ctypes.c_size_t),
         ("kept", KeptKeys),
         ("mask_bits", MaskBits),
+        ("counters", ctypes.c_void_p), ("counters_bytes", ctypes.c_size_t),
     ]
 
 
@@ -119,7 +120,7 @@ class DynBiasArgs(ctypes.Structure):
 
 
 EXPORTS = (
-    "fdma_fwd", "fdma_fwd_noalloc", "fdma_bwd", "fdma_fwd_workspace_bytes", "fdma_bwd_workspace_bytes",
+    "fdma_fwd", "fdma_fwd_noalloc", "fdma_bwd", "fdma_fwd_workspace_bytes", "fdma_fwd_counter_bytes", "fdma_bwd_workspace_bytes",
     "fdma_fwd_validate", "fdma_bwd_validate", "fdma_last_error", "fdma_abi_version",
     "fdma_sizeof_fwd_args", "fdma_sizeof_bwd_args",
     "fdma_varlen_fwd", "fdma_varlen_bwd", "fdma_varlen_fwd_validate", "fdma_varlen_bwd_validate",
@@ -134,7 +135,7 @@ EXPORTS = (
 # from the problem, 1 = never (tile skipping only), 2 = whenever the mask form allows it.  The environment variable
 # FDMA_COMPACT is read ONCE, here, as the default ("0" = never, "2" = always); set_compact_mode() changes it for
 # the process, compact_mode() for a with-block.
-NOALLOC_SCRATCH_BYTES = 8 << 20
+NOALLOC_SCRATCH_BYTES = (8 << 20) - (64 << 10)  # FDMA_NOALLOC_SCRATCH_BYTES - FDMA_NOALLOC_COUNTER_BYTES: what a problem may need
 COMPACT_AUTO, COMPACT_NEVER, COMPACT_ALWAYS = 0, 1, 2
 _compact_mode = {"0": COMPACT_NEVER, "2": COMPACT_ALWAYS}.get(os.environ.get("FDMA_COMPACT", "")[:1], COMPACT_AUTO)
 
@@ -188,6 +189,8 @@ def _load() -> ctypes.CDLL:
     lib.fdma_bwd_validate.restype = ctypes.c_int
     lib.fdma_fwd_workspace_bytes.argtypes = [ctypes.POINTER(FwdArgs)]
     lib.fdma_fwd_workspace_bytes.restype = ctypes.c_size_t
+    lib.fdma_fwd_counter_bytes.argtypes = [ctypes.POINTER(FwdArgs)]
+    lib.fdma_fwd_counter_bytes.restype = ctypes.c_size_t
     lib.fdma_bwd_workspace_bytes.argtypes = [ctypes.POINTER(BwdArgs)]
     lib.fdma_bwd_workspace_bytes.restype = ctypes.c_size_t
     lib.fdma_last_error.argtypes = []
@@ -195,8 +198,8 @@ def _load() -> ctypes.CDLL:
     lib.fdma_abi_version.restype = ctypes.c_int
     lib.fdma_sizeof_fwd_args.restype = ctypes.c_size_t
     lib.fdma_sizeof_bwd_args.restype = ctypes.c_size_t
-    if lib.fdma_abi_version() != 5:
-        raise ImportError(f"{path}: ABI version {lib.fdma_abi_version()} != 5")
+    if lib.fdma_abi_version() != 6:
+        raise ImportError(f"{path}: ABI version {lib.fdma_abi_version()} != 6")
     lib.fdma_varlen_fwd.argtypes = [ctypes.POINTER(VarlenFwdArgs), ctypes.c_void_p]
     lib.fdma_varlen_fwd.restype = ctypes.c_int
     lib.fdma_varlen_bwd.argtypes = [ctypes.POINTER(VarlenBwdArgs), ctypes.c_void_p]
@@ -261,10 +264,11 @@ def _s3(t: torch.Tensor) -> Sequence[int]:
 
 def _bcast3(t: torch.Tensor) -> Sequence[int]:
     """(batch, head, row) strides of a 4-D mask / bias, 0 for size-1 (broadcast) dims."""
-    return tuple(0 if t.size(i) == 1 else t.stride(i) for i in range(3))
+    sh, st = t.shape, t.stride()
+    return (0 if sh[0] == 1 else st[0], 0 if sh[1] == 1 else st[1], 0 if sh[2] == 1 else st[2])
 
 
-_FWD_STRUCT = struct.Struct("@7P18q10i2fiPN3Pi4xP3q")
+_FWD_STRUCT = struct.Struct("@7P18q10i2fiPN3Pi4xP3qPN")
 assert _FWD_STRUCT.size == ctypes.sizeof(FwdArgs)
 
 
@@ -277,13 +281,14 @@ def fill_fwd(a: FwdArgs, q, k, v, mask, bias, out, lse, softmax_scale, is_causal
     ms = _bcast3(mask) if mask is not None else (0, 0, 0)
     bs = _bcast3(bias) if bias is not None else (0, 0, 0)
     batch, seqlen_q, num_heads, head_dim = q.shape
+    qs, ks, vs, os_ = q.stride(), k.stride(), v.stride(), out.stride()
     _FWD_STRUCT.pack_into(
         _as_buffer(a), 0,
         q.data_ptr(), k.data_ptr(), v.data_ptr(),
         mask.data_ptr() if mask is not None else 0, bias.data_ptr() if bias is not None else 0,
         out.data_ptr(), lse.data_ptr(),
-        q.stride(0), q.stride(1), q.stride(2), k.stride(0), k.stride(1), k.stride(2),
-        v.stride(0), v.stride(1), v.stride(2), out.stride(0), out.stride(1), out.stride(2),
+        qs[0], qs[1], qs[2], ks[0], ks[1], ks[2],
+        vs[0], vs[1], vs[2], os_[0], os_[1], os_[2],
         ms[0], ms[1], ms[2], bs[0], bs[1], bs[2],
         batch, seqlen_q, k.shape[1], num_heads, k.shape[2],
         mask.shape[1] if mask is not None else 1, bias.shape[1] if bias is not None else 1,
@@ -292,6 +297,7 @@ def fill_fwd(a: FwdArgs, q, k, v, mask, bias, out, lse, softmax_scale, is_causal
         kept[0].data_ptr() if kept else 0, kept[1].data_ptr() if kept else 0, kept[2].data_ptr() if kept else 0,
         kept[3] if kept else 0,
         bits.data_ptr() if bits is not None else 0, bt[0], bt[1], bt[2],
+        0, 0,
     )
 
 

@@ -80,8 +80,39 @@ def _direct_when_eager(op, body):
     return call
 
 
+_HALF_TYPES = (torch.float16, torch.bfloat16)
+
+
+def _inputs_plainly_ok(q, k, v, mask, bias) -> bool:
+    """One pass over what _check_inputs checks, without messages: True means every rule holds (the usual case, and the
+    one that matters for calls that take a few microseconds on the device); False sends the call through _check_inputs,
+    which finds the rule that failed and raises the reference's message for it."""
+    dt = q.dtype
+    if not (dt in _HALF_TYPES and k.dtype is dt and v.dtype is dt and q.is_cuda and k.is_cuda and v.is_cuda):
+        return False
+    qs, ks = q.shape, k.shape
+    if not (len(qs) == 4 and len(ks) == 4 and ks == v.shape):
+        return False
+    batch, seqlen_q, num_heads, head_size = qs
+    seqlen_k, num_heads_k = ks[1], ks[2]
+    if not (batch > 0 and head_size <= 256 and head_size % 8 == 0 and num_heads_k > 0 and num_heads % num_heads_k == 0
+            and ks[0] == batch and ks[3] == head_size):
+        return False
+    for t, want in ((mask, torch.bool), (bias, dt)):
+        if t is None:
+            continue
+        ts = t.shape
+        if not (t.dtype is want and t.is_cuda and len(ts) == 4 and (ts[0] == batch or ts[0] == 1)
+                and (ts[1] == 1 or ts[1] == num_heads_k or ts[1] == num_heads) and (ts[2] == 1 or ts[2] == seqlen_q)
+                and ts[3] >= seqlen_k):
+            return False
+    return True
+
+
 def _check_inputs(q, k, v, mask, bias) -> None:
     """Device / dtype / rank / shape checks of mha_fwd (flash_api.cpp:371-438, 477-479)."""
+    if _inputs_plainly_ok(q, k, v, mask, bias):
+        return
     if q.dtype not in (torch.float16, torch.bfloat16):
         raise RuntimeError("FlashSparseAttention only support fp16 and bf16 data type")
     if k.dtype != q.dtype:
@@ -162,6 +193,26 @@ def _handoff_get(name):
     return items.get(name) if items else None
 
 
+# Per-(device, stream) scratch of the decode path (seqlen_q == 1), where a call takes about as long on the device as
+# three tensor allocations take on the host.  Calls on one stream run one after the other, so they can share the
+# split-KV workspace; calls on different streams may overlap on the device and get buffers of their own.  The arrival
+# counters of the one-launch decode (fdma_fwd_args.counters) are zero before a call and zero after it: they are
+# cleared when the buffer is made and then serve every later call on that stream.
+_decode_scratch = {}
+_decode_sizes = {}   # (batch, heads, kv heads, keys, head dim) -> (workspace bytes, counter bytes): pure functions of the shape
+_empty_probs = {}    # the empty S_dmask tensor per (dtype, device)
+
+
+def _decode_buffers(device: torch.device, stream: int, nbytes: int, cbytes: int):
+    key = (device.index if device.index is not None else torch.cuda.current_device(), stream)
+    ws, counters = _decode_scratch.get(key, (None, None))
+    if ws is None or ws.numel() < nbytes or counters.numel() * 4 < cbytes:
+        ws = torch.empty(max(nbytes, 1 << 20), dtype=torch.uint8, device=device)
+        counters = torch.zeros(max(1024, (cbytes + 3) // 4), dtype=torch.int32, device=device)
+        _decode_scratch[key] = (ws, counters)
+    return ws, counters
+
+
 def _flash_sparse_attn_forward_body(
     q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Optional[torch.Tensor], bias: Optional[torch.Tensor],
     softmax_scale: float, is_causal: bool, softcap: float, return_softmax: bool,
@@ -179,18 +230,34 @@ def _flash_sparse_attn_forward_body(
     softmax_lse = torch.empty((batch, num_heads, seqlen_q), dtype=torch.float32, device=q.device)
     # The attention-probability dump is a debugging aid of the reference ("for testing only",
     # interface.py:661-663); it is not produced here.
-    p = torch.empty((0,), dtype=q.dtype, device=q.device)
+    pkey = (q.dtype, q.device)
+    p = _empty_probs.get(pkey)
+    if p is None:
+        p = _empty_probs[pkey] = torch.empty((0,), dtype=q.dtype, device=q.device)
     if seqlen_q == 0:
         return out, softmax_lse, p
     args = _cabi.FwdArgs()
     _cabi.fill_fwd(args, q, k, v, mask, bias, out, softmax_lse, softmax_scale, is_causal, softcap, kept, bits)
     with _cabi.device_guard(q.device):
-        nbytes = _cabi.lib.fdma_fwd_workspace_bytes(args)
+        stream = _cabi.current_stream(q.device)
         workspace = None
-        if nbytes:
-            workspace = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
-            args.workspace, args.workspace_bytes = workspace.data_ptr(), nbytes
-        _cabi.check(_cabi.lib.fdma_fwd(args, _cabi.current_stream(q.device)))
+        if seqlen_q == 1:
+            # split-KV decode: workspace and arrival counters (with them the splits are merged by the same launch)
+            skey = (batch, num_heads, k.shape[2], k.shape[1], q.shape[3])
+            sizes = _decode_sizes.get(skey)
+            if sizes is None:
+                sizes = _decode_sizes[skey] = (_cabi.lib.fdma_fwd_workspace_bytes(args), _cabi.lib.fdma_fwd_counter_bytes(args))
+            if sizes[0]:
+                ws, counters = _decode_buffers(q.device, stream, sizes[0], sizes[1])
+                args.workspace, args.workspace_bytes = ws.data_ptr(), ws.numel()
+                if sizes[1]:
+                    args.counters, args.counters_bytes = counters.data_ptr(), counters.numel() * 4
+        else:
+            nbytes = _cabi.lib.fdma_fwd_workspace_bytes(args)
+            if nbytes:
+                workspace = torch.empty(nbytes, dtype=torch.uint8, device=q.device)
+                args.workspace, args.workspace_bytes = workspace.data_ptr(), nbytes
+        _cabi.check(_cabi.lib.fdma_fwd(args, stream))
     items = getattr(_tls, "items", None)
     if items is not None and workspace is not None and seqlen_q > 1:
         # (the compaction path's lists and copies; what identifies the problem they belong to goes with them)
@@ -389,12 +456,12 @@ class FlashDMAttnFunc(torch.autograd.Function):
         mask = _pad_key_dim(mask, k.shape[1], 16)
         bias = _pad_key_dim(bias, k.shape[1], 8)
 
-        if eager:
+        if eager and (is_grad or kept is not None or bits is not None):
             with _handoff(kept=kept, bits=bits) as side:
                 out_padded, softmax_lse, S_dmask = _wrapped_flash_sparse_attn_forward(
                     q, k, v, mask, bias, softmax_scale, is_causal=is_causal, softcap=softcap, return_softmax=return_softmax,
                 )
-        else:
+        else:  # (a traced graph, or nothing to hand over and no backward to keep the workspace for)
             side = {}
             out_padded, softmax_lse, S_dmask = _wrapped_flash_sparse_attn_forward(
                 q, k, v, mask, bias, softmax_scale, is_causal=is_causal, softcap=softcap, return_softmax=return_softmax,
@@ -412,7 +479,8 @@ class FlashDMAttnFunc(torch.autograd.Function):
             ctx.deterministic = deterministic
             ctx.seqlen_k_bias_og = seqlen_k_bias_og
 
-        out = out_padded[..., :head_size_og]
+        # (the slice is a tensor-library call of its own: skipped when nothing was padded and no graph is traced)
+        out = out_padded if (eager and out_padded.shape[-1] == head_size_og) else out_padded[..., :head_size_og]
 
         return out if not return_softmax else (out, softmax_lse, S_dmask)
 

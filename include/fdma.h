@@ -44,7 +44,7 @@
 extern "C" {
 #endif
 
-#define FDMA_ABI_VERSION 5 /* 5: fdma_mask_bits (fdma_fwd_args.mask_bits, fdma_mask_args.bits); 4: fdma_kept_keys (fdma_fwd_args.kept, fdma_mask_args.kept_*), fdma_bwd_args.fwd_workspace (the structs grew);
+#define FDMA_ABI_VERSION 6 /* 6: fdma_fwd_args.counters (split-KV decode in one launch), fdma_fwd_counter_bytes; 5: fdma_mask_bits (fdma_fwd_args.mask_bits, fdma_mask_args.bits); 4: fdma_kept_keys (fdma_fwd_args.kept, fdma_mask_args.kept_*), fdma_bwd_args.fwd_workspace (the structs grew);
                               3: fdma_fwd_args.compact_mode, fdma_fwd_noalloc; 2: fdma_varlen_*, fdma_create_mask, fdma_dyn_bias_* */
 
 enum { FDMA_DTYPE_BF16 = 0, FDMA_DTYPE_FP16 = 1 };
@@ -132,6 +132,15 @@ typedef struct fdma_fwd_args {
     size_t workspace_bytes; /* >= fdma_fwd_workspace_bytes(args) */
     fdma_kept_keys kept;    /* optional: the mask's kept columns as lists (see fdma_kept_keys) */
     fdma_mask_bits mask_bits; /* optional: a per-query mask packed to bits (see fdma_mask_bits) */
+    /* Optional: arrival counters of the split-KV decode path (seqlen_q == 1), fdma_fwd_counter_bytes(args) bytes of
+     * device memory, 4-byte aligned, that hold ZEROS when the call starts.  With them the decode is ONE launch: the
+     * workgroup that finishes last among the splits of a (batch entry, kv head) merges their partial results (the
+     * reference always runs its combine as a second kernel, flash_fwd_launch_template.h:91-143) and puts its counter
+     * back to zero, so the same buffer serves the next call as it is -- clear it once, when it is allocated.  Calls
+     * that may overlap on the device (different streams) need a buffer each.  NULL = the merge is a second launch.
+     * Results are the same bit for bit either way.  Other paths ignore the field. */
+    int32_t *counters;
+    size_t counters_bytes; /* >= fdma_fwd_counter_bytes(args) */
 } fdma_fwd_args;
 
 typedef struct fdma_bwd_args {
@@ -175,14 +184,19 @@ int fdma_bwd(const fdma_bwd_args *args, void *hip_stream);
  * A problem whose fdma_fwd_workspace_bytes() exceeds that returns FDMA_ERR_WORKSPACE and launches nothing.  The
  * call makes no hipMalloc / hipFree (nor any other allocating call); results are bit-identical to fdma_fwd's.
  * Every call on a GPU uses that GPU's one array: calls that overlap on one GPU (different streams or host
- * threads) race on it -- serialise them.  Nothing in the array needs to start at zero; every call overwrites
- * what it reads.
+ * threads) race on it -- serialise them.  The last FDMA_NOALLOC_COUNTER_BYTES of the array are the decode path's
+ * arrival counters (args->counters is ignored as well): they are zero when the library is loaded and every call
+ * leaves them zero; the rest of the array need not start at anything, every call overwrites what it reads.  The
+ * scratch a problem may need is therefore FDMA_NOALLOC_SCRATCH_BYTES - FDMA_NOALLOC_COUNTER_BYTES at most.
  */
 #define FDMA_NOALLOC_SCRATCH_BYTES (8u << 20)
+#define FDMA_NOALLOC_COUNTER_BYTES (64u << 10)
 int fdma_fwd_noalloc(const fdma_fwd_args *args, void *hip_stream);
 
 /* Scratch the caller must provide.  0 when none is needed.  Validate nothing but shapes. */
 size_t fdma_fwd_workspace_bytes(const fdma_fwd_args *args);
+/* Size of the optional arrival counters (fdma_fwd_args.counters); 0 when the call would not use them. */
+size_t fdma_fwd_counter_bytes(const fdma_fwd_args *args);
 size_t fdma_bwd_workspace_bytes(const fdma_bwd_args *args);
 
 /* Argument validation only (no GPU work, callable on a host without a device). */

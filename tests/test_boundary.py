@@ -24,7 +24,7 @@ def test_library_exports_every_declared_symbol():
     lib = ctypes.CDLL(_cabi.lib_path())
     for name in declared:
         assert hasattr(lib, name), f"{name} not exported"
-    assert lib.fdma_abi_version() == 5
+    assert lib.fdma_abi_version() == 6
 
 
 def test_struct_mirrors_match_compiled_sizes():

@@ -447,9 +447,11 @@ DECODE_CASES = {
     # 40 query heads on one kv head: two workgroups per split (32 + 8 columns)
     "mqa40_two_column_chunks": (1, 2000, 40, 1, 64, 1, 1, 300),
     "mqa40_per_head_mask_and_bias": (1, 1200, 40, 1, 128, 40, 40, 200),
-    # head dims above 128: a single query row goes through the column-mask forward (no split-KV kernel there)
+    # head dims above 128: the split-KV kernel's instantiation at 256
     "gqa4_head_dim_256": (2, 1000, 8, 2, 256, 2, 2, 128),
     "mha_head_dim_192_no_mask": (1, 300, 2, 2, 192, None, 1, None),
+    "gqa4_head_dim_256_long": (1, 9000, 8, 2, 256, 2, 8, 700),
+    "mqa_head_dim_136_per_head_mask": (2, 2100, 4, 1, 136, 4, 1, 150),
 }
 
 
@@ -556,6 +558,59 @@ def test_decode_rows_far_apart():
     assert torch.equal(out, ref) and torch.equal(lse, ref_lse)
     ro, rl = c_oracle.forward(q, k, v, mask, bias, None, False)
     assert_out_close(out.cpu(), ro)
+
+
+@pytest.mark.parametrize("name", ["gqa4_topk", "mqa40_two_column_chunks", "gqa16_per_head_bias", "gqa4_head_dim_256_long", "short"])
+def test_decode_in_one_launch_equals_the_two_launch_form(name):
+    """With arrival counters (fdma_fwd_args.counters) the last workgroup of a (batch entry, kv head) merges the splits in
+    the decode launch itself; without them the merge is a second launch.  Same bits either way, the counters are zero
+    again afterwards, and the same buffer serves the next call."""
+    from flash_sparse_attn import _cabi
+
+    B, Lk, H, Hk, D, hm, hb, W = DECODE_CASES[name]
+    q, k, v, mask, bias = make_inputs(B, 1, Lk, H, Hk, D, (B, hb, 1, Lk), (B, hm, 1, Lk) if hm else None, W, seed=13)
+    from flash_sparse_attn.flash_sparse_attn_interface import _pad_key_dim
+
+    qd, kd, vd, md, bd = _to_dev(q, k, v, mask, bias)
+    md, bd = _pad_key_dim(md, Lk, 16), _pad_key_dim(bd, Lk, 8)  # (rows of whole 16-byte vectors, as the operator makes them)
+    stream = _cabi.current_stream(qd.device)
+
+    def call(counters):
+        out = torch.full_like(qd, float("nan"))
+        lse = torch.full((B, H, 1), float("nan"), dtype=torch.float32, device=DEV)
+        a = _cabi.FwdArgs()
+        _cabi.fill_fwd(a, qd, kd, vd, md, bd, out, lse, D ** -0.5, False, 0.0)
+        need = _cabi.lib.fdma_fwd_workspace_bytes(a)
+        ws = torch.empty(max(need, 16), dtype=torch.uint8, device=DEV)
+        a.workspace, a.workspace_bytes = ws.data_ptr(), need
+        if counters is not None:
+            a.counters, a.counters_bytes = counters.data_ptr(), counters.numel() * 4
+        assert _cabi.lib.fdma_fwd(a, stream) == 0, _cabi.last_error()
+        torch.cuda.synchronize()
+        return out, lse, need
+
+    two_out, two_lse, need = call(None)
+    a = _cabi.FwdArgs()
+    _cabi.fill_fwd(a, qd, kd, vd, md, bd, two_out, two_lse, D ** -0.5, False, 0.0)
+    cbytes = _cabi.lib.fdma_fwd_counter_bytes(a)
+    if need == 0:  # a single split: nothing to merge, no counters asked for
+        assert cbytes == 0
+        return
+    assert cbytes >= 4 * B * Hk
+    counters = torch.zeros(cbytes // 4, dtype=torch.int32, device=DEV)
+    for _ in range(3):
+        one_out, one_lse, _ = call(counters)
+        assert torch.equal(one_out, two_out) and torch.equal(one_lse, two_lse)
+        assert int(counters.abs().max()) == 0
+    ro, rl = c_oracle.forward(q, k, v, mask, bias, None, False)
+    assert_out_close(one_out.cpu(), ro)
+    _check_lse(one_lse.cpu(), rl)
+    # counters that are too small are refused with a message
+    a.workspace_bytes = need
+    a.workspace = torch.empty(need, dtype=torch.uint8, device=DEV).data_ptr()
+    a.counters, a.counters_bytes = counters.data_ptr(), 4
+    if cbytes > 4:
+        assert _cabi.lib.fdma_fwd(a, stream) == -3 and "arrival counters too small" in _cabi.last_error()
 
 
 def test_direct_c_abi_call_without_the_python_operator():

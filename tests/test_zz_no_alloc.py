@@ -77,3 +77,35 @@ def test_noalloc_entry_point_rejects_what_does_not_fit():
     assert need > _cabi.NOALLOC_SCRATCH_BYTES
     assert rc == -3 and "static scratch" in _cabi.last_error()
     assert torch.isnan(out.float()).all()   # nothing was launched
+
+
+def test_noalloc_entry_point_allocates_no_device_memory():
+    """The property the entry point exists for: after one warm-up call (code object, per-device scratch address), a
+    call changes neither the device's free memory (hipMemGetInfo) nor the tensor library's allocation counters.  The
+    decode case also goes through the per-device pointer cache a second time and leaves its arrival counters (the tail
+    of the static array) at zero: a third call gives the same bits."""
+    from flash_sparse_attn import _cabi
+
+    for kind, size in (("decode", (4, 32768, 16, 4, 128)), ("compact", (1, 1024, 8, 2, 128))):
+        mode = _cabi.COMPACT_ALWAYS if kind == "compact" else _cabi.COMPACT_AUTO
+        q, k, v, mask, bias, causal = _case(kind, size, seed=300)
+        qd, kd, vd, md, bd = [t.to(DEV) for t in (q, k, v, mask, bias)]
+        B, Lq, H, D = qd.shape
+        out = torch.empty_like(qd)
+        lse = torch.empty((B, H, Lq), dtype=torch.float32, device=DEV)
+        a = _cabi.FwdArgs()
+        _cabi.fill_fwd(a, qd, kd, vd, md, bd, out, lse, D ** -0.5, causal, 0.0)
+        a.compact_mode = mode
+        stream = _cabi.current_stream(qd.device)
+        assert _cabi.lib.fdma_fwd_noalloc(a, stream) == 0, _cabi.last_error()  # warm-up
+        torch.cuda.synchronize()
+        first = (out.clone(), lse.clone())
+        free0, _ = torch.cuda.mem_get_info()
+        alloc0, reserved0 = torch.cuda.memory_allocated(), torch.cuda.memory_reserved()
+        for _ in range(2):
+            assert _cabi.lib.fdma_fwd_noalloc(a, stream) == 0, _cabi.last_error()
+        torch.cuda.synchronize()
+        free1, _ = torch.cuda.mem_get_info()
+        assert free1 == free0, (free0, free1)
+        assert (torch.cuda.memory_allocated(), torch.cuda.memory_reserved()) == (alloc0, reserved0)
+        assert torch.equal(out, first[0]) and torch.equal(lse, first[1])
