@@ -262,6 +262,12 @@ int fdma_fwd_validate(const fdma_fwd_args *a) {
     return validate_common(a, false);
 }
 
+int fdma_set_stream_min_items(int n) {
+    const int before = fdma::get_stream_min_items();
+    if (n > 0) fdma::set_stream_min_items(n);
+    return before;
+}
+
 size_t fdma_fwd_counter_bytes(const fdma_fwd_args *a) {
     if (!a || a->seqlen_k <= 0 || a->num_heads_k <= 0 || !fdma::use_decode_path(a->seqlen_q, a->num_heads, a->num_heads_k)) return 0;
     return (size_t)round_up(fdma::decode_num_counters(a->batch, a->num_heads, a->num_heads_k, a->seqlen_k) * 4, 256);

@@ -33,23 +33,37 @@ inline size_t align256(size_t x) { return (x + 255) & ~(size_t)255; }
 
 struct Layout {
     size_t off_idx, off_cnt, off_count, off_fb, off_k, off_v, off_plan, off_part_kv, off_part_db, total;
+    size_t off_bk, off_bv;  // backward on a forward workspace that holds tile images: its own row-major copies
     int ld, Hfb;
+    bool img;       // the forward part holds tile images (off_k: K | V^T per tile, off_v: side rows) instead of copies
+    int img_tiles;  // tiles per (batch, kv head) pair
 };
 
 Layout layout_of(const FwdParams &p, bool backward) {
     Layout l;
     l.ld = (p.Lk + 15) / 16 * 16;
     l.Hfb = (p.bias && p.Hb == p.H) ? p.H : p.Hk;
+    l.img = fwd_stream_applicable(p);
+    l.img_tiles = (p.Lk + IMG_BN - 1) / IMG_BN;
     const size_t pairs = (size_t)p.B * p.Hk;
     size_t o = 0;
     l.off_idx = o;   o += align256(pairs * l.ld * 4);
     l.off_cnt = o;   o += align256(pairs * l.ld * 4);
     l.off_count = o; o += align256(pairs * 4);
     l.off_fb = o;    o += align256((size_t)p.B * l.Hfb * l.ld * 4);
-    l.off_k = o;     o += align256(pairs * p.Lk * p.d * 2);
-    l.off_v = o;     o += align256(pairs * p.Lk * p.d * 2);
-    l.off_plan = l.off_part_kv = l.off_part_db = o;
+    if (l.img) {
+        l.off_k = o; o += align256(pairs * l.img_tiles * IMG_KV_BYTES);
+        l.off_v = o; o += align256((size_t)p.B * l.Hfb * l.img_tiles * IMG_X_BYTES);
+    } else {
+        l.off_k = o; o += align256(pairs * p.Lk * p.d * 2);
+        l.off_v = o; o += align256(pairs * p.Lk * p.d * 2);
+    }
+    l.off_plan = l.off_part_kv = l.off_part_db = l.off_bk = l.off_bv = o;
     if (backward) {
+        if (l.img) {  // (the backward kernels read row-major copies: made by the backward's own pre-pass)
+            l.off_bk = o; o += align256(pairs * p.Lk * p.d * 2);
+            l.off_bv = o; o += align256(pairs * p.Lk * p.d * 2);
+        }
         int grid, slots;
         dkdv_split_bounds((int)pairs, (p.Lk + 127) / 128, p.H / p.Hk, grid, slots);
         const int dpad = p.d <= 64 ? 64 : (p.d <= 128 ? 128 : 256);
@@ -73,9 +87,11 @@ __global__ void __launch_bounds__(SCAN_THREADS) compact_scan_kernel(const FwdPar
 }
 
 // orig: the caller's tensors.  kc / vc: dense [B*Hk, Lk, d] destinations.
+// copies_only: the per-pair lists and the fused bias exist already (made by the forward call whose workspace this is);
+// only the K / V rows are copied.
 template <typename T>
 __device__ __forceinline__ void gather_block(const FwdParams &p, const int32_t *idx, int32_t *cnt, const int32_t *count, float *fb,
-                                             uint16_t *kc, uint16_t *vc, int ld, int Hfb, int block_x, int pair) {
+                                             uint16_t *kc, uint16_t *vc, int ld, int Hfb, int block_x, int pair, bool copies_only = false) {
     using E = Elem<T>;
     const int b = pair / p.Hk, hk = pair % p.Hk;
     const int tid = threadIdx.x;
@@ -84,7 +100,7 @@ __device__ __forceinline__ void gather_block(const FwdParams &p, const int32_t *
     // per-pair arrays the kernels index (in place of the scan), and reads its own inputs from the source
     const int32_t *src_idx = idx + (size_t)pair * ld;
     int n;
-    if (p.kept_idx) {
+    if (p.kept_idx && !copies_only) {
         const int srow = (p.m_b == 0 ? 0 : b) * p.Hm + (p.Hm == 1 ? 0 : hk);
         src_idx = p.kept_idx + (size_t)srow * p.kept_ld;
         // (lists are device data the host cannot check: a list made for a longer key axis than this call's must not
@@ -122,6 +138,7 @@ __device__ __forceinline__ void gather_block(const FwdParams &p, const int32_t *
             *(u32x4_t *)(vd + (size_t)rr * p.d + ch * 8) = vv;
         }
     }
+    if (copies_only) return;
     // fused bias of the compacted keys, one vector per bias class of this kv head
     const int G = p.H / p.Hk;
     const int nfb = Hfb == p.H ? G : 1;
@@ -228,6 +245,167 @@ __global__ void __launch_bounds__(256) compact_scan_gather_kernel(const FwdParam
             v = E::lo((uint32_t)((const uint16_t *)p.bias)[b * p.bi_b + hb * p.bi_h + src]) * kLog2e;
         }
         fb[((size_t)b * Hfb + hfb) * ld + base + rr] = v;
+    }
+}
+
+// Tile images for the streaming forward (fdma_fwd_stream.hip), scan included, in ONE launch: workgroup j of a (batch,
+// kv head) pair owns tile j of the compacted key axis -- the kept columns of rank 64 j .. 64 j + 63.  It finds them by
+// counting the whole mask row itself (every thread a contiguous piece of it; at most 64 KB per pair, read by all
+// workgroups of the pair and served by the L2), writes its part of the lists (idx for its ranks; cnt for the original
+// columns in front of which 64 j .. 64 j + 63 kept columns lie -- every column belongs to exactly one tile that way, the
+// columns behind the last kept one included) and then the tile as the forward keeps it in LDS: K rows padded to
+// IMG_SK elements, V transposed (rows of IMG_SVT elements), and per bias class the 16-element side rows (three 16-bit
+// pieces of bias * log2(e), the mask term, two ones, zeros).  Rows beyond the last kept key are zeros with a side row
+// that says "masked": the forward needs no row limit.  With lists handed over by the caller nothing is counted.
+template <typename T>
+__global__ void __launch_bounds__(256) compact_image_kernel(const FwdParams p, int32_t *idx, int32_t *cnt, int32_t *count, float *fb,
+                                                            char *img_kv, char *img_x, int ld, int Hfb, int tiles) {
+    using E = Elem<T>;
+    __shared__ int s_wave[4], s_src[IMG_BN];
+    const int pair = blockIdx.y, b = pair / p.Hk, hk = pair % p.Hk;
+    const int j = blockIdx.x, lo = j * IMG_BN;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    int32_t *irow = idx + (size_t)pair * ld, *crow = cnt + (size_t)pair * ld;
+    if (tid < IMG_BN) s_src[tid] = -1;
+    __syncthreads();
+    int total;
+    if (p.kept_idx) {
+        const int srow = (p.m_b == 0 ? 0 : b) * p.Hm + (p.Hm == 1 ? 0 : hk);
+        const int32_t *src_idx = p.kept_idx + (size_t)srow * p.kept_ld;
+        total = p.kept_count[srow];
+        total = total < p.Lk ? total : p.Lk;  // (lists are device data: held inside [0, Lk), see gather_block)
+        if (tid < IMG_BN && lo + tid < ld) {
+            int32_t col = src_idx[lo + tid];
+            const int32_t have = p.kept_cnt[(size_t)srow * p.kept_ld + lo + tid];
+            col = col < p.Lk ? col : p.Lk - 1;
+            irow[lo + tid] = col;
+            crow[lo + tid] = have < total ? have : total;
+            if (lo + tid < total) s_src[tid] = col < 0 ? 0 : col;
+        }
+    } else {
+        const int hm = p.Hm == 1 ? 0 : hk;
+        const uint8_t *mrow = p.mask + b * p.m_b + hm * p.m_h;
+        const int cpt = (((ld + 255) >> 8) + 15) & ~15;  // columns per thread: a multiple of 16
+        const int c0 = tid * cpt, c1 = c0 + cpt < p.Lk ? c0 + cpt : p.Lk;
+        // nonzero bytes of a 4-byte word whose first byte is column c, bytes at or beyond Lk dropped: bit 8 k + 7 for byte k
+        auto kept_bits = [&](uint32_t x, int c) -> uint32_t {
+            uint32_t y = (((x & 0x7f7f7f7fu) + 0x7f7f7f7fu) | x) & 0x80808080u;
+            const int valid = p.Lk - c;
+            if (valid < 4) y &= valid <= 0 ? 0u : (0xffffffffu >> (8 * (4 - valid)));
+            return y;
+        };
+        int mine = 0;
+        for (int c = c0; c < c1; c += 16) {
+            const u32x4_t mv = *(const u32x4_t *)(mrow + c);
+#pragma unroll
+            for (int e = 0; e < 4; e++) mine += __builtin_popcount(kept_bits(mv[e], c + 4 * e));
+        }
+        int incl = mine;
+#pragma unroll
+        for (int off = 1; off < 64; off <<= 1) {
+            const int t = __shfl_up(incl, off);
+            if (lane >= off) incl += t;
+        }
+        if (lane == 63) s_wave[wave] = incl;
+        __syncthreads();
+        int woff = 0;
+        total = 0;
+#pragma unroll
+        for (int w = 0; w < 4; w++) {
+            const int v = s_wave[w];
+            if (w < wave) woff += v;
+            total += v;
+        }
+        const int r0 = woff + incl - mine;  // kept columns in front of this thread's piece
+        // this thread's columns see r0 .. r0 + mine kept columns in front of them: walk the piece again when some of
+        // them belong to this tile
+        if (c0 < c1 && r0 <= lo + IMG_BN - 1 && r0 + mine >= lo) {
+            int run = r0;
+            for (int c = c0; c < c1; c += 16) {
+                const u32x4_t mv = *(const u32x4_t *)(mrow + c);
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                    const uint32_t y = kept_bits(mv[e], c + 4 * e);
+#pragma unroll
+                    for (int k = 0; k < 4; k++) {
+                        const int col = c + 4 * e + k;
+                        const bool kept = (y >> (8 * k + 7)) & 1u;
+                        if (col < p.Lk && run >= lo && run < lo + IMG_BN) {  // `run` kept columns in front of col
+                            crow[col] = run + (kept ? 1 : 0);
+                            if (kept) {
+                                irow[run] = col;
+                                s_src[run - lo] = col;
+                            }
+                        }
+                        run += kept ? 1 : 0;
+                    }
+                }
+            }
+        }
+        // (columns from Lk to the end of the row repeat the total)
+        if (total >= lo && total < lo + IMG_BN)
+            for (int c = p.Lk + tid; c < ld; c += 256) crow[c] = total;
+    }
+    if (j == 0 && tid == 0) count[pair] = total;
+    __syncthreads();
+    const int n = total - lo < IMG_BN ? total - lo : IMG_BN;  // kept keys of this tile
+    if (n <= 0 || j >= tiles) return;
+    // ---- K rows: thread (row, 16-byte chunk), four passes; V^T: thread (key quad, d chunk) transposes 4 keys x 8 d in
+    // registers (as the forward used to while staging).  All sixteen row pieces of a thread are requested before the
+    // first is stored: one trip to memory for the tile.
+    const uint16_t *kb = (const uint16_t *)p.k + b * p.k_b + hk * p.k_h;
+    const uint16_t *vb = (const uint16_t *)p.v + b * p.v_b + hk * p.v_h;
+    char *tile = img_kv + ((size_t)pair * tiles + j) * IMG_KV_BYTES;
+    const u32x4_t zero4 = {0, 0, 0, 0};
+    {
+        const int ch = tid & 15, rr0 = tid >> 4;
+        const int vkg = tid & 15, vc = tid >> 4;
+        u32x4_t kv[4], vv[4];
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+            const int src = s_src[rr0 + 16 * it];
+            kv[it] = src >= 0 ? *(const u32x4_t *)(kb + (int64_t)src * p.k_r + ch * 8) : zero4;
+        }
+#pragma unroll
+        for (int q = 0; q < 4; q++) {
+            const int src = s_src[4 * vkg + q];
+            vv[q] = src >= 0 ? *(const u32x4_t *)(vb + (int64_t)src * p.v_r + vc * 8) : zero4;
+        }
+#pragma unroll
+        for (int it = 0; it < 4; it++) *(u32x4_t *)(tile + (rr0 + 16 * it) * (IMG_SK * 2) + ch * 16) = kv[it];
+        char *vt = tile + IMG_K_BYTES;
+#pragma unroll
+        for (int dd = 0; dd < 8; dd++) {
+            const int w = dd >> 1;
+            const uint32_t sel = (dd & 1) ? 0x07060302u : 0x05040100u;
+            u32x2_t out;
+            out[0] = __builtin_amdgcn_perm(vv[1][w], vv[0][w], sel);
+            out[1] = __builtin_amdgcn_perm(vv[3][w], vv[2][w], sel);
+            *(u32x2_t *)(vt + ((vc * 8 + dd) * IMG_SVT + 4 * vkg) * 2) = out;
+        }
+    }
+    // ---- side rows and the fused bias vector (which the backward reads), one set per bias class of this kv head
+    const int G = p.H / p.Hk;
+    const int nfb = Hfb == p.H ? G : 1;
+    for (int it = tid; it < IMG_BN * nfb; it += 256) {
+        const int gi = it / IMG_BN, rr = it - gi * IMG_BN;
+        const int src = s_src[rr];
+        const int hfb = Hfb == p.H ? hk * G + gi : hk;
+        float v = 0.f;
+        if (src >= 0 && p.bias) {
+            const int hb = p.Hb == p.H ? hfb : (p.Hb == 1 ? 0 : hk);
+            v = E::lo((uint32_t)((const uint16_t *)p.bias)[b * p.bi_b + hb * p.bi_h + src]) * kLog2e;
+        }
+        if (src >= 0) fb[((size_t)b * Hfb + hfb) * ld + lo + rr] = v;
+        const u32x2_t pc = split3<T>(v);
+        u32x4_t row;
+        row[0] = pc[0];
+        row[1] = pc[1] | (E::pack2(0.f, src >= 0 ? 0.f : -INFINITY) & 0xffff0000u);
+        row[2] = E::pack2(E::kRefWeight, 1.f);
+        row[3] = 0;
+        char *xr = img_x + (((size_t)b * Hfb + hfb) * tiles + j) * IMG_X_BYTES + rr * 32;
+        *(u32x4_t *)xr = row;
+        *(u32x4_t *)(xr + 16) = zero4;
     }
 }
 
@@ -476,7 +654,7 @@ __global__ void __launch_bounds__(256) compact_bwd_prepass_kernel(const BwdParam
     const FwdParams &f = bp.f;
     if (blockIdx.z == 0) {
         // (not when the lists and copies exist already: made by an earlier launch, or by the forward call)
-        if (do_gather) gather_block<T>(f, idx, cnt, count, fb, kc, vc, ld, Hfb, blockIdx.x, blockIdx.y);
+        if (do_gather) gather_block<T>(f, idx, cnt, count, fb, kc, vc, ld, Hfb, blockIdx.x, blockIdx.y, do_gather == 2);
     } else if (blockIdx.z == 1) {
         zero_block(bp, bp.dbias != nullptr && bp.dbias_accum == nullptr, blockIdx.x, blockIdx.y);
     } else if (blockIdx.z == 2) {
@@ -507,7 +685,8 @@ bool use_compact(const FwdParams &p) {
 
 size_t compact_bytes(const FwdParams &p, bool backward, bool reuse_fwd) {
     const Layout l = layout_of(p, backward);
-    return backward && reuse_fwd ? l.total - l.off_plan : l.total;  // (with the forward's workspace: plan and partial sums only)
+    // (with the forward's workspace: plan and partial sums only -- and the row-major copies when the forward's are images)
+    return backward && reuse_fwd ? l.total - (l.img ? l.off_bk : l.off_plan) : l.total;
 }
 
 void dkdv_split_bounds(int pairs, int n_max, int G, int &grid, int &slots) {
@@ -554,13 +733,36 @@ hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, 
     const Layout l = layout_of(p, bp != nullptr);
     // the lists and the K / V copies: in this call's workspace, or (backward) where the forward call left them
     char *w = fwd_ws ? const_cast<char *>(static_cast<const char *>(fwd_ws)) : static_cast<char *>(ws);
-    // plan and partial sums of the backward: behind the lists, or alone in `ws` when the lists are the forward's
-    char *wb = fwd_ws ? static_cast<char *>(ws) - l.off_plan : static_cast<char *>(ws);
+    // what only the backward has (its row-major copies when the forward's are tile images, the plan, the partial
+    // sums): behind the forward part, or alone in `ws` when that part is the forward call's
+    char *wb = fwd_ws ? static_cast<char *>(ws) - (l.img ? l.off_bk : l.off_plan) : static_cast<char *>(ws);
     int32_t *idx = (int32_t *)(w + l.off_idx), *cnt = (int32_t *)(w + l.off_cnt), *count = (int32_t *)(w + l.off_count);
     float *fb = (float *)(w + l.off_fb);
-    uint16_t *kc = (uint16_t *)(w + l.off_k), *vc = (uint16_t *)(w + l.off_v);
+    // row-major copies: the backward's own when the forward part holds images
+    uint16_t *kc = (uint16_t *)(l.img ? wb + l.off_bk : w + l.off_k), *vc = (uint16_t *)(l.img ? wb + l.off_bv : w + l.off_v);
     const int pairs = p.B * p.Hk;
     hipError_t e;
+    if (l.img && !bp) {
+        // forward on tile images: lists, fused bias and images in one launch
+        char *img_kv = w + l.off_k, *img_x = w + l.off_v;
+        const dim3 igrid(p.Lk / IMG_BN + 1, pairs);
+        if (dtype == 0)
+            hipLaunchKernelGGL((compact_image_kernel<bf16_tag>), igrid, dim3(256), 0, stream, p, idx, cnt, count, fb, img_kv, img_x, l.ld, l.Hfb, l.img_tiles);
+        else
+            hipLaunchKernelGGL((compact_image_kernel<fp16_tag>), igrid, dim3(256), 0, stream, p, idx, cnt, count, fb, img_kv, img_x, l.ld, l.Hfb, l.img_tiles);
+        if ((e = hipGetLastError()) != hipSuccess) return e;
+        p.cmp.idx = idx;
+        p.cmp.cnt = cnt;
+        p.cmp.count = count;
+        p.cmp.fb = fb;
+        p.cmp.ld = l.ld;
+        p.cmp.Hfb = l.Hfb;
+        p.cmp.on = 1;
+        p.cmp.img_kv = img_kv;
+        p.cmp.img_x = img_x;
+        p.cmp.img_tiles = l.img_tiles;
+        return hipSuccess;
+    }
     const bool have_lists = fwd_ws != nullptr || p.kept_idx != nullptr;
     // forward without lists: scan and gather in one launch -- up to 65536 keys: every workgroup of that launch counts the
     // mask bytes in front of its segment, Lk / 2 of them on average, which grows with the square of Lk per pair
@@ -599,7 +801,9 @@ hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, 
         const int64_t dot_layers = (dot_blocks + layer - 1) / layer;
         const bool with_dot = p.cu_q == nullptr && 3 + dot_layers <= 65535;
         const dim3 grid3(grid.x, pairs, with_dot ? (unsigned)(3 + dot_layers) : 3);
-        const int do_gather = (fwd_ws || gather_alone) ? 0 : 1;
+        // 0: lists and copies exist; 1: gather here; 2: the lists are the forward call's, whose copies are tile images --
+        // only the row-major K / V copies are made here
+        const int do_gather = fwd_ws ? (l.img ? 2 : 0) : (gather_alone ? 0 : 1);
         if (dtype == 0)
             hipLaunchKernelGGL((compact_bwd_prepass_kernel<bf16_tag>), grid3, dim3(256), 0, stream, *bp, idx, cnt, count, fb, kc, vc,
                                l.ld, l.Hfb, plan, 2 * device_cus(), plan_cap, do_gather);

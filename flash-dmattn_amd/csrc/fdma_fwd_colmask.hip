@@ -785,6 +785,7 @@ bool fwd_colmask_applicable(const FwdParams &p) {
 }
 
 hipError_t launch_fwd_colmask(const FwdParams &p, int dtype, hipStream_t stream) {
+    if (p.cmp.on && p.cmp.img_kv) return launch_fwd_stream(p, dtype, stream);  // (the pre-pass has written tile images)
     // head dims up to 64 / 128 / 256 (a head dim in between runs in the next larger instantiation)
     if (dtype == 0) return p.d <= 64 ? launch_d<bf16_tag, 64>(p, stream) : p.d <= 128 ? launch_d<bf16_tag, 128>(p, stream) : launch_d<bf16_tag, 256>(p, stream);
     return p.d <= 64 ? launch_d<fp16_tag, 64>(p, stream) : p.d <= 128 ? launch_d<fp16_tag, 128>(p, stream) : launch_d<fp16_tag, 256>(p, stream);

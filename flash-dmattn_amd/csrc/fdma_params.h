@@ -23,7 +23,21 @@ struct Compact {
     int32_t ld;            // row stride of the arrays above (Lk rounded up to 16)
     int32_t Hfb;           // heads of fb: Hk, or H when the bias differs per query head
     int32_t on;            // 0 = no compaction: k / v are the caller's tensors
+    // Tile images (forward at head dim 128 on large grids, see fwd_stream_applicable): instead of row-major copies the
+    // pre-pass writes, per 64-key tile of the compacted key axis, exactly the bytes the forward kernel keeps in LDS --
+    // the K tile with padded rows followed by V already transposed (img_kv, IMG_KV_BYTES per tile, img_tiles tiles per
+    // (batch, kv head) pair) and the 16-element side rows of the keys (img_x, IMG_X_BYTES per tile, per (batch, fb
+    // head)) -- so that the forward fetches a tile with contiguous global->LDS loads.  nullptr = row-major copies.
+    const char *img_kv;
+    const char *img_x;
+    int32_t img_tiles;
 };
+constexpr int IMG_BN = 64;                                // keys per tile image
+constexpr int IMG_SK = 128 + 8, IMG_SVT = IMG_BN + 8;     // row strides (elements) of the K tile and of V^T
+constexpr int IMG_K_BYTES = IMG_BN * IMG_SK * 2;          // 17408
+constexpr int IMG_VT_BYTES = 128 * IMG_SVT * 2;           // 18432
+constexpr int IMG_KV_BYTES = IMG_K_BYTES + IMG_VT_BYTES;  // 35840 = 35 pieces of 1 KB
+constexpr int IMG_X_BYTES = IMG_BN * 32;                  // 2048
 
 // Work split of the compacted dK/dV kernel, made on the device once the kept-key counts are known.
 // A unit is one 128-key block of one (batch, kv head) pair; U = number of units.  With few units the
@@ -244,6 +258,14 @@ hipError_t launch_fwd(const FwdParams &p, int dtype, hipStream_t stream);
 // column-mask specialisation (mask / bias absent or broadcast over queries); nq = 32-row blocks per wave
 bool fwd_colmask_applicable(const FwdParams &p);
 hipError_t launch_fwd_colmask(const FwdParams &p, int dtype, hipStream_t stream);
+// compacted forward on tile images (fdma_fwd_stream.hip): resident workgroups that walk their share of the
+// (query block, head) items with the tiles of the next item already on their way.  `fwd_stream_applicable` decides from
+// the problem alone (the pre-pass, the forward and the backward of a problem must agree on the workspace layout).
+bool fwd_stream_applicable(const FwdParams &p);
+// smallest number of (256-row query block, head) items for which it is taken (process-wide; default 512)
+void set_stream_min_items(int n);
+int get_stream_min_items();
+hipError_t launch_fwd_stream(const FwdParams &p, int dtype, hipStream_t stream);
 hipError_t launch_fwd_decode(const FwdParams &p, int dtype, hipStream_t stream);
 hipError_t launch_bwd(const BwdParams &p, int dtype, hipStream_t stream);
 // column-mask specialisations of the two main backward kernels

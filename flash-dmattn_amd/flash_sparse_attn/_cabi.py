@@ -121,6 +121,7 @@ class DynBiasArgs(ctypes.Structure):
 
 EXPORTS = (
     "fdma_fwd", "fdma_fwd_noalloc", "fdma_bwd", "fdma_fwd_workspace_bytes", "fdma_fwd_counter_bytes", "fdma_bwd_workspace_bytes",
+    "fdma_set_stream_min_items",
     "fdma_fwd_validate", "fdma_bwd_validate", "fdma_last_error", "fdma_abi_version",
     "fdma_sizeof_fwd_args", "fdma_sizeof_bwd_args",
     "fdma_varlen_fwd", "fdma_varlen_bwd", "fdma_varlen_fwd_validate", "fdma_varlen_bwd_validate",
@@ -162,6 +163,12 @@ def compact_mode(mode: int):
         set_compact_mode(previous)
 
 
+def stream_min_items(n: int = 0) -> int:
+    """Threshold (in 256-row query block x head items) from which the compacted forward at head dim 128 streams tile
+    images (fdma_set_stream_min_items); n <= 0 only queries.  Returns the value before the call."""
+    return lib.fdma_set_stream_min_items(int(n))
+
+
 def lib_path() -> str:
     return os.environ.get("FDMA_LIB", _DEFAULT_LIB)
 
@@ -191,6 +198,8 @@ def _load() -> ctypes.CDLL:
     lib.fdma_fwd_workspace_bytes.restype = ctypes.c_size_t
     lib.fdma_fwd_counter_bytes.argtypes = [ctypes.POINTER(FwdArgs)]
     lib.fdma_fwd_counter_bytes.restype = ctypes.c_size_t
+    lib.fdma_set_stream_min_items.argtypes = [ctypes.c_int]
+    lib.fdma_set_stream_min_items.restype = ctypes.c_int
     lib.fdma_bwd_workspace_bytes.argtypes = [ctypes.POINTER(BwdArgs)]
     lib.fdma_bwd_workspace_bytes.restype = ctypes.c_size_t
     lib.fdma_last_error.argtypes = []

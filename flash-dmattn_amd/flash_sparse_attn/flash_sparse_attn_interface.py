@@ -261,7 +261,7 @@ def _flash_sparse_attn_forward_body(
     items = getattr(_tls, "items", None)
     if items is not None and workspace is not None and seqlen_q > 1:
         # (the compaction path's lists and copies; what identifies the problem they belong to goes with them)
-        items["fwd_ws_out"] = (workspace, _cabi.get_compact_mode(), None if bias is None else tuple(bias.shape))
+        items["fwd_ws_out"] = (workspace, (_cabi.get_compact_mode(), _cabi.stream_min_items()), None if bias is None else tuple(bias.shape))
     return out, softmax_lse, p
 
 
@@ -335,7 +335,8 @@ def _flash_sparse_attn_backward_body(
     _cabi.fill_fwd(args.f, q, k, v, mask, bias, out, softmax_lse, softmax_scale, is_causal, softcap, _handoff_get("kept"),
                    _handoff_get("bits"))
     fwd_ws = _handoff_get("fwd_ws")
-    if fwd_ws is not None and fwd_ws[1] == _cabi.get_compact_mode() and fwd_ws[2] == (None if bias is None else tuple(bias.shape)):
+    if (fwd_ws is not None and fwd_ws[1] == (_cabi.get_compact_mode(), _cabi.stream_min_items())
+            and fwd_ws[2] == (None if bias is None else tuple(bias.shape))):
         args.fwd_workspace, args.fwd_workspace_bytes = fwd_ws[0].data_ptr(), fwd_ws[0].numel()
     args.dout = dout.data_ptr()
     args.dq, args.dk, args.dv = dq_w.data_ptr(), dk_w.data_ptr(), dv_w.data_ptr()

@@ -193,6 +193,14 @@ int fdma_bwd(const fdma_bwd_args *args, void *hip_stream);
 #define FDMA_NOALLOC_COUNTER_BYTES (64u << 10)
 int fdma_fwd_noalloc(const fdma_fwd_args *args, void *hip_stream);
 
+/* Tuning knob of the column-compaction path, process-wide.  At head dim 128 the compacted forward has two forms: one
+ * workgroup per 128 or 256 query rows of a head over row-major copies of the kept K / V rows, and -- for problems of
+ * at least `n` (256-row query block, head) items, default 512: a grid that fills the device several times -- resident
+ * workgroups that stream "tile images" written by the pre-pass (fdma_fwd_stream.hip).  The threshold decides the
+ * workspace LAYOUT: a forward call and the backward call that is handed its workspace (fwd_workspace) must run under
+ * the same value.  n <= 0 only queries.  Returns the value before the call.  No counterpart in the reference. */
+int fdma_set_stream_min_items(int n);
+
 /* Scratch the caller must provide.  0 when none is needed.  Validate nothing but shapes. */
 size_t fdma_fwd_workspace_bytes(const fdma_fwd_args *args);
 /* Size of the optional arrival counters (fdma_fwd_args.counters); 0 when the call would not use them. */
