@@ -294,11 +294,29 @@ __global__ void __launch_bounds__(256) compact_image_kernel(const FwdParams p, i
             if (valid < 4) y &= valid <= 0 ? 0u : (0xffffffffu >> (8 * (4 - valid)));
             return y;
         };
-        int mine = 0;
-        for (int c = c0; c < c1; c += 16) {
-            const u32x4_t mv = *(const u32x4_t *)(mrow + c);
+        // (a piece of up to 64 columns stays in registers for the second look; longer ones are fetched again)
+        constexpr int KEEP = 4;
+        const bool keep = cpt <= 16 * KEEP;
+        u32x4_t held[KEEP];
 #pragma unroll
-            for (int e = 0; e < 4; e++) mine += __builtin_popcount(kept_bits(mv[e], c + 4 * e));
+        for (int w = 0; w < KEEP; w++) held[w] = u32x4_t{0, 0, 0, 0};
+        int mine = 0;
+        if (keep) {
+#pragma unroll
+            for (int w = 0; w < KEEP; w++) {
+                const int c = c0 + 16 * w;
+                if (w * 16 < cpt && c < c1) held[w] = *(const u32x4_t *)(mrow + c);
+            }
+#pragma unroll
+            for (int w = 0; w < KEEP; w++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) mine += __builtin_popcount(kept_bits(held[w][e], c0 + 16 * w + 4 * e));
+        } else {
+            for (int c = c0; c < c1; c += 16) {
+                const u32x4_t mv = *(const u32x4_t *)(mrow + c);
+#pragma unroll
+                for (int e = 0; e < 4; e++) mine += __builtin_popcount(kept_bits(mv[e], c + 4 * e));
+            }
         }
         int incl = mine;
 #pragma unroll
@@ -321,8 +339,7 @@ __global__ void __launch_bounds__(256) compact_image_kernel(const FwdParams p, i
         // them belong to this tile
         if (c0 < c1 && r0 <= lo + IMG_BN - 1 && r0 + mine >= lo) {
             int run = r0;
-            for (int c = c0; c < c1; c += 16) {
-                const u32x4_t mv = *(const u32x4_t *)(mrow + c);
+            auto walk = [&](const u32x4_t mv, int c) {
 #pragma unroll
                 for (int e = 0; e < 4; e++) {
                     const uint32_t y = kept_bits(mv[e], c + 4 * e);
@@ -340,6 +357,13 @@ __global__ void __launch_bounds__(256) compact_image_kernel(const FwdParams p, i
                         run += kept ? 1 : 0;
                     }
                 }
+            };
+            if (keep) {
+#pragma unroll
+                for (int w = 0; w < KEEP; w++)
+                    if (c0 + 16 * w < c1) walk(held[w], c0 + 16 * w);
+            } else {
+                for (int c = c0; c < c1; c += 16) walk(*(const u32x4_t *)(mrow + c), c);
             }
         }
         // (columns from Lk to the end of the row repeat the total)
@@ -357,6 +381,8 @@ __global__ void __launch_bounds__(256) compact_image_kernel(const FwdParams p, i
     const uint16_t *vb = (const uint16_t *)p.v + b * p.v_b + hk * p.v_h;
     char *tile = img_kv + ((size_t)pair * tiles + j) * IMG_KV_BYTES;
     const u32x4_t zero4 = {0, 0, 0, 0};
+    const int G = p.H / p.Hk;
+    const int nfb = Hfb == p.H ? G : 1;
     {
         const int ch = tid & 15, rr0 = tid >> 4;
         const int vkg = tid & 15, vc = tid >> 4;
@@ -371,6 +397,14 @@ __global__ void __launch_bounds__(256) compact_image_kernel(const FwdParams p, i
             const int src = s_src[4 * vkg + q];
             vv[q] = src >= 0 ? *(const u32x4_t *)(vb + (int64_t)src * p.v_r + vc * 8) : zero4;
         }
+        // (the bias value of this thread's first side row travels with the rows)
+        uint32_t braw0 = 0;
+        if (p.bias && tid < IMG_BN * nfb) {
+            const int gi = tid / IMG_BN, src = s_src[tid - gi * IMG_BN];
+            const int hfb = Hfb == p.H ? hk * G + gi : hk;
+            const int hb = p.Hb == p.H ? hfb : (p.Hb == 1 ? 0 : hk);
+            if (src >= 0) braw0 = ((const uint16_t *)p.bias)[b * p.bi_b + hb * p.bi_h + src];
+        }
 #pragma unroll
         for (int it = 0; it < 4; it++) *(u32x4_t *)(tile + (rr0 + 16 * it) * (IMG_SK * 2) + ch * 16) = kv[it];
         char *vt = tile + IMG_K_BYTES;
@@ -383,29 +417,31 @@ __global__ void __launch_bounds__(256) compact_image_kernel(const FwdParams p, i
             out[1] = __builtin_amdgcn_perm(vv[3][w], vv[2][w], sel);
             *(u32x2_t *)(vt + ((vc * 8 + dd) * IMG_SVT + 4 * vkg) * 2) = out;
         }
-    }
-    // ---- side rows and the fused bias vector (which the backward reads), one set per bias class of this kv head
-    const int G = p.H / p.Hk;
-    const int nfb = Hfb == p.H ? G : 1;
-    for (int it = tid; it < IMG_BN * nfb; it += 256) {
-        const int gi = it / IMG_BN, rr = it - gi * IMG_BN;
-        const int src = s_src[rr];
-        const int hfb = Hfb == p.H ? hk * G + gi : hk;
-        float v = 0.f;
-        if (src >= 0 && p.bias) {
-            const int hb = p.Hb == p.H ? hfb : (p.Hb == 1 ? 0 : hk);
-            v = E::lo((uint32_t)((const uint16_t *)p.bias)[b * p.bi_b + hb * p.bi_h + src]) * kLog2e;
+        // ---- side rows and the fused bias vector (which the backward reads), one set per bias class of this kv head
+        for (int it = tid; it < IMG_BN * nfb; it += 256) {
+            const int gi = it / IMG_BN, rr = it - gi * IMG_BN;
+            const int src = s_src[rr];
+            const int hfb = Hfb == p.H ? hk * G + gi : hk;
+            float v = 0.f;
+            if (src >= 0 && p.bias) {
+                uint32_t braw = braw0;
+                if (it != tid) {
+                    const int hb = p.Hb == p.H ? hfb : (p.Hb == 1 ? 0 : hk);
+                    braw = ((const uint16_t *)p.bias)[b * p.bi_b + hb * p.bi_h + src];
+                }
+                v = E::lo(braw) * kLog2e;
+            }
+            if (src >= 0) fb[((size_t)b * Hfb + hfb) * ld + lo + rr] = v;
+            const u32x2_t pc = split3<T>(v);
+            u32x4_t row;
+            row[0] = pc[0];
+            row[1] = pc[1] | (E::pack2(0.f, src >= 0 ? 0.f : -INFINITY) & 0xffff0000u);
+            row[2] = E::pack2(E::kRefWeight, 1.f);
+            row[3] = 0;
+            char *xr = img_x + (((size_t)b * Hfb + hfb) * tiles + j) * IMG_X_BYTES + rr * 32;
+            *(u32x4_t *)xr = row;
+            *(u32x4_t *)(xr + 16) = zero4;
         }
-        if (src >= 0) fb[((size_t)b * Hfb + hfb) * ld + lo + rr] = v;
-        const u32x2_t pc = split3<T>(v);
-        u32x4_t row;
-        row[0] = pc[0];
-        row[1] = pc[1] | (E::pack2(0.f, src >= 0 ? 0.f : -INFINITY) & 0xffff0000u);
-        row[2] = E::pack2(E::kRefWeight, 1.f);
-        row[3] = 0;
-        char *xr = img_x + (((size_t)b * Hfb + hfb) * tiles + j) * IMG_X_BYTES + rr * 32;
-        *(u32x4_t *)xr = row;
-        *(u32x4_t *)(xr + 16) = zero4;
     }
 }
 
