@@ -274,7 +274,10 @@ __global__ void __launch_bounds__(ST_THREADS, 1) fwd_stream_kernel(const FwdPara
     const uint32_t aV = lds0 + SM::OFF_KV + IMG_K_BYTES + (uint32_t)((a_row * SVT + 8 * g) * 2);
     const uint32_t aX = lds0 + SM::OFF_X + (uint32_t)(a_row * 32 + g * 16);
     constexpr int NQK = KS + 1, NPV = 2 * DB;
-    constexpr int FR = 4;  // fragment reads run FR MFMAs ahead of their MFMAs
+#ifndef FDMA_ST_FR
+#define FDMA_ST_FR 4
+#endif
+    constexpr int FR = FDMA_ST_FR;  // fragment reads run FR MFMAs ahead of their MFMAs
     const f32x16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     const float side_mult = 1.f / E::kPieceScale;
 

@@ -101,6 +101,23 @@ def test_streaming_forward_and_its_backward_vs_oracle(name):
             assert torch.equal(a, b)
 
 
+def test_pairs_without_a_kept_key_and_a_late_first_key():
+    """One (batch, kv head) pair keeps nothing at all (its rows come out as zeros with LSE = +inf, its gradients as
+    zeros), another keeps only keys in the last quarter (under the causal rule most of its rows see nothing)."""
+    B, L, H, Hk = 2, 600, 4, 2
+    q, k, v, mask, bias = make_inputs(B, L, L, H, Hk, 128, (B, Hk, 1, L), (B, Hk, 1, L), 150, seed=12)
+    mask[0, 1] = False
+    mask[1, 0, :, : 3 * L // 4] = False
+    out, lse, grads = _run(q, k, v, mask, bias, True)
+    ro, rl = c_oracle.forward(q, k, v, mask, bias, None, True)
+    refs = c_oracle.backward(q, k, v, torch.ones_like(ro), mask, bias, None, True)
+    assert_out_close(out.cpu(), ro)
+    _check_lse(lse.cpu(), rl)
+    assert float(out[0, :, 2:].abs().max()) == 0.0 and bool(torch.isinf(lse[0, 2:]).all())
+    for g, r, n in zip(grads, refs, ("dq", "dk", "dv", "dbias")):
+        assert_grad_close(g.cpu(), r, n)
+
+
 def test_streaming_forward_with_lists_from_the_mask_builder():
     """Kept-key lists handed over by the device mask builder: the image pre-pass numbers nothing and copies the lists;
     results equal those of the same mask as a plain tensor, bit for bit."""
