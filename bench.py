@@ -599,6 +599,60 @@ def cpu_baseline(device_cfg="cfg2", groups=8, chunk=2):
             "ms_scaled_to_full": dt * 1e3 * c["Hk"] / groups}
 
 
+def run_secondary_legs(out, legs, args, device, compact, bwd, half):
+    """Every default leg but the headline: the tile-skipping path and the all-zero operands of cfg2, the matrix-pipe
+    probe, cfg3 / cfg4 / cfg5 with their roofline blocks and the forward W sweep."""
+    if compact and "tile_skip" in legs:
+        # the same workload through the tile-skipping kernel alone (one kernel per call, no pre-pass)
+        ts = run_config("cfg2", *half, device, compact=False, backward=False)
+        out["tile_skip_path"] = {"ms_fwd": ts["ms_fwd"], "n_exec_tiles": ts["n_exec"], "tflops_fwd": ts["tflops_fwd"],
+                                 "frac_of_peak": ts["tflops_fwd"] / PEAK_BF16_TFLOPS,
+                                 "kernel": "fdma::fwd_colmask_kernel<bf16, 128, causal> (compact_mode = never)"}
+    if compact and "zero" in legs:
+        # The same launches on all-zero Q / K / V / bias: identical mask, tiles and instruction stream.  The device lowers
+        # its clocks under the switching activity of real operands (a register-fed MFMA loop reaches 2.4 PFLOP/s on
+        # constant operands and 1.9 on random ones), so this is what the kernels' schedule sustains when it does not.
+        tz = run_config("cfg2", *half, device, compact=False, backward=False, zero_inputs=True)
+        out.setdefault("tile_skip_path", {})["zero_operands"] = {"ms_fwd": tz["ms_fwd"], "tflops_fwd": tz["tflops_fwd"],
+                                                                 "frac_of_peak": tz["tflops_fwd"] / PEAK_BF16_TFLOPS}
+        cz = run_config("cfg2", *half, device, compact=True, backward=bwd, zero_inputs=True)
+        out["zero_operands"] = {"ms_fwd": cz["ms_fwd"], "tflops_fwd": cz["tflops_fwd"],
+                                "frac_of_peak": cz["tflops_fwd"] / PEAK_BF16_TFLOPS, "ms_fwd_bwd": cz.get("ms_fwd_bwd"),
+                                "note": "same mask, tiles and instruction stream as the headline figures, all-zero Q / K / V / "
+                                        "bias: what the schedule sustains when the device does not lower its clock"}
+    if "probe" in legs:
+        probe = run_mfma_probe()
+        if probe is not None:
+            out["mfma_probe"] = probe
+    if args.calib_copy:
+        src = torch.empty(256 << 20, dtype=torch.uint8, device=device).fill_(1)
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+    # The other benchmark configurations, each against the roofline that bounds it: cfg3 (a bias and a mask per query
+    # row, with its dBias) and cfg5 (decode) against HBM, cfg4 (long sequence, narrow window) against the matrix pipe.
+    quarter = (max(3, args.steps // 4), max(1, args.warmup // 2))
+    configs = {}
+    for name in ("cfg3", "cfg4", "cfg5"):
+        if name not in legs:
+            continue
+        if name == "cfg5":  # (a call of some 20 us: many steps, or the two events' own resolution shows)
+            r = run_config(name, 10 * args.steps, 2 * args.warmup, device, compact, backward=False)
+            r["ms_fwd_c_abi"] = time_decode_c_abi(name, 10 * args.steps, 2 * args.warmup, device)
+        else:
+            r = run_config(name, *quarter, device, compact, backward=bwd)
+        c2 = CONFIGS[name]
+        r["workload"] = "%s: B=%d Lq=%d Lk=%d H=%d Hkv=%d d=%d bias%s top-%d%s" % (
+            name, c2["B"], c2["Lq"], c2["Lk"], c2["H"], c2["Hk"], c2["D"], list(c2["bias"]), c2["W"], " ∩ causal" if c2["causal"] else "")
+        r["roofline"] = config_roofline(name, r)
+        configs[name] = r
+        torch.cuda.empty_cache()
+    if configs:
+        out["configs"] = configs
+    if "w_sweep" in legs:
+        out["w_sweep_fwd"] = run_w_sweep_fwd(*quarter, device)
+
+
 DEFAULT_LEGS = ("cfg2", "tile_skip", "zero", "probe", "cfg3", "cfg4", "cfg5", "w_sweep", "cpu")
 
 
@@ -611,7 +665,7 @@ def main():
                     help="also: cfg1, mask builder, bias producer, hand-overs, ragged batch, forward + backward sweeps over W and L")
     ap.add_argument("--legs", default=None,
                     help="comma-separated subset of the default legs to run (" + ", ".join(DEFAULT_LEGS) + "); a profile of one "
-                         "leg then holds one workload per kernel.  cfg2 (the headline) always runs")
+                         "leg then holds one workload per kernel; without cfg2 the headline workload is not launched at all")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-probe", action="store_true", help="skip the matrix-pipe probe (MFMA rate on constant / random operands)")
     ap.add_argument("--no-backward", action="store_true", help="forward legs only")
@@ -647,6 +701,12 @@ def main():
     compact = not args.no_compact
     bwd = not args.no_backward
     half = (max(3, args.steps // 2), max(1, args.warmup // 2))
+    if "cfg2" not in legs:
+        # a profile of single legs: nothing of the headline workload is launched, and the line holds those legs only
+        out = {"metric": "single legs of bench.py (no headline value: run without --legs for the benchmark line)", "legs": sorted(legs)}
+        run_secondary_legs(out, legs, args, device, compact, bwd, half)
+        print(json.dumps(out))
+        return
     main_res = run_config("cfg2", args.steps, args.warmup, device, compact, backward=bwd)
     c = CONFIGS["cfg2"]
     if main_res["compacted"]:
@@ -695,57 +755,10 @@ def main():
     if main_res.get("ms_fwd_bwd"):
         out["roofline"]["fwd_bwd"] = {"flops_per_call": 14.0 * 64 * 64 * c["D"] * main_res["n_exec"], "duration_ms": main_res["ms_fwd_bwd"],
                                       "achieved": main_res["tflops_fwd_bwd"], "frac": main_res["tflops_fwd_bwd"] / PEAK_BF16_TFLOPS}
-    if compact and "tile_skip" in legs:
-        # the same workload through the tile-skipping kernel alone (one kernel per call, no pre-pass)
-        ts = run_config("cfg2", *half, device, compact=False, backward=False)
-        out["tile_skip_path"] = {"ms_fwd": ts["ms_fwd"], "n_exec_tiles": ts["n_exec"], "tflops_fwd": ts["tflops_fwd"],
-                                 "frac_of_peak": ts["tflops_fwd"] / PEAK_BF16_TFLOPS,
-                                 "kernel": "fdma::fwd_colmask_kernel<bf16, 128, causal> (compact_mode = never)"}
-    if compact and "zero" in legs:
-        # The same launches on all-zero Q / K / V / bias: identical mask, tiles and instruction stream.  The device lowers
-        # its clocks under the switching activity of real operands (a register-fed MFMA loop reaches 2.4 PFLOP/s on
-        # constant operands and 1.9 on random ones), so this is what the kernels' schedule sustains when it does not.
-        tz = run_config("cfg2", *half, device, compact=False, backward=False, zero_inputs=True)
-        out.setdefault("tile_skip_path", {})["zero_operands"] = {"ms_fwd": tz["ms_fwd"], "tflops_fwd": tz["tflops_fwd"],
-                                                                 "frac_of_peak": tz["tflops_fwd"] / PEAK_BF16_TFLOPS}
-        cz = run_config("cfg2", *half, device, compact=True, backward=bwd, zero_inputs=True)
-        out["zero_operands"] = {"ms_fwd": cz["ms_fwd"], "tflops_fwd": cz["tflops_fwd"],
-                                "frac_of_peak": cz["tflops_fwd"] / PEAK_BF16_TFLOPS, "ms_fwd_bwd": cz.get("ms_fwd_bwd"),
-                                "note": "same mask, tiles and instruction stream as the headline figures, all-zero Q / K / V / "
-                                        "bias: what the schedule sustains when the device does not lower its clock"}
-    if "probe" in legs:
-        probe = run_mfma_probe()
-        if probe is not None:
-            out["mfma_probe"] = probe
+    run_secondary_legs(out, legs, args, device, compact, bwd, half)
     if args.traffic_bytes is not None:
         out["roofline"]["traffic"] = args.traffic_bytes
-    if args.calib_copy:
-        src = torch.empty(256 << 20, dtype=torch.uint8, device=device).fill_(1)
-        dst = torch.empty_like(src)
-        dst.copy_(src)
-        torch.cuda.synchronize()
-    # The other benchmark configurations, each against the roofline that bounds it: cfg3 (a bias and a mask per query
-    # row, with its dBias) and cfg5 (decode) against HBM, cfg4 (long sequence, narrow window) against the matrix pipe.
     quarter = (max(3, args.steps // 4), max(1, args.warmup // 2))
-    configs = {}
-    for name in ("cfg3", "cfg4", "cfg5"):
-        if name not in legs:
-            continue
-        if name == "cfg5":  # (a call of some 20 us: many steps, or the two events' own resolution shows)
-            r = run_config(name, 10 * args.steps, 2 * args.warmup, device, compact, backward=False)
-            r["ms_fwd_c_abi"] = time_decode_c_abi(name, 10 * args.steps, 2 * args.warmup, device)
-        else:
-            r = run_config(name, *quarter, device, compact, backward=bwd)
-        c2 = CONFIGS[name]
-        r["workload"] = "%s: B=%d Lq=%d Lk=%d H=%d Hkv=%d d=%d bias%s top-%d%s" % (
-            name, c2["B"], c2["Lq"], c2["Lk"], c2["H"], c2["Hk"], c2["D"], list(c2["bias"]), c2["W"], " ∩ causal" if c2["causal"] else "")
-        r["roofline"] = config_roofline(name, r)
-        configs[name] = r
-        torch.cuda.empty_cache()
-    if configs:
-        out["configs"] = configs
-    if "w_sweep" in legs:
-        out["w_sweep_fwd"] = run_w_sweep_fwd(*quarter, device)
     if args.all:
         out["cfg1"] = run_config("cfg1", *quarter, device, compact)
         out["mask_builder"] = run_mask_builder(*half, device)

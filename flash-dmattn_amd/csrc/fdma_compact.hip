@@ -445,6 +445,111 @@ __global__ void __launch_bounds__(256) compact_image_kernel(const FwdParams p, i
     }
 }
 
+// The same images from a plain bool mask, in one launch, with the work split over ORIGINAL columns (as in
+// compact_scan_gather_kernel): a workgroup owns SEG_KEYS consecutive columns of a pair, counts the kept columns in
+// front of them (at most Lk mask bytes, served by the L2), numbers its own, writes its part of the lists and puts its
+// kept keys where their ranks say: K rows and side rows are whole pieces of a tile image, V goes in transposed, one
+// 16-bit element per (key, d) -- neighbouring ranks belong to neighbouring threads or workgroups, and the L2 merges
+// the pieces.  The workgroup that owns the end of the row also clears what is left of the pair's last tile.  (A
+// workgroup per tile, each counting the whole row for itself, took 34 us on 4 x 32768 keys; this takes a quarter.)
+template <typename T>
+__global__ void __launch_bounds__(256) compact_scan_image_kernel(const FwdParams p, int32_t *idx, int32_t *cnt, int32_t *count, float *fb,
+                                                                 char *img_kv, char *img_x, int ld, int Hfb, int tiles) {
+    using E = Elem<T>;
+    __shared__ int s_wave[4], s_src[SEG_KEYS];
+    const int pair = blockIdx.y, b = pair / p.Hk, hk = pair % p.Hk;
+    const int hm = p.Hm == 1 ? 0 : hk;
+    const uint8_t *mrow = p.mask + b * p.m_b + hm * p.m_h;
+    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int s0 = blockIdx.x * SEG_KEYS;
+    int before = 0;
+    for (int c = tid * 16; c < s0; c += 256 * 16) {
+        const u32x4_t mv = *(const u32x4_t *)(mrow + c);
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            const uint32_t x = mv[e];
+            before += __builtin_popcount((((x & 0x7f7f7f7fu) + 0x7f7f7f7fu) | x) & 0x80808080u);
+        }
+    }
+#pragma unroll
+    for (int off = 32; off > 0; off >>= 1) before += __shfl_xor(before, off);
+    if (lane == 0) s_wave[wave] = before;
+    __syncthreads();
+    const int base = s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3];
+    __syncthreads();
+    const int col = s0 + tid;
+    const bool kept = col < p.Lk && mrow[col] != 0;
+    const uint64_t vote = __ballot(kept);
+    const int excl_w = __builtin_popcountll(vote & ((1ull << lane) - 1ull));
+    if (lane == 0) s_wave[wave] = __builtin_popcountll(vote);
+    __syncthreads();
+    int woff = 0, n_seg = 0;
+#pragma unroll
+    for (int w = 0; w < 4; w++) {
+        const int v = s_wave[w];
+        if (w < wave) woff += v;
+        n_seg += v;
+    }
+    const int excl = woff + excl_w;
+    int32_t *irow = idx + (size_t)pair * ld, *crow = cnt + (size_t)pair * ld;
+    if (kept) {
+        irow[base + excl] = col;
+        s_src[excl] = col;
+    }
+    if (col < ld) crow[col] = base + excl + (kept ? 1 : 0);  // (columns from Lk to ld repeat the total)
+    const bool owns_end = s0 + SEG_KEYS >= ld;
+    const int total = base + n_seg;  // (the pair's total only where owns_end)
+    if (owns_end && tid == 0) count[pair] = total;
+    __syncthreads();
+    const uint16_t *kb = (const uint16_t *)p.k + b * p.k_b + hk * p.k_h;
+    const uint16_t *vb = (const uint16_t *)p.v + b * p.v_b + hk * p.v_h;
+    char *pair_img = img_kv + (size_t)pair * tiles * IMG_KV_BYTES;
+    const u32x4_t zero4 = {0, 0, 0, 0};
+    const int G = p.H / p.Hk;
+    const int nfb = Hfb == p.H ? G : 1;
+    // rows of rank base .. base + n_seg - 1; and (owns_end) cleared rows up to the end of the last tile
+    const int n_pad = owns_end ? ((total + IMG_BN - 1) / IMG_BN) * IMG_BN - total : 0;
+    for (int it = tid; it < (n_seg + n_pad) * 16; it += 256) {
+        const int rr = it >> 4, ch = it & 15;
+        const int rank = base + rr, tl = rank / IMG_BN, row = rank % IMG_BN;
+        char *tile = pair_img + (size_t)tl * IMG_KV_BYTES;
+        u32x4_t kv = zero4, vv = zero4;
+        if (rr < n_seg) {
+            const int src = s_src[rr];
+            kv = *(const u32x4_t *)(kb + (int64_t)src * p.k_r + ch * 8);
+            vv = *(const u32x4_t *)(vb + (int64_t)src * p.v_r + ch * 8);
+        }
+        *(u32x4_t *)(tile + row * (IMG_SK * 2) + ch * 16) = kv;
+        uint16_t *vt = (uint16_t *)(tile + IMG_K_BYTES) + (ch * 8) * IMG_SVT + row;
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+            vt[(2 * e) * IMG_SVT] = (uint16_t)(vv[e] & 0xffffu);
+            vt[(2 * e + 1) * IMG_SVT] = (uint16_t)(vv[e] >> 16);
+        }
+    }
+    for (int it = tid; it < (n_seg + n_pad) * nfb; it += 256) {
+        const int gi = it / (n_seg + n_pad), rr = it - gi * (n_seg + n_pad);
+        const int rank = base + rr, tl = rank / IMG_BN, row = rank % IMG_BN;
+        const bool real = rr < n_seg;
+        const int hfb = Hfb == p.H ? hk * G + gi : hk;
+        float v = 0.f;
+        if (real && p.bias) {
+            const int hb = p.Hb == p.H ? hfb : (p.Hb == 1 ? 0 : hk);
+            v = E::lo((uint32_t)((const uint16_t *)p.bias)[b * p.bi_b + hb * p.bi_h + s_src[rr]]) * kLog2e;
+        }
+        if (real) fb[((size_t)b * Hfb + hfb) * ld + rank] = v;
+        const u32x2_t pc = split3<T>(v);
+        u32x4_t xrow;
+        xrow[0] = pc[0];
+        xrow[1] = pc[1] | (E::pack2(0.f, real ? 0.f : -INFINITY) & 0xffff0000u);
+        xrow[2] = E::pack2(E::kRefWeight, 1.f);
+        xrow[3] = 0;
+        char *xr = img_x + (((size_t)b * Hfb + hfb) * tiles + tl) * IMG_X_BYTES + row * 32;
+        *(u32x4_t *)xr = xrow;
+        *(u32x4_t *)(xr + 16) = zero4;
+    }
+}
+
 // Gradient rows (dK, dV) and columns (dBias) of dropped keys: no workgroup of the compacted backward
 // owns them, and the operator's contract is that they come back as zeros.
 __device__ __forceinline__ void zero_block(const BwdParams &p, bool dbias_direct, int block_x, int pair) {
@@ -781,11 +886,19 @@ hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, 
     if (l.img && !bp) {
         // forward on tile images: lists, fused bias and images in one launch
         char *img_kv = w + l.off_k, *img_x = w + l.off_v;
-        const dim3 igrid(p.Lk / IMG_BN + 1, pairs);
-        if (dtype == 0)
-            hipLaunchKernelGGL((compact_image_kernel<bf16_tag>), igrid, dim3(256), 0, stream, p, idx, cnt, count, fb, img_kv, img_x, l.ld, l.Hfb, l.img_tiles);
-        else
-            hipLaunchKernelGGL((compact_image_kernel<fp16_tag>), igrid, dim3(256), 0, stream, p, idx, cnt, count, fb, img_kv, img_x, l.ld, l.Hfb, l.img_tiles);
+        if (p.kept_idx) {  // lists handed over: a workgroup per tile copies its part of them and builds the tile
+            const dim3 igrid(p.Lk / IMG_BN + 1, pairs);
+            if (dtype == 0)
+                hipLaunchKernelGGL((compact_image_kernel<bf16_tag>), igrid, dim3(256), 0, stream, p, idx, cnt, count, fb, img_kv, img_x, l.ld, l.Hfb, l.img_tiles);
+            else
+                hipLaunchKernelGGL((compact_image_kernel<fp16_tag>), igrid, dim3(256), 0, stream, p, idx, cnt, count, fb, img_kv, img_x, l.ld, l.Hfb, l.img_tiles);
+        } else {           // a plain mask: a workgroup per SEG_KEYS original columns
+            const dim3 sgrid((l.ld + SEG_KEYS - 1) / SEG_KEYS, pairs);
+            if (dtype == 0)
+                hipLaunchKernelGGL((compact_scan_image_kernel<bf16_tag>), sgrid, dim3(256), 0, stream, p, idx, cnt, count, fb, img_kv, img_x, l.ld, l.Hfb, l.img_tiles);
+            else
+                hipLaunchKernelGGL((compact_scan_image_kernel<fp16_tag>), sgrid, dim3(256), 0, stream, p, idx, cnt, count, fb, img_kv, img_x, l.ld, l.Hfb, l.img_tiles);
+        }
         if ((e = hipGetLastError()) != hipSuccess) return e;
         p.cmp.idx = idx;
         p.cmp.cnt = cnt;
