@@ -710,7 +710,7 @@ def main():
     main_res = run_config("cfg2", args.steps, args.warmup, device, compact, backward=bwd)
     c = CONFIGS["cfg2"]
     if main_res["compacted"]:
-        kernel = ("fdma::fwd_stream_kernel<bf16, causal> (compacted keys, tile images), with its pre-pass (compact_image_kernel) "
+        kernel = ("fdma::fwd_stream_kernel<bf16, causal> (compacted keys, tile images), with its pre-pass (compact_scan_image_kernel) "
                   "in the same call: the duration is that of the whole forward call")
         flops_model = ("4*64*64*d per executed 64x64 tile on the compacted key axis (kept columns packed to the front per "
                        "(batch, kv head)); a 64-row query block executes ceil(visible kept columns / 64) tiles")
