@@ -339,7 +339,7 @@ def config_roofline(name, r):
            "flops_model": "4*64*64*d per executed 64x64 tile (compacted key axis when column_compaction), 14*... forward + backward",
            "column_compaction": bool(r.get("compacted")), "n_exec_tiles": r["n_exec"],
            "achieved": r["tflops_fwd"], "frac": r["tflops_fwd"] / PEAK_BF16_TFLOPS, "duration_ms": r["ms_fwd"],
-           "kernel": "fdma::fwd_colmask_kernel with its pre-pass, whole operator call"}
+           "kernel": "fdma::fwd_stream_kernel with its pre-pass (compact_scan_image_kernel), whole operator call" if r.get("compacted") else "fdma::fwd_colmask_kernel (tile skipping), whole operator call"}
     if "ms_fwd_bwd" in r:
         blk["fwd_bwd"] = {"flops_per_call": 3.5 * flops, "duration_ms": r["ms_fwd_bwd"], "achieved": r["tflops_fwd_bwd"],
                           "frac": r["tflops_fwd_bwd"] / PEAK_BF16_TFLOPS}

@@ -257,6 +257,15 @@ __global__ void __launch_bounds__(256) compact_scan_gather_kernel(const FwdParam
 // IMG_SK elements, V transposed (rows of IMG_SVT elements), and per bias class the 16-element side rows (three 16-bit
 // pieces of bias * log2(e), the mask term, two ones, zeros).  Rows beyond the last kept key are zeros with a side row
 // that says "masked": the forward needs no row limit.  With lists handed over by the caller nothing is counted.
+// Eight 16-bit elements times a factor (the K rows of a tile image carry softmax_scale * log2(e): the streaming forward
+// then uses Q as it lies in memory, and what would be a scaling pass over Q per work item is paid once per key here)
+template <typename T> __device__ __forceinline__ u32x4_t scale8(u32x4_t v, float f) {
+    using E = Elem<T>;
+#pragma unroll
+    for (int e = 0; e < 4; e++) v[e] = E::pack2(E::lo(v[e]) * f, E::hi(v[e]) * f);
+    return v;
+}
+
 template <typename T>
 __global__ void __launch_bounds__(256) compact_image_kernel(const FwdParams p, int32_t *idx, int32_t *cnt, int32_t *count, float *fb,
                                                             char *img_kv, char *img_x, int ld, int Hfb, int tiles) {
@@ -406,7 +415,7 @@ __global__ void __launch_bounds__(256) compact_image_kernel(const FwdParams p, i
             if (src >= 0) braw0 = ((const uint16_t *)p.bias)[b * p.bi_b + hb * p.bi_h + src];
         }
 #pragma unroll
-        for (int it = 0; it < 4; it++) *(u32x4_t *)(tile + (rr0 + 16 * it) * (IMG_SK * 2) + ch * 16) = kv[it];
+        for (int it = 0; it < 4; it++) *(u32x4_t *)(tile + (rr0 + 16 * it) * (IMG_SK * 2) + ch * 16) = scale8<T>(kv[it], p.scale_log2);
         char *vt = tile + IMG_K_BYTES;
 #pragma unroll
         for (int dd = 0; dd < 8; dd++) {
@@ -519,7 +528,7 @@ __global__ void __launch_bounds__(256) compact_scan_image_kernel(const FwdParams
             kv = *(const u32x4_t *)(kb + (int64_t)src * p.k_r + ch * 8);
             vv = *(const u32x4_t *)(vb + (int64_t)src * p.v_r + ch * 8);
         }
-        *(u32x4_t *)(tile + row * (IMG_SK * 2) + ch * 16) = kv;
+        *(u32x4_t *)(tile + row * (IMG_SK * 2) + ch * 16) = scale8<T>(kv, p.scale_log2);
         uint16_t *vt = (uint16_t *)(tile + IMG_K_BYTES) + (ch * 8) * IMG_SVT + row;
 #pragma unroll
         for (int e = 0; e < 4; e++) {

@@ -6,8 +6,9 @@
 // program: scores through the matrix pipe with the softmax's bias / mask / reference point folded into one more
 // k-step (the 16-element side rows), a software pipeline over 32-key half tiles, no row maximum on the common path.
 // What differs is everything around the tile program:
-//   * Tile images.  The compaction pre-pass (compact_image_kernel, fdma_compact.hip) has written, per 64-key tile
-//     of the compacted key axis, exactly the bytes this kernel keeps in LDS: the K tile with padded rows followed
+//   * Tile images.  The compaction pre-pass (compact_scan_image_kernel / compact_image_kernel, fdma_compact.hip) has
+//     written, per 64-key tile of the compacted key axis, exactly the bytes this kernel keeps in LDS: the K tile with
+//     padded rows -- already multiplied by softmax_scale * log2(e), so Q is used as it lies in memory -- followed
 //     by V already transposed, and the side rows of the keys.  A tile is fetched with contiguous direct
 //     global->LDS loads (global_load_lds_dwordx4: a wave moves 1 KB per instruction, lane after lane): no staging
 //     registers, no permutes, no LDS stores, no staging roles -- V is transposed once per (batch, kv head) pair
@@ -20,6 +21,8 @@
 //   * The rare items whose scores leave the common path's range (or whose reference point cannot be expressed)
 //     are noted in an LDS bit set and redone at the end of the workgroup's life by a plain tile-by-tile path that
 //     reads its fragments straight from the images in global memory.
+//   * Output rows leave under the next item's matrix work: an item ends by packing its rows into registers, and the
+//     next item's first step behind a barrier issues the stores one per slot (see pack_rows / store_piece).
 // Items are dealt to the workgroups of an XCD in rounds, odd rounds reversed: heaviest query blocks first, every
 // workgroup the same causal work, K / V of a (batch, kv head) pair in one XCD's L2.
 #include <type_traits>
@@ -121,7 +124,8 @@ __global__ void __launch_bounds__(ST_THREADS, 1) fwd_stream_kernel(const FwdPara
         asm volatile("" : "+v"(x));
         return x;
     };
-    // Q fragments of an item's rows (rows beyond the end are clamped here and cleared when scaled)
+    // Q fragments of an item's rows, as they lie in memory: the K rows of the images carry softmax_scale * log2(e).  (Rows
+    // beyond the end repeat the last row; they are never stored.)
     auto load_q = [&](const Item &it) {
         const int b = it.pair / p.Hk;
         const int qrow = it.m0 + wave * 32 + opaque(r);
@@ -286,6 +290,17 @@ __global__ void __launch_bounds__(ST_THREADS, 1) fwd_stream_kernel(const FwdPara
     u32x4_t qx;
     int vis_wave = 0;
 
+    // rows of the previous item on their way out (see pack_rows)
+    u32x4_t po[2 * DB];
+    uint16_t *st_ptr = nullptr;
+    uint64_t st_mask = 0;
+    auto store_piece = [&](int k) {  // piece k: columns 32 (k / 2) + 16 (k % 2) + 8 g .. + 7 of this lane's row
+        uint64_t keep;
+        asm volatile("s_mov_b64 %0, exec\n\ts_mov_b64 exec, %1\n\ts_cbranch_execz 1f\n\t"
+                     "global_store_dwordx4 %2, %3, off offset:%4\n1:\n\ts_mov_b64 exec, %0"
+                     : "=&s"(keep) : "s"(st_mask), "v"(st_ptr), "v"(po[k]), "n"(64 * (k / 2) + 32 * (k % 2)) : "memory");
+    };
+
     auto causal_mask = [&](f32x16_t &s, int col0) {
         const int lim = vis_lane - 1 - col0 - 8 * g;
 #pragma unroll
@@ -381,8 +396,14 @@ __global__ void __launch_bounds__(ST_THREADS, 1) fwd_stream_kernel(const FwdPara
                     if (f == (SCORES ? 1 + 3 * i : 1 + i)) fetch_piece(i);
             }
 #endif
+            if (FETCH) {  // the previous item's output rows, one piece per slot (a step behind the barrier: see store_piece)
+#pragma unroll
+                for (int k = 0; k < 8; k++)
+                    if (f == (SCORES ? 2 + 3 * (k / 2) + (k & 1) : k)) store_piece(k);
+            }
             __builtin_amdgcn_sched_barrier(0);
         }
+        if (FETCH) st_mask = 0;
         const float psum = psum0 + psum1;
         row_sum += psum;
 #pragma unroll
@@ -394,8 +415,14 @@ __global__ void __launch_bounds__(ST_THREADS, 1) fwd_stream_kernel(const FwdPara
         if (__any(!(psum <= 16384.f)) && lane == 0) atomicOr(&sRedo[rd >> 5], 1u << (rd & 31));
     };
 
-    // output rows of an item: O / sum, LSE
-    auto write_rows = [&](const Item &it) {
+    // Output rows of an item.  pack_rows() turns the accumulators into 16-bit rows (O / sum) held in `po`, writes the
+    // LSE and notes which lanes have a row to store (st_mask); the stores themselves -- eight of 16 bytes per lane -- are
+    // issued one per slot by the NEXT item's first step behind a barrier (store_piece), where they travel under matrix
+    // work: issued in one go they fill the CU's store path for more than a microsecond per item with every wave waiting,
+    // and issued in front of a barrier they would be waited for there (publish() waits for everything in flight).
+    // A store is written in assembly: lanes without a row are switched off through exec (restored at once), and when no
+    // store is pending (st_mask == 0: every step but the first of an item) the instruction is jumped over.
+    auto write_rows = [&](const Item &it) {  // at once (items without tiles, the redo pass)
         const int b = it.pair / p.Hk;
         const int qrow = it.m0 + wave * 32 + opaque(r);
         const float total = xhalf_sum(row_sum);
@@ -418,6 +445,31 @@ __global__ void __launch_bounds__(ST_THREADS, 1) fwd_stream_kernel(const FwdPara
             }
         }
     };
+    auto pack_rows = [&](const Item &it) {
+        const int b = it.pair / p.Hk;
+        const int qrow = it.m0 + wave * 32 + opaque(r);
+        const float total = xhalf_sum(row_sum);
+        const float inv = total > 0.f ? 1.f / total : 0.f;
+        const bool valid = qrow < Lq;
+        st_ptr = (uint16_t *)p.o + b * p.o_b + (int64_t)(valid ? qrow : 0) * p.o_r + it.h * p.o_h + 8 * g;
+#pragma unroll
+        for (int db = 0; db < DB; db++)
+#pragma unroll
+            for (int blk = 0; blk < 2; blk++)
+#pragma unroll
+                for (int e = 0; e < 4; e++)
+                    po[2 * db + blk][e] = E::pack2(o[db][8 * blk + 2 * e] * inv, o[db][8 * blk + 2 * e + 1] * inv);
+        st_mask = __ballot(valid);
+        if (valid && g == 0) {
+            const float lse = total > 0.f ? (row_ref + __builtin_amdgcn_logf(total)) * kLn2 : INFINITY;
+            p.lse[b * p.lse_b + it.h * p.lse_h + qrow] = lse;
+        }
+    };
+    auto flush_rows = [&]() {  // whatever is pending, at once
+#pragma unroll
+        for (int k = 0; k < 8; k++) store_piece(k);
+        st_mask = 0;
+    };
     auto reset_rows = [&]() {
         row_sum = 0.f;
         row_ref = -INFINITY;
@@ -430,15 +482,6 @@ __global__ void __launch_bounds__(ST_THREADS, 1) fwd_stream_kernel(const FwdPara
         for (int db = 0; db < DB; db++)
 #pragma unroll
             for (int i = 0; i < 16; i++) o[db][i] = 0.f;
-    };
-    auto scale_q = [&](const Item &it) {
-        const bool row_ok = it.m0 + wave * 32 + opaque(r) < Lq;
-#pragma unroll
-        for (int ks = 0; ks < KS; ks++)
-#pragma unroll
-            for (int e = 0; e < 4; e++)
-                qf[ks][e] = row_ok ? E::pack2(E::lo(qf[ks][e]) * p.scale_log2, E::hi(qf[ks][e]) * p.scale_log2) : 0u;
-        if (CAUSAL) vis_wave = __builtin_amdgcn_readfirstlane(vis_lane);  // (lane 0 holds the wave's first row)
     };
 
     const std::true_type yes;
@@ -458,7 +501,7 @@ __global__ void __launch_bounds__(ST_THREADS, 1) fwd_stream_kernel(const FwdPara
         reset_rows();
         FDMA_STAMP(4 + 4 * rd);
         if (nt > 0) {
-            scale_q(cur);
+            if (CAUSAL) vis_wave = __builtin_amdgcn_readfirstlane(vis_lane);  // (lane 0 holds the wave's first row)
             FDMA_STAMP(5 + 4 * rd);
 #ifdef FDMA_DBG
             if (tid == 0 && rd < 4) g_stream_dbg[blockIdx.x * 64 + 56 + rd] = __builtin_amdgcn_s_memtime();
@@ -528,9 +571,10 @@ __global__ void __launch_bounds__(ST_THREADS, 1) fwd_stream_kernel(const FwdPara
 #ifdef FDMA_DBG
             if (tid == 0 && rd < 4) g_stream_dbg[blockIdx.x * 64 + 60 + rd] = __builtin_amdgcn_s_memtime();
 #endif
-            write_rows(cur);
+            pack_rows(cur);
             FDMA_STAMP(7 + 4 * rd);
         } else {
+            flush_rows();
             write_rows(cur);  // no visible key: zeros and LSE = +inf
             load_q(nxt);
         }
@@ -538,6 +582,7 @@ __global__ void __launch_bounds__(ST_THREADS, 1) fwd_stream_kernel(const FwdPara
         rd = rd_next;
     }
 
+    flush_rows();  // the last item's rows
     // ---- drain: nothing of this workgroup's may land in the LDS of the next one
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
@@ -568,7 +613,7 @@ __global__ void __launch_bounds__(ST_THREADS, 1) fwd_stream_kernel(const FwdPara
             const char *ximg = p.cmp.img_x + ((int64_t)b * p.cmp.Hfb + hfb) * p.cmp.img_tiles * IMG_X_BYTES;
             load_q(it);
             reset_rows();
-            scale_q(it);
+            if (CAUSAL) vis_wave = __builtin_amdgcn_readfirstlane(vis_lane);
             const uint32_t oK = (uint32_t)((a_row * SK + g * 8) * 2), oV = IMG_K_BYTES + (uint32_t)((a_row * SVT + 8 * g) * 2);
             const uint32_t oX = (uint32_t)(a_row * 32 + g * 16);
             for (int t = 0; t < nt; t++) {

@@ -25,7 +25,7 @@ struct Compact {
     int32_t on;            // 0 = no compaction: k / v are the caller's tensors
     // Tile images (forward at head dim 128 on large grids, see fwd_stream_applicable): instead of row-major copies the
     // pre-pass writes, per 64-key tile of the compacted key axis, exactly the bytes the forward kernel keeps in LDS --
-    // the K tile with padded rows followed by V already transposed (img_kv, IMG_KV_BYTES per tile, img_tiles tiles per
+    // the K tile with padded rows (times softmax_scale * log2(e)) followed by V already transposed (img_kv, IMG_KV_BYTES per tile, img_tiles tiles per
     // (batch, kv head) pair) and the 16-element side rows of the keys (img_x, IMG_X_BYTES per tile, per (batch, fb
     // head)) -- so that the forward fetches a tile with contiguous global->LDS loads.  nullptr = row-major copies.
     const char *img_kv;

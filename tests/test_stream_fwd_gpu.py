@@ -92,7 +92,9 @@ def test_streaming_forward_and_its_backward_vs_oracle(name):
     _cabi.stream_min_items(1)
     assert (out.float() - out2.float()).abs().max().item() <= 2e-2
     fin = torch.isfinite(lse2)
-    assert torch.equal(torch.isfinite(lse), fin) and (lse[fin] - lse2[fin]).abs().max().item() <= 1e-3
+    # (the streaming form reads K pre-multiplied by the softmax scale and rounded to 16 bits, the other one rounds the
+    # scaled Q: scores differ by the rounding of one operand, and so does the LSE of a row with few keys)
+    assert torch.equal(torch.isfinite(lse), fin) and (lse[fin] - lse2[fin]).abs().max().item() <= 1e-2
     # a second run gives the same bits
     out3, lse3, grads3 = _run(q, k, v, mask, bias, causal, dout=dout)
     assert torch.equal(out, out3) and torch.equal(lse, lse3)
