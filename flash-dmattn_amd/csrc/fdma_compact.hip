@@ -457,28 +457,40 @@ __global__ void __launch_bounds__(256) compact_image_kernel(const FwdParams p, i
 // The same images from a plain bool mask, in one launch, with the work split over ORIGINAL columns (as in
 // compact_scan_gather_kernel): a workgroup owns SEG_KEYS consecutive columns of a pair, counts the kept columns in
 // front of them (at most Lk mask bytes, served by the L2), numbers its own, writes its part of the lists and puts its
-// kept keys where their ranks say: K rows and side rows are whole pieces of a tile image, V goes in transposed, one
-// 16-bit element per (key, d) -- neighbouring ranks belong to neighbouring threads or workgroups, and the L2 merges
-// the pieces.  The workgroup that owns the end of the row also clears what is left of the pair's last tile.  (A
+// kept keys where their ranks say: K rows and side rows are whole pieces of a tile image, V goes in transposed through
+// LDS -- neighbouring ranks of one head-dim element are neighbours in the image, whichever workgroup owns them.  The workgroup that owns the end of the row also clears what is left of the pair's last tile.  (A
 // workgroup per tile, each counting the whole row for itself, took 34 us on 4 x 32768 keys; this takes a quarter.)
 template <typename T>
 __global__ void __launch_bounds__(256) compact_scan_image_kernel(const FwdParams p, int32_t *idx, int32_t *cnt, int32_t *count, float *fb,
                                                                  char *img_kv, char *img_x, int ld, int Hfb, int tiles) {
     using E = Elem<T>;
+    constexpr int VT_CHUNK = 128, VT_PITCH = 130;  // V rows parked in LDS at a time; their pitch in elements (odd in 32-bit words)
     __shared__ int s_wave[4], s_src[SEG_KEYS];
+    __shared__ __attribute__((aligned(16))) uint16_t s_v[VT_CHUNK * VT_PITCH];
     const int pair = blockIdx.y, b = pair / p.Hk, hk = pair % p.Hk;
     const int hm = p.Hm == 1 ? 0 : hk;
     const uint8_t *mrow = p.mask + b * p.m_b + hm * p.m_h;
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int s0 = blockIdx.x * SEG_KEYS;
+    // (this thread's own column and up to four pieces of the row in front of the segment are requested together: the
+    // launch is a chain of trips to memory, not a stream of bytes)
+    const int col = s0 + tid;
+    const uint8_t own = col < p.Lk ? mrow[col] : (uint8_t)0;
     int before = 0;
-    for (int c = tid * 16; c < s0; c += 256 * 16) {
-        const u32x4_t mv = *(const u32x4_t *)(mrow + c);
+    for (int c = tid * 16; c < s0; c += 4 * 256 * 16) {
+        u32x4_t mv[4];
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-            const uint32_t x = mv[e];
-            before += __builtin_popcount((((x & 0x7f7f7f7fu) + 0x7f7f7f7fu) | x) & 0x80808080u);
+        for (int u = 0; u < 4; u++) {
+            const int cc = c + u * 256 * 16;
+            mv[u] = cc < s0 ? *(const u32x4_t *)(mrow + cc) : u32x4_t{0, 0, 0, 0};
         }
+#pragma unroll
+        for (int u = 0; u < 4; u++)
+#pragma unroll
+            for (int e = 0; e < 4; e++) {
+                const uint32_t x = mv[u][e];
+                before += __builtin_popcount((((x & 0x7f7f7f7fu) + 0x7f7f7f7fu) | x) & 0x80808080u);
+            }
     }
 #pragma unroll
     for (int off = 32; off > 0; off >>= 1) before += __shfl_xor(before, off);
@@ -486,8 +498,7 @@ __global__ void __launch_bounds__(256) compact_scan_image_kernel(const FwdParams
     __syncthreads();
     const int base = s_wave[0] + s_wave[1] + s_wave[2] + s_wave[3];
     __syncthreads();
-    const int col = s0 + tid;
-    const bool kept = col < p.Lk && mrow[col] != 0;
+    const bool kept = own != 0;
     const uint64_t vote = __ballot(kept);
     const int excl_w = __builtin_popcountll(vote & ((1ull << lane) - 1ull));
     if (lane == 0) s_wave[wave] = __builtin_popcountll(vote);
@@ -516,25 +527,68 @@ __global__ void __launch_bounds__(256) compact_scan_image_kernel(const FwdParams
     const u32x4_t zero4 = {0, 0, 0, 0};
     const int G = p.H / p.Hk;
     const int nfb = Hfb == p.H ? G : 1;
-    // rows of rank base .. base + n_seg - 1; and (owns_end) cleared rows up to the end of the last tile
+    // rows of rank base .. base + n_seg - 1; and (owns_end) cleared rows up to the end of the last tile.  At most
+    // VT_CHUNK rows at a time: their K rows go straight to the image as 16-byte pieces (all loads of up to four pieces
+    // per thread requested before the first store), their V rows are parked in LDS and leave transposed, eight
+    // neighbouring ranks of one head-dim element per 16-byte store; only where eight ranks are shared with the
+    // neighbouring workgroup (or chunk) do they leave one by one.  (One 16-bit store per (key, d) kept the L2 busy with
+    // two million two-byte requests per launch on 8 x 2048 kept keys.)
     const int n_pad = owns_end ? ((total + IMG_BN - 1) / IMG_BN) * IMG_BN - total : 0;
-    for (int it = tid; it < (n_seg + n_pad) * 16; it += 256) {
-        const int rr = it >> 4, ch = it & 15;
-        const int rank = base + rr, tl = rank / IMG_BN, row = rank % IMG_BN;
-        char *tile = pair_img + (size_t)tl * IMG_KV_BYTES;
-        u32x4_t kv = zero4, vv = zero4;
-        if (rr < n_seg) {
-            const int src = s_src[rr];
-            kv = *(const u32x4_t *)(kb + (int64_t)src * p.k_r + ch * 8);
-            vv = *(const u32x4_t *)(vb + (int64_t)src * p.v_r + ch * 8);
-        }
-        *(u32x4_t *)(tile + row * (IMG_SK * 2) + ch * 16) = scale8<T>(kv, p.scale_log2);
-        uint16_t *vt = (uint16_t *)(tile + IMG_K_BYTES) + (ch * 8) * IMG_SVT + row;
+    const int n_rows = n_seg + n_pad;
+    // (the bias value of this thread's first side row travels with the rows)
+    uint32_t braw0 = 0;
+    if (p.bias && tid < n_rows * nfb) {
+        const int gi = tid / n_rows, rr = tid - gi * n_rows;
+        const int hfb = Hfb == p.H ? hk * G + gi : hk;
+        const int hb = p.Hb == p.H ? hfb : (p.Hb == 1 ? 0 : hk);
+        if (rr < n_seg) braw0 = ((const uint16_t *)p.bias)[b * p.bi_b + hb * p.bi_h + s_src[rr]];
+    }
+    for (int c0 = 0; c0 < n_rows; c0 += VT_CHUNK) {
+        const int nc = n_rows - c0 < VT_CHUNK ? n_rows - c0 : VT_CHUNK;
+        for (int it0 = tid; it0 < nc * 16; it0 += 256 * 4) {
+            u32x4_t kv[4], vv[4];
 #pragma unroll
-        for (int e = 0; e < 4; e++) {
-            vt[(2 * e) * IMG_SVT] = (uint16_t)(vv[e] & 0xffffu);
-            vt[(2 * e + 1) * IMG_SVT] = (uint16_t)(vv[e] >> 16);
+            for (int u = 0; u < 4; u++) {
+                const int it = it0 + 256 * u, rr = c0 + (it >> 4), ch = it & 15;
+                kv[u] = zero4;
+                vv[u] = zero4;
+                if (it < nc * 16 && rr < n_seg) {
+                    const int src = s_src[rr];
+                    kv[u] = *(const u32x4_t *)(kb + (int64_t)src * p.k_r + ch * 8);
+                    vv[u] = *(const u32x4_t *)(vb + (int64_t)src * p.v_r + ch * 8);
+                }
+            }
+#pragma unroll
+            for (int u = 0; u < 4; u++) {
+                const int it = it0 + 256 * u, lr = it >> 4, ch = it & 15;
+                if (it < nc * 16) {
+                    const int rank = base + c0 + lr, tl = rank / IMG_BN, row = rank % IMG_BN;
+                    *(u32x4_t *)(pair_img + (size_t)tl * IMG_KV_BYTES + row * (IMG_SK * 2) + ch * 16) = scale8<T>(kv[u], p.scale_log2);
+                    uint32_t *sv = (uint32_t *)(s_v + lr * VT_PITCH + ch * 8);
+#pragma unroll
+                    for (int e = 0; e < 4; e++) sv[e] = vv[u][e];
+                }
+            }
         }
+        __syncthreads();
+        const int r_lo = base + c0, r_hi = r_lo + nc;  // ranks of this chunk
+        const int o_lo = r_lo >> 3, n_oct = ((r_hi + 7) >> 3) - o_lo;
+        for (int i = tid; i < n_oct * 128; i += 256) {
+            const int d = i / n_oct, rank0 = (o_lo + (i - d * n_oct)) * 8;
+            uint16_t *dst = (uint16_t *)(pair_img + (size_t)(rank0 / IMG_BN) * IMG_KV_BYTES + IMG_K_BYTES) + d * IMG_SVT + rank0 % IMG_BN;
+            if (rank0 >= r_lo && rank0 + 8 <= r_hi) {
+                const uint16_t *src = s_v + (rank0 - r_lo) * VT_PITCH + d;
+                u32x4_t w;
+#pragma unroll
+                for (int e = 0; e < 4; e++) w[e] = (uint32_t)src[(2 * e) * VT_PITCH] | ((uint32_t)src[(2 * e + 1) * VT_PITCH] << 16);
+                *(u32x4_t *)dst = w;
+            } else {
+#pragma unroll
+                for (int e = 0; e < 8; e++)
+                    if (rank0 + e >= r_lo && rank0 + e < r_hi) dst[e] = s_v[(rank0 + e - r_lo) * VT_PITCH + d];
+            }
+        }
+        __syncthreads();
     }
     for (int it = tid; it < (n_seg + n_pad) * nfb; it += 256) {
         const int gi = it / (n_seg + n_pad), rr = it - gi * (n_seg + n_pad);
@@ -544,7 +598,8 @@ __global__ void __launch_bounds__(256) compact_scan_image_kernel(const FwdParams
         float v = 0.f;
         if (real && p.bias) {
             const int hb = p.Hb == p.H ? hfb : (p.Hb == 1 ? 0 : hk);
-            v = E::lo((uint32_t)((const uint16_t *)p.bias)[b * p.bi_b + hb * p.bi_h + s_src[rr]]) * kLog2e;
+            const uint32_t braw = it == tid ? braw0 : (uint32_t)((const uint16_t *)p.bias)[b * p.bi_b + hb * p.bi_h + s_src[rr]];
+            v = E::lo(braw) * kLog2e;
         }
         if (real) fb[((size_t)b * Hfb + hfb) * ld + rank] = v;
         const u32x2_t pc = split3<T>(v);
