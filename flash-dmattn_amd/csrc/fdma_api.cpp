@@ -276,8 +276,9 @@ size_t fdma_fwd_counter_bytes(const fdma_fwd_args *a) {
 size_t fdma_fwd_workspace_bytes(const fdma_fwd_args *a) {
     if (!a) return 0;
     if (!fdma::use_decode_path(a->seqlen_q, a->num_heads, a->num_heads_k)) {
-        fdma::FwdParams p;
+        fdma::FwdParams p, pv;
         fill_fwd_params(a, p);
+        if (fdma::compact_per_query_head(p, pv)) return fdma::compact_bytes(pv, false);
         return fdma::use_compact(p) ? fdma::compact_bytes(p, false) : 0;
     }
     const int splits = fdma::decode_num_splits(a->batch, a->num_heads_k, a->seqlen_k);
@@ -316,6 +317,10 @@ int fdma_fwd(const fdma_fwd_args *a, void *hip_stream) {
         e = fdma::launch_fwd_decode(p, a->dtype, stream);
     } else {
         // seqlen_k == 0 falls out of the kernel as O = 0, LSE = +inf (flash_api.cpp:535-539)
+        // (a query-broadcast mask with a row per query head: compacted per query head -- forward only; the backward of
+        // that form skips tiles instead)
+        fdma::FwdParams pv;
+        if (fdma::compact_per_query_head(p, pv)) p = pv;
         if (fdma::use_compact(p)) {
             const size_t need = fdma::compact_bytes(p, false);
             if (!a->workspace || a->workspace_bytes < need)

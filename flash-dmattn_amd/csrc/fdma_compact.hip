@@ -124,8 +124,8 @@ __device__ __forceinline__ void gather_block(const FwdParams &p, const int32_t *
     }
     __syncthreads();
     const int CH = p.d / 8;
-    const uint16_t *kb = (const uint16_t *)p.k + b * p.k_b + hk * p.k_h;
-    const uint16_t *vb = (const uint16_t *)p.v + b * p.v_b + hk * p.v_h;
+    const uint16_t *kb = (const uint16_t *)p.k + b * p.k_b + kv_head(p, hk) * p.k_h;
+    const uint16_t *vb = (const uint16_t *)p.v + b * p.v_b + kv_head(p, hk) * p.v_h;
     uint16_t *kd = kc + ((size_t)pair * p.Lk + c0) * p.d;
     uint16_t *vd = vc + ((size_t)pair * p.Lk + c0) * p.d;
     for (int it = tid; it < GATHER_KEYS * CH; it += 256) {
@@ -149,7 +149,7 @@ __device__ __forceinline__ void gather_block(const FwdParams &p, const int32_t *
         const int hfb = Hfb == p.H ? hk * G + gi : hk;
         float v = 0.f;
         if (p.bias) {
-            const int hb = p.Hb == p.H ? hfb : (p.Hb == 1 ? 0 : hk);
+            const int hb = p.Hb == p.H ? hfb : (p.Hb == 1 ? 0 : kv_head(p, hk));
             v = E::lo((uint32_t)((const uint16_t *)p.bias)[b * p.bi_b + hb * p.bi_h + src]) * kLog2e;
         }
         fb[((size_t)b * Hfb + hfb) * ld + c0 + rr] = v;
@@ -220,8 +220,8 @@ __global__ void __launch_bounds__(256) compact_scan_gather_kernel(const FwdParam
     __syncthreads();
     if (n_seg == 0) return;
     const int CH = p.d / 8;
-    const uint16_t *kb = (const uint16_t *)p.k + b * p.k_b + hk * p.k_h;
-    const uint16_t *vb = (const uint16_t *)p.v + b * p.v_b + hk * p.v_h;
+    const uint16_t *kb = (const uint16_t *)p.k + b * p.k_b + kv_head(p, hk) * p.k_h;
+    const uint16_t *vb = (const uint16_t *)p.v + b * p.v_b + kv_head(p, hk) * p.v_h;
     uint16_t *kd = kc + ((size_t)pair * p.Lk + base) * p.d;
     uint16_t *vd = vc + ((size_t)pair * p.Lk + base) * p.d;
     for (int it = tid; it < n_seg * CH; it += 256) {
@@ -241,7 +241,7 @@ __global__ void __launch_bounds__(256) compact_scan_gather_kernel(const FwdParam
         const int hfb = Hfb == p.H ? hk * G + gi : hk;
         float v = 0.f;
         if (p.bias) {
-            const int hb = p.Hb == p.H ? hfb : (p.Hb == 1 ? 0 : hk);
+            const int hb = p.Hb == p.H ? hfb : (p.Hb == 1 ? 0 : kv_head(p, hk));
             v = E::lo((uint32_t)((const uint16_t *)p.bias)[b * p.bi_b + hb * p.bi_h + src]) * kLog2e;
         }
         fb[((size_t)b * Hfb + hfb) * ld + base + rr] = v;
@@ -386,8 +386,8 @@ __global__ void __launch_bounds__(256) compact_image_kernel(const FwdParams p, i
     // ---- K rows: thread (row, 16-byte chunk), four passes; V^T: thread (key quad, d chunk) transposes 4 keys x 8 d in
     // registers (as the forward used to while staging).  All sixteen row pieces of a thread are requested before the
     // first is stored: one trip to memory for the tile.
-    const uint16_t *kb = (const uint16_t *)p.k + b * p.k_b + hk * p.k_h;
-    const uint16_t *vb = (const uint16_t *)p.v + b * p.v_b + hk * p.v_h;
+    const uint16_t *kb = (const uint16_t *)p.k + b * p.k_b + kv_head(p, hk) * p.k_h;
+    const uint16_t *vb = (const uint16_t *)p.v + b * p.v_b + kv_head(p, hk) * p.v_h;
     char *tile = img_kv + ((size_t)pair * tiles + j) * IMG_KV_BYTES;
     const u32x4_t zero4 = {0, 0, 0, 0};
     const int G = p.H / p.Hk;
@@ -411,7 +411,7 @@ __global__ void __launch_bounds__(256) compact_image_kernel(const FwdParams p, i
         if (p.bias && tid < IMG_BN * nfb) {
             const int gi = tid / IMG_BN, src = s_src[tid - gi * IMG_BN];
             const int hfb = Hfb == p.H ? hk * G + gi : hk;
-            const int hb = p.Hb == p.H ? hfb : (p.Hb == 1 ? 0 : hk);
+            const int hb = p.Hb == p.H ? hfb : (p.Hb == 1 ? 0 : kv_head(p, hk));
             if (src >= 0) braw0 = ((const uint16_t *)p.bias)[b * p.bi_b + hb * p.bi_h + src];
         }
 #pragma unroll
@@ -435,7 +435,7 @@ __global__ void __launch_bounds__(256) compact_image_kernel(const FwdParams p, i
             if (src >= 0 && p.bias) {
                 uint32_t braw = braw0;
                 if (it != tid) {
-                    const int hb = p.Hb == p.H ? hfb : (p.Hb == 1 ? 0 : hk);
+                    const int hb = p.Hb == p.H ? hfb : (p.Hb == 1 ? 0 : kv_head(p, hk));
                     braw = ((const uint16_t *)p.bias)[b * p.bi_b + hb * p.bi_h + src];
                 }
                 v = E::lo(braw) * kLog2e;
@@ -521,8 +521,8 @@ __global__ void __launch_bounds__(256) compact_scan_image_kernel(const FwdParams
     const int total = base + n_seg;  // (the pair's total only where owns_end)
     if (owns_end && tid == 0) count[pair] = total;
     __syncthreads();
-    const uint16_t *kb = (const uint16_t *)p.k + b * p.k_b + hk * p.k_h;
-    const uint16_t *vb = (const uint16_t *)p.v + b * p.v_b + hk * p.v_h;
+    const uint16_t *kb = (const uint16_t *)p.k + b * p.k_b + kv_head(p, hk) * p.k_h;
+    const uint16_t *vb = (const uint16_t *)p.v + b * p.v_b + kv_head(p, hk) * p.v_h;
     char *pair_img = img_kv + (size_t)pair * tiles * IMG_KV_BYTES;
     const u32x4_t zero4 = {0, 0, 0, 0};
     const int G = p.H / p.Hk;
@@ -540,7 +540,7 @@ __global__ void __launch_bounds__(256) compact_scan_image_kernel(const FwdParams
     if (p.bias && tid < n_rows * nfb) {
         const int gi = tid / n_rows, rr = tid - gi * n_rows;
         const int hfb = Hfb == p.H ? hk * G + gi : hk;
-        const int hb = p.Hb == p.H ? hfb : (p.Hb == 1 ? 0 : hk);
+        const int hb = p.Hb == p.H ? hfb : (p.Hb == 1 ? 0 : kv_head(p, hk));
         if (rr < n_seg) braw0 = ((const uint16_t *)p.bias)[b * p.bi_b + hb * p.bi_h + s_src[rr]];
     }
     for (int c0 = 0; c0 < n_rows; c0 += VT_CHUNK) {
@@ -597,7 +597,7 @@ __global__ void __launch_bounds__(256) compact_scan_image_kernel(const FwdParams
         const int hfb = Hfb == p.H ? hk * G + gi : hk;
         float v = 0.f;
         if (real && p.bias) {
-            const int hb = p.Hb == p.H ? hfb : (p.Hb == 1 ? 0 : hk);
+            const int hb = p.Hb == p.H ? hfb : (p.Hb == 1 ? 0 : kv_head(p, hk));
             const uint32_t braw = it == tid ? braw0 : (uint32_t)((const uint16_t *)p.bias)[b * p.bi_b + hb * p.bi_h + s_src[rr]];
             v = E::lo(braw) * kLog2e;
         }
@@ -874,6 +874,14 @@ __global__ void __launch_bounds__(256) compact_bwd_prepass_kernel(const BwdParam
 }
 
 }  // namespace
+
+bool compact_per_query_head(const FwdParams &p, FwdParams &pv) {
+    if (!p.mask || p.m_r != 0 || p.Hm != p.H || p.Hk <= 0 || p.H == p.Hk) return false;
+    pv = p;
+    pv.kv_share = p.H / p.Hk;
+    pv.Hk = p.H;
+    return use_compact(pv);
+}
 
 bool use_compact(const FwdParams &p) {
     const int mode = p.compact_mode;  // 0 = when it pays, 1 = never, 2 = whenever the mask form allows it

@@ -138,11 +138,19 @@ struct FwdParams {
     // (mask batch entry, mask head)
     const int32_t *kept_idx, *kept_cnt, *kept_count;
     int32_t kept_ld;
+    // Forward compaction for a query-broadcast mask with one row per QUERY head (Hm == H > kv heads): every query head
+    // keeps its own keys, so the heads of a kv group share no compacted K / V.  The compaction layer then sees H "kv
+    // heads" (Hk == H above, one compacted copy per query head) and finds the caller's K / V / bias head of such a head
+    // by dividing by kv_share (= query heads per real kv head).  0 or 1: heads are what they say.
+    int32_t kv_share;
     // the mask packed to one bit per key (fdma_mask_bits of the C ABI; nullptr = read the bool mask): strides in bytes,
     // broadcast like the mask
     const uint8_t *mbits;
     int64_t mb_b, mb_h, mb_r;
 };
+
+// the caller's kv head behind head `hk` of the compaction layer (see FwdParams::kv_share)
+__host__ __device__ inline int kv_head(const FwdParams &p, int hk) { return p.kv_share > 1 ? hk / p.kv_share : hk; }
 
 // lengths and first rows of batch entry b
 struct SeqInfo {
@@ -280,6 +288,9 @@ hipError_t launch_bwd_dq(const BwdParams &p, int dtype, hipStream_t stream);
 // p.cmp; for a backward call (bp given) the same launch zero-fills the gradient rows / columns of dropped keys
 // and makes the dK/dV plan.
 bool use_compact(const FwdParams &p);
+// forward only: `p` has a query-broadcast mask with a row per query head and grouped kv heads, and `pv` -- the same
+// problem as the compaction layer takes it (see FwdParams::kv_share) -- is one that use_compact() accepts
+bool compact_per_query_head(const FwdParams &p, FwdParams &pv);
 size_t compact_bytes(const FwdParams &p, bool backward, bool reuse_fwd = false);
 // bp != nullptr: backward -- also plans the dK/dV split and sets bp->dkv_part / bp->db_part
 // `fwd_ws` (backward only): the workspace a forward call of the same problem filled; its lists and copies are used

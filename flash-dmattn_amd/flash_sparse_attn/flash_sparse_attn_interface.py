@@ -259,8 +259,10 @@ def _flash_sparse_attn_forward_body(
                 args.workspace, args.workspace_bytes = workspace.data_ptr(), nbytes
         _cabi.check(_cabi.lib.fdma_fwd(args, stream))
     items = getattr(_tls, "items", None)
-    if items is not None and workspace is not None and seqlen_q > 1:
-        # (the compaction path's lists and copies; what identifies the problem they belong to goes with them)
+    per_query_head = mask is not None and mask.shape[1] == num_heads and num_heads != k.shape[2]
+    if items is not None and workspace is not None and seqlen_q > 1 and not per_query_head:
+        # (the compaction path's lists and copies; what identifies the problem they belong to goes with them.  A mask with
+        # a row per query head over grouped kv heads is compacted in the forward only: nothing for the backward to reuse)
         items["fwd_ws_out"] = (workspace, (_cabi.get_compact_mode(), _cabi.stream_min_items()), None if bias is None else tuple(bias.shape))
     return out, softmax_lse, p
 

@@ -252,7 +252,8 @@ def test_product_package_never_imports_the_oracle():
 
 def test_compaction_workspace_rule():
     """fdma_*_workspace_bytes is pure host arithmetic: the column-compaction path asks for scratch exactly when the
-    mask is query-broadcast with 1 or Hkv heads and the call's compact_mode allows it."""
+    mask is query-broadcast and the call's compact_mode allows it; a mask with a row per QUERY head over grouped kv heads
+    is compacted per query head in the forward (G copies of the kept K / V rows) and not at all in the backward."""
     import torch
     from flash_sparse_attn import _cabi
 
@@ -278,7 +279,13 @@ def test_compaction_workspace_rule():
         a.compact_mode = _cabi.COMPACT_ALWAYS
     assert _cabi.lib.fdma_fwd_workspace_bytes(small) > 0
     assert _cabi.lib.fdma_fwd_workspace_bytes(per_query) == 0
-    assert _cabi.lib.fdma_fwd_workspace_bytes(per_qhead) == 0
+    per_qhead_need = _cabi.lib.fdma_fwd_workspace_bytes(per_qhead)
+    big.compact_mode = _cabi.COMPACT_ALWAYS
+    assert per_qhead_need > 1.5 * _cabi.lib.fdma_fwd_workspace_bytes(big)   # a copy per query head, not per kv head
+    import ctypes
+    b = _cabi.BwdArgs()  # (the backward of that form takes the tile-skipping kernels: no compaction scratch)
+    ctypes.memmove(ctypes.byref(b.f), ctypes.byref(per_qhead), ctypes.sizeof(per_qhead))
+    assert _cabi.lib.fdma_bwd_workspace_bytes(b) == 0
     small.compact_mode = big.compact_mode = _cabi.COMPACT_AUTO
     assert _cabi.lib.fdma_fwd_workspace_bytes(small) == 0       # too small for the pre-pass to pay
     need = _cabi.lib.fdma_fwd_workspace_bytes(big)

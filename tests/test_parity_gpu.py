@@ -116,7 +116,8 @@ def _small_case(name):
 def _eligible_for_compaction(name):
     mshape, Hk = SMALL_CASES[name][7], SMALL_CASES[name][4]
     bshape = SMALL_CASES[name][6]
-    return (mshape is not None and mshape[2] == 1 and mshape[1] in (1, Hk) and (bshape is None or bshape[2] == 1)
+    H = SMALL_CASES[name][3]  # (a mask row per query head over grouped kv heads: the forward alone is compacted)
+    return (mshape is not None and mshape[2] == 1 and mshape[1] in (1, Hk, H) and (bshape is None or bshape[2] == 1)
             and SMALL_CASES[name][1] > 1)
 
 

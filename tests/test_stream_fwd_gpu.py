@@ -62,6 +62,10 @@ CASES = {
     "exactly_one_tile": (1, 300, 300, 2, 2, 2, 2, 64, True, torch.bfloat16),
     "one_key_beyond_a_tile": (1, 300, 300, 2, 2, 2, 2, 65, False, torch.bfloat16),
     "five_pairs": (5, 520, 520, 2, 1, 1, 1, 130, True, torch.bfloat16),
+    # a mask row per QUERY head over grouped kv heads: compacted per query head (forward only)
+    "mask_per_query_head_bias_per_kv_head": (1, 600, 600, 8, 2, 8, 2, 150, True, torch.bfloat16),
+    "mask_per_query_head_bias_per_query_head": (2, 300, 500, 4, 2, 4, 4, 100, True, torch.bfloat16),
+    "mask_per_query_head_shared_bias_noncausal": (1, 512, 512, 6, 3, 6, 1, 99, False, torch.bfloat16),
 }
 
 
