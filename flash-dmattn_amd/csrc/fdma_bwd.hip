@@ -525,7 +525,7 @@ hipError_t launch_bwd_t(const BwdParams &p, hipStream_t stream) {
     hipError_t e;
     // 1. D = rowsum(dO * O)  (the compacted backward has done it in its pre-pass launch)
     if (!p.dot_done) {
-        const int CH = (f.d + 7) / 8, lanes = CH <= 8 ? 8 : 16, rpb = 256 / lanes;
+        const int rpb = bwd_dot_rows_per_block(f.d);
         dim3 grid(((f.cu_q ? f.total_q : p.Lq_rounded) + rpb - 1) / rpb, f.H, f.cu_q ? 1 : f.B);
         hipLaunchKernelGGL((bwd_dot_kernel<T>), grid, dim3(256), 0, stream, p);
         if ((e = hipGetLastError()) != hipSuccess) return e;
