@@ -124,12 +124,14 @@ def test_pairs_without_a_kept_key_and_a_late_first_key():
         assert_grad_close(g.cpu(), r, n)
 
 
-def test_streaming_forward_with_lists_from_the_mask_builder():
+@pytest.mark.parametrize("bias_heads", ["kv", "query"])
+def test_streaming_forward_with_lists_from_the_mask_builder(bias_heads):
     """Kept-key lists handed over by the device mask builder: the image pre-pass numbers nothing and copies the lists;
-    results equal those of the same mask as a plain tensor, bit for bit."""
+    results equal those of the same mask as a plain tensor, bit for bit.  ("query": a bias row, hence a mask row and a
+    list, per query head over grouped kv heads -- compacted per query head.)"""
     from flash_sparse_attn.utils import mask as M
     B, Lq, Lk, H, Hk, W = 2, 520, 777, 4, 2, 250
-    q, k, v, _, bias = make_inputs(B, Lq, Lk, H, Hk, 128, (B, Hk, 1, Lk), None, None, seed=9)
+    q, k, v, _, bias = make_inputs(B, Lq, Lk, H, Hk, 128, (B, Hk if bias_heads == "kv" else H, 1, Lk), None, None, seed=9)
     bd = bias.to(DEV)
     mask = M.topk_mask(bd, None, W, torch.finfo(bd.dtype).min)
     assert M.kept_keys_of(mask) is not None
