@@ -12,7 +12,7 @@ import pytest
 import torch
 
 from oracle import c_oracle, eager
-from _util import assert_grad_close, assert_out_close, make_inputs, set_compact
+from _util import OUT_ATOL, assert_grad_close, assert_out_close, make_inputs, set_compact
 
 pytestmark = pytest.mark.gpu
 DEV = "cuda"
@@ -204,3 +204,45 @@ def test_default_threshold_takes_the_headline_shape_and_not_a_small_one():
     small = need(1, 1024, 8, 2)   # 32 items: row-major copies (2 * 64 * 256 bytes per 64 keys)
     assert abs(big - (lists(1, 8192, 8) + 8 * 128 * (35840 + 2048))) <= 4096
     assert abs(small - (lists(1, 1024, 2) + 2 * 16 * 2 * 64 * 256)) <= 4096
+
+
+def _draw_streamed(it):
+    import random
+    rng = random.Random(9100 + it)
+    Hk = rng.choice([1, 2, 3, 4])
+    H = Hk * rng.choice([1, 2, 4])
+    B = rng.choice([1, 2, 3])
+    Lq, Lk = rng.randint(2, 900), rng.randint(1, 1500)
+    hm = rng.choice([1, Hk, Hk, H])
+    hb = rng.choice([None, 1, Hk, H])
+    W = max(1, int(Lk * rng.choice([0.02, 0.1, 0.25, 0.6, 1.0])))
+    return dict(B=B, Lq=Lq, Lk=Lk, H=H, Hk=Hk, hm=hm, hb=hb, W=W, causal=rng.random() < 0.7,
+                dtype=rng.choice([torch.bfloat16, torch.bfloat16, torch.float16]), qscale=rng.choice([1.0, 1.0, 2.5]))
+
+
+@pytest.mark.parametrize("it", range(24))
+def test_streamed_random_case_vs_eager_fp32(it):
+    """Seeded random shapes through the streaming forward (every compacted call at head dim 128 takes it here): ragged
+    row and key counts, 1 to 12 (batch, kv head) pairs, mask rows per pair, per kv head or per query head, every bias
+    head count, both dtypes, larger score scales."""
+    c = _draw_streamed(it)
+    print({k: str(v) for k, v in c.items()}, flush=True)
+    q, k, v, mask, bias = make_inputs(c["B"], c["Lq"], c["Lk"], c["H"], c["Hk"], 128,
+                                      (c["B"], c["hb"], 1, c["Lk"]) if c["hb"] else None, (c["B"], c["hm"], 1, c["Lk"]), c["W"],
+                                      seed=2000 + it, dtype=c["dtype"])
+    q = (q.float() * c["qscale"]).to(c["dtype"])
+    dout = torch.randn(q.shape, generator=torch.Generator().manual_seed(3000 + it)).to(c["dtype"])
+    out, lse, grads = _run(q, k, v, mask, bias, c["causal"], dout=dout)
+    dev = [t.to(DEV) if t is not None else None for t in (q, k, v, mask, bias)]
+    ro, rl = eager.attention_forward(*dev, None, c["causal"])
+    _, *refs = eager.attention_forward_backward(*dev, None, c["causal"], dout=dout.to(DEV))
+    # (scores 2.5 times larger carry 2.5 times the rounding of their 16-bit operands: twice the bound, as in the sweep
+    # of the operator's other paths)
+    assert (out.float() - ro.float()).abs().max().item() <= OUT_ATOL * (2 if c["qscale"] > 1 else 1)
+    assert torch.equal(torch.isinf(lse), torch.isinf(rl))
+    fin = torch.isfinite(rl)
+    if fin.any():
+        assert (lse[fin] - rl[fin]).abs().max().item() <= 1e-2 * c["qscale"]
+    for g, r, n in zip(grads, refs, ("dq", "dk", "dv", "dbias")):
+        if g is not None:
+            assert_grad_close(g.cpu(), r.cpu(), n)
