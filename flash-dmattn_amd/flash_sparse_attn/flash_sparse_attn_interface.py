@@ -285,6 +285,61 @@ def _flash_sparse_attn_forward_fake(
 _wrapped_flash_sparse_attn_forward = _direct_when_eager(_flash_sparse_attn_forward, _flash_sparse_attn_forward_body)
 
 
+def _per_query_head_groups(q, k, mask, bias) -> int:
+    """Query heads per kv head when the backward of this call is to be taken apart by group member (see
+    _backward_per_query_head), else 1: a query-broadcast mask with a row per QUERY head over grouped kv heads, next to
+    no bias or a query-broadcast one, on a problem for which the library would compact a mask with a row per kv head
+    (fdma_compact.hip: use_compact -- the same rule, on what one group member sees)."""
+    if mask is None or mask.shape[2] != 1 or (bias is not None and bias.shape[2] != 1):
+        return 1
+    num_heads, num_heads_k = q.shape[2], k.shape[2]
+    if mask.shape[1] != num_heads or num_heads == num_heads_k:
+        return 1
+    mode = _cabi.get_compact_mode()
+    seqlen_q, seqlen_k = q.shape[1], k.shape[1]
+    if mode == _cabi.COMPACT_NEVER or seqlen_q < 2 or seqlen_k < 1 or q.shape[0] * num_heads_k > 65535:
+        return 1
+    if mode != _cabi.COMPACT_ALWAYS and not (seqlen_q >= 128 and seqlen_k >= 128 and seqlen_q * seqlen_k >= 1 << 21):
+        return 1
+    return num_heads // num_heads_k
+
+
+def _backward_per_query_head(dout, q, k, v, mask, bias, out, softmax_lse, dq, dk, dv, dbias, softmax_scale, is_causal,
+                             softcap, deterministic):
+    """Backward for a query-broadcast mask with a row per QUERY head over grouped kv heads.  The heads of a kv group keep
+    different keys, so the library's compacted backward -- one list of kept keys per kv head, dK / dV summed over the
+    group in registers -- does not apply to the call as a whole, and its tile-skipping kernels find hardly a tile to
+    skip.  Group member g of every kv head (query heads g, g + G, ...: strided views, no copies) together with its mask
+    rows IS a problem of the compacted form, without grouping: the call is taken apart into G of them.  dQ (and dBias
+    with a row per query head) of the members are disjoint; dK, dV (and a dBias shared by the group) are summed."""
+    G = q.shape[2] // k.shape[2]
+    batch, seqlen_q, num_heads, _ = q.shape
+    softmax_d = torch.empty((batch, num_heads, round_multiple(seqlen_q, 128)), device=q.device, dtype=torch.float32)
+    bias_per_head = bias is not None and bias.shape[1] == num_heads
+    dk_t = dv_t = dbias_t = None
+    with _handoff():  # (lists, bit rows and forward workspaces belong to the whole call, not to a member)
+        for g in range(G):
+            member = slice(g, None, G)
+            first = g == 0
+            if not first and dk_t is None:
+                dk_t, dv_t = torch.empty_like(dk), torch.empty_like(dv)
+                if bias is not None and not bias_per_head:
+                    dbias_t = torch.empty_like(dbias)
+            bias_g = bias[:, member] if bias_per_head else bias
+            dbias_g = None if bias is None else (dbias[:, member] if bias_per_head else (dbias if first else dbias_t))
+            d = _flash_sparse_attn_backward_body(
+                dout[:, :, member], q[:, :, member], k, v, mask[:, member], bias_g, out[:, :, member],
+                softmax_lse[:, member], dq[:, :, member], dk if first else dk_t, dv if first else dv_t, dbias_g,
+                softmax_scale, is_causal, softcap, deterministic)
+            softmax_d[:, member] = d
+            if not first:
+                dk.add_(dk_t)
+                dv.add_(dv_t)
+                if dbias_t is not None:
+                    dbias.add_(dbias_t)
+    return softmax_d
+
+
 def _flash_sparse_attn_backward_body(
     dout: torch.Tensor, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, mask: Optional[torch.Tensor], bias:
     Optional[torch.Tensor], out: torch.Tensor, softmax_lse: torch.Tensor, dq: Optional[torch.Tensor], dk:
@@ -298,6 +353,9 @@ def _flash_sparse_attn_backward_body(
         raise RuntimeError("query and dout must have the same dtype")
     if tuple(out.shape) != tuple(q.shape) or tuple(dout.shape) != tuple(q.shape):
         raise RuntimeError("out and dout must have the shape of q")
+    if _per_query_head_groups(q, k, mask, bias) > 1 and all(t is not None for t in (dq, dk, dv)):
+        return _backward_per_query_head(dout, q, k, v, mask, bias, out, softmax_lse, dq, dk, dv, dbias, softmax_scale,
+                                        is_causal, softcap, deterministic)
     dout, q, k, v, out = [_aligned(x, 8) for x in (dout, q, k, v, out)]
     mask = _aligned(mask, 16)
     bias = _aligned(bias, 8)
