@@ -74,7 +74,12 @@ enum {
  * num_heads_k heads, drops whole key columns; the library can then gather the kept K / V rows into dense copies
  * (in the workspace) and run attention over those alone, so that the work follows the number of kept keys.
  * The result is the same function of the inputs either way.  The mode decides the workspace size, so the
- * *_workspace_bytes call and the launch must see the same value (a mismatch is caught: FDMA_ERR_WORKSPACE). */
+ * *_workspace_bytes call and the launch must see the same value (a mismatch is caught: FDMA_ERR_WORKSPACE).
+ * A query-broadcast mask with a row per QUERY head over grouped kv heads (num_heads_mask == num_heads > num_heads_k)
+ * is compacted per query head by fdma_fwd (a copy of the kept rows per query head); fdma_bwd does not compact that
+ * form as a whole -- a caller that wants it compacted calls fdma_bwd once per member g of the kv groups, on the
+ * query heads g, g + G, ... (pointers offset by g heads, head strides times G, num_heads = num_heads_mask =
+ * num_heads_k), and sums dk / dv (and a dbias shared by the group) over the members, as the Python operator does. */
 enum {
     FDMA_COMPACT_AUTO = 0,  /* compact when the mask form allows it and the problem is large enough to pay for the pre-pass */
     FDMA_COMPACT_NEVER = 1, /* tile skipping only */
