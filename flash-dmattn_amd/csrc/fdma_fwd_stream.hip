@@ -229,27 +229,10 @@ __global__ void __launch_bounds__(ST_THREADS, 1) fwd_stream_kernel(const FwdPara
     // A wave waits for its own pieces of the tile TWO ahead -- all it has requested so far -- then the barrier publishes
     // everybody's.  (One tile more than the step behind the barrier needs: that step's first fragments are read in front
     // of the barrier, from a tile that the barrier before has published.)
-#ifdef FDMA_DBG_WAIT
-    uint64_t dbg_vm = 0, dbg_bar = 0;
-#endif
     auto publish = [&]() {
         __builtin_amdgcn_sched_barrier(0);
-#ifdef FDMA_DBG_WAIT
-        const uint64_t c0 = __builtin_amdgcn_s_memtime();
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        const uint64_t c1 = __builtin_amdgcn_s_memtime();
         __builtin_amdgcn_s_barrier();
-        const uint64_t c2 = __builtin_amdgcn_s_memtime();
-        dbg_vm += c1 - c0;
-        dbg_bar += c2 - c1;
-#else
-#ifndef FDMA_KO_DMA
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-#endif
-#ifndef FDMA_KO_BARRIER
-        __builtin_amdgcn_s_barrier();
-#endif
-#endif
         asm volatile("" ::: "memory");
         __builtin_amdgcn_sched_barrier(0);
     };
@@ -278,10 +261,7 @@ __global__ void __launch_bounds__(ST_THREADS, 1) fwd_stream_kernel(const FwdPara
     const uint32_t aV = lds0 + SM::OFF_KV + IMG_K_BYTES + (uint32_t)((a_row * SVT + 8 * g) * 2);
     const uint32_t aX = lds0 + SM::OFF_X + (uint32_t)(a_row * 32 + g * 16);
     constexpr int NQK = KS + 1, NPV = 2 * DB;
-#ifndef FDMA_ST_FR
-#define FDMA_ST_FR 4
-#endif
-    constexpr int FR = FDMA_ST_FR;  // fragment reads run FR MFMAs ahead of their MFMAs
+    constexpr int FR = 4;  // fragment reads run FR MFMAs ahead of their MFMAs (6 and 8: the same time, more registers)
     const f32x16_t zero16 = {0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f, 0.f};
     const float side_mult = 1.f / E::kPieceScale;
 
@@ -389,13 +369,11 @@ __global__ void __launch_bounds__(ST_THREADS, 1) fwd_stream_kernel(const FwdPara
                     psum1 += x1[k];
                 }
             }
-#ifndef FDMA_KO_DMA
             if (FETCH) {
 #pragma unroll
                 for (int i = 0; i < ST_NDMA; i++)
                     if (f == (SCORES ? 1 + 3 * i : 1 + i)) fetch_piece(i);
             }
-#endif
             if (FETCH) {  // the previous item's output rows, one piece per slot (a step behind the barrier: see store_piece)
 #pragma unroll
                 for (int k = 0; k < 8; k++)
@@ -587,12 +565,6 @@ __global__ void __launch_bounds__(ST_THREADS, 1) fwd_stream_kernel(const FwdPara
     asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
     __syncthreads();
     FDMA_STAMP(3);
-#ifdef FDMA_DBG_WAIT
-    if (lane == 0) {
-        g_stream_dbg[blockIdx.x * 64 + 40 + 2 * wave] = dbg_vm;
-        g_stream_dbg[blockIdx.x * 64 + 41 + 2 * wave] = dbg_bar;
-    }
-#endif
 #ifdef FDMA_DBG
     if (tid == 0) g_stream_dbg[blockIdx.x * 64 + 39] = __builtin_amdgcn_s_memtime();
 #endif
