@@ -299,9 +299,9 @@ def run_mfma_probe():
 
 
 def config_roofline(name, r):
-    """Roofline block of one of the secondary configurations (the headline's is built in main()): the bound that
-    SURVEY-style accounting assigns to the configuration, the algorithmic work per call and what the measured call
-    time makes of it.  Durations are whole operator calls (all launches of the call), timed with events on the
+    """Roofline block of one of the secondary configurations (the headline's is built in main()): the bound of
+    the configuration (matrix pipe for the column-mask shapes, HBM for per-query bias and for decode), the algorithmic
+    work per call and what the measured call time makes of it.  Durations are whole operator calls (all launches of the call), timed with events on the
     launch stream."""
     c = CONFIGS[name]
     if c["Lq"] == 1:  # decode: HBM, touched K / V rows + side inputs
