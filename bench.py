@@ -298,6 +298,29 @@ def run_mfma_probe():
     return out
 
 
+def run_hbm_probe():
+    """What rate of bytes the device delivers to a kernel that only reads 256-byte rows (a K or V row at head dim 128),
+    one launch each, launch ramp included: a stream of 1 GiB, 1 GiB of rows at scattered positions, and cfg5's volume
+    (2 x 131072 kept rows = 67 MB) at scattered positions of a 2 GiB buffer -- what the gather of a decode call looks
+    like to the memory, without the mask, the lists, the arithmetic and the merge.  The HBM roofline fractions (always
+    against the published 8 TB/s) are to be read next to these.  None when the probe is not built."""
+    import ctypes
+
+    path = os.path.join(ROOT, "flash-dmattn_amd", "lib", "libfdma_probe.so")
+    if not os.path.exists(path):
+        return None
+    lib = ctypes.CDLL(path)
+    if not hasattr(lib, "fdma_probe_read_gbs"):
+        return None
+    lib.fdma_probe_read_gbs.restype = ctypes.c_double
+    lib.fdma_probe_read_gbs.argtypes = [ctypes.c_int64, ctypes.c_int, ctypes.c_int]
+    return {"unit": "GB/s", "row_bytes": 256,
+            "stream_1GiB": lib.fdma_probe_read_gbs(1 << 22, 0, 1024),
+            "scattered_rows_1GiB": lib.fdma_probe_read_gbs(1 << 22, 1, 2048),
+            "scattered_rows_cfg5_volume_67MB": lib.fdma_probe_read_gbs(2 * 131072, 1, 2048),
+            "note": "read-only kernels, best of five launches each; scattered = hashed row positions in a 2 GiB buffer"}
+
+
 def config_roofline(name, r):
     """Roofline block of one of the secondary configurations (the headline's is built in main()): the bound of
     the configuration (matrix pipe for the column-mask shapes, HBM for per-query bias and for decode), the algorithmic
@@ -624,6 +647,9 @@ def run_secondary_legs(out, legs, args, device, compact, bwd, half):
         probe = run_mfma_probe()
         if probe is not None:
             out["mfma_probe"] = probe
+        probe = run_hbm_probe()
+        if probe is not None:
+            out["hbm_probe"] = probe
     if args.calib_copy:
         src = torch.empty(256 << 20, dtype=torch.uint8, device=device).fill_(1)
         dst = torch.empty_like(src)

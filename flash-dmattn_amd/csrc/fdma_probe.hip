@@ -112,3 +112,68 @@ extern "C" double fdma_probe_mfma_tflops(int mode, int random) {
     const double mfmas = (double)wgs * 8 * iters * 16;
     return mfmas * 32768.0 / (ms * 1e-3) / 1e12;
 }
+
+// ---- HBM probes: what rate of bytes the device delivers to kernels that do nothing but read, as context for the
+// HBM-bound shapes (per-query bias, decode).  `rows` rows of 256 bytes (a K or V row at head dim 128) are read from a
+// buffer of `total_rows` rows, 16 lanes x 16 bytes per row, eight rows of a wave in flight per lane -- one after the
+// other (a streaming read) or at hashed positions (what decode's gather of the kept keys looks like to the memory).
+namespace {
+
+__global__ void __launch_bounds__(256) read_rows_kernel(const u32x4 *base, uint32_t total_rows, uint32_t rows_per_wave, int scattered,
+                                                        uint32_t seed, uint32_t *out) {
+    const uint32_t wave = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const uint32_t first = wave * rows_per_wave;
+    u32x4 acc = {0, 0, 0, 0};
+    for (uint32_t i = 0; i < rows_per_wave; i += 32) {
+        u32x4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; j++) {
+            const uint32_t n = first + i + 4 * j + (lane >> 4);
+            const uint32_t row = (scattered ? hash(n ^ seed) : n) & (total_rows - 1);  // (a power of two)
+            v[j] = base[(size_t)row * 16 + (lane & 15)];
+        }
+#pragma unroll
+        for (int j = 0; j < 8; j++) acc ^= v[j];
+    }
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x12345678u) out[wave] = acc[0];  // (keeps the loads alive)
+}
+
+}  // namespace
+
+// GB/s of one launch that reads `rows` rows of 256 bytes from a buffer of `buffer_mib` MiB (a power of two), scattered or
+// not: 32 / 64 / 128 / 256 rows per wave are tried (more, smaller workgroups ramp up faster; fewer, fatter ones issue
+// fewer instructions per byte), five timed launches each, and the best launch counts -- launch ramp included (< 0 on error)
+extern "C" double fdma_probe_read_gbs(int64_t rows, int scattered, int buffer_mib) {
+    const size_t bytes = (size_t)buffer_mib << 20;
+    void *buf = nullptr;
+    uint32_t *d_out = nullptr;
+    if (rows <= 0 || buffer_mib <= 0 || (buffer_mib & (buffer_mib - 1)) || hipMalloc(&buf, bytes) != hipSuccess) return -1.0;
+    const size_t max_waves = (size_t)((rows + 31) / 32) + 4;
+    if (hipMalloc((void **)&d_out, max_waves * sizeof(uint32_t)) != hipSuccess) { (void)hipFree(buf); return -1.0; }
+    (void)hipMemset(buf, 0x5a, bytes);
+    hipEvent_t e0, e1;
+    (void)hipEventCreate(&e0);
+    (void)hipEventCreate(&e1);
+    double best_gbs = -1.0;
+    for (uint32_t rows_per_wave = 32; rows_per_wave <= 256; rows_per_wave *= 2) {
+        const uint32_t wgs = (uint32_t)((rows + 4 * rows_per_wave - 1) / (4 * rows_per_wave));
+        float best = 1e30f;
+        for (int rep = 0; rep < 7; rep++) {
+            (void)hipEventRecord(e0, 0);
+            hipLaunchKernelGGL(read_rows_kernel, dim3(wgs), dim3(256), 0, 0, (const u32x4 *)buf, (uint32_t)(bytes / 256), rows_per_wave,
+                               scattered, 0x9e3779b9u * (uint32_t)(rep + 1), d_out);
+            (void)hipEventRecord(e1, 0);
+            (void)hipEventSynchronize(e1);
+            float ms = 0.f;
+            (void)hipEventElapsedTime(&ms, e0, e1);
+            if (rep >= 2 && ms < best) best = ms;
+        }
+        const double gbs = (double)wgs * 4 * rows_per_wave * 256.0 / (best * 1e-3) / 1e9;
+        if (best > 0.f && best < 1e29f && gbs > best_gbs) best_gbs = gbs;
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipFree(d_out);
+    (void)hipFree(buf);
+    return hipGetLastError() == hipSuccess ? best_gbs : -1.0;
+}
