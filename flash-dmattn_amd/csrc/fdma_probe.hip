@@ -120,17 +120,18 @@ extern "C" double fdma_probe_mfma_tflops(int mode, int random) {
 namespace {
 
 __global__ void __launch_bounds__(256) read_rows_kernel(const u32x4 *base, uint32_t total_rows, uint32_t rows_per_wave, int scattered,
-                                                        uint32_t seed, uint32_t *out) {
+                                                        uint32_t seed, uint32_t *out, int lanes_log2) {
     const uint32_t wave = blockIdx.x * 4 + (threadIdx.x >> 6), lane = threadIdx.x & 63;
     const uint32_t first = wave * rows_per_wave;
+    const uint32_t rows_per_load = 64u >> lanes_log2, lanes_mask = (1u << lanes_log2) - 1u;  // (lanes_log2 = 4: rows of 256 bytes)
     u32x4 acc = {0, 0, 0, 0};
-    for (uint32_t i = 0; i < rows_per_wave; i += 32) {
+    for (uint32_t i = 0; i < rows_per_wave; i += 8 * rows_per_load) {
         u32x4 v[8];
 #pragma unroll
         for (int j = 0; j < 8; j++) {
-            const uint32_t n = first + i + 4 * j + (lane >> 4);
+            const uint32_t n = first + i + rows_per_load * j + (lane >> lanes_log2);
             const uint32_t row = (scattered ? hash(n ^ seed) : n) & (total_rows - 1);  // (a power of two)
-            v[j] = base[(size_t)row * 16 + (lane & 15)];
+            v[j] = base[((size_t)row << lanes_log2) + (lane & lanes_mask)];
         }
 #pragma unroll
         for (int j = 0; j < 8; j++) acc ^= v[j];
@@ -143,32 +144,40 @@ __global__ void __launch_bounds__(256) read_rows_kernel(const u32x4 *base, uint3
 // GB/s of one launch that reads `rows` rows of 256 bytes from a buffer of `buffer_mib` MiB (a power of two), scattered or
 // not: 32 / 64 / 128 / 256 rows per wave are tried (more, smaller workgroups ramp up faster; fewer, fatter ones issue
 // fewer instructions per byte), five timed launches each, and the best launch counts -- launch ramp included (< 0 on error)
+extern "C" double fdma_probe_read_rows_gbs(int64_t rows, int row_bytes, int scattered, int buffer_mib);
 extern "C" double fdma_probe_read_gbs(int64_t rows, int scattered, int buffer_mib) {
+    return fdma_probe_read_rows_gbs(rows, 256, scattered, buffer_mib);
+}
+// ... the same with rows of 64, 128, 256 or 512 bytes (a mask / bias row of a 64-key tile is 64 / 128 bytes)
+extern "C" double fdma_probe_read_rows_gbs(int64_t rows, int row_bytes, int scattered, int buffer_mib) {
+    const int lanes_log2 = row_bytes == 64 ? 2 : row_bytes == 128 ? 3 : row_bytes == 256 ? 4 : row_bytes == 512 ? 5 : -1;
+    if (lanes_log2 < 0) return -1.0;
     const size_t bytes = (size_t)buffer_mib << 20;
     void *buf = nullptr;
     uint32_t *d_out = nullptr;
     if (rows <= 0 || buffer_mib <= 0 || (buffer_mib & (buffer_mib - 1)) || hipMalloc(&buf, bytes) != hipSuccess) return -1.0;
-    const size_t max_waves = (size_t)((rows + 31) / 32) + 4;
+    const size_t max_waves = (size_t)(rows / (8u * (64u >> lanes_log2)) + 8);
     if (hipMalloc((void **)&d_out, max_waves * sizeof(uint32_t)) != hipSuccess) { (void)hipFree(buf); return -1.0; }
     (void)hipMemset(buf, 0x5a, bytes);
     hipEvent_t e0, e1;
     (void)hipEventCreate(&e0);
     (void)hipEventCreate(&e1);
     double best_gbs = -1.0;
-    for (uint32_t rows_per_wave = 32; rows_per_wave <= 256; rows_per_wave *= 2) {
+    const uint32_t rows_per_pass = 8u * (64u >> lanes_log2);  // rows a wave has in flight
+    for (uint32_t rows_per_wave = rows_per_pass; rows_per_wave <= 8 * rows_per_pass; rows_per_wave *= 2) {
         const uint32_t wgs = (uint32_t)((rows + 4 * rows_per_wave - 1) / (4 * rows_per_wave));
         float best = 1e30f;
         for (int rep = 0; rep < 7; rep++) {
             (void)hipEventRecord(e0, 0);
-            hipLaunchKernelGGL(read_rows_kernel, dim3(wgs), dim3(256), 0, 0, (const u32x4 *)buf, (uint32_t)(bytes / 256), rows_per_wave,
-                               scattered, 0x9e3779b9u * (uint32_t)(rep + 1), d_out);
+            hipLaunchKernelGGL(read_rows_kernel, dim3(wgs), dim3(256), 0, 0, (const u32x4 *)buf, (uint32_t)(bytes / row_bytes), rows_per_wave,
+                               scattered, 0x9e3779b9u * (uint32_t)(rep + 1), d_out, lanes_log2);
             (void)hipEventRecord(e1, 0);
             (void)hipEventSynchronize(e1);
             float ms = 0.f;
             (void)hipEventElapsedTime(&ms, e0, e1);
             if (rep >= 2 && ms < best) best = ms;
         }
-        const double gbs = (double)wgs * 4 * rows_per_wave * 256.0 / (best * 1e-3) / 1e9;
+        const double gbs = (double)wgs * 4 * rows_per_wave * row_bytes / (best * 1e-3) / 1e9;
         if (best > 0.f && best < 1e29f && gbs > best_gbs) best_gbs = gbs;
     }
     (void)hipEventDestroy(e0);
