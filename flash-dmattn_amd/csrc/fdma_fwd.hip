@@ -170,8 +170,8 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) fwd_ker
         }
         return any != 0;
     };
-    // bias, K and V of tile j into registers
-    auto load_rest = [&](int j) {
+    // bias of tile j into registers
+    auto load_bias = [&](int j, u32x4_t (&dst)[F_IT]) {
         const int n0 = j * BN;
         if (bbase) {
             int kk = n0 + 8 * fc;
@@ -180,12 +180,16 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) fwd_ker
             for (int it = 0; it < F_IT; it++) {
                 int row = m0 + fr0 + F_RPP * it;
                 row = row < p.Lq ? row : p.Lq - 1;
-                breg[it] = *(const u32x4_t *)(bbase + (int64_t)row * p.bi_r + kk);
+                dst[it] = *(const u32x4_t *)(bbase + (int64_t)row * p.bi_r + kk);
             }
         } else {
 #pragma unroll
-            for (int it = 0; it < F_IT; it++) breg[it] = u32x4_t{0, 0, 0, 0};
+            for (int it = 0; it < F_IT; it++) dst[it] = u32x4_t{0, 0, 0, 0};
         }
+    };
+    // K and V of tile j into registers
+    auto load_kv = [&](int j) {
+        const int n0 = j * BN;
 #pragma unroll
         for (int it = 0; it < K_IT; it++) {
             int key = n0 + kr0 + it * K_RPP;
@@ -201,8 +205,12 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) fwd_ker
             }
         }
     };
+    auto load_rest = [&](int j) {
+        load_bias(j, breg);
+        load_kv(j);
+    };
     // registers -> LDS stage `buf`: K rows, V transposed, mask and bias fused (bias where kept, -inf elsewhere)
-    auto store_stage = [&](int buf, const u32x2_t (&mv)[F_IT]) {
+    auto store_stage = [&](int buf, const u32x2_t (&mv)[F_IT], const u32x4_t (&bsrc)[F_IT]) {
         char *sK = smem + buf * SM::STAGE;
         char *sVt = sK + SM::K_BYTES;
         char *sF = sVt + SM::VT_BYTES;
@@ -222,7 +230,7 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) fwd_ker
         }
 #pragma unroll
         for (int it = 0; it < F_IT; it++) {
-            u32x4_t bv = breg[it];
+            u32x4_t bv = bsrc[it];
 #pragma unroll
             for (int hlf = 0; hlf < 2; hlf++) {
                 uint32_t x = mv[it][hlf];
@@ -338,13 +346,59 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) fwd_ker
 
     // ---- main loop.  At the top of iteration j: tile j sits in LDS stage j&1 if it is active, `mreg` holds
     // the mask of tile j+1 and `act_next` says whether that tile has any kept element.
-    if (n_end > 0) {
+    // DEEP (head dims up to 64, where the registers are there): mask and bias -- the bytes that come from HBM -- stay in
+    // flight for TWO iterations instead of one.  With one, every iteration contained a whole trip to memory (the mask
+    // requested at its top decided, at its end, whether the tile after the next is fetched at all), and the launch moved
+    // what it had in flight once per trip: 64 KB per CU every 3.5 us.  Now the mask of tile j+4 and the bias of tile
+    // j+2 are requested at the top of iteration j, behind K / V of tile j+1 (cache hits; waiting for those must not
+    // mean waiting for the younger requests: loads come back in the order they were issued).
+    constexpr bool DEEP = D <= 64;
+    if (n_end > 0 && DEEP) {
+        u32x2_t m1[F_IT], m2[F_IT], m3[F_IT], m4[F_IT];  // masks of tiles j+1 .. j+4 at the top of iteration j
+        u32x4_t b1[F_IT], b2[F_IT];                      // bias of tiles j+1 (requested an iteration ago), j+2
+        load_mask(0, mreg);
+        load_mask(1, m1);
+        load_mask(2, m2);
+        load_mask(3, m3);
+        bool act_cur = __syncthreads_or(finish_mask(0, mreg));
+        if (act_cur) {
+            load_rest(0);
+            store_stage(0, mreg, breg);
+        }
+        bool act_1 = __syncthreads_or(n_end > 1 && finish_mask(1, m1));
+        if (act_1) load_bias(1, b1);
+        bool act_2 = __syncthreads_or(n_end > 2 && finish_mask(2, m2));
+#pragma unroll 1
+        for (int j = 0; j < n_end; j++) {
+            const bool have_next = j + 1 < n_end && act_1;
+            if (have_next) load_kv(j + 1);
+            __builtin_amdgcn_sched_barrier(0);
+            if (j + 4 < n_end) load_mask(j + 4, m4);
+            __builtin_amdgcn_sched_barrier(0);
+            if (j + 2 < n_end && act_2) load_bias(j + 2, b2);
+            __builtin_amdgcn_sched_barrier(0);
+            if (act_cur) compute(j, j & 1);
+            __builtin_amdgcn_sched_barrier(0);
+            if (have_next) store_stage((j + 1) & 1, m1, b1);
+            const bool act_3 = __syncthreads_or(j + 3 < n_end && finish_mask(j + 3, m3));
+            act_cur = have_next;
+            act_1 = act_2;
+            act_2 = act_3;
+#pragma unroll
+            for (int it = 0; it < F_IT; it++) {
+                m1[it] = m2[it];
+                m2[it] = m3[it];
+                m3[it] = m4[it];
+                b1[it] = b2[it];
+            }
+        }
+    } else if (n_end > 0) {
         load_mask(0, mreg);
         if (n_end > 1) load_mask(1, mnext);
         bool act_cur = __syncthreads_or(finish_mask(0, mreg));
         if (act_cur) {
             load_rest(0);
-            store_stage(0, mreg);
+            store_stage(0, mreg, breg);
         }
         bool act_next = __syncthreads_or(n_end > 1 && finish_mask(1, mnext));
         // one iteration; `m_next` holds the (finished) mask of tile j+1, `m_new` receives the mask of tile j+2.
@@ -357,7 +411,7 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) fwd_ker
             __builtin_amdgcn_sched_barrier(0);
             if (act_cur) compute(j, j & 1);
             __builtin_amdgcn_sched_barrier(0);
-            if (have_next) store_stage((j + 1) & 1, m_next);
+            if (have_next) store_stage((j + 1) & 1, m_next, breg);
             const bool act_nn = __syncthreads_or(j + 2 < n_end && finish_mask(j + 2, m_new));
             act_cur = have_next;
             act_next = act_nn;
