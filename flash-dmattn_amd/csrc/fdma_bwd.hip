@@ -560,6 +560,9 @@ hipError_t launch_bwd_t(const BwdParams &p, hipStream_t stream) {
     // 3. dQ (the launch of a compacted backward also sums the dK / dV / dBias partial results of step 2)
     if (colmask) {
         if ((e = launch_bwd_dq_colmask(p, dtype_code, stream)) != hipSuccess) return e;
+    } else if (f.Lk > 0 && bwd_dq_from_ds_applicable(p)) {
+        // (step 2 has written dS itself as dBias: dQ = scale * dS K without a second pass over mask and bias)
+        if ((e = launch_bwd_dq_from_ds(p, dtype_code, stream)) != hipSuccess) return e;
     } else {
         if ((e = launch_bwd_dq(p, dtype_code, stream)) != hipSuccess) return e;
     }

@@ -354,7 +354,7 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) fwd_ker
     // mean waiting for the younger requests: loads come back in the order they were issued).
     constexpr bool DEEP = D <= 64;
     if (n_end > 0 && DEEP) {
-        u32x2_t m1[F_IT], m2[F_IT], m3[F_IT], m4[F_IT];  // masks of tiles j+1 .. j+4 at the top of iteration j
+        u32x2_t m1[F_IT], m2[F_IT], m3[F_IT];            // with mreg: the masks of tiles j .. j+3 at the top of iteration j
         u32x4_t b1[F_IT], b2[F_IT];                      // bias of tiles j+1 (requested an iteration ago), j+2
         load_mask(0, mreg);
         load_mask(1, m1);
@@ -368,29 +368,32 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) fwd_ker
         bool act_1 = __syncthreads_or(n_end > 1 && finish_mask(1, m1));
         if (act_1) load_bias(1, b1);
         bool act_2 = __syncthreads_or(n_end > 2 && finish_mask(2, m2));
-#pragma unroll 1
-        for (int j = 0; j < n_end; j++) {
+        // one iteration; the register sets change roles from one iteration to the next (written out four iterations
+        // at a time: a move between sets would have to wait for a load that is still in flight)
+        auto step = [&](int j, u32x2_t (&ma)[F_IT], u32x2_t (&mc)[F_IT], u32x2_t (&md)[F_IT], u32x4_t (&ba)[F_IT], u32x4_t (&bb)[F_IT]) {
+            // ma: mask of tile j+1 (finished); mc: of tile j+3 (in flight since the iteration before); md: receives tile j+4
+            // ba: bias of tile j+1 (requested an iteration ago); bb: receives tile j+2
             const bool have_next = j + 1 < n_end && act_1;
             if (have_next) load_kv(j + 1);
             __builtin_amdgcn_sched_barrier(0);
-            if (j + 4 < n_end) load_mask(j + 4, m4);
+            if (j + 4 < n_end) load_mask(j + 4, md);
             __builtin_amdgcn_sched_barrier(0);
-            if (j + 2 < n_end && act_2) load_bias(j + 2, b2);
+            if (j + 2 < n_end && act_2) load_bias(j + 2, bb);
             __builtin_amdgcn_sched_barrier(0);
             if (act_cur) compute(j, j & 1);
             __builtin_amdgcn_sched_barrier(0);
-            if (have_next) store_stage((j + 1) & 1, m1, b1);
-            const bool act_3 = __syncthreads_or(j + 3 < n_end && finish_mask(j + 3, m3));
+            if (have_next) store_stage((j + 1) & 1, ma, ba);
+            const bool act_3 = __syncthreads_or(j + 3 < n_end && finish_mask(j + 3, mc));
             act_cur = have_next;
             act_1 = act_2;
             act_2 = act_3;
-#pragma unroll
-            for (int it = 0; it < F_IT; it++) {
-                m1[it] = m2[it];
-                m2[it] = m3[it];
-                m3[it] = m4[it];
-                b1[it] = b2[it];
-            }
+        };
+#pragma unroll 1
+        for (int j = 0; j < n_end; j += 4) {
+            step(j, m1, m3, mreg, b1, b2);  // (mreg, the set of tile j, is free: it receives tile j+4)
+            if (j + 1 < n_end) step(j + 1, m2, mreg, m1, b2, b1);
+            if (j + 2 < n_end) step(j + 2, m3, m1, m2, b1, b2);
+            if (j + 3 < n_end) step(j + 3, mreg, m2, m3, b2, b1);
         }
     } else if (n_end > 0) {
         load_mask(0, mreg);

@@ -280,6 +280,10 @@ hipError_t launch_bwd(const BwdParams &p, int dtype, hipStream_t stream);
 bool bwd_colmask_applicable(const BwdParams &p);
 hipError_t launch_bwd_dkdv_colmask(const BwdParams &p, int dtype, hipStream_t stream);
 hipError_t launch_bwd_dq_colmask(const BwdParams &p, int dtype, hipStream_t stream);
+// dQ from the dS tiles that the general dK/dV kernel has written as dBias (a per-query bias with a row per query head
+// and batch entry, dBias written directly): one tile GEMM and no second pass over mask, bias, Q, V, dO
+bool bwd_dq_from_ds_applicable(const BwdParams &p);
+hipError_t launch_bwd_dq_from_ds(const BwdParams &p, int dtype, hipStream_t stream);
 // general dQ kernel (mask / bias per query row), fdma_bwd_dq.hip
 hipError_t launch_bwd_dq(const BwdParams &p, int dtype, hipStream_t stream);
 

@@ -130,7 +130,14 @@ __global__ void __launch_bounds__(256) read_rows_kernel(const u32x4 *base, uint3
 #pragma unroll
         for (int j = 0; j < 8; j++) {
             const uint32_t n = first + i + rows_per_load * j + (lane >> lanes_log2);
-            const uint32_t row = (scattered ? hash(n ^ seed) : n) & (total_rows - 1);  // (a power of two)
+            uint32_t row = (scattered == 1 ? hash(n ^ seed) : n) & (total_rows - 1);  // (a power of two)
+            if (scattered == 2) {
+                // the walk of a kernel over tiles of a row-major matrix with rows of 8 KB: a wave's 32 matrix rows, one
+                // piece of each, then the next piece of the same rows
+                const uint32_t pieces_per_row = 8192u >> (lanes_log2 + 4);
+                const uint32_t i = n - first, mrow = (wave * 32 + (i & 31)) & (total_rows / pieces_per_row - 1);
+                row = mrow * pieces_per_row + ((i >> 5) & (pieces_per_row - 1));
+            }
             v[j] = base[((size_t)row << lanes_log2) + (lane & lanes_mask)];
         }
 #pragma unroll
