@@ -348,7 +348,7 @@ def config_roofline(name, r):
         blk = {"bound": "hbm", "unit": "GB/s", "peak": PEAK_HBM_GBS, "bytes_per_call": fwd,
                "bytes_model": "forward: mask bytes of every causal 64x64 tile + bias of every executed tile + q, k, v, out, lse; "
                               "forward + backward adds the same tiles once more, the full dBias write, dout and the gradients "
-                              "(the two backward kernels each read the tiles: the measured traffic is higher)",
+                              "(measured traffic is higher: the dQ kernel reads the written dS tiles back, see profiles/)",
                "achieved": fwd / r["ms_fwd"] / 1e6, "frac": fwd / r["ms_fwd"] / 1e6 / PEAK_HBM_GBS, "duration_ms": r["ms_fwd"],
                "kernel": "fdma::fwd_kernel (per-query mask / bias), whole operator call"}
         if "ms_fwd_bwd" in r:
