@@ -215,7 +215,7 @@ def _draw_streamed(it):
     Lq, Lk = rng.randint(2, 900), rng.randint(1, 1500)
     hm = rng.choice([1, Hk, Hk, H])
     hb = rng.choice([None, 1, Hk, H])
-    W = max(1, int(Lk * rng.choice([0.02, 0.1, 0.25, 0.6, 1.0])))
+    W = max(2, int(Lk * rng.choice([0.02, 0.1, 0.25, 0.6, 1.0])))  # (one kept key: P = 1, dS = 0, nothing to compare dQ with)
     return dict(B=B, Lq=Lq, Lk=Lk, H=H, Hk=Hk, hm=hm, hb=hb, W=W, causal=rng.random() < 0.7,
                 dtype=rng.choice([torch.bfloat16, torch.bfloat16, torch.float16]), qscale=rng.choice([1.0, 1.0, 2.5]))
 
