@@ -902,33 +902,6 @@ size_t compact_bytes(const FwdParams &p, bool backward, bool reuse_fwd) {
     return backward && reuse_fwd ? l.total - (l.img ? l.off_bk : l.off_plan) : l.total;
 }
 
-void dkdv_split_bounds(int pairs, int n_max, int G, int &grid, int &slots) {
-    const int k = dkdv_lists_per_pair(pairs);
-    const int lists_per_xcd = pairs * k / 8;
-    // n = units of the largest pair; the total U is then between n and pairs * n, and the split factor does
-    // not grow with U: the split of U = n bounds the workgroups, U * split(U) bounds the partial slots
-    int64_t items = 1, sl = 1;
-    for (int n = 1; n <= n_max; n++) {
-        int Gs, Sm;
-        dkdv_split(n, G, Gs, Sm);
-        const int64_t it = (int64_t)dkdv_list_len(n, k) * Gs * Sm;
-        if (it > items) items = it;
-        if (n >= DKDV_ENOUGH_UNITS) {  // no split from here on: the bound grows with n alone
-            const int64_t last = dkdv_list_len(n_max, k);
-            if (last > items) items = last;
-            break;
-        }
-    }
-    const int U_max = pairs * n_max < DKDV_ENOUGH_UNITS ? pairs * n_max : DKDV_ENOUGH_UNITS - 1;
-    for (int U = 1; U <= U_max; U++) {
-        int Gs, Sm;
-        dkdv_split(U, G, Gs, Sm);
-        if (Gs * Sm > 1 && (int64_t)U * Gs * Sm > sl) sl = (int64_t)U * Gs * Sm;
-    }
-    grid = (int)(8 * lists_per_xcd * items);
-    slots = (int)sl;
-}
-
 // compute units of the current device (cached per device)
 static int device_cus() {
     static std::atomic<int> cus[16];

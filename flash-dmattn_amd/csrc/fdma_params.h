@@ -303,7 +303,32 @@ hipError_t compact_setup(FwdParams &p, void *ws, int dtype, hipStream_t stream, 
                          const void *fwd_ws = nullptr);
 // host-side bounds over every possible unit count 1..U_max: workgroups to launch, partial slots to hold
 // (n_max = units of one pair at most)
-void dkdv_split_bounds(int pairs, int n_max, int G, int &grid, int &slots);
+inline void dkdv_split_bounds(int pairs, int n_max, int G, int &grid, int &slots) {
+    const int k = dkdv_lists_per_pair(pairs);
+    const int lists_per_xcd = pairs * k / 8;
+    // n = units of the largest pair; the total U is then between n and pairs * n, and the split factor does
+    // not grow with U: the split of U = n bounds the workgroups, U * split(U) bounds the partial slots
+    int64_t items = 1, sl = 1;
+    for (int n = 1; n <= n_max; n++) {
+        int Gs, Sm;
+        dkdv_split(n, G, Gs, Sm);
+        const int64_t it = (int64_t)dkdv_list_len(n, k) * Gs * Sm;
+        if (it > items) items = it;
+        if (n >= DKDV_ENOUGH_UNITS) {  // no split from here on: the bound grows with n alone
+            const int64_t last = dkdv_list_len(n_max, k);
+            if (last > items) items = last;
+            break;
+        }
+    }
+    const int U_max = pairs * n_max < DKDV_ENOUGH_UNITS ? pairs * n_max : DKDV_ENOUGH_UNITS - 1;
+    for (int U = 1; U <= U_max; U++) {
+        int Gs, Sm;
+        dkdv_split(U, G, Gs, Sm);
+        if (Gs * Sm > 1 && (int64_t)U * Gs * Sm > sl) sl = (int64_t)U * Gs * Sm;
+    }
+    grid = (int)(8 * lists_per_xcd * items);
+    slots = (int)sl;
+}
 
 // number of KV splits the decode path uses for this shape (1 = no workspace needed)
 int decode_num_splits(int B, int Hk, int Lk);
