@@ -314,11 +314,20 @@ def run_hbm_probe():
         return None
     lib.fdma_probe_read_gbs.restype = ctypes.c_double
     lib.fdma_probe_read_gbs.argtypes = [ctypes.c_int64, ctypes.c_int, ctypes.c_int]
-    return {"unit": "GB/s", "row_bytes": 256,
-            "stream_1GiB": lib.fdma_probe_read_gbs(1 << 22, 0, 1024),
-            "scattered_rows_1GiB": lib.fdma_probe_read_gbs(1 << 22, 1, 2048),
-            "scattered_rows_cfg5_volume_67MB": lib.fdma_probe_read_gbs(2 * 131072, 1, 2048),
-            "note": "read-only kernels, best of five launches each; scattered = hashed row positions in a 2 GiB buffer"}
+    out = {"unit": "GB/s", "row_bytes": 256,
+           "stream_1GiB": lib.fdma_probe_read_gbs(1 << 22, 0, 1024),
+           "scattered_rows_1GiB": lib.fdma_probe_read_gbs(1 << 22, 1, 2048),
+           "scattered_rows_cfg5_volume_67MB": lib.fdma_probe_read_gbs(2 * 131072, 1, 2048),
+           "note": "read-only kernels, best of five launches each; scattered = hashed row positions in a 2 GiB buffer"}
+    if hasattr(lib, "fdma_probe_tile_walk_gbs"):
+        # cfg3's access pattern alone: 128-row workgroups walking a [4096, 4096] bias and mask 64 columns at a time, at the
+        # general forward kernel's occupancy and depth (two workgroups of four waves per CU, one step in flight)
+        lib.fdma_probe_tile_walk_gbs.restype = ctypes.c_double
+        lib.fdma_probe_tile_walk_gbs.argtypes = [ctypes.c_int, ctypes.c_int, ctypes.c_int]
+        out["tile_walk_mask_and_bias_cfg3_pattern"] = lib.fdma_probe_tile_walk_gbs(1, 1, 64)
+        out["tile_walk_mask_and_bias_4_workgroups_per_cu"] = lib.fdma_probe_tile_walk_gbs(1, 1, 0)
+        out["tile_walk_bias_only"] = lib.fdma_probe_tile_walk_gbs(0, 1, 64)
+    return out
 
 
 def config_roofline(name, r):

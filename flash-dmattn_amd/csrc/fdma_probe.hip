@@ -193,3 +193,86 @@ extern "C" double fdma_probe_read_rows_gbs(int64_t rows, int row_bytes, int scat
     (void)hipFree(buf);
     return hipGetLastError() == hipSuccess ? best_gbs : -1.0;
 }
+
+// ---- the walk of the general forward kernel over a per-query bias (2 bytes) and mask (1 byte), without the kernel: 32
+// matrices of 4096 x 4096 (cfg3's shapes); a workgroup of four waves owns 128 rows of one matrix and reads 64 columns
+// per step -- 128 pieces of 128 bytes at a pitch of 8 KB and 128 pieces of 64 bytes at a pitch of 4 KB, eight rows per
+// load instruction --, the next step's loads in flight while it waits for this step's, one barrier per step; with two
+// workgroups per CU that is the kernel's own occupancy and depth.  What this reaches is what the access pattern leaves of the
+// HBM rate at that occupancy; the kernel's own rate is to be read against it.
+namespace {
+
+template <bool MASK, bool BIAS>
+__global__ void __launch_bounds__(256, 2) tile_walk_kernel(const char *bias, const char *mask, uint32_t steps, uint32_t *out) {
+    const uint32_t tid = threadIdx.x, fc = tid % 8, fr0 = tid / 8;
+    const uint32_t mat = blockIdx.x % 32, mblk = (blockIdx.x / 32) % 32;
+    const char *bb = bias + (size_t)mat * (4096u * 8192u) + (size_t)(mblk * 128 + fr0) * 8192 + fc * 16;
+    const char *mb = mask + (size_t)mat * (4096u * 4096u) + (size_t)(mblk * 128 + fr0) * 4096 + fc * 8;
+    u32x4 acc = {0, 0, 0, 0};
+    u32x4 b0[4], b1[4];
+    uint2 m0[4], m1[4];
+    auto ld = [&](uint32_t st, u32x4 (&b)[4], uint2 (&m)[4]) {
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+            if (MASK) m[it] = *(const uint2 *)(mb + (size_t)it * 32 * 4096 + st * 64);
+            if (BIAS) b[it] = *(const u32x4 *)(bb + (size_t)it * 32 * 8192 + st * 128);
+        }
+    };
+    auto use = [&](u32x4 (&b)[4], uint2 (&m)[4]) {
+#pragma unroll
+        for (int it = 0; it < 4; it++) {
+            if (BIAS) acc ^= b[it];
+            if (MASK) { acc[0] ^= m[it].x; acc[1] ^= m[it].y; }
+        }
+    };
+    ld(0, b0, m0);
+    for (uint32_t st = 0; st < steps; st += 2) {  // (steps is even and at most 62: step `steps` still lies inside the row)
+        ld(st + 1, b1, m1);
+        use(b0, m0);
+        __builtin_amdgcn_s_barrier();
+        ld(st + 2, b0, m0);
+        use(b1, m1);
+        __builtin_amdgcn_s_barrier();
+    }
+    use(b0, m0);
+    if ((acc[0] ^ acc[1] ^ acc[2] ^ acc[3]) == 0x12345678u) out[blockIdx.x] = acc[0];  // (keeps the loads alive)
+}
+
+}  // namespace
+
+// GB/s of that walk: 1024 workgroups x 32 steps (0.8 GB with mask and bias), best of four timed launches (< 0 on error).
+// `lds_kb`: LDS per workgroup, which sets how many a CU holds (64: two, as the forward kernel; 0: as many as the launch has, four)
+extern "C" double fdma_probe_tile_walk_gbs(int with_mask, int with_bias, int lds_kb) {
+    if ((!with_mask && !with_bias) || lds_kb > 64) return -1.0;
+    void *bias = nullptr, *mask = nullptr;
+    uint32_t *d_out = nullptr;
+    if (hipMalloc(&bias, (size_t)32 * 4096 * 8192) != hipSuccess) return -1.0;
+    if (hipMalloc(&mask, (size_t)32 * 4096 * 4096) != hipSuccess) { (void)hipFree(bias); return -1.0; }
+    if (hipMalloc((void **)&d_out, 1024 * sizeof(uint32_t)) != hipSuccess) { (void)hipFree(bias); (void)hipFree(mask); return -1.0; }
+    (void)hipMemset(bias, 0x5a, (size_t)32 * 4096 * 8192);
+    (void)hipMemset(mask, 0x01, (size_t)32 * 4096 * 4096);
+    hipEvent_t e0, e1;
+    (void)hipEventCreate(&e0);
+    (void)hipEventCreate(&e1);
+    const uint32_t steps = 32;
+    const size_t lds = lds_kb > 0 ? (size_t)lds_kb << 10 : 0;  // (dynamic LDS nobody touches: it only limits the workgroups a CU holds)
+    float best = 1e30f;
+    for (int rep = 0; rep < 6; rep++) {
+        (void)hipEventRecord(e0, 0);
+        if (with_mask && with_bias) hipLaunchKernelGGL((tile_walk_kernel<true, true>), dim3(1024), dim3(256), lds, 0, (const char *)bias, (const char *)mask, steps, d_out);
+        else if (with_bias) hipLaunchKernelGGL((tile_walk_kernel<false, true>), dim3(1024), dim3(256), lds, 0, (const char *)bias, (const char *)mask, steps, d_out);
+        else hipLaunchKernelGGL((tile_walk_kernel<true, false>), dim3(1024), dim3(256), lds, 0, (const char *)bias, (const char *)mask, steps, d_out);
+        (void)hipEventRecord(e1, 0);
+        (void)hipEventSynchronize(e1);
+        float ms = 0.f;
+        (void)hipEventElapsedTime(&ms, e0, e1);
+        if (rep >= 2 && ms < best) best = ms;
+    }
+    (void)hipEventDestroy(e0);
+    (void)hipEventDestroy(e1);
+    (void)hipFree(d_out);
+    (void)hipFree(mask);
+    (void)hipFree(bias);
+    const double bytes = 1024.0 * steps * 128 * ((with_bias ? 128 : 0) + (with_mask ? 64 : 0));
+    return hipGetLastError() == hipSuccess && best < 1e29f ? bytes / (best * 1e-3) / 1e9 : -1.0;
+}
