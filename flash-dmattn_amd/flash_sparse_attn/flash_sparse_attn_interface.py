@@ -316,27 +316,33 @@ def _backward_per_query_head(dout, q, k, v, mask, bias, out, softmax_lse, dq, dk
     batch, seqlen_q, num_heads, _ = q.shape
     softmax_d = torch.empty((batch, num_heads, round_multiple(seqlen_q, 128)), device=q.device, dtype=torch.float32)
     bias_per_head = bias is not None and bias.shape[1] == num_heads
-    dk_t = dv_t = dbias_t = None
+    # The members' dK, dV (and shared dBias) are summed in fp32 and rounded once, as the reference sums its per-head
+    # dK / dV over a group (flash_api.cpp:1027-1047); summed in the 16-bit type they would be rounded G times.
+    dk_t, dv_t = torch.empty_like(dk), torch.empty_like(dv)
+    dk_sum = torch.zeros(dk.shape, device=dk.device, dtype=torch.float32)
+    dv_sum = torch.zeros(dv.shape, device=dv.device, dtype=torch.float32)
+    dbias_t = dbias_sum = None
+    if bias is not None and not bias_per_head:
+        dbias_t = torch.empty_like(dbias)
+        dbias_sum = torch.zeros(dbias.shape, device=dbias.device, dtype=torch.float32)
     with _handoff():  # (lists, bit rows and forward workspaces belong to the whole call, not to a member)
         for g in range(G):
             member = slice(g, None, G)
-            first = g == 0
-            if not first and dk_t is None:
-                dk_t, dv_t = torch.empty_like(dk), torch.empty_like(dv)
-                if bias is not None and not bias_per_head:
-                    dbias_t = torch.empty_like(dbias)
             bias_g = bias[:, member] if bias_per_head else bias
-            dbias_g = None if bias is None else (dbias[:, member] if bias_per_head else (dbias if first else dbias_t))
+            dbias_g = None if bias is None else (dbias[:, member] if bias_per_head else dbias_t)
             d = _flash_sparse_attn_backward_body(
                 dout[:, :, member], q[:, :, member], k, v, mask[:, member], bias_g, out[:, :, member],
-                softmax_lse[:, member], dq[:, :, member], dk if first else dk_t, dv if first else dv_t, dbias_g,
+                softmax_lse[:, member], dq[:, :, member], dk_t, dv_t, dbias_g,
                 softmax_scale, is_causal, softcap, deterministic)
             softmax_d[:, member] = d
-            if not first:
-                dk.add_(dk_t)
-                dv.add_(dv_t)
-                if dbias_t is not None:
-                    dbias.add_(dbias_t)
+            dk_sum.add_(dk_t)
+            dv_sum.add_(dv_t)
+            if dbias_sum is not None:
+                dbias_sum.add_(dbias_t)
+    dk.copy_(dk_sum)
+    dv.copy_(dv_sum)
+    if dbias_sum is not None:
+        dbias.copy_(dbias_sum)
     return softmax_d
 
 

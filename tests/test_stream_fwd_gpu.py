@@ -66,6 +66,9 @@ CASES = {
     "mask_per_query_head_bias_per_kv_head": (1, 600, 600, 8, 2, 8, 2, 150, True, torch.bfloat16),
     "mask_per_query_head_bias_per_query_head": (2, 300, 500, 4, 2, 4, 4, 100, True, torch.bfloat16),
     "mask_per_query_head_shared_bias_noncausal": (1, 512, 512, 6, 3, 6, 1, 99, False, torch.bfloat16),
+    # ... many rows over few keys and one bias row for sixteen heads: four members whose dK / dV / dBias are summed
+    # (in fp32, rounded once), with sums of thousands of terms per dBias element
+    "mask_per_query_head_shared_bias_many_rows_few_keys": (2, 549, 33, 16, 4, 16, 1, 8, True, torch.bfloat16),
 }
 
 
