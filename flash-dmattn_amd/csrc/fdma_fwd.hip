@@ -10,7 +10,8 @@
 // One workgroup = 4 waves = 128 query rows of one (batch, head); each wave owns 32 rows and computes the
 // TRANSPOSED score tile S^T = K Q^T (K rows from LDS as the MFMA A operand, its pre-scaled Q rows in
 // registers as the B operand), so a lane owns one query row and row max / row sum are in-lane reductions
-// plus one cross-half swap.  P^T feeds O^T = V^T P^T straight from the accumulator registers.
+// plus one cross-half swap.  P^T feeds O^T = V^T P^T straight from the accumulator registers; V^T comes out of the
+// row-major V tile through transposing LDS reads.
 //
 // With a [Lq, Lk] bias (2 B) and mask (1 B) per score this path is bound by HBM, not by the matrix pipe, so the
 // kernel is built around the mask / bias stream:
@@ -33,14 +34,12 @@ namespace {
 // in-order issue of that wave -- a second wave per SIMD does.
 constexpr int BN_DEFAULT = 64;  // keys per tile (32 at head dims above 128: LDS)
 
-template <int D, int BN, int NT> struct KQ_OK { static constexpr bool value = (BN / 4) * (D / 8) <= NT; };
-
 template <int D, int BM, int BN> struct FwdSmem {
     static constexpr int SK = D + 8;     // K tile row stride (elements): conflict-free 16-byte row reads
-    static constexpr int SVT = BN + 8;   // V^T tile row stride
+    static constexpr int SV = LdsTile<D>::S;  // V tile row stride (row-major like K, read through transposing LDS reads)
     static constexpr int SF = BN + 8;    // fused mask+bias tile row stride
     static constexpr int K_BYTES = BN * SK * 2;
-    static constexpr int VT_BYTES = D * SVT * 2;
+    static constexpr int VT_BYTES = BN * SV * 2;
     static constexpr int F_BYTES = BM * SF * 2;
     static constexpr int STAGE = K_BYTES + VT_BYTES + F_BYTES;
     static constexpr int TOTAL = 2 * STAGE;
@@ -57,14 +56,12 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) fwd_ker
     constexpr int F_RPP = NTHREADS / FCH;   // mask / bias rows staged per pass (FCH threads cover the keys of a row)
     using E = Elem<T>;
     using SM = FwdSmem<D, BM, BN>;
-    static_assert(KQ_OK<D, BN, 64 * NW>::value, "a V tile is one (key quad, d chunk) item per thread at most");
     constexpr int KS = D / 16;  // contraction steps of Q K^T
     constexpr int DB = D / 32;  // 32-wide blocks of the head dimension
-    constexpr int MB = BN / 32, KB = BN / 16, KQ = BN / 4;
+    constexpr int MB = BN / 32, KB = BN / 16;
     constexpr int CH = D / 8;               // 16-byte chunks per K row
     constexpr int K_RPP = NTHREADS / CH;    // K rows staged per pass
     constexpr int K_IT = BN / K_RPP;
-    constexpr int V_ITEMS = KQ * CH;        // (key quad, d chunk) items of a V tile
     constexpr int F_IT = BM * (BN / 8) / NTHREADS;  // 8-key chunks of the mask / bias tile per thread (4)
 
     extern __shared__ __attribute__((aligned(16))) char smem[];
@@ -124,17 +121,16 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) fwd_ker
 
     // ---- staging maps
     const int kc = tid % CH, kr0 = tid / CH;             // K: d chunk, first row
-    const int vkg = tid % KQ, vc = (tid / KQ) % CH;      // V: key quad, d chunk
-    const bool k_dvalid = kc * 8 < p.d, v_dvalid = vc * 8 < p.d;
+    const bool k_dvalid = kc * 8 < p.d;
     const int fc = tid % FCH, fr0 = tid / FCH;           // mask / bias: 8-key chunk, first row (rows fr0 + F_RPP it)
-    u32x4_t kreg[K_IT], vreg[4], breg[F_IT];
+    u32x4_t kreg[K_IT], vreg[K_IT], breg[F_IT];
     u32x2_t mreg[F_IT], mnext[F_IT];
 
     // All tile loads are unconditional, from clamped (always valid) addresses, so that they can be issued early and
     // stay in flight; what a clamped load fetched in place of a missing element is neutralised later: the mask
     // words are ANDed with a validity pattern when they are consumed, rows of K / V beyond Lk and head-dim chunks
     // beyond d are finite duplicates that meet a -inf score or a zero Q fragment.
-    const int kcol = k_dvalid ? kc * 8 : 0, vcol = v_dvalid ? vc * 8 : 0;
+    const int kcol = k_dvalid ? kc * 8 : 0;
     // (a mask that comes packed to bits: one byte per 8-key chunk instead of eight, expanded where it is looked at)
     const uint8_t *mbits = (mbase && p.mbits) ? p.mbits + b * p.mb_b + hm * p.mb_h : nullptr;
     auto load_mask = [&](int j, u32x2_t (&dst)[F_IT]) {
@@ -195,38 +191,24 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) fwd_ker
             int key = n0 + kr0 + it * K_RPP;
             key = key < p.Lk ? key : p.Lk - 1;
             kreg[it] = *(const u32x4_t *)(kbase + (int64_t)key * p.k_r + kcol);
-        }
-        if (tid < V_ITEMS) {
-#pragma unroll
-            for (int i = 0; i < 4; i++) {
-                int key = n0 + 4 * vkg + i;
-                key = key < p.Lk ? key : p.Lk - 1;
-                vreg[i] = *(const u32x4_t *)(vbase + (int64_t)key * p.v_r + vcol);
-            }
+            // (V rows the same way: a wave's load covers whole rows -- one cache line per row at head dim 64 -- where a
+            // (key quad, d chunk) item per thread, as a transposition in registers wants it, touched every line twice)
+            vreg[it] = *(const u32x4_t *)(vbase + (int64_t)key * p.v_r + kcol);
         }
     };
     auto load_rest = [&](int j) {
         load_bias(j, breg);
         load_kv(j);
     };
-    // registers -> LDS stage `buf`: K rows, V transposed, mask and bias fused (bias where kept, -inf elsewhere)
+    // registers -> LDS stage `buf`: K and V rows, mask and bias fused (bias where kept, -inf elsewhere)
     auto store_stage = [&](int buf, const u32x2_t (&mv)[F_IT], const u32x4_t (&bsrc)[F_IT]) {
         char *sK = smem + buf * SM::STAGE;
         char *sVt = sK + SM::K_BYTES;
         char *sF = sVt + SM::VT_BYTES;
 #pragma unroll
-        for (int it = 0; it < K_IT; it++)
+        for (int it = 0; it < K_IT; it++) {
             *(u32x4_t *)(sK + ((kr0 + it * K_RPP) * SM::SK + kc * 8) * 2) = kreg[it];
-        if (tid < V_ITEMS) {
-#pragma unroll
-            for (int dd = 0; dd < 8; dd++) {
-                const int w = dd >> 1;
-                const uint32_t sel = (dd & 1) ? 0x07060302u : 0x05040100u;
-                u32x2_t out;
-                out[0] = __builtin_amdgcn_perm(vreg[1][w], vreg[0][w], sel);
-                out[1] = __builtin_amdgcn_perm(vreg[3][w], vreg[2][w], sel);
-                *(u32x2_t *)(sVt + ((vc * 8 + dd) * SM::SVT + 4 * vkg) * 2) = out;
-            }
+            *(u32x4_t *)(sVt + LdsTile<D>::chunk(kr0 + it * K_RPP, kc)) = vreg[it];
         }
 #pragma unroll
         for (int it = 0; it < F_IT; it++) {
@@ -246,6 +228,8 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) fwd_ker
     };
 
     const int a_row = pi_row(r);
+    // (this lane's part of the address of a transposing read of the V tile)
+    const uint32_t tr_lane = LdsTile<D>::tr_base(g, (lane & 15) >> 2, (lane >> 4) & 1, (lane & 3) == 1 ? 2 : ((lane & 3) == 2 ? 1 : (lane & 3)));
 
     // ---- one tile from LDS stage `buf`
     auto compute = [&](int j, int buf) {
@@ -326,11 +310,14 @@ __global__ void __launch_bounds__(64 * NW, (D <= 64 && NW == 4) ? 2 : 1) fwd_ker
             }
         row_sum += psum;
         {
+            // V^T (rows of the A operand = head dim) through transposing reads of the row-major V tile
             constexpr int NF = KB * DB, FR = NF < 8 ? NF : 8;
             u32x4_t a[NF];
+            const uint32_t tr_v = lds_addr(sVt) + tr_lane;
             auto frag = [&](int f) {
                 const int kb = f / DB, db = f % DB;
-                return *(const u32x4_t *)(sVt + ((32 * db + a_row) * SM::SVT + 16 * kb + 8 * g) * 2);
+                const u32x2_t lo = lds_ld_tr16(LdsTile<D>::tr_at(tr_v, kb, db, 0)), hi = lds_ld_tr16(LdsTile<D>::tr_at(tr_v, kb, db, 1));
+                return u32x4_t{lo[0], lo[1], hi[0], hi[1]};
             };
 #pragma unroll
             for (int f = 0; f < FR; f++) a[f] = frag(f);
