@@ -364,7 +364,7 @@ def config_roofline(name, r):
             tot = fwd + bwd
             blk["fwd_bwd"] = {"bytes_per_call": tot, "duration_ms": r["ms_fwd_bwd"], "achieved": tot / r["ms_fwd_bwd"] / 1e6,
                               "frac": tot / r["ms_fwd_bwd"] / 1e6 / PEAK_HBM_GBS,
-                              "kernels": "fwd_kernel, bwd_dot_kernel, bwd_dkdv_kernel, bwd_dq_kernel"}
+                              "kernels": "fwd_kernel, bwd_dot_kernel, bwd_dkdv_kernel, bwd_dq_ds_kernel (dQ from the dS tiles that dK/dV wrote as dBias)"}
         return blk
     flops = 4.0 * 64 * 64 * c["D"] * r["n_exec"]
     blk = {"bound": "mfma", "unit": "TFLOP/s", "peak": PEAK_BF16_TFLOPS, "flops_per_call": flops,
